@@ -1,0 +1,183 @@
+/*
+ * ptoamd — C ABI of the MI355X (gfx950) backend for the PTO tile-matmul hot path.
+ *
+ * Everything below is `extern "C"`, plain pointers and sizes.  Device pointers are ordinary HIP device
+ * addresses (from ptoamd_malloc, hipMalloc or a framework allocator); `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  Every function returns 0 on success and a negative PTOAMD_E_* code on
+ * failure; ptoamd_last_error() gives the text.  Launches are asynchronous on `stream`.
+ *
+ * Two groups of entry points:
+ *   1. the host runtime the reference's tests and demos reach through `aclrt*`
+ *      (reference: include/pto/common/cpu_stub.hpp:73-120, 524-555);
+ *   2. whole-kernel launchers, the counterpart of the reference's per-kernel
+ *      `Launch...(uint8_t* out, uint8_t* src..., void* stream)` host functions
+ *      (reference: tests/cpu/st/testcase/tmatmul/tmatmul_kernel.cpp:175-203,
+ *       kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:360-380),
+ *      each of which runs one TLOAD -> TMATMUL/TMATMUL_ACC -> TSTORE pipeline (or one TQUANT / TDEQUANT pass)
+ *      over whole matrices in HBM.
+ */
+#ifndef PTOAMD_H
+#define PTOAMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes ---------------------------------------------------------------------------------------- */
+#define PTOAMD_OK 0
+#define PTOAMD_E_INVALID (-1)     /* bad argument (null pointer, non-positive size, unknown enum) */
+#define PTOAMD_E_UNSUPPORTED (-2) /* combination the backend has no kernel for */
+#define PTOAMD_E_ALIGNMENT (-3)   /* pointer / leading dimension not aligned as the kernel needs */
+#define PTOAMD_E_HIP (-4)         /* a HIP runtime call failed */
+#define PTOAMD_E_NODEVICE (-5)    /* no gfx950 device */
+
+/* ---- enums ---------------------------------------------------------------------------------------------- */
+/* element types of GEMM operands / results */
+enum {
+    PTOAMD_F32 = 0,
+    PTOAMD_F16 = 1,
+    PTOAMD_BF16 = 2,
+    PTOAMD_I32 = 3,
+    PTOAMD_I8 = 4,
+    PTOAMD_U8 = 5,
+    PTOAMD_E4M3 = 6, /* float8_e4m3_t (OCP E4M3FN)        reference: include/pto/cpu/MXTypes.hpp:344 */
+    PTOAMD_E5M2 = 7, /* float8_e5m2_t                      reference: MXTypes.hpp:345 */
+    PTOAMD_E2M1 = 8, /* float4_e2m1x2_t, two per byte, even element in the low nibble   MXTypes.hpp:341,350-372 */
+    PTOAMD_E1M2 = 9, /* float4_e1m2x2_t                    MXTypes.hpp:342 */
+    PTOAMD_I16 = 10
+};
+
+/* memory layout of the B operand ([K, N] logical) — reference Layout::ND / Layout::DN (common/type.hpp:163-165) */
+enum {
+    PTOAMD_B_ND = 0, /* row-major [K][N], element (k, n) at b[k * ldb + n] */
+    PTOAMD_B_DN = 1  /* column-major, i.e. [N][K] in memory, element (k, n) at b[n * ldb + k] */
+};
+
+/* GM layouts of E8M0 block scales — reference Layout::MX_* (common/type.hpp:167-172, cpu/tile_offsets.hpp:233-268) */
+enum {
+    PTOAMD_MX_A_ZZ = 0,
+    PTOAMD_MX_A_ND = 1, /* [M][K/32] */
+    PTOAMD_MX_A_DN = 2,
+    PTOAMD_MX_B_NN = 3,
+    PTOAMD_MX_B_ND = 4, /* [K/64][N][2] */
+    PTOAMD_MX_B_DN = 5  /* [N][K/32] */
+};
+
+/* TQUANT algorithms — reference MxQuantAlg (common/type.hpp:213-219) */
+enum { PTOAMD_OCP_MXFP8 = 0, PTOAMD_NV_MXFP8 = 1, PTOAMD_OCP_MXFP4 = 2, PTOAMD_NV_MXFP4 = 3 };
+
+/* aclrtMemcpy kinds (cpu_stub.hpp) */
+enum { PTOAMD_MEMCPY_H2H = 0, PTOAMD_MEMCPY_H2D = 1, PTOAMD_MEMCPY_D2H = 2, PTOAMD_MEMCPY_D2D = 3 };
+
+/* =========================================================================================================
+ * 1. Host runtime  (replaces the fake aclrt* runtime, include/pto/common/cpu_stub.hpp:73-120, 524-555)
+ * ========================================================================================================= */
+int ptoamd_init(int device);                    /* aclInit + aclrtSetDevice: selects the device, checks it is gfx950 */
+int ptoamd_finalize(void);                      /* aclrtResetDevice + aclFinalize */
+const char* ptoamd_last_error(void);            /* text of the calling thread's last failure */
+int ptoamd_device_info(int* compute_units, int* clock_khz, size_t* hbm_bytes, char* arch, size_t arch_len);
+
+int ptoamd_malloc(void** dev_ptr, size_t bytes);      /* aclrtMalloc */
+int ptoamd_free(void* dev_ptr);                       /* aclrtFree */
+int ptoamd_malloc_host(void** host_ptr, size_t bytes); /* aclrtMallocHost (pinned) */
+int ptoamd_free_host(void* host_ptr);                 /* aclrtFreeHost */
+int ptoamd_memcpy(void* dst, size_t dst_bytes, const void* src, size_t count, int kind); /* aclrtMemcpy (blocking) */
+int ptoamd_memcpy_async(void* dst, size_t dst_bytes, const void* src, size_t count, int kind, void* stream);
+int ptoamd_memset(void* dev_ptr, size_t dst_bytes, int value, size_t count);             /* aclrtMemset */
+
+int ptoamd_stream_create(void** stream);        /* aclrtCreateStream (default priority) */
+int ptoamd_stream_destroy(void* stream);        /* aclrtDestroyStream */
+int ptoamd_stream_synchronize(void* stream);    /* aclrtSynchronizeStream */
+
+/* HIP events on a stream, for timing a launch region */
+int ptoamd_event_create(void** event);
+int ptoamd_event_destroy(void* event);
+int ptoamd_event_record(void* event, void* stream);
+int ptoamd_event_synchronize(void* event);
+int ptoamd_event_elapsed_ms(float* ms, void* start, void* stop);
+
+/* =========================================================================================================
+ * 2. Kernel launchers
+ * ========================================================================================================= */
+
+/*
+ * C[M, N] = A[M, K] * B[K, N] (+ Cin) : the TLOAD -> TMATMUL / TMATMUL_ACC -> TSTORE pipeline.
+ * reference: include/pto/cpu/TMatmul.hpp:77-113, 207-217 (arithmetic), cpu/TLoad.hpp:287-321, cpu/TStore.hpp:41-79.
+ *   ab_type : PTOAMD_F16 | PTOAMD_BF16 | PTOAMD_F32 | PTOAMD_I8 | PTOAMD_E4M3 | PTOAMD_E5M2  (A and B alike)
+ *   c_type  : PTOAMD_F32 | PTOAMD_F16 | PTOAMD_BF16 for float inputs (TSTORE's static_cast, round to nearest even);
+ *             PTOAMD_I32 for int8 (raw accumulators, bit-exact)
+ *   a       : row-major, leading dimension lda (elements)
+ *   b       : b_layout PTOAMD_B_ND ([K][N], ldb >= N) or PTOAMD_B_DN ([N][K], ldb >= K)
+ *   c_in    : optional accumulator input (TMATMUL_ACC), same type as the accumulator (f32 / i32), ld = ldc; may be NULL
+ *   relu    : TSTORE's ReluPreMode::NormalRelu
+ */
+int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, int m, int n, int k,
+                int lda, int ldb, int ldc, int b_layout, int relu, void* stream);
+
+/*
+ * W8A8: int8 x int8 -> int32 accumulate, then the dequantising drain fused in registers:
+ *   out(i, j) = bf16( (float(acc(i, j)) * scale_a[i]) * scale_b[j] )
+ * i.e. TMATMUL (cpu/TMatmul.hpp:106) -> TDEQUANT with offset 0 (cpu/TDeQuant.hpp:31-34) -> per-column multiply
+ * (cpu/TColExpandOp.hpp:57-63) -> TCVT f32->bf16 RINT.  acc_out (optional, may be NULL) receives the raw int32
+ * accumulators so parity can be checked bit for bit.
+ */
+int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const int8_t* b, const float* scale_a,
+                     const float* scale_b, int m, int n, int k, int lda, int ldb, int ldc, int b_layout, void* stream);
+
+/*
+ * Block-scaled matmul, TMATMUL_MX (cpu/TMatmul.hpp:169-205, 254-292):
+ *   C(i, j) = sum_k A(i, k) * B(k, j) * 2^(sa(i, k/32) - 127) * 2^(sb(k/32, j) - 127)   (+ Cin)
+ *   a_type / b_type : both fp8 (PTOAMD_E4M3 | PTOAMD_E5M2) or both fp4 (PTOAMD_E2M1 | PTOAMD_E1M2; E1M2 runs on
+ *                     the order-exact generic kernel only)
+ *   a  : [M][K] codes row-major (fp4: K/2 bytes per row);  b : PTOAMD_B_DN ([N][K]) or PTOAMD_B_ND ([K][N])
+ *   sa : E8M0 bytes in sa_layout (PTOAMD_MX_A_*), logical [M][K/32];  sb : sb_layout (PTOAMD_MX_B_*), [K/32][N]
+ *   c_type : PTOAMD_F32 | PTOAMD_BF16 | PTOAMD_F16
+ * lda / ldb are in elements.  K must be a multiple of 64 (CheckMadMxValid, TMatmul.hpp:121-142).
+ */
+int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
+                   const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n, int k, int lda,
+                   int ldb, int ldc, int b_layout, void* stream);
+
+/*
+ * Decode-shaped weight-only MXFP4 GEMV/GEMM (m <= 16):
+ *   out(i, j) = sum_k bf16 A(i, k) * ( e2m1 W(j, k) * 2^(sw(j, k/32) - 127) )      fp32 accumulate
+ * The dequantised weight is exact in bf16, so this is TMATMUL on bf16 operands (cpu/TMatmul.hpp:77-113) fed by the
+ * MX decode of cpu/MXTypes.hpp:232-274, with the dequantisation done in registers.
+ *   a : bf16 [m][k] (lda elements);  w : packed e2m1 [n][k/2] bytes (ldw elements);  sw : E8M0 [n][k/32]
+ *   c_type : PTOAMD_F32 | PTOAMD_BF16
+ */
+int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, const uint8_t* w, const uint8_t* sw, int m, int n,
+                      int k, int lda, int ldw, int ldc, void* stream);
+
+/* TQUANT<INT8_SYM / INT8_ASYM> (cpu/TQuant.hpp:496-522): dst = clamp(nearbyint(src * scale[row] (+ offset[row]))).
+ * offset == NULL selects the symmetric form (int8 output); otherwise the output is uint8.  src is [rows][cols] f32. */
+int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const float* offset, int rows, int cols,
+                       void* stream);
+
+/* TQUANT<MXFP8 | MXFP4_E2M1> (cpu/TQuant.hpp:461-493, 524-547).  src [rows][cols] of src_type (F32 | F16 | BF16);
+ * axis 1 groups 32 elements along a row (exp / max / scaling are [rows][cols/32]), axis 0 along a column
+ * ([rows/32][cols]).  dst: one byte per element (fp8) or packed nibbles (fp4).  max / scaling may be NULL. */
+int ptoamd_tquant_mx(uint8_t* dst, uint8_t* exp, float* max, float* scaling, const void* src, int src_type, int rows,
+                     int cols, int alg, int axis, void* stream);
+
+/* TDEQUANT (cpu/TDeQuant.hpp:18-37): dst(r, c) = (float(src(r, c)) - offset[r]) * scale[r];
+ * src_type PTOAMD_I8 | PTOAMD_I16 | PTOAMD_I32. */
+int ptoamd_tdequant(float* dst, const void* src, int src_type, const float* scale, const float* offset, int rows,
+                    int cols, void* stream);
+
+/* Copies an E8M0 scale matrix between GM layouts (the TLOAD + TMOV of a scale tile, cpu/tile_offsets.hpp:233-268):
+ * rows x cols is the logical extent ([M][K/32] for the A side, [K/32][N] for the B side). */
+int ptoamd_mx_scale_relayout(uint8_t* dst, int dst_layout, const uint8_t* src, int src_layout, int rows, int cols,
+                             void* stream);
+
+/* Names the kernel the last ptoamd_gemm* / ptoamd_gemv* call on this thread dispatched to ("tile256x256_bf16", ...,
+ * "generic"): lets tests assert that the MFMA path, not the order-exact generic kernel, produced a result. */
+const char* ptoamd_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PTOAMD_H */

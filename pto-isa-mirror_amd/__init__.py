@@ -1,0 +1,166 @@
+"""Python host side of the MI355X (gfx950) backend for the PTO tile-matmul hot path.
+
+Thin ctypes binding of the C ABI in ``include/ptoamd.h`` (``lib/libptoamd.so``).  PyTorch is used for device memory
+and streams only; every operator below hands raw device pointers and sizes to the library, which runs hand-written
+HIP kernels.  There is no CPU or PyTorch fallback: if the library is missing, importing this package raises.
+
+Operator names and argument meaning mirror the reference's tile instructions for this path
+(``TMATMUL`` / ``TMATMUL_ACC`` / ``TMATMUL_MX`` / ``TQUANT`` / ``TDEQUANT``, reference ``include/pto/common/pto_instr.hpp``).
+"""
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libptoamd.so")
+
+# element types (include/ptoamd.h)
+F32, F16, BF16, I32, I8, U8, E4M3, E5M2, E2M1, E1M2, I16 = range(11)
+B_ND, B_DN = 0, 1
+MX_A_ZZ, MX_A_ND, MX_A_DN, MX_B_NN, MX_B_ND, MX_B_DN = range(6)
+OCP_MXFP8, NV_MXFP8, OCP_MXFP4, NV_MXFP4 = range(4)
+
+
+class PtoAmdError(RuntimeError):
+    pass
+
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(f"{LIB_PATH} is missing: build it with `make -C pto-isa-mirror_amd -j8` "
+                      "(or __graft_entry__.build()); this package has no fallback path")
+
+_lib = C.CDLL(LIB_PATH)
+_lib.ptoamd_last_error.restype = C.c_char_p
+_lib.ptoamd_last_kernel.restype = C.c_char_p
+
+EXPORTS = [
+    "ptoamd_init", "ptoamd_finalize", "ptoamd_last_error", "ptoamd_device_info", "ptoamd_malloc", "ptoamd_free",
+    "ptoamd_malloc_host", "ptoamd_free_host", "ptoamd_memcpy", "ptoamd_memcpy_async", "ptoamd_memset",
+    "ptoamd_stream_create", "ptoamd_stream_destroy", "ptoamd_stream_synchronize", "ptoamd_event_create",
+    "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
+    "ptoamd_gemm", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
+    "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_mx_scale_relayout", "ptoamd_last_kernel",
+]
+
+
+def lib():
+    return _lib
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise PtoAmdError(f"{what} failed ({rc}): {_lib.ptoamd_last_error().decode()}")
+
+
+def last_kernel():
+    return _lib.ptoamd_last_kernel().decode()
+
+
+def init(device=0):
+    _check(_lib.ptoamd_init(int(device)), "ptoamd_init")
+
+
+def _ptr(t):
+    if t is None:
+        return C.c_void_p(0)
+    assert t.is_cuda and t.is_contiguous(), "operands must be contiguous device tensors"
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream(stream):
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return C.c_void_p(s.cuda_stream)
+
+
+_TORCH_OUT = {F32: torch.float32, F16: torch.float16, BF16: torch.bfloat16, I32: torch.int32}
+
+
+def gemm(a, b, ab_type, c_type=F32, b_layout=B_DN, c_in=None, relu=False, m=None, n=None, k=None, stream=None, out=None):
+    """TLOAD -> TMATMUL / TMATMUL_ACC -> TSTORE.  a: [m, k]; b: [n, k] (B_DN) or [k, n] (B_ND), raw-typed tensors."""
+    m = a.shape[0] if m is None else m
+    k = a.shape[1] if k is None else k
+    n = (b.shape[0] if b_layout == B_DN else b.shape[1]) if n is None else n
+    if out is None:
+        out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
+    _check(_lib.ptoamd_gemm(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), m, n, k, a.stride(0), b.stride(0),
+                            out.stride(0), b_layout, int(relu), _stream(stream)), "ptoamd_gemm")
+    return out
+
+
+def gemm_w8a8(a, b, scale_a, scale_b, b_layout=B_DN, want_acc=False, stream=None, out=None):
+    """int8 x int8 -> int32 accumulate with the fused dequantising drain to bf16."""
+    m, k = a.shape
+    n = b.shape[0] if b_layout == B_DN else b.shape[1]
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    acc = torch.empty((m, n), dtype=torch.int32, device=a.device) if want_acc else None
+    _check(_lib.ptoamd_gemm_w8a8(_ptr(out), _ptr(acc), _ptr(a), _ptr(b), _ptr(scale_a), _ptr(scale_b), m, n, k,
+                                 a.stride(0), b.stride(0), out.stride(0), b_layout, _stream(stream)), "ptoamd_gemm_w8a8")
+    return (out, acc) if want_acc else out
+
+
+def gemm_mx(a, b, sa, sb, m, n, k, a_type, b_type, c_type=F32, sa_layout=MX_A_ND, sb_layout=MX_B_DN, b_layout=B_DN,
+            c_in=None, stream=None, out=None):
+    """TMATMUL_MX.  a / b hold element codes (uint8; fp4 packed two per byte); sa / sb hold E8M0 bytes."""
+    if out is None:
+        out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
+    lda = k
+    ldb = k if b_layout == B_DN else n
+    _check(_lib.ptoamd_gemm_mx(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
+                               sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),
+           "ptoamd_gemm_mx")
+    return out
+
+
+def gemv_mxfp4(a_bf16, w, sw, n, k, c_type=F32, stream=None, out=None):
+    """Decode GEMV: bf16 activations [m <= 16, k] times MXFP4 weights [n, k/2] with E8M0 scales [n, k/32]."""
+    m = a_bf16.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=w.device)
+    _check(_lib.ptoamd_gemv_mxfp4(_ptr(out), c_type, _ptr(a_bf16), _ptr(w), _ptr(sw), m, n, k, a_bf16.stride(0), k,
+                                  out.stride(0), _stream(stream)), "ptoamd_gemv_mxfp4")
+    return out
+
+
+def tquant_int8(src, scale, offset=None, stream=None):
+    rows, cols = src.shape
+    out = torch.empty((rows, cols), dtype=torch.int8 if offset is None else torch.uint8, device=src.device)
+    _check(_lib.ptoamd_tquant_int8(_ptr(out), _ptr(src), _ptr(scale), _ptr(offset), rows, cols, _stream(stream)),
+           "ptoamd_tquant_int8")
+    return out
+
+
+_SRC_TYPE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+
+
+def tquant_mx(src, alg, axis=1, want_aux=True, stream=None):
+    """TQUANT<MXFP8 | MXFP4_E2M1>: returns (codes, exp[, max, scaling])."""
+    rows, cols = src.shape
+    fp4 = alg in (OCP_MXFP4, NV_MXFP4)
+    codes = torch.empty((rows, cols // 2 if fp4 else cols), dtype=torch.uint8, device=src.device)
+    gshape = (rows, cols // 32) if axis == 1 else (rows // 32, cols)
+    exp = torch.empty(gshape, dtype=torch.uint8, device=src.device)
+    mx = torch.empty(gshape, dtype=torch.float32, device=src.device) if want_aux else None
+    sc = torch.empty(gshape, dtype=torch.float32, device=src.device) if want_aux else None
+    _check(_lib.ptoamd_tquant_mx(_ptr(codes), _ptr(exp), _ptr(mx), _ptr(sc), _ptr(src), _SRC_TYPE[src.dtype], rows, cols,
+                                 alg, axis, _stream(stream)), "ptoamd_tquant_mx")
+    return (codes, exp, mx, sc) if want_aux else (codes, exp)
+
+
+_INT_TYPE = {torch.int8: I8, torch.int16: I16, torch.int32: I32}
+
+
+def tdequant(src, scale, offset, stream=None):
+    rows, cols = src.shape
+    out = torch.empty((rows, cols), dtype=torch.float32, device=src.device)
+    _check(_lib.ptoamd_tdequant(_ptr(out), _ptr(src), _INT_TYPE[src.dtype], _ptr(scale), _ptr(offset), rows, cols,
+                                _stream(stream)), "ptoamd_tdequant")
+    return out
+
+
+def mx_scale_relayout(src, src_layout, dst_layout, rows, cols, stream=None):
+    out = torch.empty_like(src)
+    _check(_lib.ptoamd_mx_scale_relayout(_ptr(out), dst_layout, _ptr(src), src_layout, rows, cols, _stream(stream)),
+           "ptoamd_mx_scale_relayout")
+    return out

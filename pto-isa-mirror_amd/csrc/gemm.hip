@@ -1,0 +1,471 @@
+// C-ABI launchers of the matmul family (ptoamd_gemm, ptoamd_gemm_w8a8, ptoamd_gemm_mx) and the kernels around the
+// tiled MFMA kernel: an order-exact generic kernel for shapes/layouts the tiled kernel does not take, the B-operand
+// transpose (Layout::ND -> the K-contiguous form the MFMA path reads) and the MX scale re-layout.
+#include "common_host.hpp"
+#include "gemm_tile.hpp"
+
+#include <stdlib.h>
+#include <string.h>
+
+namespace ptoamd {
+
+hipError_t launch_gemm_tile_bf16(int, const TileGemmParams&, hipStream_t);
+hipError_t launch_gemm_tile_f16(int, const TileGemmParams&, hipStream_t);
+hipError_t launch_gemm_tile_i8(int, const TileGemmParams&, hipStream_t);
+hipError_t launch_gemm_tile_fp8_e4e4(int, const TileGemmParams&, hipStream_t);
+hipError_t launch_gemm_tile_fp8_e5e5(int, const TileGemmParams&, hipStream_t);
+hipError_t launch_gemm_tile_fp8_e4e5(int, const TileGemmParams&, hipStream_t);
+hipError_t launch_gemm_tile_fp8_e5e4(int, const TileGemmParams&, hipStream_t);
+hipError_t launch_gemm_tile_fp4(int, const TileGemmParams&, hipStream_t);
+
+hipError_t launch_gemm_tile(int tile, int op, const TileGemmParams& p, hipStream_t stream)
+{
+    switch (op) {
+        case TOP_BF16: return launch_gemm_tile_bf16(tile, p, stream);
+        case TOP_F16: return launch_gemm_tile_f16(tile, p, stream);
+        case TOP_I8: return launch_gemm_tile_i8(tile, p, stream);
+        case TOP_FP8_E4E4: return launch_gemm_tile_fp8_e4e4(tile, p, stream);
+        case TOP_FP8_E5E5: return launch_gemm_tile_fp8_e5e5(tile, p, stream);
+        case TOP_FP8_E4E5: return launch_gemm_tile_fp8_e4e5(tile, p, stream);
+        case TOP_FP8_E5E4: return launch_gemm_tile_fp8_e5e4(tile, p, stream);
+        case TOP_FP4: return launch_gemm_tile_fp4(tile, p, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+void tile_shape(int tile, int* bm, int* bn)
+{
+    static const int shapes[3] = {256, 128, 64};
+    *bm = *bn = shapes[tile < 0 || tile > 2 ? 2 : tile];
+}
+
+// ---- MX scale GM layouts (reference: cpu/tile_offsets.hpp:233-268 with the strides of pto_tile.hpp:849-1102) ----
+__host__ __device__ inline long mx_scale_offset(int layout, int rows, int cols, int r, int c)
+{
+    switch (layout) {
+        case PTOAMD_MX_A_ZZ: return (long)(r / 16) * cols * 16 + (c / 2) * 32 + (r % 16) * 2 + c % 2;
+        case PTOAMD_MX_A_ND: return (long)r * cols + c;
+        case PTOAMD_MX_A_DN: return (long)(c / 2) * rows * 2 + r * 2 + c % 2;
+        case PTOAMD_MX_B_NN: return (long)(c / 16) * rows * 16 + (r / 2) * 32 + (c % 16) * 2 + r % 2;
+        case PTOAMD_MX_B_ND: return (long)(r / 2) * cols * 2 + c * 2 + r % 2;
+        default: return (long)c * rows + r;  // PTOAMD_MX_B_DN
+    }
+}
+
+__global__ void mx_scale_relayout_kernel(uint8_t* dst, int dst_layout, const uint8_t* src, int src_layout, int rows,
+                                         int cols)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long)rows * cols)
+        return;
+    const int r = (int)(idx / cols), c = (int)(idx % cols);
+    dst[mx_scale_offset(dst_layout, rows, cols, r, c)] = src[mx_scale_offset(src_layout, rows, cols, r, c)];
+}
+
+// ---- B operand: [K][N] row-major -> [N][K] so both operands are read K-contiguous -----------------------------
+template <typename T>
+__global__ void transpose_kernel(T* dst, const T* src, int rows, int cols, long ld_src, long ld_dst)
+{
+    __shared__ T tile[32][33];
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    for (int i = threadIdx.y; i < 32; i += blockDim.y) {
+        const int r = r0 + i, c = c0 + threadIdx.x;
+        if (r < rows && c < cols)
+            tile[i][threadIdx.x] = src[(long)r * ld_src + c];
+    }
+    __syncthreads();
+    for (int i = threadIdx.y; i < 32; i += blockDim.y) {
+        const int c = c0 + i, r = r0 + threadIdx.x;
+        if (r < rows && c < cols)
+            dst[(long)c * ld_dst + r] = tile[threadIdx.x][i];
+    }
+}
+
+// ---- order-exact generic kernel -------------------------------------------------------------------------------
+// One thread per output element, k ascending, one rounding per step exactly as the reference CPU simulator does
+// (cpu/TMatmul.hpp:96-110 and :191-200).  Slow; it serves the shapes, layouts and element types the MFMA kernel
+// does not take, and matches the simulator bit for bit on every type.
+struct GenericParams {
+    const void* a;
+    const void* b;
+    void* c;
+    const void* c_in;
+    int32_t* acc_out;
+    const uint8_t* sa;
+    const uint8_t* sb;
+    const float* row_scale;
+    const float* col_scale;
+    int m, n, k;
+    long lda, sbk, sbn;  // element strides: A row pitch; B(k, j) = b[k * sbk + j * sbn]
+    int ldc;
+    int a_type, b_type, out_kind, relu;
+    int sa_layout, sb_layout, mx;
+};
+
+__device__ __forceinline__ float load_elem_f32(const void* p, long idx, int type)
+{
+    switch (type) {
+        case PTOAMD_F32: return reinterpret_cast<const float*>(p)[idx];
+        case PTOAMD_F16: return f16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[idx]);
+        case PTOAMD_BF16: return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[idx]);
+        case PTOAMD_E4M3: return e4m3_to_f32(reinterpret_cast<const uint8_t*>(p)[idx]);
+        case PTOAMD_E5M2: return e5m2_to_f32(reinterpret_cast<const uint8_t*>(p)[idx]);
+        case PTOAMD_E2M1: return e2m1_to_f32((reinterpret_cast<const uint8_t*>(p)[idx >> 1] >> ((idx & 1) * 4)) & 0xFu);
+        case PTOAMD_E1M2: return e1m2_to_f32((reinterpret_cast<const uint8_t*>(p)[idx >> 1] >> ((idx & 1) * 4)) & 0xFu);
+        default: return (float)reinterpret_cast<const int8_t*>(p)[idx];
+    }
+}
+
+__device__ __forceinline__ void store_out(const GenericParams& p, long o, float v, int gi, int gj)
+{
+    if (p.relu)
+        v = v > 0 ? v : 0;
+    switch (p.out_kind) {
+        case OUT_F32: reinterpret_cast<float*>(p.c)[o] = v; break;
+        case OUT_F16: reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits(v); break;
+        default: reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(v); break;
+    }
+    (void)gi;
+    (void)gj;
+}
+
+__global__ void gemm_generic_kernel(const GenericParams p)
+{
+    const int gj = blockIdx.x * blockDim.x + threadIdx.x;
+    const int gi = blockIdx.y * blockDim.y + threadIdx.y;
+    if (gi >= p.m || gj >= p.n)
+        return;
+    const long o = (long)gi * p.ldc + gj;
+    if (p.a_type == PTOAMD_I8 && !p.mx) {
+        uint32_t acc = p.c_in ? (uint32_t) reinterpret_cast<const int32_t*>(p.c_in)[o] : 0u;
+        const int8_t* a = reinterpret_cast<const int8_t*>(p.a) + (long)gi * p.lda;
+        const int8_t* b = reinterpret_cast<const int8_t*>(p.b) + (long)gj * p.sbn;
+        for (int kk = 0; kk < p.k; ++kk)
+            acc += (uint32_t)((int32_t)a[kk] * (int32_t)b[(long)kk * p.sbk]);
+        int32_t v = (int32_t)acc;
+        if (p.relu)
+            v = v > 0 ? v : 0;
+        if (p.out_kind == OUT_I32) {
+            reinterpret_cast<int32_t*>(p.c)[o] = v;
+        } else {
+            if (p.acc_out)
+                p.acc_out[o] = v;
+            const float t = __fmul_rn((float)v, p.row_scale[gi]);
+            reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(__fmul_rn(t, p.col_scale[gj]));
+        }
+        return;
+    }
+    float acc = p.c_in ? reinterpret_cast<const float*>(p.c_in)[o] : 0.0f;
+    if (!p.mx) {
+        for (int kk = 0; kk < p.k; ++kk) {
+            const float av = load_elem_f32(p.a, (long)gi * p.lda + kk, p.a_type);
+            const float bv = load_elem_f32(p.b, (long)kk * p.sbk + (long)gj * p.sbn, p.b_type);
+            acc = __fmaf_rn(av, bv, acc);
+        }
+    } else {
+        const int kg = p.k / 32;
+        for (int kk = 0; kk < p.k; ++kk) {
+            const double sf = e8m0_to_f64(p.sa[mx_scale_offset(p.sa_layout, p.m, kg, gi, kk / 32)]) *
+                              e8m0_to_f64(p.sb[mx_scale_offset(p.sb_layout, kg, p.n, kk / 32, gj)]);
+            const double av = (double)load_elem_f32(p.a, (long)gi * p.lda + kk, p.a_type);
+            const double bv = (double)load_elem_f32(p.b, (long)kk * p.sbk + (long)gj * p.sbn, p.b_type);
+            acc = (float)((double)acc + av * bv * sf);  // double add, then one rounding to float per k
+        }
+    }
+    store_out(p, o, acc, gi, gj);
+}
+
+static int launch_generic(const GenericParams& p, hipStream_t stream)
+{
+    dim3 block(32, 8), grid((p.n + 31) / 32, (p.m + 7) / 8);
+    hipLaunchKernelGGL(gemm_generic_kernel, grid, block, 0, stream, p);
+    PTOAMD_HIP_CHECK(hipGetLastError());
+    set_last_kernel("generic");
+    return PTOAMD_OK;
+}
+
+static int elem_bits(int type)
+{
+    switch (type) {
+        case PTOAMD_F32: case PTOAMD_I32: return 32;
+        case PTOAMD_F16: case PTOAMD_BF16: case PTOAMD_I16: return 16;
+        case PTOAMD_E2M1: case PTOAMD_E1M2: return 4;
+        default: return 8;
+    }
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Which tile shape to run: the largest whose grid still fills most of the 256 CUs.  PTOAMD_TILE=0|1|2 overrides,
+// PTOAMD_FORCE_GENERIC=1 sends everything to the order-exact kernel (used by the parity tests).
+static int pick_tile(int m, int n)
+{
+    const char* env = getenv("PTOAMD_TILE");
+    if (env && env[0] >= '0' && env[0] <= '2')
+        return env[0] - '0';
+    const long t256 = (long)((m + 255) / 256) * ((n + 255) / 256);
+    if (t256 >= 128)
+        return 0;
+    const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128);
+    if (t128 >= 96)
+        return 1;
+    return 2;
+}
+
+static bool force_generic()
+{
+    const char* env = getenv("PTOAMD_FORCE_GENERIC");
+    return env && env[0] == '1';
+}
+
+static const char* tile_kernel_name(int tile, int op)
+{
+    static const char* ops[TOP_COUNT] = {"bf16", "f16", "i8", "fp8_e4m3_e4m3", "fp8_e5m2_e5m2", "fp8_e4m3_e5m2",
+                                         "fp8_e5m2_e4m3", "fp4_e2m1"};
+    static const char* tiles[3] = {"tile256x256", "tile128x128", "tile64x64"};
+    static thread_local char buf[64];
+    snprintf(buf, sizeof buf, "%s_%s", tiles[tile], ops[op]);
+    return buf;
+}
+
+// Temporary device buffers (transposed B, re-laid scales) are stream-ordered allocations released after the launch.
+struct StreamTemp {
+    void* ptr = nullptr;
+    hipStream_t stream;
+    explicit StreamTemp(hipStream_t s) : stream(s) {}
+    hipError_t alloc(size_t bytes) { return hipMallocAsync(&ptr, bytes, stream); }
+    ~StreamTemp()
+    {
+        if (ptr)
+            (void)hipFreeAsync(ptr, stream);
+    }
+};
+
+template <typename T>
+static int transpose_b(void* dst, const void* src, int k, int n, long ldb, hipStream_t stream)
+{
+    dim3 block(32, 8), grid((n + 31) / 32, (k + 31) / 32);
+    hipLaunchKernelGGL(transpose_kernel<T>, grid, block, 0, stream, reinterpret_cast<T*>(dst),
+                       reinterpret_cast<const T*>(src), k, n, ldb, (long)k);
+    PTOAMD_HIP_CHECK(hipGetLastError());
+    return PTOAMD_OK;
+}
+
+}  // namespace ptoamd
+
+using namespace ptoamd;
+
+extern "C" {
+
+int ptoamd_mx_scale_relayout(uint8_t* dst, int dst_layout, const uint8_t* src, int src_layout, int rows, int cols,
+                             void* stream)
+{
+    PTOAMD_REQUIRE(dst && src && rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_mx_scale_relayout: bad argument");
+    PTOAMD_REQUIRE(dst_layout >= 0 && dst_layout <= 5 && src_layout >= 0 && src_layout <= 5, PTOAMD_E_INVALID,
+                   "ptoamd_mx_scale_relayout: unknown layout");
+    const bool a_side = src_layout <= PTOAMD_MX_A_DN;
+    PTOAMD_REQUIRE(a_side == (dst_layout <= PTOAMD_MX_A_DN), PTOAMD_E_INVALID,
+                   "ptoamd_mx_scale_relayout: source and destination must both be A-side or both B-side layouts");
+    const int pair_dim = a_side ? cols : rows;   // the K/32 axis is stored in pairs
+    const int box_dim = a_side ? rows : cols;    // ZZ / NN box the other axis by 16
+    PTOAMD_REQUIRE(pair_dim % 2 == 0, PTOAMD_E_INVALID, "ptoamd_mx_scale_relayout: K/32 must be even");
+    const bool boxed = src_layout == PTOAMD_MX_A_ZZ || dst_layout == PTOAMD_MX_A_ZZ || src_layout == PTOAMD_MX_B_NN ||
+                       dst_layout == PTOAMD_MX_B_NN;
+    PTOAMD_REQUIRE(!boxed || box_dim % 16 == 0, PTOAMD_E_INVALID,
+                   "ptoamd_mx_scale_relayout: ZZ/NN layouts need the row (A) / column (B) count to be a multiple of 16");
+    const long total = (long)rows * cols;
+    hipLaunchKernelGGL(mx_scale_relayout_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       dst, dst_layout, src, src_layout, rows, cols);
+    PTOAMD_HIP_CHECK(hipGetLastError());
+    return PTOAMD_OK;
+}
+
+int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, int m, int n, int k,
+                int lda, int ldb, int ldc, int b_layout, int relu, void* stream_)
+{
+    hipStream_t stream = as_stream(stream_);
+    PTOAMD_REQUIRE(c && a && b, PTOAMD_E_INVALID, "ptoamd_gemm: null operand");
+    PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemm: m, n, k must be positive (%d, %d, %d)", m, n, k);
+    PTOAMD_REQUIRE(b_layout == PTOAMD_B_ND || b_layout == PTOAMD_B_DN, PTOAMD_E_INVALID, "ptoamd_gemm: unknown b_layout");
+    PTOAMD_REQUIRE(lda >= k && ldc >= n && ldb >= (b_layout == PTOAMD_B_DN ? k : n), PTOAMD_E_INVALID,
+                   "ptoamd_gemm: leading dimension smaller than the row length");
+    const bool is_int = ab_type == PTOAMD_I8;
+    const bool is_float = ab_type == PTOAMD_F16 || ab_type == PTOAMD_BF16 || ab_type == PTOAMD_F32 ||
+                          ab_type == PTOAMD_E4M3 || ab_type == PTOAMD_E5M2;
+    PTOAMD_REQUIRE(is_int || is_float, PTOAMD_E_UNSUPPORTED,
+                   "ptoamd_gemm: operand type %d is not a TMATMUL input type (s8, f16, bf16, f32, e4m3, e5m2)", ab_type);
+    int out_kind;
+    if (is_int) {
+        PTOAMD_REQUIRE(c_type == PTOAMD_I32, PTOAMD_E_UNSUPPORTED, "ptoamd_gemm: int8 operands accumulate to int32 only");
+        out_kind = OUT_I32;
+    } else {
+        PTOAMD_REQUIRE(c_type == PTOAMD_F32 || c_type == PTOAMD_F16 || c_type == PTOAMD_BF16, PTOAMD_E_UNSUPPORTED,
+                       "ptoamd_gemm: float accumulators store as f32, f16 or bf16");
+        out_kind = c_type == PTOAMD_F32 ? OUT_F32 : (c_type == PTOAMD_F16 ? OUT_F16 : OUT_BF16);
+    }
+    const int ebytes = elem_bits(ab_type) / 8;
+    const long k_bytes = (long)k * ebytes, lda_b = (long)lda * ebytes, ldb_b = (long)ldb * ebytes;
+    const bool tile_ok = !force_generic() && ab_type != PTOAMD_F32 && aligned16(a) && aligned16(b) && (lda_b % 16) == 0 &&
+                         (k_bytes % 16) == 0 &&
+                         (b_layout == PTOAMD_B_DN ? (ldb_b % 16) == 0 : true);
+    if (!tile_ok) {
+        GenericParams g{};
+        g.a = a; g.b = b; g.c = c; g.c_in = c_in;
+        g.m = m; g.n = n; g.k = k; g.lda = lda; g.ldc = ldc;
+        g.sbk = b_layout == PTOAMD_B_DN ? 1 : ldb;
+        g.sbn = b_layout == PTOAMD_B_DN ? ldb : 1;
+        g.a_type = g.b_type = ab_type; g.out_kind = out_kind; g.relu = relu;
+        return launch_generic(g, stream);
+    }
+    StreamTemp bt(stream);
+    const uint8_t* b_kmajor = reinterpret_cast<const uint8_t*>(b);
+    long ldb_kmajor = ldb_b;
+    if (b_layout == PTOAMD_B_ND) {  // TLOAD of an ND B panel: re-order once so the MFMA path reads K-contiguous rows
+        PTOAMD_HIP_CHECK(bt.alloc((size_t)n * k_bytes));
+        const int rc = ebytes == 2 ? transpose_b<uint16_t>(bt.ptr, b, k, n, ldb, stream)
+                                   : transpose_b<uint8_t>(bt.ptr, b, k, n, ldb, stream);
+        if (rc != PTOAMD_OK)
+            return rc;
+        b_kmajor = reinterpret_cast<const uint8_t*>(bt.ptr);
+        ldb_kmajor = k_bytes;
+    }
+    TileGemmParams p{};
+    p.a = reinterpret_cast<const uint8_t*>(a);
+    p.b = b_kmajor;
+    p.c = c; p.c_in = c_in;
+    p.m = m; p.n = n; p.k_bytes = (int)k_bytes;
+    p.lda_bytes = lda_b; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
+    p.relu = relu; p.out_kind = out_kind; p.group_m = 4;
+    const int op = ab_type == PTOAMD_BF16 ? TOP_BF16
+                   : ab_type == PTOAMD_F16 ? TOP_F16
+                   : ab_type == PTOAMD_I8 ? TOP_I8
+                   : ab_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E5E5;
+    const int tile = pick_tile(m, n);
+    PTOAMD_HIP_CHECK(launch_gemm_tile(tile, op, p, stream));
+    set_last_kernel(tile_kernel_name(tile, op));
+    return PTOAMD_OK;
+}
+
+int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const int8_t* b, const float* scale_a,
+                     const float* scale_b, int m, int n, int k, int lda, int ldb, int ldc, int b_layout, void* stream_)
+{
+    hipStream_t stream = as_stream(stream_);
+    PTOAMD_REQUIRE(out_bf16 && a && b && scale_a && scale_b, PTOAMD_E_INVALID, "ptoamd_gemm_w8a8: null operand");
+    PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemm_w8a8: m, n, k must be positive");
+    PTOAMD_REQUIRE(b_layout == PTOAMD_B_ND || b_layout == PTOAMD_B_DN, PTOAMD_E_INVALID, "ptoamd_gemm_w8a8: unknown b_layout");
+    PTOAMD_REQUIRE(lda >= k && ldc >= n && ldb >= (b_layout == PTOAMD_B_DN ? k : n), PTOAMD_E_INVALID,
+                   "ptoamd_gemm_w8a8: leading dimension smaller than the row length");
+    const bool tile_ok = !force_generic() && aligned16(a) && aligned16(b) && (lda % 16) == 0 && (k % 16) == 0 &&
+                         (b_layout == PTOAMD_B_DN ? (ldb % 16) == 0 : true);
+    if (!tile_ok) {
+        GenericParams g{};
+        g.a = a; g.b = b; g.c = out_bf16; g.acc_out = acc_out; g.row_scale = scale_a; g.col_scale = scale_b;
+        g.m = m; g.n = n; g.k = k; g.lda = lda; g.ldc = ldc;
+        g.sbk = b_layout == PTOAMD_B_DN ? 1 : ldb;
+        g.sbn = b_layout == PTOAMD_B_DN ? ldb : 1;
+        g.a_type = g.b_type = PTOAMD_I8; g.out_kind = OUT_W8A8_BF16;
+        return launch_generic(g, stream);
+    }
+    StreamTemp bt(stream);
+    const uint8_t* b_kmajor = reinterpret_cast<const uint8_t*>(b);
+    long ldb_kmajor = ldb;
+    if (b_layout == PTOAMD_B_ND) {
+        PTOAMD_HIP_CHECK(bt.alloc((size_t)n * k));
+        const int rc = transpose_b<uint8_t>(bt.ptr, b, k, n, ldb, stream);
+        if (rc != PTOAMD_OK)
+            return rc;
+        b_kmajor = reinterpret_cast<const uint8_t*>(bt.ptr);
+        ldb_kmajor = k;
+    }
+    TileGemmParams p{};
+    p.a = reinterpret_cast<const uint8_t*>(a);
+    p.b = b_kmajor;
+    p.c = out_bf16; p.acc_out = acc_out; p.row_scale = scale_a; p.col_scale = scale_b;
+    p.m = m; p.n = n; p.k_bytes = k; p.lda_bytes = lda; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
+    p.out_kind = OUT_W8A8_BF16; p.group_m = 4;
+    const int tile = pick_tile(m, n);
+    PTOAMD_HIP_CHECK(launch_gemm_tile(tile, TOP_I8, p, stream));
+    set_last_kernel(tile_kernel_name(tile, TOP_I8));
+    return PTOAMD_OK;
+}
+
+int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
+                   const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n, int k, int lda,
+                   int ldb, int ldc, int b_layout, void* stream_)
+{
+    hipStream_t stream = as_stream(stream_);
+    PTOAMD_REQUIRE(c && a && b && sa && sb, PTOAMD_E_INVALID, "ptoamd_gemm_mx: null operand");
+    PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemm_mx: m, n, k must be positive");
+    PTOAMD_REQUIRE(k % 64 == 0, PTOAMD_E_INVALID, "ptoamd_gemm_mx: k = %d must be a multiple of 64", k);
+    PTOAMD_REQUIRE(b_layout == PTOAMD_B_ND || b_layout == PTOAMD_B_DN, PTOAMD_E_INVALID, "ptoamd_gemm_mx: unknown b_layout");
+    PTOAMD_REQUIRE(sa_layout >= PTOAMD_MX_A_ZZ && sa_layout <= PTOAMD_MX_A_DN && sb_layout >= PTOAMD_MX_B_NN &&
+                       sb_layout <= PTOAMD_MX_B_DN,
+                   PTOAMD_E_INVALID, "ptoamd_gemm_mx: sa_layout must be an MX_A_* and sb_layout an MX_B_* layout");
+    const bool a8 = a_type == PTOAMD_E4M3 || a_type == PTOAMD_E5M2, b8 = b_type == PTOAMD_E4M3 || b_type == PTOAMD_E5M2;
+    const bool a4 = a_type == PTOAMD_E2M1 || a_type == PTOAMD_E1M2, b4 = b_type == PTOAMD_E2M1 || b_type == PTOAMD_E1M2;
+    PTOAMD_REQUIRE((a8 && b8) || (a4 && b4), PTOAMD_E_UNSUPPORTED,
+                   "ptoamd_gemm_mx: operands must both be fp8 (e4m3/e5m2) or both fp4 (e2m1/e1m2)");
+    PTOAMD_REQUIRE(c_type == PTOAMD_F32 || c_type == PTOAMD_F16 || c_type == PTOAMD_BF16, PTOAMD_E_UNSUPPORTED,
+                   "ptoamd_gemm_mx: the accumulator stores as f32, f16 or bf16");
+    PTOAMD_REQUIRE(lda >= k && ldc >= n && ldb >= (b_layout == PTOAMD_B_DN ? k : n), PTOAMD_E_INVALID,
+                   "ptoamd_gemm_mx: leading dimension smaller than the row length");
+    PTOAMD_REQUIRE(sa_layout != PTOAMD_MX_A_ZZ || m % 16 == 0, PTOAMD_E_INVALID, "ptoamd_gemm_mx: MX_A_ZZ needs m %% 16 == 0");
+    PTOAMD_REQUIRE(sb_layout != PTOAMD_MX_B_NN || n % 16 == 0, PTOAMD_E_INVALID, "ptoamd_gemm_mx: MX_B_NN needs n %% 16 == 0");
+    if (a4)
+        PTOAMD_REQUIRE(lda % 2 == 0 && ldb % 2 == 0, PTOAMD_E_ALIGNMENT, "ptoamd_gemm_mx: fp4 leading dimensions must be even");
+    const int out_kind = c_type == PTOAMD_F32 ? OUT_F32 : (c_type == PTOAMD_F16 ? OUT_F16 : OUT_BF16);
+    const int bits = a8 ? 8 : 4;
+    const long k_bytes = (long)k * bits / 8, lda_b = (long)lda * bits / 8, ldb_b = (long)ldb * bits / 8;
+    const bool e1m2 = a_type == PTOAMD_E1M2 || b_type == PTOAMD_E1M2;  // the scaled MFMA has no E1M2 format
+    const bool tile_ok = !force_generic() && !e1m2 && b_layout == PTOAMD_B_DN && aligned16(a) && aligned16(b) &&
+                         (lda_b % 16) == 0 && (ldb_b % 16) == 0 && (k_bytes % 128) == 0;
+    if (!tile_ok) {
+        GenericParams g{};
+        g.a = a; g.b = b; g.c = c; g.c_in = c_in; g.sa = sa; g.sb = sb;
+        g.m = m; g.n = n; g.k = k; g.lda = lda; g.ldc = ldc;
+        g.sbk = b_layout == PTOAMD_B_DN ? 1 : ldb;
+        g.sbn = b_layout == PTOAMD_B_DN ? ldb : 1;
+        g.a_type = a_type; g.b_type = b_type; g.out_kind = out_kind; g.mx = 1;
+        g.sa_layout = sa_layout; g.sb_layout = sb_layout;
+        return launch_generic(g, stream);
+    }
+    const int kg = k / 32;
+    StreamTemp ta(stream), tb(stream);
+    const uint8_t* sa_nd = sa;
+    const uint8_t* sb_dn = sb;
+    if (sa_layout != PTOAMD_MX_A_ND) {  // the kernel streams scales as [M][K/32] and [N][K/32]
+        PTOAMD_HIP_CHECK(ta.alloc((size_t)m * kg));
+        const int rc = ptoamd_mx_scale_relayout(reinterpret_cast<uint8_t*>(ta.ptr), PTOAMD_MX_A_ND, sa, sa_layout, m, kg, stream_);
+        if (rc != PTOAMD_OK)
+            return rc;
+        sa_nd = reinterpret_cast<const uint8_t*>(ta.ptr);
+    }
+    if (sb_layout != PTOAMD_MX_B_DN) {
+        PTOAMD_HIP_CHECK(tb.alloc((size_t)n * kg));
+        const int rc = ptoamd_mx_scale_relayout(reinterpret_cast<uint8_t*>(tb.ptr), PTOAMD_MX_B_DN, sb, sb_layout, kg, n, stream_);
+        if (rc != PTOAMD_OK)
+            return rc;
+        sb_dn = reinterpret_cast<const uint8_t*>(tb.ptr);
+    }
+    PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(sa_nd) & 3u) == 0 && (reinterpret_cast<uintptr_t>(sb_dn) & 3u) == 0,
+                   PTOAMD_E_ALIGNMENT, "ptoamd_gemm_mx: scale arrays must be 4-byte aligned");
+    TileGemmParams p{};
+    p.a = reinterpret_cast<const uint8_t*>(a);
+    p.b = reinterpret_cast<const uint8_t*>(b);
+    p.c = c; p.c_in = c_in; p.sa = sa_nd; p.sb = sb_dn;
+    p.m = m; p.n = n; p.k_bytes = (int)k_bytes; p.lda_bytes = lda_b; p.ldb_bytes = ldb_b; p.ldc = ldc;
+    p.scale_ld = kg; p.out_kind = out_kind; p.group_m = 4;
+    int op;
+    if (a4)
+        op = TOP_FP4;
+    else if (a_type == PTOAMD_E4M3)
+        op = b_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E4E5;
+    else
+        op = b_type == PTOAMD_E5M2 ? TOP_FP8_E5E5 : TOP_FP8_E5E4;
+    const int tile = pick_tile(m, n);
+    PTOAMD_HIP_CHECK(launch_gemm_tile(tile, op, p, stream));
+    set_last_kernel(tile_kernel_name(tile, op));
+    return PTOAMD_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,361 @@
+// Tiled MFMA GEMM for gfx950: the TLOAD -> TMATMUL_ACC -> TSTORE pipeline of one PTO kernel as one HIP kernel.
+//
+//   TLOAD (GM -> L1 Mat tile)        128-bit coalesced global loads of a [rows][128 B] K-slab, staged into LDS
+//   TMOV/TEXTRACT (L1 -> L0A/L0B)    ds_read_b128 of MFMA operand fragments from the swizzled LDS slab
+//   TMATMUL / TMATMUL_ACC (Cube)     v_mfma_* on 32x32 blocks, accumulators (the L0C Acc tile) live in registers
+//   TSTORE (L0C -> GM, fix-pipe)     register epilogue: relu / dequant scales / f32->bf16|f16 RNE, then global stores
+//
+// Both operands are read K-contiguous: A is [M][K] row-major and B is [N][K] (Layout::DN).  A K-slab is 128 bytes per
+// row whatever the element type (64 bf16/f16, 128 fp8/int8, 256 fp4), so one loader and one LDS layout serve all types.
+// The LDS slab is double buffered: slab kt+1 is fetched into registers while slab kt is multiplied, then written to
+// the other buffer; one __syncthreads per slab replaces the MTE2/MTE1/M event chain of the reference kernels
+// (kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:115-150).
+#pragma once
+#include "device_types.hpp"
+
+namespace ptoamd {
+
+struct TileGemmParams {
+    const uint8_t* a;       // [m][lda_bytes]
+    const uint8_t* b;       // [n][ldb_bytes]
+    void* c;                // [m][ldc] of the output type
+    const void* c_in;       // optional accumulator input, [m][ldc] f32 / i32
+    int32_t* acc_out;       // optional raw int32 accumulators (W8A8), [m][ldc]
+    const uint8_t* sa;      // MX: [m][k/32] E8M0
+    const uint8_t* sb;      // MX: [n][k/32] E8M0
+    const float* row_scale; // W8A8: [m]
+    const float* col_scale; // W8A8: [n]
+    int m, n;
+    int k_bytes;            // bytes per operand row that take part in the contraction
+    long lda_bytes, ldb_bytes;
+    int ldc;
+    int scale_ld;           // MX: bytes per scale row (k / 32)
+    int relu;
+    int out_kind;           // OutKind
+    int group_m;            // tile-order grouping for L2 reuse
+};
+
+enum OutKind { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2, OUT_I32 = 3, OUT_W8A8_BF16 = 4 };
+
+// ---- MFMA operand traits ------------------------------------------------------------------------------------
+// FRAG_BYTES: operand bytes one lane feeds one MFMA; a k-step spans 2 * FRAG_BYTES of a slab row (lanes 0-31 take
+// the first half, lanes 32-63 the second), so a 128-byte slab is 128 / (2 * FRAG_BYTES) k-steps.
+struct OpBF16 {
+    using Acc = f32x16;
+    using Elem = float;
+    static constexpr int FRAG_BYTES = 16;
+    static constexpr bool SCALED = false;
+    static constexpr int GROUPS_PER_SLAB = 0;
+    __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t, uint32_t)
+    {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]),
+                                                    c, 0, 0, 0);
+    }
+};
+struct OpF16 {
+    using Acc = f32x16;
+    using Elem = float;
+    static constexpr int FRAG_BYTES = 16;
+    static constexpr bool SCALED = false;
+    static constexpr int GROUPS_PER_SLAB = 0;
+    __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t, uint32_t)
+    {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c,
+                                                   0, 0, 0);
+    }
+};
+struct OpI8 {
+    using Acc = i32x16;
+    using Elem = int32_t;
+    static constexpr int FRAG_BYTES = 16;
+    static constexpr bool SCALED = false;
+    static constexpr int GROUPS_PER_SLAB = 0;
+    __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t, uint32_t)
+    {
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a[0]), __builtin_bit_cast(i32x4, b[0]), c,
+                                                  0, 0, 0);
+    }
+};
+// fp8 (E4M3 = format 0, E5M2 = format 1) through the block-scaled MFMA; each lane's 32 bytes are one MX group.
+// Without scale pointers both scales are 2^0 (E8M0 127) and the instruction is a plain fp8 TMATMUL.
+template <int AFMT, int BFMT>
+struct OpFP8 {
+    using Acc = f32x16;
+    using Elem = float;
+    static constexpr int FRAG_BYTES = 32;
+    static constexpr bool SCALED = true;
+    static constexpr int GROUPS_PER_SLAB = 4;
+    __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        i32x8 av, bv;
+        av.s0 = a[0].x; av.s1 = a[0].y; av.s2 = a[0].z; av.s3 = a[0].w;
+        av.s4 = a[1].x; av.s5 = a[1].y; av.s6 = a[1].z; av.s7 = a[1].w;
+        bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
+        bv.s4 = b[1].x; bv.s5 = b[1].y; bv.s6 = b[1].z; bv.s7 = b[1].w;
+        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, AFMT, BFMT, 0, (int)sa, 0, (int)sb);
+    }
+};
+// fp4 E2M1 (format 4): 32 elements = 16 bytes per lane = one MX group
+struct OpFP4 {
+    using Acc = f32x16;
+    using Elem = float;
+    static constexpr int FRAG_BYTES = 16;
+    static constexpr bool SCALED = true;
+    static constexpr int GROUPS_PER_SLAB = 8;
+    __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        i32x8 av = {0, 0, 0, 0, 0, 0, 0, 0}, bv = {0, 0, 0, 0, 0, 0, 0, 0};
+        av.s0 = a[0].x; av.s1 = a[0].y; av.s2 = a[0].z; av.s3 = a[0].w;
+        bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
+        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 4, 4, 0, (int)sa, 0, (int)sb);
+    }
+};
+
+// 16-byte chunk swizzle inside a 128-byte slab row: consecutive rows land in different banks for ds_read_b128
+__device__ __forceinline__ int swizzle_chunk(int row, int chunk) { return chunk ^ ((row >> 1) & 7) ^ ((row & 1) << 2); }
+
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, class Op_>
+struct TileCfg {
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    using Op = Op_;
+    static constexpr int THREADS = WAVES_M * WAVES_N * 64;
+    static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;  // per-wave output tile
+    static constexpr int MB = WTM / 32, NB = WTN / 32;            // 32x32 MFMA blocks per wave
+    static constexpr int SLAB = 128;                              // bytes of K per slab row
+    static constexpr int KSTEPS = SLAB / (2 * Op::FRAG_BYTES);
+    static constexpr int A_BYTES = BM * SLAB, B_BYTES = BN * SLAB, STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    static constexpr int LA = BM * 8 / THREADS, LB = BN * 8 / THREADS;  // 16-byte chunks per thread per slab
+    static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "wave tiles are made of 32x32 blocks");
+    static_assert((BM * 8) % THREADS == 0 && (BN * 8) % THREADS == 0, "slab chunks must divide over the workgroup");
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmParams p)
+{
+    using Op = typename Cfg::Op;
+    using Acc = typename Op::Acc;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, LA = Cfg::LA, LB = Cfg::LB;
+    constexpr int NT = Cfg::THREADS, FR = Op::FRAG_BYTES / 16;
+    extern __shared__ __align__(16) uint8_t smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % Cfg::WAVES_M, wn = wave / Cfg::WAVES_M;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    // ---- workgroup -> output tile.  Workgroups are dealt round-robin to the 8 XCDs, so ids congruent mod 8 share an
+    // L2; give each XCD a contiguous run of tiles and walk tiles in groups of group_m rows so a run reuses few panels.
+    const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+    const int grid = tiles_m * tiles_n;
+    int lid = blockIdx.x;
+    if ((grid & 7) == 0)
+        lid = (lid & 7) * (grid >> 3) + (lid >> 3);
+    const int per_group = p.group_m * tiles_n;
+    const int first_m = (lid / per_group) * p.group_m;
+    const int gsize = min(tiles_m - first_m, p.group_m);
+    const int tm = first_m + (lid % per_group) % gsize;
+    const int tn = (lid % per_group) / gsize;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // ---- TLOAD addressing: thread t moves chunk (t % 8) of rows t / 8 + i * NT / 8
+    const int ld_chunk = tid & 7, ld_row = tid >> 3;
+    const uint8_t* ga[LA];
+    const uint8_t* gb[LB];
+    int sa_off[LA], sb_off[LB];
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int r = ld_row + i * (NT / 8);
+        ga[i] = p.a + (long)min(m0 + r, p.m - 1) * p.lda_bytes + ld_chunk * 16;
+        sa_off[i] = r * 128 + swizzle_chunk(r, ld_chunk) * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int r = ld_row + i * (NT / 8);
+        gb[i] = p.b + (long)min(n0 + r, p.n - 1) * p.ldb_bytes + ld_chunk * 16;
+        sb_off[i] = Cfg::A_BYTES + r * 128 + swizzle_chunk(r, ld_chunk) * 16;
+    }
+    const int k_slabs = (p.k_bytes + 127) / 128;
+
+    uint4 ra[LA], rb[LB];
+    auto tload = [&](int kt) {
+        const bool live = kt * 128 + ld_chunk * 16 < p.k_bytes;  // partial last slab: missing chunks are zero
+#pragma unroll
+        for (int i = 0; i < LA; ++i)
+            ra[i] = live ? *reinterpret_cast<const uint4*>(ga[i] + (long)kt * 128) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < LB; ++i)
+            rb[i] = live ? *reinterpret_cast<const uint4*>(gb[i] + (long)kt * 128) : make_uint4(0, 0, 0, 0);
+    };
+    auto stage = [&](int buf) {
+        uint8_t* base = smem + buf * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < LA; ++i)
+            *reinterpret_cast<uint4*>(base + sa_off[i]) = ra[i];
+#pragma unroll
+        for (int i = 0; i < LB; ++i)
+            *reinterpret_cast<uint4*>(base + sb_off[i]) = rb[i];
+    };
+
+    // ---- MX block scales: one E8M0 byte per row per 32 elements, fetched per slab straight into registers
+    constexpr int SW = Op::SCALED ? Op::GROUPS_PER_SLAB / 4 : 1;  // dwords of scales per row per slab
+    uint32_t sca[MB][SW], scb[NB][SW], sca_n[MB][SW], scb_n[NB][SW];
+    const uint8_t* gsa[MB];
+    const uint8_t* gsb[NB];
+    const bool has_scales = Op::SCALED && p.sa != nullptr;
+    if (has_scales) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+            gsa[i] = p.sa + (long)min(m0 + wm * Cfg::WTM + i * 32 + l32, p.m - 1) * p.scale_ld;
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+            gsb[j] = p.sb + (long)min(n0 + wn * Cfg::WTN + j * 32 + l32, p.n - 1) * p.scale_ld;
+    }
+    auto load_scales = [&](int kt) {
+        if (has_scales) {
+#pragma unroll
+            for (int w = 0; w < SW; ++w) {
+#pragma unroll
+                for (int i = 0; i < MB; ++i)
+                    sca_n[i][w] = *reinterpret_cast<const uint32_t*>(gsa[i] + (long)kt * (SW * 4) + w * 4);
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+                    scb_n[j][w] = *reinterpret_cast<const uint32_t*>(gsb[j] + (long)kt * (SW * 4) + w * 4);
+            }
+        }
+    };
+
+    // ---- Acc tile (L0C) in registers
+    Acc acc[MB][NB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0;
+        }
+    if (p.c_in != nullptr) {  // TMATMUL_ACC: start from the caller's accumulator
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int gi = m0 + wm * Cfg::WTM + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                    const int gj = n0 + wn * Cfg::WTN + j * 32 + l32;
+                    if (gi < p.m && gj < p.n)
+                        acc[i][j][r] = reinterpret_cast<const typename Op::Elem*>(p.c_in)[(long)gi * p.ldc + gj];
+                }
+    }
+
+    // ---- fragment addressing (TMOV/TEXTRACT): lane reads row l32 of a 32-row block, half lhi of the k-step
+    int fa_row[MB], fb_row[NB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+        fa_row[i] = wm * Cfg::WTM + i * 32 + l32;
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+        fb_row[j] = wn * Cfg::WTN + j * 32 + l32;
+
+    tload(0);
+    load_scales(0);
+    stage(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < k_slabs; ++kt) {
+        const int cur = kt & 1;
+        if (has_scales) {
+#pragma unroll
+            for (int w = 0; w < SW; ++w) {
+#pragma unroll
+                for (int i = 0; i < MB; ++i)
+                    sca[i][w] = sca_n[i][w];
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+                    scb[j][w] = scb_n[j][w];
+            }
+        }
+        if (kt + 1 < k_slabs) {
+            tload(kt + 1);
+            load_scales(kt + 1);
+        }
+        const uint8_t* sA = smem + cur * Cfg::STAGE_BYTES;
+        const uint8_t* sB = sA + Cfg::A_BYTES;
+#pragma unroll
+        for (int s = 0; s < Cfg::KSTEPS; ++s) {
+            uint4 fa[MB][FR], fb[NB][FR];
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+#pragma unroll
+                for (int f = 0; f < FR; ++f) {
+                    const int chunk = (2 * s + lhi) * FR + f;
+                    fa[i][f] = *reinterpret_cast<const uint4*>(sA + fa_row[i] * 128 + swizzle_chunk(fa_row[i], chunk) * 16);
+                }
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+#pragma unroll
+                for (int f = 0; f < FR; ++f) {
+                    const int chunk = (2 * s + lhi) * FR + f;
+                    fb[j][f] = *reinterpret_cast<const uint4*>(sB + fb_row[j] * 128 + swizzle_chunk(fb_row[j], chunk) * 16);
+                }
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    uint32_t xa = 127u, xb = 127u;
+                    if (has_scales) {
+                        const int g = 2 * s + lhi;  // MX group of this lane inside the slab
+                        xa = (sca[i][g >> 2] >> ((g & 3) * 8)) & 0xFFu;
+                        xb = (scb[j][g >> 2] >> ((g & 3) * 8)) & 0xFFu;
+                    }
+                    Op::mma(acc[i][j], fa[i], fb[j], xa, xb);
+                }
+        }
+        if (kt + 1 < k_slabs)
+            stage(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- TSTORE: drain the accumulators through the epilogue
+    const int out_kind = p.out_kind;
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int gj = n0 + wn * Cfg::WTN + j * 32 + l32;
+            float cs = 1.0f;
+            if (out_kind == OUT_W8A8_BF16)
+                cs = gj < p.n ? p.col_scale[gj] : 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int gi = m0 + wm * Cfg::WTM + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                if (gi >= p.m || gj >= p.n)
+                    continue;
+                const long o = (long)gi * p.ldc + gj;
+                auto v = acc[i][j][r];
+                if (p.relu)
+                    v = v > 0 ? v : 0;
+                switch (out_kind) {
+                    case OUT_F32: reinterpret_cast<float*>(p.c)[o] = (float)v; break;
+                    case OUT_F16: reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits((float)v); break;
+                    case OUT_BF16: reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits((float)v); break;
+                    case OUT_I32: reinterpret_cast<int32_t*>(p.c)[o] = (int32_t)v; break;
+                    default: {  // W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16, each step rounded to f32
+                        if (p.acc_out != nullptr)
+                            p.acc_out[o] = (int32_t)v;
+                        const float t = __fmul_rn((float)v, p.row_scale[gi]);
+                        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(__fmul_rn(t, cs));
+                        break;
+                    }
+                }
+            }
+        }
+}
+
+// One launcher per (tile shape, operand type); defined in gemm_tile_<op>.hip, called from gemm.hip.
+// tile: 0 = 256x256 (8 waves), 1 = 128x128 (4 waves), 2 = 64x64 (4 waves)
+enum TileOp { TOP_BF16 = 0, TOP_F16, TOP_I8, TOP_FP8_E4E4, TOP_FP8_E5E5, TOP_FP8_E4E5, TOP_FP8_E5E4, TOP_FP4, TOP_COUNT };
+hipError_t launch_gemm_tile(int tile, int op, const TileGemmParams& p, hipStream_t stream);
+void tile_shape(int tile, int* bm, int* bn);
+
+}  // namespace ptoamd

@@ -1,0 +1,4 @@
+// gemm_tile_kernel instantiated for OpI8
+#define PTOAMD_TILE_OP OpI8
+#define PTOAMD_TILE_FN launch_gemm_tile_i8
+#include "gemm_tile_inst.hpp"

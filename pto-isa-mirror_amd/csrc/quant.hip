@@ -1,0 +1,372 @@
+// TQUANT (INT8 symmetric / asymmetric, MXFP8, MXFP4) and TDEQUANT as HBM-streaming gfx950 kernels.
+// Arithmetic follows the reference CPU simulator step for step (include/pto/cpu/TQuant.hpp, cpu/TDeQuant.hpp) so the
+// codes, shared exponents, group maxima and scalings are bit-identical; citations are given per function.
+#include "common_host.hpp"
+#include "device_types.hpp"
+
+namespace ptoamd {
+
+// ---- scalar pieces (TQuant.hpp:118-252) ---------------------------------------------------------------------
+
+// EncodeE4M3Fn (TQuant.hpp:118-153): nearest finite E4M3 code to clamp(v, +-448), ties to the even code, and a result
+// of zero is always code 0x00.  NV flushes |v| < 2^-10 to a signed zero first.
+template <bool NV>
+__device__ __forceinline__ uint32_t encode_e4m3fn(float v)
+{
+    const uint32_t vb = f2u(v);
+    if ((vb & 0x7FFFFFFFu) > 0x7F800000u)
+        return 0x7Fu;
+    const uint32_t ab0 = vb & 0x7FFFFFFFu;
+    if (NV && ab0 < 0x3A800000u /* 2^-10 */)
+        return (vb >> 31) ? 0x80u : 0x00u;
+    const uint32_t ab = ab0 > 0x43E00000u /* 448 */ ? 0x43E00000u : ab0;
+    uint32_t code;
+    if (ab < 0x3C800000u /* 2^-6: subnormal codes, step 2^-9 */) {
+        code = (uint32_t)__float2int_rn(u2f(ab) * 512.0f);
+    } else {
+        const uint32_t r = ab + 0x7FFFFu + ((ab >> 20) & 1u);  // keep 3 mantissa bits, round to nearest even
+        code = (r >> 20) - (120u << 3);
+    }
+    if (code == 0)
+        return 0;
+    return ((vb >> 31) << 7) | code;
+}
+
+// EncodeE2M1Magic (TQuant.hpp:155-176)
+__device__ __forceinline__ uint32_t encode_e2m1_magic(float v)
+{
+    const uint32_t vb = f2u(v);
+    const uint32_t ab = vb & 0x7FFFFFFFu;
+    if (ab > 0x7F800000u)
+        return 0x7u;
+    const uint32_t sign = (vb >> 28) & 0x8u;
+    if (ab == 0x7F800000u)
+        return sign | 0x7u;
+    uint32_t be = ab >> 23;
+    be = be < 127u ? 127u : (be > 129u ? 129u : be);
+    const uint32_t magic = (be + 22u) << 23;
+    const uint32_t q = f2u(__fadd_rn(u2f(ab), u2f(magic))) - magic;
+    const uint32_t mag = q + ((be - 127u) << 1);
+    return sign | (mag < 7u ? mag : 7u);
+}
+
+// ComputeSharedExponent / ComputeE2M1SharedExponent / ComputeNvSharedExponent (TQuant.hpp:178-222)
+template <int ALG>
+__device__ __forceinline__ uint32_t shared_exponent(float maxabs)
+{
+    const uint32_t bits = f2u(maxabs);
+    if (ALG == PTOAMD_OCP_MXFP8 || ALG == PTOAMD_OCP_MXFP4) {
+        const uint32_t e = (bits & 0x7F800000u) >> 23, mant = bits & 0x7FFFFFu;
+        const uint32_t sub = ALG == PTOAMD_OCP_MXFP8 ? 8u : 2u;
+        if (e == 0xFFu && mant != 0)
+            return 0xFFu;
+        return e <= sub ? 0u : e - sub;
+    }
+    if (maxabs == 0.0f)
+        return 0;
+    const float descale = __fmul_rn(maxabs, ALG == PTOAMD_NV_MXFP8 ? (1.0f / 448.0f) : (1.0f / 6.0f));
+    const uint32_t db = f2u(descale);
+    const uint32_t e = (db & 0x7F800000u) >> 23, mant = db & 0x7FFFFFu;
+    if (e == 0xFFu)
+        return mant == 0 ? 0xFEu : 0xFFu;
+    const bool up = mant > 0 && e != 0xFEu && !(e == 0 && mant <= 0x00400000u);
+    return (e + (up ? 1u : 0u)) & 0xFFu;
+}
+
+// ComputeMxGroupScaling (TQuant.hpp:226-252, 336-347)
+template <int ALG>
+__device__ __forceinline__ float group_scaling(float maxabs, uint32_t e8m0)
+{
+    if (e8m0 == 0xFFu)
+        return maxabs;
+    if ((ALG == PTOAMD_NV_MXFP8 || ALG == PTOAMD_NV_MXFP4) && e8m0 == 0xFEu)
+        return u2f(0x00400000u);  // 2^-127
+    const uint32_t b = (254u - e8m0) << 23;
+    return b == 0 ? u2f(0x00400000u) : u2f(b);
+}
+
+// ComputeMxGroupMax's per-element step (TQuant.hpp:280-306).  The running value is kept as bits: for OCP-FP4 it is
+// the maximum of truncated-bf16 magnitude patterns, otherwise max(fabs) where NaN never wins (NV-FP4: NaN wins).
+template <int ALG>
+__device__ __forceinline__ uint32_t max_step(uint32_t run, float v)
+{
+    const uint32_t ab = f2u(v) & 0x7FFFFFFFu;
+    if (ALG == PTOAMD_OCP_MXFP4) {
+        const uint32_t t = ab & 0x7FFF0000u;
+        return t > run ? t : run;
+    }
+    if (ab > 0x7F800000u)                               // NaN
+        return ALG == PTOAMD_NV_MXFP4 ? 0xFFFFFFFFu : run;  // sentinel: the group maximum is NaN
+    return (run != 0xFFFFFFFFu && ab > run) ? ab : run;
+}
+template <int ALG>
+__device__ __forceinline__ uint32_t max_merge(uint32_t a, uint32_t b)
+{
+    return a > b ? a : b;  // bit patterns of non-negative floats order like the floats; the NaN sentinel is largest
+}
+template <int ALG>
+__device__ __forceinline__ float max_value(uint32_t run, float first_nan)
+{
+    if (ALG == PTOAMD_NV_MXFP4 && run == 0xFFFFFFFFu)
+        return first_nan;
+    return u2f(run);
+}
+
+template <typename T>
+__device__ __forceinline__ float widen(T v);
+template <>
+__device__ __forceinline__ float widen<float>(float v) { return v; }
+struct half_bits { uint16_t b; };
+struct bf16_bits { uint16_t b; };
+template <>
+__device__ __forceinline__ float widen<half_bits>(half_bits v) { return f16_bits_to_f32(v.b); }
+template <>
+__device__ __forceinline__ float widen<bf16_bits>(bf16_bits v) { return bf16_bits_to_f32(v.b); }
+
+// StoreMxEncodedValue (TQuant.hpp:349-372)
+template <int ALG, bool SRC_BF16>
+__device__ __forceinline__ uint32_t encode_mx(float v, float scaling)
+{
+    if (ALG == PTOAMD_OCP_MXFP8 || ALG == PTOAMD_NV_MXFP8)
+        return encode_e4m3fn<ALG == PTOAMD_NV_MXFP8>(__fmul_rn(v, scaling));
+    const uint32_t sb = f2u(scaling);
+    if ((sb & 0x7FFFFFFFu) == 0x7F800000u)
+        return (sb >> 31) ? 0xFu : 0x7u;
+    if ((sb & 0x7FFFFFFFu) > 0x7F800000u)
+        return 0x7u;
+    float scaled = __fmul_rn(v, scaling);
+    if (SRC_BF16)  // bf16 sources re-round the scaled value to bf16 (TQuant.hpp:68-76)
+        scaled = bf16_bits_to_f32(f32_to_bf16_bits(scaled));
+    return encode_e2m1_magic(scaled);
+}
+
+// ---- axis 1: 32-element groups along a row.  8 lanes own one group, 4 consecutive elements each. --------------
+template <int ALG, typename T, bool SRC_BF16>
+__global__ void tquant_mx_rows_kernel(uint8_t* dst, uint8_t* exp, float* mx, float* scaling, const T* src, long groups)
+{
+    constexpr bool FP4 = ALG == PTOAMD_OCP_MXFP4 || ALG == PTOAMD_NV_MXFP4;
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long g = t >> 3;  // all 8 lanes of a group are in or out together (blockDim is a multiple of 8)
+    const bool live = g < groups;
+    float v[4] = {0, 0, 0, 0};
+    if (live) {
+        const T* p = src + g * 32 + (t & 7) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            v[i] = widen<T>(p[i]);
+    }
+    uint32_t run = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        run = max_step<ALG>(run, v[i]);
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1)
+        run = max_merge<ALG>(run, (uint32_t)__shfl_xor((int)run, off, 8));
+    if (!live)
+        return;
+    const float maxabs = max_value<ALG>(run, u2f(0x7FC00000u));
+    const uint32_t e = shared_exponent<ALG>(maxabs);
+    const float sc = group_scaling<ALG>(maxabs, e);
+    if ((t & 7) == 0) {
+        exp[g] = (uint8_t)e;
+        if (mx)
+            mx[g] = maxabs;
+        if (scaling)
+            scaling[g] = sc;
+    }
+    uint32_t c[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        c[i] = encode_mx<ALG, SRC_BF16>(v[i], sc);
+    if (FP4) {
+        reinterpret_cast<uint16_t*>(dst)[g * 8 + (t & 7)] = (uint16_t)(c[0] | (c[1] << 4) | (c[2] << 8) | (c[3] << 12));
+    } else {
+        reinterpret_cast<uint32_t*>(dst)[g * 8 + (t & 7)] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+    }
+}
+
+// ---- axis 0: 32-element groups along a column.  One thread owns two adjacent columns of one group. -----------
+template <int ALG, typename T, bool SRC_BF16>
+__global__ void tquant_mx_cols_kernel(uint8_t* dst, uint8_t* exp, float* mx, float* scaling, const T* src, int rows,
+                                      int cols)
+{
+    constexpr bool FP4 = ALG == PTOAMD_OCP_MXFP4 || ALG == PTOAMD_NV_MXFP4;
+    const int cp = blockIdx.x * blockDim.x + threadIdx.x;  // column pair
+    const int g = blockIdx.y;
+    if (cp * 2 >= cols)
+        return;
+    const T* p = src + (long)g * 32 * cols + cp * 2;
+    uint32_t run[2] = {0, 0};
+    for (int r = 0; r < 32; ++r) {
+        run[0] = max_step<ALG>(run[0], widen<T>(p[(long)r * cols]));
+        run[1] = max_step<ALG>(run[1], widen<T>(p[(long)r * cols + 1]));
+    }
+    float sc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const float maxabs = max_value<ALG>(run[j], u2f(0x7FC00000u));
+        const uint32_t e = shared_exponent<ALG>(maxabs);
+        sc[j] = group_scaling<ALG>(maxabs, e);
+        const long gi = (long)g * cols + cp * 2 + j;
+        exp[gi] = (uint8_t)e;
+        if (mx)
+            mx[gi] = maxabs;
+        if (scaling)
+            scaling[gi] = sc[j];
+    }
+    for (int r = 0; r < 32; ++r) {
+        const uint32_t c0 = encode_mx<ALG, SRC_BF16>(widen<T>(p[(long)r * cols]), sc[0]);
+        const uint32_t c1 = encode_mx<ALG, SRC_BF16>(widen<T>(p[(long)r * cols + 1]), sc[1]);
+        const long idx = ((long)g * 32 + r) * cols + cp * 2;
+        if (FP4)
+            dst[idx >> 1] = (uint8_t)(c0 | (c1 << 4));
+        else
+            reinterpret_cast<uint16_t*>(dst)[idx >> 1] = (uint16_t)(c0 | (c1 << 8));
+    }
+}
+
+// ---- TQUANT INT8 (TQuant.hpp:86-96, 496-522): the "scale" operand multiplies -----------------------------------
+template <bool ASYM>
+__global__ void tquant_int8_kernel(uint8_t* dst, const float* src, const float* scale, const float* offset, int rows,
+                                   int cols)
+{
+    const long idx4 = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    const long total = (long)rows * cols;
+    if (idx4 >= total)
+        return;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const long idx = idx4 + i;
+        if (idx >= total)
+            break;
+        const int r = (int)(idx / cols);
+        float v = __fmul_rn(src[idx], scale[r]);
+        if (ASYM)
+            v = __fadd_rn(v, offset[r]);
+        v = rintf(v);
+        const float lo = ASYM ? 0.0f : -128.0f, hi = ASYM ? 255.0f : 127.0f;
+        v = v < lo ? lo : (v > hi ? hi : v);
+        const int q = (int)v;
+        packed |= ((uint32_t)q & 0xFFu) << (8 * i);
+    }
+    if (idx4 + 4 <= total && (total & 3) == 0) {
+        reinterpret_cast<uint32_t*>(dst)[idx4 >> 2] = packed;
+    } else {
+        for (int i = 0; i < 4 && idx4 + i < total; ++i)
+            dst[idx4 + i] = (uint8_t)(packed >> (8 * i));
+    }
+}
+
+// ---- TDEQUANT (TDeQuant.hpp:18-37) ---------------------------------------------------------------------------
+template <typename T>
+__global__ void tdequant_kernel(float* dst, const T* src, const float* scale, const float* offset, int rows, int cols)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long)rows * cols)
+        return;
+    const int r = (int)(idx / cols);
+    dst[idx] = __fmul_rn(__fsub_rn((float)src[idx], offset[r]), scale[r]);
+}
+
+template <int ALG, typename T, bool SRC_BF16>
+static int launch_tquant_mx(uint8_t* dst, uint8_t* exp, float* mx, float* scaling, const void* src, int rows, int cols,
+                            int axis, hipStream_t stream)
+{
+    const T* s = reinterpret_cast<const T*>(src);
+    if (axis == 1) {
+        const long groups = (long)rows * (cols / 32);
+        const long threads = groups * 8;
+        hipLaunchKernelGGL((tquant_mx_rows_kernel<ALG, T, SRC_BF16>), dim3((unsigned)((threads + 255) / 256)), dim3(256),
+                           0, stream, dst, exp, mx, scaling, s, groups);
+    } else {
+        dim3 block(128), grid((cols / 2 + 127) / 128, rows / 32);
+        hipLaunchKernelGGL((tquant_mx_cols_kernel<ALG, T, SRC_BF16>), grid, block, 0, stream, dst, exp, mx, scaling, s,
+                           rows, cols);
+    }
+    PTOAMD_HIP_CHECK(hipGetLastError());
+    return PTOAMD_OK;
+}
+
+template <int ALG>
+static int dispatch_src(uint8_t* dst, uint8_t* exp, float* mx, float* scaling, const void* src, int src_type, int rows,
+                        int cols, int axis, hipStream_t stream)
+{
+    switch (src_type) {
+        case PTOAMD_F32: return launch_tquant_mx<ALG, float, false>(dst, exp, mx, scaling, src, rows, cols, axis, stream);
+        case PTOAMD_F16: return launch_tquant_mx<ALG, half_bits, false>(dst, exp, mx, scaling, src, rows, cols, axis, stream);
+        default: return launch_tquant_mx<ALG, bf16_bits, true>(dst, exp, mx, scaling, src, rows, cols, axis, stream);
+    }
+}
+
+}  // namespace ptoamd
+
+using namespace ptoamd;
+
+extern "C" {
+
+int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const float* offset, int rows, int cols,
+                       void* stream)
+{
+    PTOAMD_REQUIRE(dst && src && scale, PTOAMD_E_INVALID, "ptoamd_tquant_int8: null operand");
+    PTOAMD_REQUIRE(rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_tquant_int8: rows and cols must be positive");
+    const long total = (long)rows * cols;
+    const unsigned blocks = (unsigned)((total / 4 + 256) / 256);
+    if (offset)
+        hipLaunchKernelGGL(tquant_int8_kernel<true>, dim3(blocks), dim3(256), 0, as_stream(stream),
+                           reinterpret_cast<uint8_t*>(dst), src, scale, offset, rows, cols);
+    else
+        hipLaunchKernelGGL(tquant_int8_kernel<false>, dim3(blocks), dim3(256), 0, as_stream(stream),
+                           reinterpret_cast<uint8_t*>(dst), src, scale, offset, rows, cols);
+    PTOAMD_HIP_CHECK(hipGetLastError());
+    return PTOAMD_OK;
+}
+
+int ptoamd_tquant_mx(uint8_t* dst, uint8_t* exp, float* max, float* scaling, const void* src, int src_type, int rows,
+                     int cols, int alg, int axis, void* stream)
+{
+    PTOAMD_REQUIRE(dst && exp && src, PTOAMD_E_INVALID, "ptoamd_tquant_mx: null operand");
+    PTOAMD_REQUIRE(rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_tquant_mx: rows and cols must be positive");
+    PTOAMD_REQUIRE(axis == 0 || axis == 1, PTOAMD_E_INVALID, "ptoamd_tquant_mx: axis must be 0 or 1");
+    PTOAMD_REQUIRE(src_type == PTOAMD_F32 || src_type == PTOAMD_F16 || src_type == PTOAMD_BF16, PTOAMD_E_UNSUPPORTED,
+                   "ptoamd_tquant_mx: the source must be f32, f16 or bf16");
+    PTOAMD_REQUIRE(axis == 1 ? cols % 32 == 0 : rows % 32 == 0, PTOAMD_E_INVALID,
+                   "ptoamd_tquant_mx: the grouped axis must be a multiple of 32 (rows %d, cols %d, axis %d)", rows, cols, axis);
+    PTOAMD_REQUIRE(cols % 2 == 0, PTOAMD_E_INVALID, "ptoamd_tquant_mx: cols must be even");
+    PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(dst) & 3u) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0,
+                   PTOAMD_E_ALIGNMENT, "ptoamd_tquant_mx: dst must be 4-byte and src 16-byte aligned");
+    hipStream_t s = as_stream(stream);
+    switch (alg) {
+        case PTOAMD_OCP_MXFP8: return dispatch_src<PTOAMD_OCP_MXFP8>(dst, exp, max, scaling, src, src_type, rows, cols, axis, s);
+        case PTOAMD_NV_MXFP8: return dispatch_src<PTOAMD_NV_MXFP8>(dst, exp, max, scaling, src, src_type, rows, cols, axis, s);
+        case PTOAMD_OCP_MXFP4: return dispatch_src<PTOAMD_OCP_MXFP4>(dst, exp, max, scaling, src, src_type, rows, cols, axis, s);
+        case PTOAMD_NV_MXFP4: return dispatch_src<PTOAMD_NV_MXFP4>(dst, exp, max, scaling, src, src_type, rows, cols, axis, s);
+        default: set_error("ptoamd_tquant_mx: unknown algorithm %d", alg); return PTOAMD_E_INVALID;
+    }
+}
+
+int ptoamd_tdequant(float* dst, const void* src, int src_type, const float* scale, const float* offset, int rows,
+                    int cols, void* stream)
+{
+    PTOAMD_REQUIRE(dst && src && scale && offset, PTOAMD_E_INVALID, "ptoamd_tdequant: null operand");
+    PTOAMD_REQUIRE(rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_tdequant: rows and cols must be positive");
+    const long total = (long)rows * cols;
+    const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    hipStream_t s = as_stream(stream);
+    switch (src_type) {
+        case PTOAMD_I8:
+            hipLaunchKernelGGL(tdequant_kernel<int8_t>, grid, block, 0, s, dst, reinterpret_cast<const int8_t*>(src), scale, offset, rows, cols);
+            break;
+        case PTOAMD_I16:
+            hipLaunchKernelGGL(tdequant_kernel<int16_t>, grid, block, 0, s, dst, reinterpret_cast<const int16_t*>(src), scale, offset, rows, cols);
+            break;
+        case PTOAMD_I32:
+            hipLaunchKernelGGL(tdequant_kernel<int32_t>, grid, block, 0, s, dst, reinterpret_cast<const int32_t*>(src), scale, offset, rows, cols);
+            break;
+        default: set_error("ptoamd_tdequant: source type %d is not int8, int16 or int32", src_type); return PTOAMD_E_UNSUPPORTED;
+    }
+    PTOAMD_HIP_CHECK(hipGetLastError());
+    return PTOAMD_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,193 @@
+// Host runtime of the gfx950 backend: the counterpart of the fake aclrt* runtime the reference's tests and demos use
+// (include/pto/common/cpu_stub.hpp:73-120, 524-555), on the HIP runtime.
+#include <string.h>
+
+#include "common_host.hpp"
+
+namespace ptoamd {
+static thread_local char g_error[512] = "";
+static thread_local char g_kernel[64] = "";
+
+void set_error(const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+}
+void set_last_kernel(const char* name)
+{
+    strncpy(g_kernel, name, sizeof g_kernel - 1);
+    g_kernel[sizeof g_kernel - 1] = 0;
+}
+}  // namespace ptoamd
+
+using namespace ptoamd;
+
+extern "C" {
+
+const char* ptoamd_last_error(void) { return g_error; }
+const char* ptoamd_last_kernel(void) { return g_kernel; }
+
+int ptoamd_init(int device)
+{
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        set_error("no HIP device visible");
+        return PTOAMD_E_NODEVICE;
+    }
+    PTOAMD_REQUIRE(device >= 0 && device < count, PTOAMD_E_INVALID, "device %d out of range (0..%d)", device, count - 1);
+    PTOAMD_HIP_CHECK(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    PTOAMD_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+        return PTOAMD_E_NODEVICE;
+    }
+    return PTOAMD_OK;
+}
+
+int ptoamd_finalize(void)
+{
+    PTOAMD_HIP_CHECK(hipDeviceSynchronize());
+    return PTOAMD_OK;
+}
+
+int ptoamd_device_info(int* compute_units, int* clock_khz, size_t* hbm_bytes, char* arch, size_t arch_len)
+{
+    int dev = 0;
+    PTOAMD_HIP_CHECK(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    PTOAMD_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+    if (compute_units)
+        *compute_units = prop.multiProcessorCount;
+    if (clock_khz)
+        *clock_khz = prop.clockRate;
+    if (hbm_bytes)
+        *hbm_bytes = prop.totalGlobalMem;
+    if (arch && arch_len) {
+        strncpy(arch, prop.gcnArchName, arch_len - 1);
+        arch[arch_len - 1] = 0;
+    }
+    return PTOAMD_OK;
+}
+
+int ptoamd_malloc(void** dev_ptr, size_t bytes)
+{
+    PTOAMD_REQUIRE(dev_ptr != nullptr && bytes > 0, PTOAMD_E_INVALID, "ptoamd_malloc: null result pointer or zero size");
+    PTOAMD_HIP_CHECK(hipMalloc(dev_ptr, bytes));
+    return PTOAMD_OK;
+}
+int ptoamd_free(void* dev_ptr)
+{
+    PTOAMD_HIP_CHECK(hipFree(dev_ptr));
+    return PTOAMD_OK;
+}
+int ptoamd_malloc_host(void** host_ptr, size_t bytes)
+{
+    PTOAMD_REQUIRE(host_ptr != nullptr && bytes > 0, PTOAMD_E_INVALID, "ptoamd_malloc_host: null result pointer or zero size");
+    PTOAMD_HIP_CHECK(hipHostMalloc(host_ptr, bytes, hipHostMallocDefault));
+    return PTOAMD_OK;
+}
+int ptoamd_free_host(void* host_ptr)
+{
+    PTOAMD_HIP_CHECK(hipHostFree(host_ptr));
+    return PTOAMD_OK;
+}
+
+static int to_kind(int kind, hipMemcpyKind* out)
+{
+    switch (kind) {
+        case PTOAMD_MEMCPY_H2H: *out = hipMemcpyHostToHost; return 0;
+        case PTOAMD_MEMCPY_H2D: *out = hipMemcpyHostToDevice; return 0;
+        case PTOAMD_MEMCPY_D2H: *out = hipMemcpyDeviceToHost; return 0;
+        case PTOAMD_MEMCPY_D2D: *out = hipMemcpyDeviceToDevice; return 0;
+        default: return -1;
+    }
+}
+
+int ptoamd_memcpy(void* dst, size_t dst_bytes, const void* src, size_t count, int kind)
+{
+    hipMemcpyKind k;
+    PTOAMD_REQUIRE(to_kind(kind, &k) == 0, PTOAMD_E_INVALID, "ptoamd_memcpy: unknown kind %d", kind);
+    PTOAMD_REQUIRE(count <= dst_bytes, PTOAMD_E_INVALID, "ptoamd_memcpy: count %zu exceeds destination size %zu", count,
+                   dst_bytes);
+    if (count == 0)
+        return PTOAMD_OK;
+    PTOAMD_REQUIRE(dst != nullptr && src != nullptr, PTOAMD_E_INVALID, "ptoamd_memcpy: null pointer");
+    PTOAMD_HIP_CHECK(hipMemcpy(dst, src, count, k));
+    return PTOAMD_OK;
+}
+int ptoamd_memcpy_async(void* dst, size_t dst_bytes, const void* src, size_t count, int kind, void* stream)
+{
+    hipMemcpyKind k;
+    PTOAMD_REQUIRE(to_kind(kind, &k) == 0, PTOAMD_E_INVALID, "ptoamd_memcpy_async: unknown kind %d", kind);
+    PTOAMD_REQUIRE(count <= dst_bytes, PTOAMD_E_INVALID, "ptoamd_memcpy_async: count %zu exceeds destination size %zu",
+                   count, dst_bytes);
+    if (count == 0)
+        return PTOAMD_OK;
+    PTOAMD_REQUIRE(dst != nullptr && src != nullptr, PTOAMD_E_INVALID, "ptoamd_memcpy_async: null pointer");
+    PTOAMD_HIP_CHECK(hipMemcpyAsync(dst, src, count, k, as_stream(stream)));
+    return PTOAMD_OK;
+}
+int ptoamd_memset(void* dev_ptr, size_t dst_bytes, int value, size_t count)
+{
+    PTOAMD_REQUIRE(count <= dst_bytes, PTOAMD_E_INVALID, "ptoamd_memset: count %zu exceeds destination size %zu", count,
+                   dst_bytes);
+    if (count == 0)
+        return PTOAMD_OK;
+    PTOAMD_REQUIRE(dev_ptr != nullptr, PTOAMD_E_INVALID, "ptoamd_memset: null pointer");
+    PTOAMD_HIP_CHECK(hipMemset(dev_ptr, value, count));
+    return PTOAMD_OK;
+}
+
+int ptoamd_stream_create(void** stream)
+{
+    PTOAMD_REQUIRE(stream != nullptr, PTOAMD_E_INVALID, "ptoamd_stream_create: null result pointer");
+    hipStream_t s;
+    PTOAMD_HIP_CHECK(hipStreamCreate(&s));
+    *stream = s;
+    return PTOAMD_OK;
+}
+int ptoamd_stream_destroy(void* stream)
+{
+    PTOAMD_HIP_CHECK(hipStreamDestroy(as_stream(stream)));
+    return PTOAMD_OK;
+}
+int ptoamd_stream_synchronize(void* stream)
+{
+    PTOAMD_HIP_CHECK(hipStreamSynchronize(as_stream(stream)));
+    return PTOAMD_OK;
+}
+
+int ptoamd_event_create(void** event)
+{
+    PTOAMD_REQUIRE(event != nullptr, PTOAMD_E_INVALID, "ptoamd_event_create: null result pointer");
+    hipEvent_t e;
+    PTOAMD_HIP_CHECK(hipEventCreate(&e));
+    *event = e;
+    return PTOAMD_OK;
+}
+int ptoamd_event_destroy(void* event)
+{
+    PTOAMD_HIP_CHECK(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+    return PTOAMD_OK;
+}
+int ptoamd_event_record(void* event, void* stream)
+{
+    PTOAMD_HIP_CHECK(hipEventRecord(reinterpret_cast<hipEvent_t>(event), as_stream(stream)));
+    return PTOAMD_OK;
+}
+int ptoamd_event_synchronize(void* event)
+{
+    PTOAMD_HIP_CHECK(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)));
+    return PTOAMD_OK;
+}
+int ptoamd_event_elapsed_ms(float* ms, void* start, void* stop)
+{
+    PTOAMD_REQUIRE(ms != nullptr, PTOAMD_E_INVALID, "ptoamd_event_elapsed_ms: null result pointer");
+    PTOAMD_HIP_CHECK(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(stop)));
+    return PTOAMD_OK;
+}
+
+}  // extern "C"
