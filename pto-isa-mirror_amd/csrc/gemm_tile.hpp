@@ -114,6 +114,18 @@ struct OpFP4 {
 // 16-byte chunk swizzle inside a 128-byte slab row: consecutive rows land in different banks for ds_read_b128
 __device__ __forceinline__ int swizzle_chunk(int row, int chunk) { return chunk ^ ((row >> 1) & 7) ^ ((row & 1) << 2); }
 
+// Which 16-byte chunk of a slab row holds piece f of lane-half lhi's fragment for k-step s.
+// 16-byte fragments: the two lane halves take consecutive chunks.  32-byte fp8 fragments of the 32x32x64 scaled MFMA:
+// registers 0-3 of a lane belong to the k-step's first MX block (32 elements) and registers 4-7 to its second, each
+// block being split 16 + 16 bytes over the two lane halves, while lane half h supplies the E8M0 scale of block h.
+template <int FR>
+__device__ __forceinline__ int frag_chunk(int s, int lhi, int f)
+{
+    if (FR == 1)
+        return 2 * s + lhi;
+    return 4 * s + 2 * f + lhi;
+}
+
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, class Op_>
 struct TileCfg {
     static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
@@ -288,14 +300,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
             for (int i = 0; i < MB; ++i)
 #pragma unroll
                 for (int f = 0; f < FR; ++f) {
-                    const int chunk = (2 * s + lhi) * FR + f;
+                    const int chunk = frag_chunk<FR>(s, lhi, f);
                     fa[i][f] = *reinterpret_cast<const uint4*>(sA + fa_row[i] * 128 + swizzle_chunk(fa_row[i], chunk) * 16);
                 }
 #pragma unroll
             for (int j = 0; j < NB; ++j)
 #pragma unroll
                 for (int f = 0; f < FR; ++f) {
-                    const int chunk = (2 * s + lhi) * FR + f;
+                    const int chunk = frag_chunk<FR>(s, lhi, f);
                     fb[j][f] = *reinterpret_cast<const uint4*>(sB + fb_row[j] * 128 + swizzle_chunk(fb_row[j], chunk) * 16);
                 }
 #pragma unroll
