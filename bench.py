@@ -1,0 +1,209 @@
+"""Throughput of the PTO tile-matmul hot path on one MI355X, with roofline fraction and a CPU baseline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+A "step" is one TLOAD -> TMATMUL_ACC -> TSTORE pass over one synthetic batch.  The headline workload is
+BASELINE.json configs[1] (bf16 GEMM, M = N = K = 4096, A row-major, B column-major, N(0,1) * 0.02, fp32 accumulate,
+bf16 output); inputs are resident in HBM before the timed region.  The other configs are measured once each after the
+headline and reported under "per_config" (the metric is "per GEMM config").  One JSON line goes to stdout.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as ge  # noqa: E402
+
+METRIC = "TFLOP/s (or GB/s) + % of MI355X roofline per GEMM config, 1 GPU"
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "int8": 5000.0, "fp8": 5000.0, "fp4": 10100.0}
+PEAK_HBM_GBPS = 8000.0
+DEV = "cuda:0"
+
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of
+# known size); filled in from profiles/ once measured, None until then.
+HEADLINE_TRAFFIC_BYTES = None
+
+
+class Events:
+    """HIP events recorded on torch's current stream through the library's C ABI."""
+
+    def __init__(self, pa):
+        import ctypes as C
+        self.C, self.lib = C, pa.lib()
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        assert self.lib.ptoamd_event_create(C.byref(self.e0)) == 0 and self.lib.ptoamd_event_create(C.byref(self.e1)) == 0
+
+    def _stream(self):
+        return self.C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def start(self):
+        assert self.lib.ptoamd_event_record(self.e0, self._stream()) == 0
+
+    def stop_ms(self):
+        assert self.lib.ptoamd_event_record(self.e1, self._stream()) == 0
+        assert self.lib.ptoamd_event_synchronize(self.e1) == 0
+        ms = self.C.c_float()
+        assert self.lib.ptoamd_event_elapsed_ms(self.C.byref(ms), self.e0, self.e1) == 0
+        return float(ms.value)
+
+
+def time_launches(ev, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev.start()
+    for _ in range(steps):
+        fn()
+    kernel_ms = ev.stop_ms() / steps
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return wall_ms, kernel_ms
+
+
+def randn_bf16(shape, gen, scale=1.0):
+    return (torch.randn(shape, generator=gen, device=DEV) * scale).to(torch.bfloat16)
+
+
+def config1(pa, ev, gen, steps, warmup):
+    a = (torch.rand((512, 512), generator=gen, device=DEV) * 2 - 1).to(torch.float16)
+    b = (torch.rand((512, 512), generator=gen, device=DEV) * 2 - 1).to(torch.float16)
+    out = torch.empty((512, 512), dtype=torch.float32, device=DEV)
+    wall, ker = time_launches(ev, lambda: pa.gemm(a, b, pa.F16, pa.F32, pa.B_ND, out=out), steps, warmup)
+    flops = 2 * 512 ** 3
+    return dict(config="configs[0] fp16 512^3 -> fp32, B row-major", kernel=pa.last_kernel(), ms=ker, wall_ms=wall,
+                tflops=flops / ker / 1e9, bound="latency", frac_of_peak=flops / ker / 1e9 / PEAK_TFLOPS["f16"])
+
+
+def config3(pa, ev, gen, steps, warmup):
+    m, n, k = 2048, 8192, 8192
+    a = torch.randint(-127, 128, (m, k), generator=gen, device=DEV, dtype=torch.int8)
+    b = torch.randint(-127, 128, (n, k), generator=gen, device=DEV, dtype=torch.int8)
+    sa = torch.rand(m, generator=gen, device=DEV) * 0.01 + 0.001
+    sb = torch.rand(n, generator=gen, device=DEV) * 0.01 + 0.001
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    wall, ker = time_launches(ev, lambda: pa.gemm_w8a8(a, b, sa, sb, out=out), steps, warmup)
+    ops = 2 * m * n * k
+    return dict(config="configs[2] W8A8 int8 2048x8192x8192 -> bf16, fused dequant", kernel=pa.last_kernel(), ms=ker,
+                wall_ms=wall, tflops=ops / ker / 1e9, bound="mfma", frac_of_peak=ops / ker / 1e9 / PEAK_TFLOPS["int8"])
+
+
+def config4(pa, ev, gen, steps, warmup):
+    m, n, k = 4096, 14336, 4096
+    a, sa = pa.tquant_mx(torch.randn((m, k), generator=gen, device=DEV), pa.OCP_MXFP8, want_aux=False)
+    b, sb = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP8, want_aux=False)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    wall, ker = time_launches(ev, lambda: pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E4M3, pa.E4M3, pa.BF16, out=out), steps,
+                              warmup)
+    flops = 2 * m * n * k
+    return dict(config="configs[3] MXFP8 E4M3 4096x14336x4096 -> bf16", kernel=pa.last_kernel(), ms=ker, wall_ms=wall,
+                tflops=flops / ker / 1e9, bound="mfma", frac_of_peak=flops / ker / 1e9 / PEAK_TFLOPS["fp8"])
+
+
+def config5(pa, ev, gen, steps, warmup):
+    m, n, k = 16, 28672, 8192
+    a = randn_bf16((m, k), gen)
+    # four weight copies (4 x 125 MB) rotated between launches so every launch streams from HBM, not the 256 MB MALL
+    copies = []
+    for _ in range(4):
+        w, sw = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
+        copies.append((w, sw))
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    state = {"i": 0}
+
+    def step():
+        w, sw = copies[state["i"] % 4]
+        state["i"] += 1
+        pa.gemv_mxfp4(a, w, sw, n, k, pa.BF16, out=out)
+
+    wall, ker = time_launches(ev, step, steps, warmup)
+    nbytes = n * k // 2 + n * k // 32 + m * k * 2 + m * n * 2
+    return dict(config="configs[4] MXFP4 decode GEMV 16x28672x8192 -> bf16 (weights rotated over 4 copies)",
+                kernel=pa.last_kernel(), ms=ker, wall_ms=wall, gbps=nbytes / ker / 1e6, bound="hbm",
+                frac_of_peak=nbytes / ker / 1e6 / PEAK_HBM_GBPS)
+
+
+def cpu_baseline():
+    """The CPU-simulator-shaped port (oracle/pto_oracle.c: per-element fractal addressing, per-TMATMUL thread
+    fan-out) on a bounded slab of the headline workload: 256 output rows x 4096 columns x K = 4096."""
+    from oracle.binding import Oracle, ST_BF16
+
+    orc = Oracle()
+    rng = np.random.default_rng(0)
+    m, n, k = 256, 4096, 4096
+    a = ((rng.standard_normal((m, k)) * 0.02).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    b = ((rng.standard_normal((n, k)) * 0.02).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    t0 = time.perf_counter()
+    _, threads = orc.sim_gemm_tiled(a, b, 1, ST_BF16, b_dn=True, max_threads=16)
+    dt = time.perf_counter() - t0
+    gflops = 2 * m * n * k / dt / 1e9
+    return {"value": gflops / 1e3, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"256 of 4096 output rows x N=4096 x K=4096 (8.6 GFLOP) in {dt:.1f} s; "
+                      f"full 4096^3 extrapolates to {dt * 16:.0f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the per-config measurements after the headline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: every box of this build has one MI355X and the path needs no second "
+                 "(C tiles are independent; see DESIGN.md on sharding). Run with --gpus 1.")
+
+    pa = ge.load_package()
+    pa.init(0)
+    ev = Events(pa)
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=DEV)  # 256 MiB read + 256 MiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    gen = torch.Generator(device=DEV).manual_seed(1)
+
+    m = n = k = 4096
+    a = randn_bf16((m, k), gen, 0.02)
+    b = randn_bf16((n, k), gen, 0.02)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    wall_ms, kernel_ms = time_launches(ev, lambda: pa.gemm(a, b, pa.BF16, pa.BF16, pa.B_DN, out=out), args.steps,
+                                       args.warmup)
+    kernel = pa.last_kernel()
+    flops = 2 * m * n * k
+    value = flops / wall_ms / 1e9
+    achieved = flops / kernel_ms / 1e9
+    line = {
+        "metric": METRIC, "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: bf16 GEMM M=N=K=4096, A row-major, B column-major, N(0,1)*0.02, "
+                               "fp32 accumulate, bf16 output", "kernel": kernel},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_TFLOPS["bf16"], "traffic": HEADLINE_TRAFFIC_BYTES,
+                     "kernel_ms": kernel_ms, "algorithmic_flops_per_launch": flops},
+    }
+    if not args.no_extra:
+        per = []
+        for fn in (config1, config3, config4, config5):
+            per.append(fn(pa, ev, gen, 20, 5))
+            torch.cuda.empty_cache()
+        line["per_config"] = per
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
