@@ -35,8 +35,11 @@ hipError_t launch_gemm_tile(int tile, int op, const TileGemmParams& p, hipStream
 
 void tile_shape(int tile, int* bm, int* bn)
 {
-    static const int shapes[3] = {256, 128, 64};
-    *bm = *bn = shapes[tile < 0 || tile > 2 ? 2 : tile];
+    static const int bms[7] = {256, 128, 64, 256, 256, 128, 256};
+    static const int bns[7] = {256, 128, 64, 256, 256, 128, 128};
+    const int t = tile < 0 || tile > 6 ? 2 : tile;
+    *bm = bms[t];
+    *bn = bns[t];
 }
 
 // ---- MX scale GM layouts (reference: cpu/tile_offsets.hpp:233-268 with the strides of pto_tile.hpp:849-1102) ----
@@ -198,17 +201,28 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 // Which tile shape to run: the largest whose grid still fills most of the 256 CUs.  PTOAMD_TILE=0|1|2 overrides,
 // PTOAMD_FORCE_GENERIC=1 sends everything to the order-exact kernel (used by the parity tests).
-static int pick_tile(int m, int n)
+// Tiles 0-2 stage slabs through registers (any K that is a multiple of 16 bytes); tiles 3-6 DMA slabs straight into
+// LDS and need K to be a whole number of 128-byte slabs.  Measured on MI355X: the 8-wave 256x256 DMA tile (4) is the
+// fastest for bf16 / f16 / int8 once the grid fills the chip; the block-scaled operand types keep more registers live
+// per MFMA and run best on the 128x128 DMA tile (5), two workgroups per CU.
+static int pick_tile(int m, int n, long k_bytes, bool scaled)
 {
+    const bool dtl_ok = (k_bytes % 128) == 0;
     const char* env = getenv("PTOAMD_TILE");
-    if (env && env[0] >= '0' && env[0] <= '2')
-        return env[0] - '0';
+    if (env && env[0] >= '0' && env[0] <= '6') {
+        const int t = env[0] - '0';
+        if (t < 3 || dtl_ok)
+            return t;
+        return t == 5 ? 1 : 0;
+    }
     const long t256 = (long)((m + 255) / 256) * ((n + 255) / 256);
-    if (t256 >= 128)
-        return 0;
     const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128);
+    if (scaled)
+        return t128 >= 96 ? (dtl_ok ? 5 : 1) : 2;
+    if (t256 >= 128)
+        return dtl_ok ? 4 : 0;
     if (t128 >= 96)
-        return 1;
+        return dtl_ok ? 5 : 1;
     return 2;
 }
 
@@ -222,7 +236,8 @@ static const char* tile_kernel_name(int tile, int op)
 {
     static const char* ops[TOP_COUNT] = {"bf16", "f16", "i8", "fp8_e4m3_e4m3", "fp8_e5m2_e5m2", "fp8_e4m3_e5m2",
                                          "fp8_e5m2_e4m3", "fp4_e2m1"};
-    static const char* tiles[3] = {"tile256x256", "tile128x128", "tile64x64"};
+    static const char* tiles[7] = {"tile256x256", "tile128x128", "tile64x64", "tile256x256w4_dtl", "tile256x256w8_dtl",
+                                   "tile128x128_dtl", "tile256x128_dtl"};
     static thread_local char buf[64];
     snprintf(buf, sizeof buf, "%s_%s", tiles[tile], ops[op]);
     return buf;
@@ -340,7 +355,7 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
                    : ab_type == PTOAMD_F16 ? TOP_F16
                    : ab_type == PTOAMD_I8 ? TOP_I8
                    : ab_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E5E5;
-    const int tile = pick_tile(m, n);
+    const int tile = pick_tile(m, n, k_bytes, false);
     PTOAMD_HIP_CHECK(launch_gemm_tile(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;
@@ -383,7 +398,7 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
     p.c = out_bf16; p.acc_out = acc_out; p.row_scale = scale_a; p.col_scale = scale_b;
     p.m = m; p.n = n; p.k_bytes = k; p.lda_bytes = lda; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
     p.out_kind = OUT_W8A8_BF16; p.group_m = 4;
-    const int tile = pick_tile(m, n);
+    const int tile = pick_tile(m, n, k, false);
     PTOAMD_HIP_CHECK(launch_gemm_tile(tile, TOP_I8, p, stream));
     set_last_kernel(tile_kernel_name(tile, TOP_I8));
     return PTOAMD_OK;
@@ -462,7 +477,7 @@ int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type
         op = b_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E4E5;
     else
         op = b_type == PTOAMD_E5M2 ? TOP_FP8_E5E5 : TOP_FP8_E5E4;
-    const int tile = pick_tile(m, n);
+    const int tile = pick_tile(m, n, k_bytes, true);
     PTOAMD_HIP_CHECK(launch_gemm_tile(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;

@@ -142,6 +142,78 @@ struct TileCfg {
     static_assert((BM * 8) % THREADS == 0 && (BN * 8) % THREADS == 0, "slab chunks must divide over the workgroup");
 };
 
+// ---- TSTORE: drains one wave's accumulator blocks through the fix-pipe epilogue ------------------------------------
+// KIND (OutKind) and FULL (no bounds checks: the wave's tile lies inside the matrix) are compile-time so that each form
+// is a short, fully unrolled store sequence; a run-time switch inside the 16-register loop keeps the compiler from
+// unrolling it and pushes the accumulators into scratch memory.  The TMATMUL_ACC input is folded in here: C = Cin + A.B.
+template <int KIND, bool FULL, class Cfg, class Acc>
+__device__ __forceinline__ void tstore_blocks(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0,
+                                              int l32, int lhi)
+{
+    using Elem = typename Cfg::Op::Elem;
+    const Elem* cin = reinterpret_cast<const Elem*>(p.c_in);
+#pragma unroll
+    for (int i = 0; i < Cfg::MB; ++i)
+#pragma unroll
+        for (int j = 0; j < Cfg::NB; ++j) {
+            // keep the address arithmetic of one 32x32 block from being hoisted over the others (register pressure)
+            __builtin_amdgcn_sched_barrier(0);
+            const int gj = col0 + j * 32 + l32;
+            float cs = 1.0f;
+            if (KIND == OUT_W8A8_BF16)
+                cs = (FULL || gj < p.n) ? p.col_scale[gj] : 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int gi = row0 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                if (FULL || (gi < p.m && gj < p.n)) {
+                    const long o = (long)gi * p.ldc + gj;
+                    auto v = acc[i][j][r];
+                    if (cin != nullptr)
+                        v += cin[o];
+                    if (p.relu)
+                        v = v > 0 ? v : 0;
+                    if (KIND == OUT_F32) {
+                        reinterpret_cast<float*>(p.c)[o] = (float)v;
+                    } else if (KIND == OUT_F16) {
+                        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits((float)v);
+                    } else if (KIND == OUT_BF16) {
+                        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits((float)v);
+                    } else if (KIND == OUT_I32) {
+                        reinterpret_cast<int32_t*>(p.c)[o] = (int32_t)v;
+                    } else {  // W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16, each step rounded to f32
+                        if (p.acc_out != nullptr)
+                            p.acc_out[o] = (int32_t)v;
+                        const float t = __fmul_rn((float)v, p.row_scale[gi]);
+                        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(__fmul_rn(t, cs));
+                    }
+                }
+            }
+        }
+}
+
+template <bool FULL, class Cfg, class Acc>
+__device__ __forceinline__ void tstore_kind(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0,
+                                            int l32, int lhi)
+{
+    switch (p.out_kind) {
+        case OUT_F32: tstore_blocks<OUT_F32, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
+        case OUT_F16: tstore_blocks<OUT_F16, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
+        case OUT_BF16: tstore_blocks<OUT_BF16, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
+        case OUT_I32: tstore_blocks<OUT_I32, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
+        default: tstore_blocks<OUT_W8A8_BF16, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
+    }
+}
+
+template <class Cfg, class Acc>
+__device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0, int l32,
+                                       int lhi)
+{
+    if (row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n)
+        tstore_kind<true, Cfg>(p, acc, row0, col0, l32, lhi);
+    else
+        tstore_kind<false, Cfg>(p, acc, row0, col0, l32, lhi);
+}
+
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmParams p)
 {
@@ -246,20 +318,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
             for (int r = 0; r < 16; ++r)
                 acc[i][j][r] = 0;
         }
-    if (p.c_in != nullptr) {  // TMATMUL_ACC: start from the caller's accumulator
-#pragma unroll
-        for (int i = 0; i < MB; ++i)
-#pragma unroll
-            for (int j = 0; j < NB; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int gi = m0 + wm * Cfg::WTM + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-                    const int gj = n0 + wn * Cfg::WTN + j * 32 + l32;
-                    if (gi < p.m && gj < p.n)
-                        acc[i][j][r] = reinterpret_cast<const typename Op::Elem*>(p.c_in)[(long)gi * p.ldc + gj];
-                }
-    }
-
     // ---- fragment addressing (TMOV/TEXTRACT): lane reads row l32 of a 32-row block, half lhi of the k-step
     int fa_row[MB], fb_row[NB];
 #pragma unroll
@@ -329,39 +387,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
     }
 
     // ---- TSTORE: drain the accumulators through the epilogue
-    const int out_kind = p.out_kind;
-#pragma unroll
-    for (int i = 0; i < MB; ++i)
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
-            const int gj = n0 + wn * Cfg::WTN + j * 32 + l32;
-            float cs = 1.0f;
-            if (out_kind == OUT_W8A8_BF16)
-                cs = gj < p.n ? p.col_scale[gj] : 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int gi = m0 + wm * Cfg::WTM + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-                if (gi >= p.m || gj >= p.n)
-                    continue;
-                const long o = (long)gi * p.ldc + gj;
-                auto v = acc[i][j][r];
-                if (p.relu)
-                    v = v > 0 ? v : 0;
-                switch (out_kind) {
-                    case OUT_F32: reinterpret_cast<float*>(p.c)[o] = (float)v; break;
-                    case OUT_F16: reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits((float)v); break;
-                    case OUT_BF16: reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits((float)v); break;
-                    case OUT_I32: reinterpret_cast<int32_t*>(p.c)[o] = (int32_t)v; break;
-                    default: {  // W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16, each step rounded to f32
-                        if (p.acc_out != nullptr)
-                            p.acc_out[o] = (int32_t)v;
-                        const float t = __fmul_rn((float)v, p.row_scale[gi]);
-                        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(__fmul_rn(t, cs));
-                        break;
-                    }
-                }
-            }
-        }
+    tstore<Cfg>(p, acc, m0 + wm * Cfg::WTM, n0 + wn * Cfg::WTN, l32, lhi);
 }
 
 // One launcher per (tile shape, operand type); defined in gemm_tile_<op>.hip, called from gemm.hip.

@@ -1,0 +1,285 @@
+// Tiled MFMA GEMM, direct-to-LDS form: the steady-state kernel for shapes whose K extent is a whole number of
+// 128-byte slabs.  Same tile instructions as gemm_tile.hpp, different engines:
+//
+//   TLOAD      global_load_lds_dwordx4: each wave DMAs 1 KiB pieces of the next K-slab straight into the LDS ring
+//              (no register staging); the bank swizzle is applied on the global-address side, because the DMA
+//              writes lanes linearly.
+//   TEXTRACT   operand fragments of k-step s+1 are read (ds_read_b128) while the MFMAs of k-step s run; two register
+//              sets alternate, so the matrix pipe never waits on LDS inside a slab.
+//   sync       one workgroup barrier per slab, placed before the last k-step: by then every wave has drained its reads
+//              of the current slab (so it can be overwritten by slab kt+2) and its DMA of slab kt+1 has landed, and the
+//              last k-step's MFMAs cover the first fragment reads of slab kt+1.  This replaces the four-flag
+//              MTE2/MTE1/M hand-shake of the reference kernels.
+#pragma once
+#include <type_traits>
+#include <utility>
+
+#include "gemm_tile.hpp"
+
+namespace ptoamd {
+
+// Scheduling recipe for one k-step: NM MFMAs interleaved evenly with ND LDS reads (next k-step's fragments) and NV
+// LDS-DMA issues (a later slab).  Without it the compiler shortens the fragment live ranges, re-uses the registers and
+// puts the reads right in front of the MFMAs that need them, which exposes the LDS latency on every k-step.
+template <int I, int NM, int ND, int NV>
+struct SchedKStep {
+    __device__ static __forceinline__ void run()
+    {
+        constexpr int nd = (I + 1) * ND / NM - I * ND / NM;
+        constexpr int nv = (I + 1) * NV / NM - I * NV / NM;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        if constexpr (nd > 0)
+            __builtin_amdgcn_sched_group_barrier(0x100, nd, 0);  // LDS reads
+        if constexpr (nv > 0)
+            __builtin_amdgcn_sched_group_barrier(0x020, nv, 0);  // VMEM reads (LDS-DMA)
+        SchedKStep<I + 1, NM, ND, NV>::run();
+    }
+};
+template <int NM, int ND, int NV>
+struct SchedKStep<NM, NM, ND, NV> {
+    __device__ static __forceinline__ void run() {}
+};
+template <int NM, int ND, int NV>
+__device__ __forceinline__ void sched_kstep()
+{
+    SchedKStep<0, NM, ND, NV>::run();
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// Compile-time loop: f(std::integral_constant<int, I>{}) for I = 0 .. N-1.  Keeps every register-array index a literal
+// (a `#pragma unroll` the compiler declines leaves the accumulators indexed at run time, i.e. in scratch memory).
+template <int... Is, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f)
+{
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
+}
+
+// One LDS-DMA: 64 lanes x 16 bytes from per-lane global addresses to LDS bytes [lds_base, lds_base + 1024), lane-linear.
+// Issued as inline assembly on purpose: when the compiler sees an LDS-DMA it makes every later LDS read wait for it
+// (vmcnt(0)), since it cannot prove that the reads touch the other half of the ring; that wait would serialise the
+// slab prefetch with the MFMAs.  The kernel waits for its DMAs itself, right before the barrier that publishes a slab.
+__device__ __forceinline__ void lds_dma16(const uint8_t* gptr, uint32_t lds_base)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);  // wave-uniform by construction
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_address(const void* generic_ptr)
+{
+    return (uint32_t)(uintptr_t)(lds_ptr_t)(generic_ptr);
+}
+
+template <class Cfg>
+__global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileGemmParams p)
+{
+    using Op = typename Cfg::Op;
+    using Acc = typename Op::Acc;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, LA = Cfg::LA, LB = Cfg::LB;
+    constexpr int NT = Cfg::THREADS, FR = Op::FRAG_BYTES / 16, KS = Cfg::KSTEPS;
+    static_assert(KS % 2 == 0, "fragment register sets alternate per k-step");
+    static_assert((NT / 8) % 16 == 0, "the swizzle of a lane's row must not depend on the piece index");
+    extern __shared__ __align__(16) uint8_t smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % Cfg::WAVES_M, wn = wave / Cfg::WAVES_M;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+    const int grid = tiles_m * tiles_n;
+    int lid = blockIdx.x;
+    if ((grid & 7) == 0)
+        lid = (lid & 7) * (grid >> 3) + (lid >> 3);
+    const int per_group = p.group_m * tiles_n;
+    const int first_m = (lid / per_group) * p.group_m;
+    const int gsize = min(tiles_m - first_m, p.group_m);
+    const int tm = first_m + (lid % per_group) % gsize;
+    const int tn = (lid % per_group) / gsize;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // ---- TLOAD addressing.  Piece i of a slab is rows i * NT/8 .. + NT/8; lane `tid` lands at LDS position
+    // (row = tid / 8, slot = tid % 8) of the piece and therefore fetches logical chunk slot ^ swizzle(row).
+    const int ld_row = tid >> 3;
+    const int ld_chunk = swizzle_chunk(ld_row, tid & 7);
+    uint32_t goff_a[LA], goff_b[LB];
+#pragma unroll
+    for (int i = 0; i < LA; ++i)
+        goff_a[i] = (uint32_t)((long)min(m0 + ld_row + i * (NT / 8), p.m - 1) * p.lda_bytes + ld_chunk * 16);
+#pragma unroll
+    for (int i = 0; i < LB; ++i)
+        goff_b[i] = (uint32_t)((long)min(n0 + ld_row + i * (NT / 8), p.n - 1) * p.ldb_bytes + ld_chunk * 16);
+    const int k_slabs = p.k_bytes / 128;
+
+    const uint32_t lds_wave_base = __builtin_amdgcn_readfirstlane(lds_address(smem) + wave * 1024);
+    // DMA number q (0 .. LA + LB - 1) of slab kt into ring buffer buf
+    auto tload_piece = [&](int kt, int buf, int q) {
+        const uint32_t dst = lds_wave_base + buf * Cfg::STAGE_BYTES;
+        if (q < LA)
+            lds_dma16(p.a + goff_a[q] + (long)kt * 128, dst + q * (NT * 16));
+        else
+            lds_dma16(p.b + goff_b[q - LA] + (long)kt * 128, dst + Cfg::A_BYTES + (q - LA) * (NT * 16));
+    };
+    auto tload = [&](int kt, int buf) {
+#pragma unroll
+        for (int q = 0; q < LA + LB; ++q)
+            tload_piece(kt, buf, q);
+    };
+
+    // ---- MX block scales
+    constexpr int SW = Op::SCALED ? Op::GROUPS_PER_SLAB / 4 : 1;
+    uint32_t sca[MB][SW], scb[NB][SW], sca_n[MB][SW], scb_n[NB][SW];
+    const uint8_t* gsa[MB];
+    const uint8_t* gsb[NB];
+    const bool has_scales = Op::SCALED && p.sa != nullptr;
+    if (has_scales) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+            gsa[i] = p.sa + (long)min(m0 + wm * Cfg::WTM + i * 32 + l32, p.m - 1) * p.scale_ld;
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+            gsb[j] = p.sb + (long)min(n0 + wn * Cfg::WTN + j * 32 + l32, p.n - 1) * p.scale_ld;
+    }
+    auto load_scales = [&](int kt) {
+        if (has_scales) {
+#pragma unroll
+            for (int w = 0; w < SW; ++w) {
+#pragma unroll
+                for (int i = 0; i < MB; ++i)
+                    sca_n[i][w] = *reinterpret_cast<const uint32_t*>(gsa[i] + (long)kt * (SW * 4) + w * 4);
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+                    scb_n[j][w] = *reinterpret_cast<const uint32_t*>(gsb[j] + (long)kt * (SW * 4) + w * 4);
+            }
+        }
+    };
+
+    // ---- Acc tile
+    Acc acc[MB][NB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0;
+    // ---- fragment addressing: byte offset of (row, chunk 0) and the row's swizzle, per 32-row block
+    int fa_off[MB], fb_off[NB], fa_swz[MB], fb_swz[NB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i) {
+        const int r = wm * Cfg::WTM + i * 32 + l32;
+        fa_off[i] = r * 128;
+        fa_swz[i] = swizzle_chunk(r, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int r = wn * Cfg::WTN + j * 32 + l32;
+        fb_off[j] = Cfg::A_BYTES + r * 128;
+        fb_swz[j] = swizzle_chunk(r, 0);
+    }
+    // Two fragment register sets (next k-step's reads overlap this k-step's MFMAs) unless 32-byte fragments of a
+    // large wave tile would not fit the register file next to the accumulators; then one set is refilled piecewise,
+    // each block right after the last MFMA that reads it, and the second wave of the SIMD covers the LDS latency.
+    constexpr int SETS = (FR == 2 && MB * NB >= 8) ? 1 : 2;
+    uint4 fa[SETS][MB][FR], fb[SETS][NB][FR];
+    constexpr int NREAD = (MB + NB) * FR, NMMA = MB * NB, NDMA = LA + LB;
+    // fragment read number q of k-step s of ring buffer buf into register set `set`; B fragments come first because the
+    // first MFMAs of a k-step need all of B's first block but only A's first
+    auto textract_piece = [&](int set, int buf, int s, int q) {
+        const uint8_t* base = smem + buf * Cfg::STAGE_BYTES;
+        if (q < NB * FR) {
+            const int j = q / FR, f = q % FR;
+            fb[set][j][f] = *reinterpret_cast<const uint4*>(base + fb_off[j] + ((frag_chunk<FR>(s, lhi, f) ^ fb_swz[j]) << 4));
+        } else {
+            const int i = (q - NB * FR) / FR, f = (q - NB * FR) % FR;
+            fa[set][i][f] = *reinterpret_cast<const uint4*>(base + fa_off[i] + ((frag_chunk<FR>(s, lhi, f) ^ fa_swz[i]) << 4));
+        }
+    };
+    // One k-step: the MFMAs of step s (register set s & 1), with the fragment reads of the next step (register set
+    // (s + 1) & 1, from buffer rbuf step rs) and, in a slab's last step, the DMAs of slab dkt spread between them.
+    auto kstep = [&](int s, bool reads, int rbuf, int rs, bool dmas, int dkt, int dbuf) {
+        const int set = SETS == 2 ? (s & 1) : 0;
+        const int nset = SETS == 2 ? (set ^ 1) : 0;
+        static_for<NMMA>([&](auto xc) {
+            constexpr int x = decltype(xc)::value;
+            constexpr int i = x / NB, j = x % NB;
+            uint32_t xa = 127u, xb = 127u;
+            if (has_scales) {
+                const int g = 2 * s + lhi;
+                xa = (sca[i][g >> 2] >> ((g & 3) * 8)) & 0xFFu;
+                xb = (scb[j][g >> 2] >> ((g & 3) * 8)) & 0xFFu;
+            }
+            Op::mma(acc[i][j], fa[set][i], fb[set][j], xa, xb);
+            if (reads) {
+                if constexpr (SETS == 2) {
+                    constexpr int q0 = x * NREAD / NMMA, q1 = (x + 1) * NREAD / NMMA;
+                    static_for<q1 - q0>([&](auto qc) { textract_piece(nset, rbuf, rs, q0 + decltype(qc)::value); });
+                } else {
+                    if constexpr (j == NB - 1)  // row i of A is free once its last MFMA has issued
+                        static_for<FR>([&](auto fc) { textract_piece(0, rbuf, rs, NB * FR + i * FR + decltype(fc)::value); });
+                    if constexpr (x == NMMA - 1)  // B is free after the last MFMA
+                        static_for<NB * FR>([&](auto qc) { textract_piece(0, rbuf, rs, decltype(qc)::value); });
+                }
+            }
+            if (dmas) {
+                constexpr int q0 = x * NDMA / NMMA, q1 = (x + 1) * NDMA / NMMA;
+                static_for<q1 - q0>([&](auto qc) { tload_piece(dkt, dbuf, q0 + decltype(qc)::value); });
+            }
+        });
+        if constexpr (SETS == 2)
+            sched_kstep<NMMA, NREAD, 0>();
+    };
+
+    // ---- prologue: slabs 0 and 1 in flight, first fragments in registers
+    tload(0, 0);
+    load_scales(0);
+    if (k_slabs > 1)
+        tload(1, 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMAs have landed
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < NREAD; ++q)
+        textract_piece(0, 0, 0, q);
+
+    // One slab.  `more` = slab kt+1 exists (read its first fragments in the last k-step), `dma` = slab kt+2 exists
+    // (start its DMA into the buffer this slab frees); both are literal at the call sites so the branches fold.
+    auto slab = [&](int kt, bool more, bool dma) {
+        const int cur = kt & 1;
+        if (has_scales) {
+#pragma unroll
+            for (int w = 0; w < SW; ++w) {
+#pragma unroll
+                for (int i = 0; i < MB; ++i)
+                    sca[i][w] = sca_n[i][w];
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+                    scb[j][w] = scb_n[j][w];
+            }
+            if (more)
+                load_scales(kt + 1);
+        }
+#pragma unroll
+        for (int s = 0; s < KS - 1; ++s)
+            kstep(s, true, cur, s + 1, false, 0, 0);
+        // every wave is done reading slab kt, and its DMAs of slab kt+1 (issued one slab ago) have landed
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        kstep(KS - 1, more, cur ^ 1, 0, dma, kt + 2, cur);
+    };
+    int kt = 0;
+    for (; kt + 2 < k_slabs; ++kt)
+        slab(kt, true, true);
+    if (kt + 1 < k_slabs) {
+        slab(kt, true, false);
+        ++kt;
+    }
+    slab(kt, false, false);
+
+    // ---- TSTORE
+    tstore<Cfg>(p, acc, m0 + wm * Cfg::WTM, n0 + wn * Cfg::WTN, l32, lhi);
+}
+
+}  // namespace ptoamd

@@ -1,7 +1,7 @@
 // Instantiates gemm_tile_kernel for one operand type at the three tile shapes.  Included by gemm_tile_<op>.hip with
 // PTOAMD_TILE_OP (the traits type) and PTOAMD_TILE_FN (the launcher's name) defined, so the operand types compile in
 // parallel translation units.
-#include "gemm_tile.hpp"
+#include "gemm_tile_dtl.hpp"
 
 namespace ptoamd {
 
@@ -21,9 +21,29 @@ static hipError_t launch_cfg(const TileGemmParams& p, hipStream_t stream)
     return hipGetLastError();
 }
 
+template <class Cfg>
+static hipError_t launch_dtl(const TileGemmParams& p, hipStream_t stream)
+{
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_dtl_kernel<Cfg>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+        if (e != hipSuccess)
+            return e;
+        attr_set = true;
+    }
+    const int tiles = ((p.m + Cfg::BM - 1) / Cfg::BM) * ((p.n + Cfg::BN - 1) / Cfg::BN);
+    hipLaunchKernelGGL(gemm_tile_dtl_kernel<Cfg>, dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
+    return hipGetLastError();
+}
+
 hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 {
     switch (tile) {
+        case 3: return launch_dtl<TileCfg<256, 256, 2, 2, PTOAMD_TILE_OP>>(p, stream);
+        case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>>(p, stream);
+        case 5: return launch_dtl<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>>(p, stream);
+        case 6: return launch_dtl<TileCfg<256, 128, 4, 2, PTOAMD_TILE_OP>>(p, stream);
         case 0: return launch_cfg<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>>(p, stream);
         case 1: return launch_cfg<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>>(p, stream);
         default: return launch_cfg<TileCfg<64, 64, 2, 2, PTOAMD_TILE_OP>>(p, stream);

@@ -90,8 +90,22 @@ def test_config1_fp16_512_cubed(pa, oracle):
     assert np.array_equal(exact.view(np.uint32), ref.view(np.uint32))  # k-order-exact kernel: bit for bit
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2])
-@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (300, 200, 136), (64, 520, 1024), (1, 64, 64)])
+TILE_NAMES = ("tile256x256_", "tile128x128_", "tile64x64_", "tile256x256w4_dtl", "tile256x256w8_dtl", "tile128x128_dtl",
+              "tile256x128_dtl")
+ALL_TILES = [0, 1, 2, 3, 4, 5, 6]
+
+
+def expect_tile(pa, tile, k_bytes):
+    """Tiles 3-6 need whole 128-byte K slabs; otherwise the dispatcher falls back to the register-staged tile."""
+    name = pa.last_kernel()
+    if tile >= 3 and k_bytes % 128:
+        assert name.startswith("tile128x128_" if tile == 5 else "tile256x256_"), name
+    else:
+        assert name.startswith(TILE_NAMES[tile]), name
+
+
+@pytest.mark.parametrize("tile", ALL_TILES)
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (300, 200, 136), (64, 520, 1024), (1, 64, 64), (512, 384, 448)])
 def test_bf16_gemm_every_tile_shape(pa, oracle, tile, m, n, k):
     r = np.random.default_rng(m * 7 + n)
     a = bf16_bits(r.standard_normal((m, k)) * 0.02)
@@ -99,7 +113,7 @@ def test_bf16_gemm_every_tile_shape(pa, oracle, tile, m, n, k):
     ref = oracle.matmul_bf16(a, b, b_dn=True)
     with tile_env(PTOAMD_TILE=tile):
         got32 = host(pa.gemm(dev(a).view(torch.bfloat16), dev(b).view(torch.bfloat16), pa.BF16, pa.F32, pa.B_DN))
-        assert pa.last_kernel().startswith(("tile256", "tile128", "tile64")[tile])
+        expect_tile(pa, tile, 2 * k)
         got16 = host(pa.gemm(dev(a).view(torch.bfloat16), dev(b).view(torch.bfloat16), pa.BF16, pa.BF16, pa.B_DN))
     assert relerr(got32, ref) <= 1e-2
     # TSTORE f32 -> bf16 is round-to-nearest-even of the same accumulator
@@ -137,7 +151,7 @@ def test_config2_bf16_4096_cubed(pa, oracle):
     a = (torch.randn((m, k), generator=gen, device=DEV) * 0.02).to(torch.bfloat16)
     b = (torch.randn((n, k), generator=gen, device=DEV) * 0.02).to(torch.bfloat16)
     out = pa.gemm(a, b, pa.BF16, pa.BF16, pa.B_DN)
-    assert pa.last_kernel() == "tile256x256_bf16"
+    assert pa.last_kernel() == "tile256x256w8_dtl_bf16"
     rows = np.array([0, 1, 255, 256, 1000, 2047, 2048, 3333, 4095])
     cols = np.arange(0, 4096, 37)
     ref = oracle.matmul_bf16(host(sel(a, rows)), host(sel(b, cols)), b_dn=True)
@@ -157,7 +171,7 @@ def test_config2_bf16_4096_cubed(pa, oracle):
 
 
 # ------------------------------------------------------------------------------------------- int8 / W8A8
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("tile", ALL_TILES)
 def test_int8_accumulators_bit_exact(pa, oracle, tile):
     r = np.random.default_rng(tile)
     for m, n, k in ((256, 256, 512), (130, 70, 208), (33, 500, 4096)):
@@ -216,7 +230,7 @@ def test_config3_w8a8_full_size(pa, oracle):
     sa = torch.rand(m, generator=gen, device=DEV) * 0.01 + 0.001
     sb = torch.rand(n, generator=gen, device=DEV) * 0.01 + 0.001
     out, acc = pa.gemm_w8a8(a, b, sa, sb, want_acc=True)
-    assert pa.last_kernel() == "tile256x256_i8"
+    assert pa.last_kernel() == "tile256x256w8_dtl_i8"
     rows = np.array([0, 255, 256, 1023, 2047])
     cols = np.arange(0, n, 257)
     ra, rb = host(sel(a, rows)), host(sel(b, cols))
@@ -250,7 +264,7 @@ PA_T = {ob.E4M3: 6, ob.E5M2: 7, ob.E2M1: 8, ob.E1M2: 9}
 
 @pytest.mark.parametrize("ta,tb", [(ob.E4M3, ob.E4M3), (ob.E5M2, ob.E5M2), (ob.E4M3, ob.E5M2), (ob.E5M2, ob.E4M3),
                                    (ob.E2M1, ob.E2M1)])
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("tile", ALL_TILES)
 def test_mx_gemm(pa, oracle, ta, tb, tile):
     r = np.random.default_rng(ta * 16 + tb + tile)
     for m, n, k in ((128, 128, 256), (200, 72, 512)):
@@ -318,7 +332,7 @@ def test_config4_mxfp8_full_size(pa, oracle):
     a, sa = pa.tquant_mx(xa, pa.OCP_MXFP8, want_aux=False)
     b, sb = pa.tquant_mx(xb, pa.OCP_MXFP8, want_aux=False)
     out = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E4M3, pa.E4M3, pa.BF16)
-    assert pa.last_kernel() == "tile256x256_fp8_e4m3_e4m3"
+    assert pa.last_kernel() == "tile128x128_dtl_fp8_e4m3_e4m3"
     rows = np.array([0, 255, 256, 2049, 4095])
     cols = np.arange(0, n, 449)
     ref = oracle.matmul_mx(host(sel(a, rows)), host(sel(b, cols)), host(sel(sa, rows)), host(sel(sb, cols)), len(rows), k, len(cols),
