@@ -1,14 +1,15 @@
 // Decode-shaped weight-only MXFP4 GEMV/GEMM (m <= 16): out[m][n] = sum_k A[m][k] * (e2m1 W[n][k] * 2^(sw[n][k/32]-127)).
 //
-// The shape is HBM-bound (every weight byte is read once, ~60 FLOP per byte), so the kernel is built around the
-// weight stream:
-//   * the K range is split over the 8 waves of a workgroup; each wave keeps its [16][K/8] slice of the bf16
-//     activations in registers for the whole kernel (the TLOAD of the Left operand happens once per workgroup);
-//   * a workgroup walks groups of 16 weight rows; each lane streams 16-byte pieces (32 fp4 = one MX group) with the
-//     loads of the next row group in flight while the current one is multiplied;
+// The shape is HBM-bound (every weight byte is read once, ~60 FLOP per byte), so the kernel is built around keeping
+// enough weight bytes in flight:
+//   * a workgroup owns WAVES x 16 weight rows over the full K; each wave streams its 16 rows in 512-k chunks, four
+//     16-byte loads (32 fp4 = one MX group each) plus one 16-byte scale load per lane per chunk, with DEPTH chunks of
+//     loads outstanding per wave (registers are cheap here: the accumulator is 4 VGPRs);
+//   * the bf16 activations (the Left operand, shared by every wave) are staged per chunk into a double-buffered LDS
+//     strip already laid out as MFMA operand fragments, so a ds_read_b128 per MFMA is conflict-free;
 //   * dequantisation happens in registers (v_cvt_scalef32_pk_bf16_fp4: fp4 pair * 2^e -> bf16 pair, exact), the
-//     product runs on v_mfma_f32_16x16x32_bf16 with fp32 accumulation, and the 8 partial 16x16 tiles are summed
-//     through LDS in a fixed order before the store (TSTORE f32 -> f32 | bf16).
+//     product runs on v_mfma_f32_16x16x32_bf16 with fp32 accumulation, and each wave stores its own 16 x 16 result
+//     (TSTORE f32 -> f32 | bf16): no cross-wave reduction, one barrier per chunk for the activation strip.
 // Operand k-slots are assigned so that a lane's 32 consecutive k (one MX group, one scale byte) feed 4 MFMAs.
 #include "common_host.hpp"
 #include "device_types.hpp"
@@ -31,8 +32,8 @@ struct GemvParams {
     int n_groups;       // ceil(n / 16)
 };
 
-constexpr int GEMV_WAVES = 8;
-constexpr int GEMV_MAX_CHUNKS = 8;  // 128-k chunks per wave: K <= 8 * 8 * 128 = 8192
+constexpr int GEMV_CHUNK = 512;  // k per chunk
+constexpr int GEMV_DEPTH = 4;    // chunks of weight loads in flight per wave
 
 // 8 packed fp4 (one dword) times 2^(e-127) -> 8 bf16, exact.  HW: one v_cvt_scalef32_pk_bf16_fp4 per byte.
 template <bool HW_CVT>
@@ -57,92 +58,104 @@ __device__ __forceinline__ uint4 dequant8(uint32_t x, float scale)
     return r;
 }
 
-template <bool HW_CVT>
-__global__ void __launch_bounds__(GEMV_WAVES * 64) gemv_mxfp4_kernel(const GemvParams p)
+// LDS strip of one activation chunk: [4 sub-chunks of 128 k][4 MFMAs][64 lanes] x 16 bytes = 16 KiB.  Lane (row l16,
+// quarter g) of MFMA j of sub-chunk c holds A[l16][128 c + 32 g + 8 j .. + 7].
+template <bool HW_CVT, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64) gemv_mxfp4_kernel(const GemvParams p)
 {
-    __shared__ float red[GEMV_WAVES][64][4];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int NT = WAVES * 64;
+    __shared__ uint4 astrip[2][16 * 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
-    const int ks = p.k / GEMV_WAVES;  // this wave's K slice, a multiple of 128
-    const int chunks = ks / 128;
-    const int k0 = wave * ks;
+    const int chunks = p.k / GEMV_CHUNK;
+    const int row = min((blockIdx.x * WAVES + wave) * 16 + l16, p.n - 1);
+    const uint8_t* wp = p.w + (long)row * p.ldw_bytes + g * 16;   // + chunk * 256 + c * 64
+    const uint8_t* sp = p.sw + (long)row * (p.k / 32);            // + chunk * 16
 
-    // Left operand slice -> registers: lane (row l16, quarter g) holds k0 + 128c + 32g .. +31 of its row, per chunk c
-    uint4 areg[GEMV_MAX_CHUNKS][4];
+    // activation chunk -> registers -> LDS (fragment-major); 1024 pieces of 16 bytes per chunk
+    constexpr int APIECES = (1024 + NT - 1) / NT;
+    // The activation pieces of chunk kc are fetched together with the weights of chunk kc (DEPTH chunks ahead), not one
+    // chunk ahead: vmcnt retires loads in issue order, so waiting for a young activation load would also wait for
+    // every older weight prefetch and collapse the prefetch depth to one chunk.
+    uint4 areg[GEMV_DEPTH][APIECES];
+    auto a_fetch = [&](int stage, int kc) {
 #pragma unroll
-    for (int c = 0; c < GEMV_MAX_CHUNKS; ++c) {
+        for (int x = 0; x < APIECES; ++x) {
+            const int piece = tid + x * NT;            // m = piece % 16, q = piece / 16 (q-th group of 8 k)
+            const int m = piece & 15, q = piece >> 4;
+            areg[stage][x] = make_uint4(0, 0, 0, 0);
+            if (piece < 1024 && m < p.m)
+                areg[stage][x] = *reinterpret_cast<const uint4*>(p.a + (long)m * p.lda + kc * GEMV_CHUNK + q * 8);
+        }
+    };
+    auto a_stage = [&](int stage, int buf) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            areg[c][j] = make_uint4(0, 0, 0, 0);
-        if (c < chunks && l16 < p.m) {
-            const uint4* src = reinterpret_cast<const uint4*>(p.a + (long)l16 * p.lda + k0 + c * 128 + g * 32);
+        for (int x = 0; x < APIECES; ++x) {
+            const int piece = tid + x * NT;
+            const int m = piece & 15, q = piece >> 4;  // q = 16 c + 4 g + j; 16 rows of one q are contiguous in LDS
+            if (piece < 1024)
+                astrip[buf][((q >> 4) * 4 + (q & 3)) * 64 + ((q >> 2) & 3) * 16 + m] = areg[stage][x];
+        }
+    };
+
+    uint4 wreg[GEMV_DEPTH][4], sreg[GEMV_DEPTH];
+    auto w_fetch = [&](int stage, int kc) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                areg[c][j] = src[j];
+        for (int c = 0; c < 4; ++c)
+            wreg[stage][c] = *reinterpret_cast<const uint4*>(wp + (long)kc * (GEMV_CHUNK / 2) + c * 64);
+        sreg[stage] = *reinterpret_cast<const uint4*>(sp + kc * (GEMV_CHUNK / 32));
+    };
+
+    f32x4 acc = {0, 0, 0, 0};
+#pragma unroll
+    for (int d = 0; d < GEMV_DEPTH; ++d)
+        if (d < chunks) {
+            a_fetch(d, d);
+            w_fetch(d, d);
+        }
+    a_stage(0, 0);
+    __syncthreads();
+
+    for (int kc0 = 0; kc0 < chunks; kc0 += GEMV_DEPTH) {
+#pragma unroll
+        for (int d = 0; d < GEMV_DEPTH; ++d) {
+            const int kc = kc0 + d;
+            if (kc < chunks) {
+                const int buf = kc & 1;
+                const uint32_t sw4[4] = {sreg[d].x, sreg[d].y, sreg[d].z, sreg[d].w};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float scale = e8m0_to_f32((sw4[c] >> (8 * g)) & 0xFFu);  // MX group 4 c + g of the chunk
+                    const uint32_t xs[4] = {wreg[d][c].x, wreg[d][c].y, wreg[d][c].z, wreg[d][c].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint4 wv = dequant8<HW_CVT>(xs[j], scale);
+                        const uint4 av = astrip[buf][(c * 4 + j) * 64 + lane];
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av),
+                                                                     __builtin_bit_cast(bf16x8, wv), acc, 0, 0, 0);
+                    }
+                }
+                if (kc + 1 < chunks)
+                    a_stage((d + 1) % GEMV_DEPTH, buf ^ 1);  // chunk kc + 1's activations, fetched DEPTH - 1 chunks ago
+                if (kc + GEMV_DEPTH < chunks) {  // refill this stage: DEPTH chunks of loads stay in flight
+                    a_fetch(d, kc + GEMV_DEPTH);
+                    w_fetch(d, kc + GEMV_DEPTH);
+                }
+                __syncthreads();
+            }
         }
     }
 
-    uint4 wreg[GEMV_MAX_CHUNKS];
-    uint32_t sreg[GEMV_MAX_CHUNKS];
-    auto load_group = [&](int ng) {
-        const int row = min(ng * 16 + l16, p.n - 1);
-        const uint8_t* wp = p.w + (long)row * p.ldw_bytes + (k0 + g * 32) / 2;
-        const uint8_t* sp = p.sw + (long)row * (p.k / 32) + k0 / 32 + g;
+    const int n0 = (blockIdx.x * WAVES + wave) * 16;
 #pragma unroll
-        for (int c = 0; c < GEMV_MAX_CHUNKS; ++c)
-            if (c < chunks) {
-                wreg[c] = *reinterpret_cast<const uint4*>(wp + c * 64);
-                sreg[c] = sp[c * 4];
-            }
-    };
-
-    int ng = blockIdx.x;
-    if (ng < p.n_groups)
-        load_group(ng);
-    for (; ng < p.n_groups; ng += gridDim.x) {
-        uint4 wcur[GEMV_MAX_CHUNKS];
-        uint32_t scur[GEMV_MAX_CHUNKS];
-#pragma unroll
-        for (int c = 0; c < GEMV_MAX_CHUNKS; ++c) {
-            wcur[c] = wreg[c];
-            scur[c] = sreg[c];
+    for (int r = 0; r < 4; ++r) {
+        const int gi = 4 * g + r, gj = n0 + l16;
+        if (gi < p.m && gj < p.n) {
+            if (p.out_bf16)
+                reinterpret_cast<uint16_t*>(p.out)[(long)gi * p.ldc + gj] = f32_to_bf16_bits(acc[r]);
+            else
+                reinterpret_cast<float*>(p.out)[(long)gi * p.ldc + gj] = acc[r];
         }
-        if (ng + (int)gridDim.x < p.n_groups)
-            load_group(ng + gridDim.x);  // next row group's weights are in flight during the multiply
-
-        f32x4 acc = {0, 0, 0, 0};
-#pragma unroll
-        for (int c = 0; c < GEMV_MAX_CHUNKS; ++c)
-            if (c < chunks) {
-                const float scale = e8m0_to_f32(scur[c]);
-                const uint32_t xs[4] = {wcur[c].x, wcur[c].y, wcur[c].z, wcur[c].w};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint4 wv = dequant8<HW_CVT>(xs[j], scale);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, areg[c][j]),
-                                                                 __builtin_bit_cast(bf16x8, wv), acc, 0, 0, 0);
-                }
-            }
-        // sum the 8 K-slice partials in wave order (deterministic), then TSTORE
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-            red[wave][lane][r] = acc[r];
-        __syncthreads();
-        if (threadIdx.x < 256) {
-            const int ol = threadIdx.x >> 2, r = threadIdx.x & 3;
-            float s = 0.0f;
-#pragma unroll
-            for (int w8 = 0; w8 < GEMV_WAVES; ++w8)
-                s += red[w8][ol][r];
-            const int gi = 4 * (ol >> 4) + r, gj = ng * 16 + (ol & 15);
-            if (gi < p.m && gj < p.n) {
-                if (p.out_bf16)
-                    reinterpret_cast<uint16_t*>(p.out)[(long)gi * p.ldc + gj] = f32_to_bf16_bits(s);
-                else
-                    reinterpret_cast<float*>(p.out)[(long)gi * p.ldc + gj] = s;
-            }
-        }
-        __syncthreads();
     }
 }
 
@@ -188,8 +201,8 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
     p.out_bf16 = c_type == PTOAMD_BF16;
     p.n_groups = (n + 15) / 16;
     const char* fg = getenv("PTOAMD_FORCE_GENERIC");
-    const bool stream_ok = !(fg && fg[0] == '1') && k % (GEMV_WAVES * 128) == 0 && k <= GEMV_WAVES * GEMV_MAX_CHUNKS * 128 &&
-                           (reinterpret_cast<uintptr_t>(a_bf16) & 15u) == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0 &&
+    const bool stream_ok = !(fg && fg[0] == '1') && k % GEMV_CHUNK == 0 && (reinterpret_cast<uintptr_t>(a_bf16) & 15u) == 0 &&
+                           (reinterpret_cast<uintptr_t>(w) & 15u) == 0 && (reinterpret_cast<uintptr_t>(sw) & 15u) == 0 &&
                            (lda % 8) == 0 && (p.ldw_bytes % 16) == 0;
     if (!stream_ok) {
         dim3 block(128), grid((n + 127) / 128, m);
@@ -198,19 +211,28 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
         set_last_kernel("gemv_mxfp4_generic");
         return PTOAMD_OK;
     }
+    // 16 rows per wave; 7 waves per workgroup when that tiles the row groups more evenly over the CUs than 8
+    // (N = 28672: 1792 groups = 256 workgroups of 7), else 8
     int dev = 0, cus = 256;
     PTOAMD_HIP_CHECK(hipGetDevice(&dev));
     PTOAMD_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    // one workgroup per CU walks its share of the row groups; a grid that divides the groups evenly avoids a tail
-    int grid = p.n_groups < cus ? p.n_groups : cus;
+    const int g7 = (p.n_groups + 6) / 7, g8 = (p.n_groups + 7) / 8;
+    const auto rounds = [&](int blocks) { return (blocks + cus - 1) / cus; };
+    const bool use7 = rounds(g7) * 7 < rounds(g8) * 8;
     const char* sw_cvt = getenv("PTOAMD_GEMV_SW_CVT");
-    if (sw_cvt && sw_cvt[0] == '1') {
-        hipLaunchKernelGGL(gemv_mxfp4_kernel<false>, dim3(grid), dim3(GEMV_WAVES * 64), 0, stream, p);
-        set_last_kernel("gemv_mxfp4_stream_swcvt");
+    const bool swc = sw_cvt && sw_cvt[0] == '1';
+    if (use7) {
+        if (swc)
+            hipLaunchKernelGGL((gemv_mxfp4_kernel<false, 7>), dim3(g7), dim3(7 * 64), 0, stream, p);
+        else
+            hipLaunchKernelGGL((gemv_mxfp4_kernel<true, 7>), dim3(g7), dim3(7 * 64), 0, stream, p);
     } else {
-        hipLaunchKernelGGL(gemv_mxfp4_kernel<true>, dim3(grid), dim3(GEMV_WAVES * 64), 0, stream, p);
-        set_last_kernel("gemv_mxfp4_stream");
+        if (swc)
+            hipLaunchKernelGGL((gemv_mxfp4_kernel<false, 8>), dim3(g8), dim3(8 * 64), 0, stream, p);
+        else
+            hipLaunchKernelGGL((gemv_mxfp4_kernel<true, 8>), dim3(g8), dim3(8 * 64), 0, stream, p);
     }
+    set_last_kernel(swc ? "gemv_mxfp4_stream_swcvt" : "gemv_mxfp4_stream");
     PTOAMD_HIP_CHECK(hipGetLastError());
     return PTOAMD_OK;
 }
