@@ -15,6 +15,7 @@
 #include <utility>
 
 #include "gemm_tile.hpp"
+#include "lds_dma.hpp"
 
 namespace ptoamd {
 
@@ -43,35 +44,6 @@ template <int NM, int ND, int NV>
 __device__ __forceinline__ void sched_kstep()
 {
     SchedKStep<0, NM, ND, NV>::run();
-}
-
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-
-// Compile-time loop: f(std::integral_constant<int, I>{}) for I = 0 .. N-1.  Keeps every register-array index a literal
-// (a `#pragma unroll` the compiler declines leaves the accumulators indexed at run time, i.e. in scratch memory).
-template <int... Is, class F>
-__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f)
-{
-    (f(std::integral_constant<int, Is>{}), ...);
-}
-template <int N, class F>
-__device__ __forceinline__ void static_for(F&& f)
-{
-    static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
-}
-
-// One LDS-DMA: 64 lanes x 16 bytes from per-lane global addresses to LDS bytes [lds_base, lds_base + 1024), lane-linear.
-// Issued as inline assembly on purpose: when the compiler sees an LDS-DMA it makes every later LDS read wait for it
-// (vmcnt(0)), since it cannot prove that the reads touch the other half of the ring; that wait would serialise the
-// slab prefetch with the MFMAs.  The kernel waits for its DMAs itself, right before the barrier that publishes a slab.
-__device__ __forceinline__ void lds_dma16(const uint8_t* gptr, uint32_t lds_base)
-{
-    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);  // wave-uniform by construction
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(base) : "memory", "m0");
-}
-__device__ __forceinline__ uint32_t lds_address(const void* generic_ptr)
-{
-    return (uint32_t)(uintptr_t)(lds_ptr_t)(generic_ptr);
 }
 
 template <class Cfg>

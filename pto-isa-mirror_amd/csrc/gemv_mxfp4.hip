@@ -1,18 +1,23 @@
 // Decode-shaped weight-only MXFP4 GEMV/GEMM (m <= 16): out[m][n] = sum_k A[m][k] * (e2m1 W[n][k] * 2^(sw[n][k/32]-127)).
 //
-// The shape is HBM-bound (every weight byte is read once, ~60 FLOP per byte), so the kernel is built around keeping
-// enough weight bytes in flight:
-//   * a workgroup owns WAVES x 16 weight rows over the full K; each wave streams its 16 rows in 512-k chunks, four
-//     16-byte loads (32 fp4 = one MX group each) plus one 16-byte scale load per lane per chunk, with DEPTH chunks of
-//     loads outstanding per wave (registers are cheap here: the accumulator is 4 VGPRs);
-//   * the bf16 activations (the Left operand, shared by every wave) are staged per chunk into a double-buffered LDS
-//     strip already laid out as MFMA operand fragments, so a ds_read_b128 per MFMA is conflict-free;
-//   * dequantisation happens in registers (v_cvt_scalef32_pk_bf16_fp4: fp4 pair * 2^e -> bf16 pair, exact), the
-//     product runs on v_mfma_f32_16x16x32_bf16 with fp32 accumulation, and each wave stores its own 16 x 16 result
-//     (TSTORE f32 -> f32 | bf16): no cross-wave reduction, one barrier per chunk for the activation strip.
-// Operand k-slots are assigned so that a lane's 32 consecutive k (one MX group, one scale byte) feed 4 MFMAs.
+// The shape is HBM-bound (every weight byte is read once, ~60 FLOP per byte).  What limits a streaming read on this
+// memory system is the shape of each wave's load: 16 rows x 64 bytes per instruction (the natural MFMA operand
+// pattern) tops out near 3.4 TB/s, 512 contiguous bytes per half wave reaches 5+ TB/s.  Two kernels:
+//
+//   * split-K (k % 1024 == 0, the decode shapes): a workgroup of 8 waves owns a run of 16-row strips; wave s owns
+//     k-slice s (1024 k) of every strip and keeps its activation fragments for that slice in registers for the whole
+//     kernel (128 VGPRs, loaded once).  Weights and scales stream global -> LDS by LDS-DMA into a per-wave
+//     double-buffered region (512 contiguous bytes per row, two rows per instruction, no VGPRs, no barriers: a wave
+//     reads back only what it wrote), are re-read as MFMA operand fragments (16-byte chunks XOR-swizzled by row on
+//     the global side, so the reads are conflict-free), dequantised in registers and multiplied on
+//     v_mfma_f32_16x16x32_bf16.  The 8 k-slice partials of a strip are summed through LDS in a fixed order.
+//   * streaming (k % 512 == 0 otherwise): a wave owns 16 rows over the full K, register prefetch four chunks deep,
+//     activations staged per chunk through LDS.
+// Dequantisation: v_cvt_scalef32_pk_bf16_fp4 (fp4 pair * 2^e -> bf16 pair, exact).  Operand k-slots are assigned so
+// that a lane's 32 consecutive k (one MX group, one scale byte) feed 4 MFMAs.
 #include "common_host.hpp"
 #include "device_types.hpp"
+#include "lds_dma.hpp"
 
 #include <stdlib.h>
 
@@ -159,6 +164,153 @@ __global__ void __launch_bounds__(WAVES * 64) gemv_mxfp4_kernel(const GemvParams
     }
 }
 
+// ---- split-K kernel -------------------------------------------------------------------------------------------
+constexpr int SK_SLICE = 1024;                     // k per wave slice
+constexpr int SK_WAVES = 8;
+constexpr int SK_RMAX = 8;                         // strips whose accumulators a wave holds at once
+constexpr int SK_PAIR = 2 * (SK_SLICE / 2) + 16;   // LDS bytes of a row pair: 2 x 512 plus one 16-byte pad
+constexpr int SK_WBYTES = 8 * SK_PAIR;             // one strip's weight slice: 16 rows x 512 bytes (+ pads)
+constexpr int SK_SBYTES = 16 * (SK_SLICE / 32);    // and its scales: 16 rows x 32 bytes
+constexpr int SK_STAGE = SK_WBYTES + SK_SBYTES;
+constexpr int SK_WAVE_LDS = 2 * SK_STAGE;          // double buffer, private to the wave
+constexpr int SK_LDS = SK_WAVES * SK_WAVE_LDS;     // 138 KiB of the CU's 160 KiB
+constexpr int SK_VM_PER_STRIP = 10;                // LDS-DMA instructions per strip: 8 weight + 2 scale
+static_assert(SK_RMAX * 64 * 16 <= SK_WAVE_LDS, "a wave's partial sums reuse its own staging region");
+
+// ksw = 1 << ksw_log2 waves share one strip's K (wave & (ksw - 1) = first k-slice, then every ksw-th);
+// 8 / ksw row groups work on different strips.  Workgroup b owns strips [b * strips_per_wg, (b + 1) * strips_per_wg).
+template <bool HW_CVT>
+__global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const GemvParams p, int ksw_log2, int strips_per_wg)
+{
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l16 = lane & 15, q = lane >> 4;
+    const int ksw = 1 << ksw_log2, rgs = SK_WAVES >> ksw_log2;
+    const int slice = wave & (ksw - 1), rg = wave >> ksw_log2;
+    const int s_begin = blockIdx.x * strips_per_wg, s_end = min(s_begin + strips_per_wg, p.n_groups);
+    const int ks = p.k / SK_SLICE, sb = p.k / 32;
+    uint8_t* my = smem + wave * SK_WAVE_LDS;
+    const uint32_t my_lds = lds_address(my);
+    const int wread = (l16 >> 1) * SK_PAIR + (l16 & 1) * 512 + ((8 * q) ^ (8 * (l16 & 1))) * 16;  // row l16, chunk 8 q
+    const int mine = s_end > s_begin + rg ? (s_end - s_begin - rg + rgs - 1) / rgs : 0;  // strips of this row group
+    const int most = (s_end - s_begin + rgs - 1) / rgs;                                   // ... of row group 0
+
+    for (int b0 = 0; b0 < most; b0 += SK_RMAX) {
+        const int cnt = max(0, min(SK_RMAX, mine - b0));
+        f32x4 acc[SK_RMAX];
+#pragma unroll
+        for (int i = 0; i < SK_RMAX; ++i)
+            acc[i] = f32x4{0, 0, 0, 0};
+
+        for (int kb = slice; kb < ks; kb += ksw) {
+            // activation fragments of this k-slice: lane (m = l16, quarter q) holds A[m][1024 kb + 256 q .. + 255];
+            // lanes past the last activation row re-read it (their output rows are never stored)
+            uint4 areg[32];
+            const uint4* ap = reinterpret_cast<const uint4*>(p.a + (long)min(l16, p.m - 1) * p.lda + kb * SK_SLICE + q * 256);
+#pragma unroll
+            for (int x = 0; x < 32; ++x)
+                areg[x] = ap[x];
+
+            // strip i of the batch -> buffer i & 1.  One LDS-DMA moves a row pair (2 x 512 contiguous bytes); pairs
+            // are 16 bytes apart in LDS and odd rows swap their 128-byte halves (chunk ^ 8), so that 16 lanes reading
+            // one chunk index of the 16 rows hit 16 different bank groups with a lane-constant base address.
+            // Addresses are a wave-uniform strip base plus a 32-bit lane offset (rows past n - 1 re-read row n - 1).
+            auto issue = [&](int i) {
+                const int strip = s_begin + rg + rgs * (b0 + i);
+                const int rlim = min(15, p.n - 1 - strip * 16);
+                const uint8_t* wbase = p.w + (long)strip * 16 * p.ldw_bytes + kb * (SK_SLICE / 2);
+                const uint8_t* sbase = p.sw + (long)strip * 16 * sb + kb * (SK_SLICE / 32);
+                const uint32_t dst = my_lds + (i & 1) * SK_STAGE;
+                // (the lane id is made opaque here so that these few VALU ops are redone per strip rather than
+                // precomputed for all strips of the batch and parked in scratch memory)
+                int ln = lane;
+                asm volatile("" : "+v"(ln));
+                const int hi = ln >> 5;
+                const uint32_t chunk_off = ((ln & 31) ^ (8 * hi)) * 16;
+#pragma unroll
+                for (int d = 0; d < 8; ++d)
+                    lds_dma16_off(wbase, __umul24(min(2 * d + hi, rlim), (uint32_t)p.ldw_bytes) + chunk_off, dst + d * SK_PAIR);
+#pragma unroll
+                for (int d = 0; d < 2; ++d)
+                    lds_dma4_off(sbase, __umul24(min(8 * d + (ln >> 3), rlim), (uint32_t)sb) + (ln & 7) * 4,
+                                 dst + SK_WBYTES + d * 256);
+            };
+            if (cnt > 0)
+                issue(0);
+            if (cnt > 1)
+                issue(1);
+            static_for<SK_RMAX>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                if (i < cnt) {
+                    // LDS-DMAs retire in issue order: strip i is complete once only strip i + 1's are outstanding
+                    if (i + 1 < cnt)
+                        __builtin_amdgcn_s_waitcnt(0x0F70 | SK_VM_PER_STRIP);
+                    else
+                        __builtin_amdgcn_s_waitcnt(0x0F70);
+                    asm volatile("" ::: "memory");
+                    const uint8_t* buf = my + (i & 1) * SK_STAGE;
+                    const uint2 sc = *reinterpret_cast<const uint2*>(buf + SK_WBYTES + l16 * 32 + 8 * q);
+                    static_for<2>([&](auto hc) {
+                        constexpr int h = decltype(hc)::value;
+                        uint4 wv[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)  // MX group 8 q + 4 h + j of the slice, row l16
+                            wv[j] = *reinterpret_cast<const uint4*>(buf + wread + (4 * h + j) * 16);
+                        if (h == 1) {
+                            // the buffer is refilled only after every read of it has returned
+                            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                            if (i + 2 < cnt)
+                                issue(i + 2);
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const float scale = e8m0_to_f32(((h ? sc.y : sc.x) >> (8 * j)) & 0xFFu);
+                            const uint32_t xs[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) {
+                                const uint4 w8 = dequant8<HW_CVT>(xs[t], scale);
+                                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                    __builtin_bit_cast(bf16x8, areg[(4 * h + j) * 4 + t]), __builtin_bit_cast(bf16x8, w8), acc[i], 0, 0, 0);
+                            }
+                        }
+                    });
+                }
+            });
+        }
+
+        // sum the k-slice partials of each strip in slice order; every wave parks its accumulators in its own region
+        f32x4* part = reinterpret_cast<f32x4*>(my);
+#pragma unroll
+        for (int i = 0; i < SK_RMAX; ++i)
+            part[i * 64 + lane] = acc[i];
+        __syncthreads();
+        for (int idx = tid; idx < rgs * SK_RMAX * 64; idx += SK_WAVES * 64) {
+            const int rg2 = idx / (SK_RMAX * 64), i = (idx >> 6) & (SK_RMAX - 1), ln = idx & 63;
+            const int strip = s_begin + rg2 + rgs * (b0 + i);
+            if (strip >= s_end)
+                continue;
+            f32x4 sum = {0, 0, 0, 0};
+            for (int s = 0; s < ksw; ++s) {
+                const f32x4 v = reinterpret_cast<const f32x4*>(smem + (rg2 * ksw + s) * SK_WAVE_LDS)[i * 64 + ln];
+                sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
+            }
+            const int gj = strip * 16 + (ln & 15);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int gi = 4 * (ln >> 4) + r;
+                if (gi < p.m && gj < p.n) {
+                    if (p.out_bf16)
+                        reinterpret_cast<uint16_t*>(p.out)[(long)gi * p.ldc + gj] = f32_to_bf16_bits(sum[r]);
+                    else
+                        reinterpret_cast<float*>(p.out)[(long)gi * p.ldc + gj] = sum[r];
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // Generic form for shapes the streaming kernel does not take: one thread per output, k ascending, fp32 fma
 // (the same order as the reference TMATMUL on the dequantised bf16 weights).
 __global__ void gemv_mxfp4_generic_kernel(const GemvParams p)
@@ -211,16 +363,42 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
         set_last_kernel("gemv_mxfp4_generic");
         return PTOAMD_OK;
     }
-    // 16 rows per wave; 7 waves per workgroup when that tiles the row groups more evenly over the CUs than 8
-    // (N = 28672: 1792 groups = 256 workgroups of 7), else 8
     int dev = 0, cus = 256;
     PTOAMD_HIP_CHECK(hipGetDevice(&dev));
     PTOAMD_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const char* sw_cvt = getenv("PTOAMD_GEMV_SW_CVT");
+    const bool swc = sw_cvt && sw_cvt[0] == '1';
+    const char* no_sk = getenv("PTOAMD_GEMV_NO_SPLITK");
+    if (k % SK_SLICE == 0 && (reinterpret_cast<uintptr_t>(sw) & 3u) == 0 && !(no_sk && no_sk[0] == '1')) {
+        const int ks = k / SK_SLICE;
+        int ksw_log2 = 0;
+        while (ksw_log2 < 3 && (2 << ksw_log2) <= ks)
+            ++ksw_log2;
+        const int rgs = SK_WAVES >> ksw_log2;
+        int spw = (p.n_groups + cus - 1) / cus;          // strips per workgroup, a multiple of the row-group count
+        spw = (spw + rgs - 1) / rgs * rgs;
+        const int grid = (p.n_groups + spw - 1) / spw;
+        static bool attr_set[2] = {false, false};
+        if (!attr_set[swc]) {
+            PTOAMD_HIP_CHECK(swc ? hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mxfp4_splitk_kernel<false>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS)
+                                 : hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mxfp4_splitk_kernel<true>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS));
+            attr_set[swc] = true;
+        }
+        if (swc)
+            hipLaunchKernelGGL(gemv_mxfp4_splitk_kernel<false>, dim3(grid), dim3(SK_WAVES * 64), SK_LDS, stream, p, ksw_log2, spw);
+        else
+            hipLaunchKernelGGL(gemv_mxfp4_splitk_kernel<true>, dim3(grid), dim3(SK_WAVES * 64), SK_LDS, stream, p, ksw_log2, spw);
+        PTOAMD_HIP_CHECK(hipGetLastError());
+        set_last_kernel(swc ? "gemv_mxfp4_splitk_swcvt" : "gemv_mxfp4_splitk");
+        return PTOAMD_OK;
+    }
+    // streaming kernel: 16 rows per wave; 7 waves per workgroup when that tiles the row groups more evenly over the
+    // CUs than 8, else 8
     const int g7 = (p.n_groups + 6) / 7, g8 = (p.n_groups + 7) / 8;
     const auto rounds = [&](int blocks) { return (blocks + cus - 1) / cus; };
     const bool use7 = rounds(g7) * 7 < rounds(g8) * 8;
-    const char* sw_cvt = getenv("PTOAMD_GEMV_SW_CVT");
-    const bool swc = sw_cvt && sw_cvt[0] == '1';
     if (use7) {
         if (swc)
             hipLaunchKernelGGL((gemv_mxfp4_kernel<false, 7>), dim3(g7), dim3(7 * 64), 0, stream, p);

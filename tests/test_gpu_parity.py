@@ -357,24 +357,51 @@ def _gemv_reference(oracle, a_bits, w, sw, n, k):
     return oracle.matmul_bf16(a_bits, wbits, b_dn=True)
 
 
-@pytest.mark.parametrize("m,n,k", [(16, 256, 1024), (16, 1000, 8192), (5, 48, 2048), (1, 16, 1024)])
-def test_gemv_mxfp4(pa, oracle, m, n, k):
+def _gemv_case(m, n, k):
     r = np.random.default_rng(m + n)
     a = bf16_bits(r.standard_normal((m, k)))
     w = r.integers(0, 256, (n, k // 2)).astype(np.uint8)
     sw = r.integers(118, 132, (n, k // 32)).astype(np.uint8)
-    ref = _gemv_reference(oracle, a, w, sw, n, k)
+    return a, w, sw
+
+
+def _check_gemv(pa, oracle, m, n, k, kernel):
+    a, w, sw = _gemv_case(m, n, k)
+    # big cases: the oracle sees a spread of weight rows plus the ragged tail
+    cols = np.arange(n) if n * k <= (1 << 25) else np.unique(np.r_[np.arange(0, n, 61), np.arange(n - 40, n)])
+    ref = _gemv_reference(oracle, a, w[cols], sw[cols], len(cols), k)
     got = host(pa.gemv_mxfp4(dev(a).view(torch.bfloat16), dev(w), dev(sw), n, k, pa.F32))
-    assert pa.last_kernel() == "gemv_mxfp4_stream"
-    assert relerr(got, ref) <= 2e-2
+    assert pa.last_kernel() == kernel
+    assert relerr(got[:, cols], ref) <= 2e-2
     with tile_env(PTOAMD_GEMV_SW_CVT=1):
         sw_path = host(pa.gemv_mxfp4(dev(a).view(torch.bfloat16), dev(w), dev(sw), n, k, pa.F32))
+        assert pa.last_kernel() == kernel + "_swcvt"
     assert np.array_equal(got.view(np.uint32), sw_path.view(np.uint32))  # the hardware fp4->bf16 conversion is exact
     with tile_env(PTOAMD_FORCE_GENERIC=1):
         exact = host(pa.gemv_mxfp4(dev(a).view(torch.bfloat16), dev(w), dev(sw), n, k, pa.F32))
-    assert np.array_equal(exact.view(np.uint32), ref.view(np.uint32))
+    assert np.array_equal(exact[:, cols].view(np.uint32), ref.view(np.uint32))
     got16 = host(pa.gemv_mxfp4(dev(a).view(torch.bfloat16), dev(w), dev(sw), n, k, pa.BF16))
     assert np.array_equal(got16, oracle.store_f32(got, ob.ST_BF16))
+    return got
+
+
+# k a multiple of 1024: 1, 2, 3, 4, 8, 12 and 16 k-slices (1, 2, 2, 4, 8, 8, 8 waves per strip), ragged n and m,
+# more strips per workgroup than one accumulator batch holds (n = 40000: 2500 strips over 256 workgroups, 10 each)
+@pytest.mark.parametrize("m,n,k", [(16, 256, 1024), (16, 1000, 8192), (5, 48, 2048), (1, 16, 1024), (7, 333, 3072),
+                                   (16, 4096, 4096), (2, 40000, 1024), (16, 520, 12288), (3, 36, 16384),
+                                   (16, 40000, 8192)])
+def test_gemv_mxfp4_splitk(pa, oracle, m, n, k):
+    got = _check_gemv(pa, oracle, m, n, k, "gemv_mxfp4_splitk")
+    with tile_env(PTOAMD_GEMV_NO_SPLITK=1):  # the streaming kernel agrees to rounding
+        a, w, sw = _gemv_case(m, n, k)
+        other = host(pa.gemv_mxfp4(dev(a).view(torch.bfloat16), dev(w), dev(sw), n, k, pa.F32))
+        assert pa.last_kernel() == "gemv_mxfp4_stream"
+    assert relerr(other, got) <= 1e-5
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 256, 512), (5, 1000, 1536), (1, 16, 2560), (16, 2049, 512)])
+def test_gemv_mxfp4_stream(pa, oracle, m, n, k):
+    _check_gemv(pa, oracle, m, n, k, "gemv_mxfp4_stream")
 
 
 def test_gemv_ragged_k_takes_the_generic_kernel(pa, oracle):
@@ -396,7 +423,7 @@ def test_config5_mxfp4_decode_full_size(pa, oracle):
     xw = torch.randn((n, k), generator=gen, device=DEV)
     w, sw = pa.tquant_mx(xw, pa.OCP_MXFP4, want_aux=False)
     out = pa.gemv_mxfp4(a, w, sw, n, k, pa.F32)
-    assert pa.last_kernel() == "gemv_mxfp4_stream"
+    assert pa.last_kernel() == "gemv_mxfp4_splitk"
     cols = np.arange(0, n, 97)
     ref = _gemv_reference(oracle, host(a), host(sel(w, cols)), host(sel(sw, cols)), len(cols), k)
     assert relerr(host(out)[:, cols], ref) <= 2e-2
