@@ -8,13 +8,13 @@
 //     k-slice s (1024 k) of every strip and keeps its activation fragments for that slice in registers for the whole
 //     kernel (128 VGPRs, loaded once).  Weights and scales stream global -> LDS by LDS-DMA into a per-wave
 //     double-buffered region (512 contiguous bytes per row, two rows per instruction, no VGPRs, no barriers: a wave
-//     reads back only what it wrote), are re-read as MFMA operand fragments (16-byte chunks XOR-swizzled by row on
-//     the global side, so the reads are conflict-free), dequantised in registers and multiplied on
+//     reads back only what it wrote), are re-read as MFMA operand fragments (4 bytes = 8 fp4 per lane and MFMA; row
+//     pairs padded and odd rows half-swapped on the global side, so the reads are conflict-free), dequantised in
+//     registers and multiplied on
 //     v_mfma_f32_16x16x32_bf16.  The 8 k-slice partials of a strip are summed through LDS in a fixed order.
 //   * streaming (k % 512 == 0 otherwise): a wave owns 16 rows over the full K, register prefetch four chunks deep,
 //     activations staged per chunk through LDS.
-// Dequantisation: v_cvt_scalef32_pk_bf16_fp4 (fp4 pair * 2^e -> bf16 pair, exact).  Operand k-slots are assigned so
-// that a lane's 32 consecutive k (one MX group, one scale byte) feed 4 MFMAs.
+// Dequantisation: v_cvt_scalef32_pk_bf16_fp4 (fp4 pair * 2^e -> bf16 pair, exact).
 #include "common_host.hpp"
 #include "device_types.hpp"
 #include "lds_dma.hpp"
@@ -192,7 +192,13 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
     const int ks = p.k / SK_SLICE, sb = p.k / 32;
     uint8_t* my = smem + wave * SK_WAVE_LDS;
     const uint32_t my_lds = lds_address(my);
-    const int wread = (l16 >> 1) * SK_PAIR + (l16 & 1) * 512 + ((8 * q) ^ (8 * (l16 & 1))) * 16;  // row l16, chunk 8 q
+    // LDS byte of (row l16, chunk t, byte 4 q) is wread0 + 16 t for chunks with (t & 8) == 0, wread1 + 16 t for the others
+    // (odd rows keep their 128-byte halves swapped: 64 lanes reading one chunk index hit 64 different banks)
+    const int wrow = (l16 >> 1) * SK_PAIR + (l16 & 1) * 512 + 4 * q;
+    const int wread0 = wrow + 128 * (l16 & 1), wread1 = wrow - 128 * (l16 & 1);
+    // activation stages use the same row layout with 16-byte pieces: (row l16, step tt of the quarter, piece q)
+    const int arow = (l16 >> 1) * SK_PAIR + (l16 & 1) * 512 + 16 * q;
+    const int aread0 = arow + 128 * (l16 & 1), aread1 = arow - 128 * (l16 & 1);
     const int mine = s_end > s_begin + rg ? (s_end - s_begin - rg + rgs - 1) / rgs : 0;  // strips of this row group
     const int most = (s_end - s_begin + rgs - 1) / rgs;                                   // ... of row group 0
 
@@ -203,19 +209,19 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
         for (int i = 0; i < SK_RMAX; ++i)
             acc[i] = f32x4{0, 0, 0, 0};
 
-        for (int kb = slice; kb < ks; kb += ksw) {
-            // activation fragments of this k-slice: lane (m = l16, quarter q) holds A[m][1024 kb + 256 q .. + 255];
-            // lanes past the last activation row re-read it (their output rows are never stored)
-            uint4 areg[32];
-            const uint4* ap = reinterpret_cast<const uint4*>(p.a + (long)min(l16, p.m - 1) * p.lda + kb * SK_SLICE + q * 256);
+        for (int kb = slice; kb < ks && cnt > 0; kb += ksw) {
+            // 16 rows x 512 bytes -> one LDS stage.  One LDS-DMA moves a row pair (2 x 512 contiguous bytes); pairs are
+            // 16 bytes apart in LDS and odd rows swap their 128-byte halves (chunk ^ 8), so that the fragment reads
+            // below are conflict-free with lane-constant base addresses.  Addresses are a wave-uniform base plus a
+            // 32-bit lane offset; rows past rlim re-read row rlim.
+            auto issue_rows = [&](const uint8_t* base, uint32_t row_bytes, int rlim, uint32_t dst, int ln) {
+                const int hi = ln >> 5;
+                const uint32_t chunk_off = ((ln & 31) ^ (8 * hi)) * 16;
 #pragma unroll
-            for (int x = 0; x < 32; ++x)
-                areg[x] = ap[x];
-
-            // strip i of the batch -> buffer i & 1.  One LDS-DMA moves a row pair (2 x 512 contiguous bytes); pairs
-            // are 16 bytes apart in LDS and odd rows swap their 128-byte halves (chunk ^ 8), so that 16 lanes reading
-            // one chunk index of the 16 rows hit 16 different bank groups with a lane-constant base address.
-            // Addresses are a wave-uniform strip base plus a 32-bit lane offset (rows past n - 1 re-read row n - 1).
+                for (int d = 0; d < 8; ++d)
+                    lds_dma16_off(base, __umul24(min(2 * d + hi, rlim), row_bytes) + chunk_off, dst + d * SK_PAIR);
+            };
+            // weight strip i of the batch (and its scales) -> buffer i & 1
             auto issue = [&](int i) {
                 const int strip = s_begin + rg + rgs * (b0 + i);
                 const int rlim = min(15, p.n - 1 - strip * 16);
@@ -226,20 +232,45 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
                 // precomputed for all strips of the batch and parked in scratch memory)
                 int ln = lane;
                 asm volatile("" : "+v"(ln));
-                const int hi = ln >> 5;
-                const uint32_t chunk_off = ((ln & 31) ^ (8 * hi)) * 16;
-#pragma unroll
-                for (int d = 0; d < 8; ++d)
-                    lds_dma16_off(wbase, __umul24(min(2 * d + hi, rlim), (uint32_t)p.ldw_bytes) + chunk_off, dst + d * SK_PAIR);
+                issue_rows(wbase, (uint32_t)p.ldw_bytes, rlim, dst, ln);
 #pragma unroll
                 for (int d = 0; d < 2; ++d)
                     lds_dma4_off(sbase, __umul24(min(8 * d + (ln >> 3), rlim), (uint32_t)sb) + (ln & 7) * 4,
                                  dst + SK_WBYTES + d * 256);
             };
-            if (cnt > 0)
-                issue(0);
-            if (cnt > 1)
-                issue(1);
+            // activation quarter j (256 k of the slice, 16 rows x 512 bytes) -> buffer j & 1; rows past m - 1 re-read
+            // row m - 1 (their output rows are never stored)
+            auto issue_a = [&](int j) {
+                int ln = lane;
+                asm volatile("" : "+v"(ln));
+                issue_rows(reinterpret_cast<const uint8_t*>(p.a) + (long)kb * (SK_SLICE * 2) + j * 512, (uint32_t)p.lda * 2,
+                           p.m - 1, my_lds + (j & 1) * SK_STAGE, ln);
+            };
+
+            // Activation fragments of this k-slice, in the MFMA's own k order: step t multiplies k = 32 t .. 32 t + 31 of
+            // the slice and lane (m = l16, quarter q) holds A[m][32 t + 8 q .. + 7].  Loading them straight from global
+            // memory would make 64 separate 16-byte requests per instruction (the row index is the fast lane index);
+            // instead the four quarters run through the same LDS-DMA pipeline as the weight strips, ahead of them.
+            uint4 areg[32];
+            issue_a(0);
+            issue_a(1);
+            static_for<4>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                if (j < 3 || cnt > 0)
+                    __builtin_amdgcn_s_waitcnt(0x0F70 | (j < 3 ? 8 : SK_VM_PER_STRIP));  // all but the next stage's DMAs
+                else
+                    __builtin_amdgcn_s_waitcnt(0x0F70);
+                asm volatile("" ::: "memory");
+                const uint8_t* buf = my + (j & 1) * SK_STAGE;
+#pragma unroll
+                for (int tt = 0; tt < 8; ++tt)
+                    areg[8 * j + tt] = *reinterpret_cast<const uint4*>(buf + ((tt & 2) ? aread1 : aread0) + 64 * tt);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (j + 2 < 4)
+                    issue_a(j + 2);
+                else if (j - 2 < cnt)
+                    issue(j - 2);
+            });
             static_for<SK_RMAX>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
                 if (i < cnt) {
@@ -250,13 +281,17 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
                         __builtin_amdgcn_s_waitcnt(0x0F70);
                     asm volatile("" ::: "memory");
                     const uint8_t* buf = my + (i & 1) * SK_STAGE;
-                    const uint2 sc = *reinterpret_cast<const uint2*>(buf + SK_WBYTES + l16 * 32 + 8 * q);
+                    const uint4 sc0 = *reinterpret_cast<const uint4*>(buf + SK_WBYTES + l16 * 32);
+                    const uint4 sc1 = *reinterpret_cast<const uint4*>(buf + SK_WBYTES + l16 * 32 + 16);
+                    const uint32_t sc[8] = {sc0.x, sc0.y, sc0.z, sc0.w, sc1.x, sc1.y, sc1.z, sc1.w};
                     static_for<2>([&](auto hc) {
                         constexpr int h = decltype(hc)::value;
-                        uint4 wv[4];
+                        uint32_t wv[16];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j)  // MX group 8 q + 4 h + j of the slice, row l16
-                            wv[j] = *reinterpret_cast<const uint4*>(buf + wread + (4 * h + j) * 16);
+                        for (int j = 0; j < 16; ++j) {  // step t = 16 h + j: MX group t of the slice, 8 fp4 at byte 4 q
+                            const int t = 16 * h + j;
+                            wv[j] = *reinterpret_cast<const uint32_t*>(buf + ((t & 8) ? wread1 : wread0) + t * 16);
+                        }
                         if (h == 1) {
                             // the buffer is refilled only after every read of it has returned
                             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -264,15 +299,12 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
                                 issue(i + 2);
                         }
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const float scale = e8m0_to_f32(((h ? sc.y : sc.x) >> (8 * j)) & 0xFFu);
-                            const uint32_t xs[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
-#pragma unroll
-                            for (int t = 0; t < 4; ++t) {
-                                const uint4 w8 = dequant8<HW_CVT>(xs[t], scale);
-                                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                                    __builtin_bit_cast(bf16x8, areg[(4 * h + j) * 4 + t]), __builtin_bit_cast(bf16x8, w8), acc[i], 0, 0, 0);
-                            }
+                        for (int j = 0; j < 16; ++j) {
+                            const int t = 16 * h + j;
+                            const float scale = e8m0_to_f32((sc[t >> 2] >> (8 * (t & 3))) & 0xFFu);
+                            const uint4 w8 = dequant8<HW_CVT>(wv[j], scale);
+                            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, areg[t]),
+                                                                            __builtin_bit_cast(bf16x8, w8), acc[i], 0, 0, 0);
                         }
                     });
                 }
@@ -369,7 +401,9 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
     const char* sw_cvt = getenv("PTOAMD_GEMV_SW_CVT");
     const bool swc = sw_cvt && sw_cvt[0] == '1';
     const char* no_sk = getenv("PTOAMD_GEMV_NO_SPLITK");
-    if (k % SK_SLICE == 0 && (reinterpret_cast<uintptr_t>(sw) & 3u) == 0 && !(no_sk && no_sk[0] == '1')) {
+    // (row pitches are multiplied as 24-bit integers in the kernel's address arithmetic)
+    if (k % SK_SLICE == 0 && (reinterpret_cast<uintptr_t>(sw) & 3u) == 0 && (long)lda * 2 < (1L << 24) && p.ldw_bytes < (1L << 24) &&
+        !(no_sk && no_sk[0] == '1')) {
         const int ks = k / SK_SLICE;
         int ksw_log2 = 0;
         while (ksw_log2 < 3 && (2 << ksw_log2) <= ks)
