@@ -1,0 +1,346 @@
+// The tile instructions of the matmul path as workgroup-collective device functions.
+// Reference semantics: TLOAD cpu/TLoad.hpp:287-321; TMOV cpu/TMov.hpp:21-35; TEXTRACT cpu/TExtract.hpp:21-46;
+// TMATMUL / _ACC / _BIAS / TGEMV* cpu/TMatmul.hpp:77-113,207-252; TSTORE cpu/TStore.hpp:41-79,
+// cpu/common.hpp:187-198 (relu then static_cast).  Wrapper signatures: common/pto_instr.hpp:257-268,377-447,952-1010.
+//
+// Ordering: every instruction that writes LDS ends with a workgroup barrier, and starts with one (earlier readers of
+// the bytes it overwrites are done); instructions that only read LDS need no barrier of their own.
+#pragma once
+#include "tile.hpp"
+
+namespace pto {
+namespace amd {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4v __attribute__((ext_vector_type(4)));
+
+template <typename D, typename S>
+PTO_INST D convert(S v)
+{
+    return static_cast<D>(v);  // float -> _Float16 / __bf16: round to nearest even, as the reference's static_cast
+}
+
+// number of bytes one logical element occupies for plain (non-packed) types
+template <typename T>
+constexpr bool is_packed4 = std::is_same_v<T, float4_e2m1x2_t> || std::is_same_v<T, float4_e1m2x2_t>;
+
+// ---- generic element movement between global memory and an LDS tile ------------------------------------------------
+template <typename TileData, typename GlobalData>
+PTO_INST void tload_lds(TileData& dst, GlobalData& src)
+{
+    using T = typename TileData::DType;
+    static_assert(sizeof(T) == sizeof(typename GlobalData::DType), "TLOAD: tile and global element sizes differ");
+    static_assert(!is_packed4<T>, "TLOAD of packed fp4 tiles is not implemented on this backend yet");
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    const auto* g = reinterpret_cast<const T*>(src.data());
+    uint8_t* base = dst.Storage();
+    __syncthreads();
+    if constexpr (GlobalData::layout == Layout::DN) {  // rows are the contiguous direction in memory
+        for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
+            const int c = idx / vr, r = idx - c * vr;
+            *reinterpret_cast<T*>(base + dst.ByteOffset(r, c)) = g[src.Offset(r, c)];
+        }
+    } else {
+        for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
+            const int r = idx / vc, c = idx - r * vc;
+            *reinterpret_cast<T*>(base + dst.ByteOffset(r, c)) = g[src.Offset(r, c)];
+        }
+    }
+    __syncthreads();
+}
+
+template <typename TileData, typename GlobalData, AtomicType atomic, ReluPreMode relu>
+PTO_INST void tstore_lds(GlobalData& dst, TileData& src)
+{
+    using T = typename TileData::DType;
+    using G = typename GlobalData::DType;
+    static_assert(!is_packed4<T>, "TSTORE of packed fp4 tiles is not implemented on this backend yet");
+    static_assert(atomic == AtomicType::AtomicNone, "TSTORE AtomicAdd from an LDS tile is not implemented on this backend");
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    auto* g = reinterpret_cast<G*>(dst.data());
+    const uint8_t* base = src.Storage();
+    for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
+        const int r = idx / vc, c = idx - r * vc;
+        T v = *reinterpret_cast<const T*>(base + src.ByteOffset(r, c));
+        if constexpr (relu == ReluPreMode::NormalRelu)
+            v = v > T(0) ? v : T(0);
+        g[dst.Offset(r, c)] = convert<G>(v);
+    }
+}
+
+// dst(r, c) = src(r + row0, c + col0) over dst's static extent, zero outside src's valid region: the zero fill is what
+// lets TMATMUL walk the padded K of Left / Right tiles
+template <typename DstTile, typename SrcTile>
+PTO_INST void textract_lds(DstTile& dst, SrcTile& src, int row0, int col0)
+{
+    using T = typename DstTile::DType;
+    static_assert(std::is_same_v<T, typename SrcTile::DType>, "TMOV / TEXTRACT: element types differ");
+    static_assert(!is_packed4<T>, "TMOV of packed fp4 tiles is not implemented on this backend yet");
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    const uint8_t* s = src.Storage();
+    uint8_t* d = dst.Storage();
+    __syncthreads();
+    if constexpr (DstTile::Loc == TileType::Right) {  // stored transposed: walk k (rows) fastest
+        for (int idx = threadIdx.x; idx < DstTile::Rows * DstTile::Cols; idx += PTO_AMD_THREADS) {
+            const int c = idx / DstTile::Rows, r = idx - c * DstTile::Rows;
+            const int sr = r + row0, sc = c + col0;
+            T v{};
+            if (sr < vr && sc < vc && r < dst.GetValidRow() && c < dst.GetValidCol())
+                v = *reinterpret_cast<const T*>(s + src.ByteOffset(sr, sc));
+            *reinterpret_cast<T*>(d + dst.ByteOffset(r, c)) = v;
+        }
+    } else {
+        for (int idx = threadIdx.x; idx < DstTile::Rows * DstTile::Cols; idx += PTO_AMD_THREADS) {
+            const int r = idx / DstTile::Cols, c = idx - r * DstTile::Cols;
+            const int sr = r + row0, sc = c + col0;
+            T v{};
+            if (sr < vr && sc < vc && r < dst.GetValidRow() && c < dst.GetValidCol())
+                v = *reinterpret_cast<const T*>(s + src.ByteOffset(sr, sc));
+            *reinterpret_cast<T*>(d + dst.ByteOffset(r, c)) = v;
+        }
+    }
+    __syncthreads();
+}
+
+// ---- the contraction ------------------------------------------------------------------------------------------------
+// One 32 x 32 block per MFMA chain: lane (l32, lhi) feeds row l32 of the Left block and column l32 of the Right block;
+// its k-slots inside a step are lhi * (STEP / 2) .. + STEP / 2 - 1.
+template <typename T>
+struct Mfma;
+template <>
+struct Mfma<_Float16> {
+    static constexpr int STEP = 16;
+    template <typename Acc>
+    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const f16x8*>(a), *reinterpret_cast<const f16x8*>(b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma<__bf16> {
+    static constexpr int STEP = 16;
+    template <typename Acc>
+    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(a), *reinterpret_cast<const bf16x8*>(b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma<int8_t> {
+    static constexpr int STEP = 32;
+    template <typename Acc>
+    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
+    {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const i32x4v*>(a), *reinterpret_cast<const i32x4v*>(b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma<float> {
+    static constexpr int STEP = 2;
+    template <typename Acc>
+    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(*reinterpret_cast<const float*>(a), *reinterpret_cast<const float*>(b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma<float8_e4m3_t> {
+    static constexpr int STEP = 16;
+    template <typename Acc>
+    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(*reinterpret_cast<const long*>(a), *reinterpret_cast<const long*>(b), c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma<float8_e5m2_t> {
+    static constexpr int STEP = 16;
+    template <typename Acc>
+    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(*reinterpret_cast<const long*>(a), *reinterpret_cast<const long*>(b), c, 0, 0, 0);
+    }
+};
+
+template <bool INIT, typename TileRes, typename TileLeftT, typename TileRightT>
+PTO_INST void tmatmul(TileRes& c, TileLeftT& a, TileRightT& b)
+{
+    using T = typename TileLeftT::DType;
+    static_assert(TileRes::Loc == TileType::Acc && TileLeftT::Loc == TileType::Left && TileRightT::Loc == TileType::Right,
+                  "TMATMUL takes (Acc, Left, Right) tiles");
+    static_assert(std::is_same_v<T, typename TileRightT::DType>, "TMATMUL: Left and Right element types differ");
+    static_assert(TileLeftT::Cols == TileRightT::Rows && TileRes::Rows == TileLeftT::Rows && TileRes::Cols == TileRightT::Cols,
+                  "TMATMUL: static tile shapes do not chain (M x K) . (K x N) -> (M x N)");
+    static_assert(std::is_integral_v<typename TileRes::DType> == std::is_integral_v<T>,
+                  "TMATMUL: int8 operands accumulate in int32, floating operands in float");
+    using M = Mfma<T>;
+    static_assert(TileLeftT::Cols % M::STEP == 0, "TMATMUL: the static K of the tiles must be a multiple of the MFMA k-step");
+    const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kpad = min((a.GetValidCol() + M::STEP - 1) / M::STEP * M::STEP, TileLeftT::Cols);
+    const uint8_t* pa = a.Storage();
+    const uint8_t* pb = b.Storage();
+    constexpr int RB = TileRes::RB, CB = TileRes::CB;
+#pragma unroll
+    for (int slot = 0; slot < TileRes::NBLK; ++slot) {
+        const int blk = slot * WAVES + wave;
+        if (blk < RB * CB) {
+            const int bi = blk / CB, bj = blk - bi * CB;
+            const int arow = min(bi * 32 + l32, TileLeftT::Rows - 1);
+            const int bcol = min(bj * 32 + l32, TileRightT::Cols - 1);
+            typename TileRes::Vec16 acc = c.regs[slot];
+            if constexpr (INIT)
+                acc = typename TileRes::Vec16(0);
+            for (int k0 = 0; k0 < kpad; k0 += M::STEP) {
+                const int k = k0 + lhi * (M::STEP / 2);
+                acc = M::run(pa + a.ByteOffset(arow, k), pb + b.ByteOffset(k, bcol), acc);
+            }
+            c.regs[slot] = acc;
+        }
+    }
+}
+
+// visits every accumulator element this lane owns: f(slot, reg index, row, col)
+template <typename TileRes, typename F>
+PTO_INST void for_each_acc(TileRes& c, F&& f)
+{
+    const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    constexpr int CB = TileRes::CB;
+#pragma unroll
+    for (int slot = 0; slot < TileRes::NBLK; ++slot) {
+        const int blk = slot * WAVES + wave;
+        if (blk < TileRes::RB * CB) {
+            const int bi = blk / CB, bj = blk - bi * CB;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                f(slot, r, bi * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3), bj * 32 + l32);
+        }
+    }
+}
+
+template <typename TileRes, typename GlobalData, AtomicType atomic, ReluPreMode relu>
+PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
+{
+    using G = typename GlobalData::DType;
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    auto* g = reinterpret_cast<G*>(dst.data());
+    for_each_acc(src, [&](int slot, int r, int row, int col) {
+        if (row < vr && col < vc) {
+            auto v = src.regs[slot][r];
+            if constexpr (relu == ReluPreMode::NormalRelu)
+                v = v > 0 ? v : 0;
+            if constexpr (atomic == AtomicType::AtomicAdd) {
+                static_assert(atomic != AtomicType::AtomicAdd || std::is_same_v<G, float> || std::is_same_v<G, int32_t>,
+                              "TSTORE AtomicAdd targets float or int32 on this backend");
+                atomicAdd(&g[dst.Offset(row, col)], convert<G>(v));
+            } else {
+                g[dst.Offset(row, col)] = convert<G>(v);
+            }
+        }
+    });
+}
+
+}  // namespace amd
+
+// ---- TLOAD ---------------------------------------------------------------------------------------------------------
+template <typename TileData, typename GlobalData, typename... WaitEvents>
+PTO_INST RecordEvent TLOAD(TileData& dst, GlobalData& src, WaitEvents&...)
+{
+    static_assert(TileData::Loc != TileType::Acc, "TLOAD targets an on-chip buffer tile, not an accumulator");
+    amd::tload_lds(dst, src);
+    return {};
+}
+
+// ---- TSTORE --------------------------------------------------------------------------------------------------------
+template <typename TileData, typename GlobalData, AtomicType atomicType = AtomicType::AtomicNone,
+          ReluPreMode reluPreMode = ReluPreMode::NoRelu, typename... WaitEvents>
+PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, WaitEvents&...)
+{
+    if constexpr (TileData::Loc == TileType::Acc)
+        amd::tstore_acc<TileData, GlobalData, atomicType, reluPreMode>(dst, src);
+    else
+        amd::tstore_lds<TileData, GlobalData, atomicType, reluPreMode>(dst, src);
+    return {};
+}
+
+// ---- TMOV / TEXTRACT -----------------------------------------------------------------------------------------------
+template <typename DstTileData, typename SrcTileData, typename... WaitEvents>
+PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, WaitEvents&...)
+{
+    static_assert(DstTileData::Loc != TileType::Acc && SrcTileData::Loc != TileType::Acc,
+                  "TMOV from / to accumulator tiles is not implemented on this backend yet");
+    amd::textract_lds(dst, src, 0, 0);
+    return {};
+}
+template <typename DstTileData, typename SrcTileData, typename... WaitEvents>
+PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, uint16_t indexRow = 0, uint16_t indexCol = 0, WaitEvents&...)
+{
+    static_assert(DstTileData::Loc != TileType::Acc && SrcTileData::Loc != TileType::Acc,
+                  "TEXTRACT from / to accumulator tiles is not implemented on this backend yet");
+    amd::textract_lds(dst, src, indexRow, indexCol);
+    return {};
+}
+
+// ---- TMATMUL family ------------------------------------------------------------------------------------------------
+template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
+PTO_INST RecordEvent TMATMUL(TileRes& cMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, WaitEvents&...)
+{
+    amd::tmatmul<true>(cMatrix, aMatrix, bMatrix);
+    return {};
+}
+template <AccPhase Phase, typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
+PTO_INST RecordEvent TMATMUL(TileRes& cMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, WaitEvents&...)
+{
+    amd::tmatmul<true>(cMatrix, aMatrix, bMatrix);
+    return {};
+}
+template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
+PTO_INST RecordEvent TMATMUL_ACC(TileRes& cOutMatrix, TileRes& cInMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, WaitEvents&...)
+{
+    if (&cOutMatrix != &cInMatrix) {
+#pragma unroll
+        for (int s = 0; s < TileRes::NBLK; ++s)
+            cOutMatrix.regs[s] = cInMatrix.regs[s];
+    }
+    amd::tmatmul<false>(cOutMatrix, aMatrix, bMatrix);
+    return {};
+}
+template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
+PTO_INST RecordEvent TMATMUL_ACC(TileRes& cMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, WaitEvents&...)
+{
+    amd::tmatmul<false>(cMatrix, aMatrix, bMatrix);
+    return {};
+}
+// bias (1 x N, any LDS tile) is added after the K loop, per column (reference: cpu/TMatmul.hpp:219-230)
+template <typename TileRes, typename TileLeftT, typename TileRightT, typename TileBias, typename... WaitEvents>
+PTO_INST RecordEvent TMATMUL_BIAS(TileRes& cMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, TileBias& biasData, WaitEvents&...)
+{
+    amd::tmatmul<true>(cMatrix, aMatrix, bMatrix);
+    using B = typename TileBias::DType;
+    const uint8_t* pb = biasData.Storage();
+    const int vc = cMatrix.GetValidCol();
+    amd::for_each_acc(cMatrix, [&](int slot, int r, int, int col) {
+        if (col < vc)
+            cMatrix.regs[slot][r] += static_cast<typename TileRes::Reg>(*reinterpret_cast<const B*>(pb + biasData.ByteOffset(0, col)));
+    });
+    return {};
+}
+template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
+PTO_INST RecordEvent TGEMV(TileRes& c, TileLeftT& a, TileRightT& b, WaitEvents&...)
+{
+    return TMATMUL(c, a, b);
+}
+template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
+PTO_INST RecordEvent TGEMV_ACC(TileRes& cOut, TileRes& cIn, TileLeftT& a, TileRightT& b, WaitEvents&...)
+{
+    return TMATMUL_ACC(cOut, cIn, a, b);
+}
+template <typename TileRes, typename TileLeftT, typename TileRightT, typename TileBias, typename... WaitEvents>
+PTO_INST RecordEvent TGEMV_BIAS(TileRes& c, TileLeftT& a, TileRightT& b, TileBias& bias, WaitEvents&...)
+{
+    return TMATMUL_BIAS(c, a, b, bias);
+}
+
+}  // namespace pto

@@ -1,0 +1,198 @@
+// Tile<>: a 2-D on-chip operand.  Reference: include/pto/common/pto_tile.hpp:1422-1835 (template parameters, aliases,
+// valid-shape accessors), cpu/TAssign.hpp:21-36 (address binding).
+//
+// Where a tile lives on gfx950:
+//   Mat (L1), Vec (UB), Bias, Scaling, ScaleLeft/Right : LDS, plain row-major [Rows][Cols]
+//   Left  (L0A) : LDS, [Rows = M][Cols = K], k contiguous, 16-byte chunks XOR-swizzled by row (MFMA fragment reads)
+//   Right (L0B) : LDS, stored transposed [Cols = N][Rows = K], k contiguous, same swizzle
+//   Acc   (L0C) : registers; the tile is cut into 32 x 32 MFMA blocks, block b belongs to wave b % WAVES
+// BLayout / SLayout / fractal size are accepted for source compatibility; the internal layouts above are the backend's
+// own (they are invisible in global-memory results).
+#pragma once
+#include "base.hpp"
+
+namespace pto {
+namespace amd {
+
+constexpr int WAVES = PTO_AMD_THREADS / 64;
+
+// the core's LDS arena and its regions
+__device__ __forceinline__ uint8_t* lds_arena()
+{
+    extern __shared__ __align__(16) uint8_t pto_amd_lds[];
+    return pto_amd_lds;
+}
+template <TileType L>
+struct Region {
+    static constexpr bool in_lds = L != TileType::Acc && L != TileType::Ctrl;
+    static constexpr uint32_t base = L == TileType::Mat       ? 0u
+                                     : L == TileType::Left    ? PTO_AMD_L1_BYTES
+                                     : L == TileType::Right   ? PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES
+                                     : L == TileType::Vec     ? PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES
+                                     : L == TileType::Bias    ? PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES
+                                     : L == TileType::Scaling ? PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES + PTO_AMD_BIAS_BYTES
+                                                              : PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES + PTO_AMD_BIAS_BYTES + PTO_AMD_FB_BYTES;
+    static constexpr uint32_t size = L == TileType::Mat       ? PTO_AMD_L1_BYTES
+                                     : L == TileType::Left    ? PTO_AMD_L0A_BYTES
+                                     : L == TileType::Right   ? PTO_AMD_L0B_BYTES
+                                     : L == TileType::Vec     ? PTO_AMD_UB_BYTES
+                                     : L == TileType::Bias    ? PTO_AMD_BIAS_BYTES
+                                     : L == TileType::Scaling ? PTO_AMD_FB_BYTES
+                                                              : PTO_AMD_L0S_BYTES;  // ScaleLeft and ScaleRight share it
+};
+constexpr uint32_t LDS_TOTAL = PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES +
+                               PTO_AMD_BIAS_BYTES + PTO_AMD_FB_BYTES + PTO_AMD_L0S_BYTES;
+static_assert(LDS_TOTAL <= 160 * 1024, "the on-chip regions must fit the 160 KiB LDS of a CU");
+
+// Sticky status word of the kernels of this translation unit: 0, or the first constraint a core violated
+// (1: TASSIGN address outside its region).  pto::amd::device_status() reads it on the host.
+static __device__ int g_status = 0;
+__device__ __forceinline__ void report(int code)
+{
+    if (threadIdx.x == 0)
+        atomicCAS(&g_status, 0, code);
+}
+
+template <typename T>
+struct ElemTraits {
+    static constexpr int bytes2 = 2 * (int)sizeof(T);  // bytes of two elements
+};
+template <>
+struct ElemTraits<float4_e2m1x2_t> {
+    static constexpr int bytes2 = 1;
+};
+template <>
+struct ElemTraits<float4_e1m2x2_t> {
+    static constexpr int bytes2 = 1;
+};
+
+// register storage of an accumulator tile
+template <typename T, int Rows, int Cols>
+struct AccStorage {
+    static constexpr int RB = (Rows + 31) / 32, CB = (Cols + 31) / 32, NBLK = (RB * CB + WAVES - 1) / WAVES;
+    using Reg = std::conditional_t<std::is_integral_v<T>, int32_t, float>;
+    typedef Reg Vec16 __attribute__((ext_vector_type(16)));
+    Vec16 regs[NBLK];
+};
+struct LdsStorage {
+    uint32_t lds_ = 0;  // byte offset of the tile in the arena
+};
+
+}  // namespace amd
+
+template <TileType Loc_, typename Element_, const int Rows_, const int Cols_, const BLayout BFractal_ = BLayout::RowMajor,
+          const int RowValid_ = Rows_, const int ColValid_ = Cols_, const SLayout SFractal_ = SLayout::NoneBox,
+          const int SFractalSize_ = TileConfig::fractalABSize, auto PadVal_ = PadValue::Null,
+          const CompactMode Compact_ = CompactMode::Null>
+struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_, Rows_, Cols_>, amd::LdsStorage> {
+    using DType = Element_;
+    static constexpr TileType Loc = Loc_;
+    static constexpr int Rows = Rows_, Cols = Cols_, ValidRow = RowValid_, ValidCol = ColValid_;
+    static constexpr BLayout BFractal = BFractal_;
+    static constexpr SLayout SFractal = SFractal_;
+    static constexpr int SFractalSize = SFractalSize_;
+    static constexpr int Numel = Rows_ * Cols_;
+    static constexpr uint32_t Bytes = (uint32_t)((int64_t)Rows_ * Cols_ * amd::ElemTraits<Element_>::bytes2 / 2);
+    static constexpr bool isRowMajor = BFractal_ == BLayout::RowMajor;
+
+    int vrow_ = RowValid_, vcol_ = ColValid_;
+
+    PTO_INST Tile() {}
+    // dynamic valid extents, in declaration order (reference: pto_tile.hpp:1654-1676)
+    PTO_INST Tile(int a)
+    {
+        if constexpr (RowValid_ == DYNAMIC)
+            vrow_ = a;
+        else
+            vcol_ = a;
+    }
+    PTO_INST Tile(int r, int c) : vrow_(r), vcol_(c) {}
+    PTO_INST int GetValidRow() const { return vrow_; }
+    PTO_INST int GetValidCol() const { return vcol_; }
+
+    // byte offset of logical element (r, c) inside the tile's LDS storage (fp4: of the byte holding it)
+    PTO_INST uint32_t ByteOffset(int r, int c) const
+    {
+        constexpr int b2 = amd::ElemTraits<Element_>::bytes2;
+        if constexpr (Loc_ == TileType::Left)
+            return KContiguous<Cols_>(r, c);
+        else if constexpr (Loc_ == TileType::Right)
+            return KContiguous<Rows_>(c, r);
+        else
+            return (uint32_t)(((int64_t)r * Cols_ + c) * b2 / 2);
+    }
+    // [row][KC] with k contiguous; 16-byte chunk index XORed with the row when the row holds a power-of-two number of
+    // chunks (<= 8 of its low bits), so 32 rows read at one k land in different banks
+    template <int KC>
+    PTO_INST static uint32_t KContiguous(int row, int k)
+    {
+        constexpr int b2 = amd::ElemTraits<Element_>::bytes2;
+        constexpr int row_bytes = KC * b2 / 2, chunks = row_bytes / 16;
+        constexpr bool swz = row_bytes % 16 == 0 && chunks >= 2 && (chunks & (chunks - 1)) == 0;
+        const int kb = k * b2 / 2;
+        if constexpr (swz) {
+            constexpr int mask = chunks < 8 ? chunks - 1 : 7;
+            return (uint32_t)(row * row_bytes + ((((kb >> 4) ^ (row & mask))) << 4) + (kb & 15));
+        } else {
+            return (uint32_t)(row * row_bytes + kb);
+        }
+    }
+    PTO_INST uint8_t* Storage() const
+    {
+        static_assert(Loc_ != TileType::Acc, "accumulator tiles live in registers");
+        return amd::lds_arena() + this->lds_;
+    }
+};
+
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileLeft = Tile<TileType::Left, Element_, Rows_, Cols_, BLayout::ColMajor, RowValid_, ColValid_, SLayout::RowMajor,
+                      TileConfig::fractalABSize>;
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileRight = Tile<TileType::Right, Element_, Rows_, Cols_, BLayout::RowMajor, RowValid_, ColValid_, SLayout::ColMajor,
+                       TileConfig::fractalABSize>;
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileAcc = Tile<TileType::Acc, Element_, Rows_, Cols_, BLayout::ColMajor, RowValid_, ColValid_, SLayout::RowMajor,
+                     TileConfig::fractalCSize>;
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileLeftScale = Tile<TileType::ScaleLeft, Element_, Rows_, Cols_, BLayout::RowMajor, RowValid_, ColValid_,
+                           SLayout::RowMajor, TileConfig::fractalMxSize>;
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileRightScale = Tile<TileType::ScaleRight, Element_, Rows_, Cols_, BLayout::ColMajor, RowValid_, ColValid_,
+                            SLayout::ColMajor, TileConfig::fractalMxSize>;
+
+template <typename T>
+struct is_tile : std::false_type {};
+template <TileType L, typename E, int R, int C, BLayout B, int RV, int CV, SLayout S, int F, auto P, CompactMode M>
+struct is_tile<Tile<L, E, R, C, B, RV, CV, S, F, P, M>> : std::true_type {};
+template <typename T>
+constexpr bool is_tile_data_v = is_tile<std::remove_cv_t<T>>::value;
+
+struct RecordEvent {};
+
+// TASSIGN: binds a tile to a byte address of its on-chip buffer (reference: cpu/TAssign.hpp:21-36,
+// common/pto_instr.hpp:104-121).  Accumulator tiles are register-resident: the address is accepted and ignored.
+template <typename T, typename AddrType>
+PTO_INST void TASSIGN(T& obj, AddrType addr)
+{
+    if constexpr (T::Loc != TileType::Acc) {
+        using R = amd::Region<T::Loc>;
+        uint32_t a = (uint32_t)(uint64_t)addr;
+        if (a + T::Bytes > R::size || (a & 15u) != 0) {
+            amd::report(1);
+            a = 0;
+        }
+        static_assert(T::Bytes <= R::size, "tile larger than its on-chip region (raise PTO_AMD_*_BYTES)");
+        obj.lds_ = R::base + a;
+    }
+}
+template <std::size_t Addr, typename T>
+PTO_INST std::enable_if_t<is_tile_data_v<T>> TASSIGN(T& obj)
+{
+    if constexpr (T::Loc != TileType::Acc) {
+        static_assert(Addr + T::Bytes <= amd::Region<T::Loc>::size && Addr % 16 == 0,
+                      "TASSIGN: address outside the tile's on-chip region or not 16-byte aligned");
+    }
+    TASSIGN(obj, Addr);
+}
+
+}  // namespace pto

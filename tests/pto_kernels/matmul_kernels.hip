@@ -1,0 +1,194 @@
+// PTO-style kernel sources for the gfx950 backend, written against <pto/pto-inst.hpp> the way the reference's own test
+// kernels are (tests/cpu/st/testcase/tmatmul/tmatmul_kernel.cpp:25-173 is the model for the single-tile and split-K
+// programs, demos/cpu/gemm_demo/gemm_demo.cpp:83-121 for the tiled GEMM), plus the extern "C" launchers the parity
+// tests call.  Inputs and outputs are device pointers.
+#include <pto/pto-inst.hpp>
+#include <pto/common/constants.hpp>
+
+using namespace pto;
+
+template <typename T>
+AICORE constexpr inline T CeilAlign(T a, T b)
+{
+    return b == 0 ? 0 : (a + b - 1) / b * b;
+}
+
+// One tile: C[validM, validN] = A[validM, validK] . B[validK, validN] (+ bias), all row-major in global memory.
+template <typename OutT, typename AT, typename BT, typename BiasT, int validM, int validK, int validN, bool isBias>
+__global__ AICORE void RunTMATMUL(__gm__ OutT* out, __gm__ AT* src0, __gm__ BT* src1, __gm__ BiasT* src2)
+{
+    constexpr int blockAlign = (sizeof(AT) == 1) ? 32 : 16;
+    constexpr int M = CeilAlign<int>(validM, 16);
+    constexpr int N = CeilAlign<int>(validN, blockAlign);
+    constexpr int K = CeilAlign<int>(validK, blockAlign);
+
+    using GlobalA = GlobalTensor<AT, Shape<1, 1, 1, validM, validK>, Stride<validM * validK, validM * validK, validM * validK, validK, 1>>;
+    using GlobalB = GlobalTensor<BT, Shape<1, 1, 1, validK, validN>, Stride<validK * validN, validK * validN, validK * validN, validN, 1>>;
+    using GlobalBias = GlobalTensor<BiasT, Shape<1, 1, 1, 1, validN>, Stride<validN, validN, validN, validN, 1>>;
+    using GlobalOut = GlobalTensor<OutT, Shape<1, 1, 1, validM, validN>, Stride<validM * validN, validM * validN, validM * validN, validN, 1>>;
+    GlobalA aGlobal(src0);
+    GlobalB bGlobal(src1);
+    GlobalOut outGlobal(out);
+
+    using MatA = Tile<TileType::Mat, AT, M, K, BLayout::ColMajor, validM, validK, SLayout::RowMajor, 512>;
+    using MatB = Tile<TileType::Mat, BT, K, N, BLayout::ColMajor, validK, validN, SLayout::RowMajor, 512>;
+    using LeftT = TileLeft<AT, M, K, validM, validK>;
+    using RightT = TileRight<BT, K, N, validK, validN>;
+    using AccT = TileAcc<OutT, M, N, validM, validN>;
+    using BiasTile = Tile<TileType::Bias, BiasT, 1, N, BLayout::RowMajor, 1, validN>;
+
+    MatA aMat;
+    MatB bMat;
+    TASSIGN(aMat, 0x0);
+    TASSIGN(bMat, 0x10000);
+    LeftT aTile;
+    RightT bTile;
+    AccT cTile;
+    BiasTile biasTile;
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(cTile, 0x0);
+    TASSIGN(biasTile, 0x0);
+
+    TLOAD(aMat, aGlobal);
+    TLOAD(bMat, bGlobal);
+    set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+
+    TMOV(aTile, aMat);
+    TMOV(bTile, bMat);
+    set_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
+    wait_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
+
+    if constexpr (isBias) {
+        GlobalBias biasGlobal(src2);
+        TLOAD(biasTile, biasGlobal);
+        if constexpr (validM == 1)
+            TGEMV_BIAS(cTile, aTile, bTile, biasTile);
+        else
+            TMATMUL_BIAS(cTile, aTile, bTile, biasTile);
+    } else {
+        if constexpr (validM == 1)
+            TGEMV(cTile, aTile, bTile);
+        else
+            TMATMUL(cTile, aTile, bTile);
+    }
+    set_flag(PIPE_M, PIPE_FIX, EVENT_ID0);
+    wait_flag(PIPE_M, PIPE_FIX, EVENT_ID0);
+    TSTORE(outGlobal, cTile);
+}
+
+// numRepeats K-slabs accumulated into one accumulator tile: TMATMUL for the first, TMATMUL_ACC after
+template <typename OutT, typename AT, typename BT, int M, int K, int N>
+__global__ AICORE void RunTMATMUL_SPLIT_K(__gm__ OutT* out, __gm__ AT* src0, __gm__ BT* src1, uint32_t numRepeats)
+{
+    using GlobalA = GlobalTensor<AT, Shape<1, 1, 1, M, K>, Stride<M * K, M * K, M * K, K, 1>>;
+    using GlobalB = GlobalTensor<BT, Shape<1, 1, 1, K, N>, Stride<K * N, K * N, K * N, N, 1>>;
+    using GlobalOut = GlobalTensor<OutT, Shape<1, 1, 1, M, N>, Stride<M * N, M * N, M * N, N, 1>>;
+    GlobalOut outGlobal(out);
+    using MatA = Tile<TileType::Mat, AT, M, K, BLayout::ColMajor, M, K, SLayout::RowMajor, 512>;
+    using MatB = Tile<TileType::Mat, BT, K, N, BLayout::ColMajor, K, N, SLayout::RowMajor, 512>;
+    MatA aMat;
+    MatB bMat;
+    TASSIGN(aMat, 0x0);
+    TASSIGN(bMat, 0x10000);
+    TileLeft<AT, M, K> aTile;
+    TileRight<BT, K, N> bTile;
+    TileAcc<OutT, M, N> cTile;
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(cTile, 0x0);
+    for (uint32_t i = 0; i < numRepeats; i++) {
+        GlobalA aGlobal(src0 + i * M * K);
+        GlobalB bGlobal(src1 + i * K * N);
+        TLOAD(aMat, aGlobal);
+        TLOAD(bMat, bGlobal);
+        TMOV(aTile, aMat);
+        TMOV(bTile, bMat);
+        if (i == 0)
+            TMATMUL(cTile, aTile, bTile);
+        else
+            TMATMUL_ACC(cTile, cTile, aTile, bTile);
+    }
+    TSTORE(outGlobal, cTile);
+}
+
+// The tiled GEMM of the CPU-simulator demo at full problem size: C[M, N] = A[M, K] . B[K, N], one core per BM x BN
+// output tile, K walked in BK slabs through TLOAD -> TMOV -> TMATMUL / TMATMUL_ACC, then TSTORE of the tile.
+template <typename OutT, typename InT, int M, int K, int N, int BM, int BN, int BK, bool B_IS_DN>
+__global__ AICORE void RunTiledGemm(__gm__ OutT* out, __gm__ InT* a, __gm__ InT* b)
+{
+    constexpr int tilesN = N / BN;
+    const int tile = (int)get_block_idx();
+    const int tm = tile / tilesN, tn = tile % tilesN;
+
+    using GlobalA = GlobalTensor<InT, Shape<1, 1, 1, BM, BK>, Stride<M * K, M * K, M * K, K, 1>>;
+    // B is [K][N] row-major (ND view) or [N][K] in memory (the DN view of the same logical K x N matrix)
+    using GlobalB = std::conditional_t<B_IS_DN, GlobalTensor<InT, Shape<1, 1, 1, BK, BN>, Stride<K * N, K * N, K * N, 1, K>, Layout::DN>,
+                                       GlobalTensor<InT, Shape<1, 1, 1, BK, BN>, Stride<K * N, K * N, K * N, N, 1>>>;
+    using GlobalOut = GlobalTensor<OutT, Shape<1, 1, 1, BM, BN>, Stride<M * N, M * N, M * N, N, 1>>;
+
+    using MatA = Tile<TileType::Mat, InT, BM, BK, BLayout::ColMajor, BM, BK, SLayout::RowMajor, 512>;
+    using MatB = Tile<TileType::Mat, InT, BK, BN, BLayout::ColMajor, BK, BN, SLayout::RowMajor, 512>;
+    MatA aMat;
+    MatB bMat;
+    TASSIGN(aMat, 0x0);
+    TASSIGN(bMat, 0x8000);
+    TileLeft<InT, BM, BK> aTile;
+    TileRight<InT, BK, BN> bTile;
+    TileAcc<float, BM, BN> cTile;
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(cTile, 0x0);
+
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        GlobalA aGlobal(a + (size_t)tm * BM * K + k0);
+        GlobalB bGlobal(B_IS_DN ? b + (size_t)tn * BN * K + k0 : b + (size_t)k0 * N + tn * BN);
+        TLOAD(aMat, aGlobal);
+        TLOAD(bMat, bGlobal);
+        TMOV(aTile, aMat);
+        TMOV(bTile, bMat);
+        if (k0 == 0)
+            TMATMUL(cTile, aTile, bTile);
+        else
+            TMATMUL_ACC(cTile, cTile, aTile, bTile);
+    }
+    GlobalOut outGlobal(out + (size_t)tm * BM * N + tn * BN);
+    TSTORE(outGlobal, cTile);
+}
+
+// ---- launchers ------------------------------------------------------------------------------------------------------
+// case ids follow the reference's tmatmul test list (tests/cpu/st/testcase/tmatmul/main.cpp:96-252):
+//   1: f16 40x50x60 -> f32      2: int8 6x7x8 -> i32        3: f16 128x128x64, 5 K-slabs (split-K) -> f32
+//   4: f32 56x110x40 -> f32     5: f16 gemv 1x110x50        6: f32 gemv 1x128x48       7: bf16 40x50x60 -> f32
+//   8: fp8 e4m3 33x64x70 -> f32 (f32 shapes are smaller than the reference's: three copies of a tile - L1, L0 and
+//   the accumulator - share 160 KiB of LDS here, not 512 + 64 + 64 KiB)
+//   11: f16 + f32 bias 26x100x94          12: int8 + i32 bias 8x7x6 ... (bias cases)
+//   100: tiled f16 512^3 -> f32 (B row-major)   101: tiled bf16 512x512x512 -> bf16 out (B column-major)
+template <auto Kernel, typename... Args>
+static int run(void* stream, int blocks, Args... args)
+{
+    return pto::amd::launch<Kernel>(blocks, stream, args...);
+}
+
+extern "C" int pto_kernels_launch(int id, void* out, void* src0, void* src1, void* src2, void* stream)
+{
+    switch (id) {
+    case 1: return run<&RunTMATMUL<float, half, half, float, 40, 50, 60, false>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)nullptr);
+    case 2: return run<&RunTMATMUL<int32_t, int8_t, int8_t, int32_t, 6, 7, 8, false>>(stream, 1, (int32_t*)out, (int8_t*)src0, (int8_t*)src1, (int32_t*)nullptr);
+    case 3: return run<&RunTMATMUL_SPLIT_K<float, half, half, 128, 128, 64>>(stream, 1, (float*)out, (half*)src0, (half*)src1, 5u);
+    case 4: return run<&RunTMATMUL<float, float, float, float, 56, 110, 40, false>>(stream, 1, (float*)out, (float*)src0, (float*)src1, (float*)nullptr);
+    case 5: return run<&RunTMATMUL<float, half, half, float, 1, 110, 50, false>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)nullptr);
+    case 6: return run<&RunTMATMUL<float, float, float, float, 1, 128, 48, false>>(stream, 1, (float*)out, (float*)src0, (float*)src1, (float*)nullptr);
+    case 7: return run<&RunTMATMUL<float, bfloat16_t, bfloat16_t, float, 40, 50, 60, false>>(stream, 1, (float*)out, (bfloat16_t*)src0, (bfloat16_t*)src1, (float*)nullptr);
+    case 8: return run<&RunTMATMUL<float, float8_e4m3_t, float8_e4m3_t, float, 33, 64, 70, false>>(stream, 1, (float*)out, (float8_e4m3_t*)src0, (float8_e4m3_t*)src1, (float*)nullptr);
+    case 11: return run<&RunTMATMUL<float, half, half, float, 26, 100, 94, true>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)src2);
+    case 12: return run<&RunTMATMUL<int32_t, int8_t, int8_t, int32_t, 8, 7, 6, true>>(stream, 1, (int32_t*)out, (int8_t*)src0, (int8_t*)src1, (int32_t*)src2);
+    case 13: return run<&RunTMATMUL<float, half, half, float, 1, 64, 96, true>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)src2);
+    case 100: return run<&RunTiledGemm<float, half, 512, 512, 512, 128, 128, 64, false>>(stream, 16, (float*)out, (half*)src0, (half*)src1);
+    case 101: return run<&RunTiledGemm<bfloat16_t, bfloat16_t, 512, 512, 512, 128, 128, 64, true>>(stream, 16, (bfloat16_t*)out, (bfloat16_t*)src0, (bfloat16_t*)src1);
+    default: return -1;
+    }
+}
+
+extern "C" int pto_kernels_status() { return pto::amd::device_status(); }
