@@ -10,9 +10,9 @@
 #define PTO_AMD_THREADS 256  // threads of one core (4 waves)
 #endif
 // LDS regions (bytes) standing in for the Ascend on-chip buffers (L1, L0A, L0B, UB, bias table, fix-pipe buffer,
-// L0 scale buffer); together they must fit the CU's 160 KiB.  Override before including this header.
+// L0 scale buffer, split evenly between the Left and the Right scales); together they must fit the CU's 160 KiB.  Override before including this header.
 #ifndef PTO_AMD_L1_BYTES
-#define PTO_AMD_L1_BYTES (88 * 1024)
+#define PTO_AMD_L1_BYTES (80 * 1024)
 #endif
 #ifndef PTO_AMD_L0A_BYTES
 #define PTO_AMD_L0A_BYTES (32 * 1024)
@@ -21,16 +21,16 @@
 #define PTO_AMD_L0B_BYTES (32 * 1024)
 #endif
 #ifndef PTO_AMD_UB_BYTES
-#define PTO_AMD_UB_BYTES (4 * 1024)
+#define PTO_AMD_UB_BYTES (8 * 1024)
 #endif
 #ifndef PTO_AMD_BIAS_BYTES
 #define PTO_AMD_BIAS_BYTES (2 * 1024)
 #endif
 #ifndef PTO_AMD_FB_BYTES
-#define PTO_AMD_FB_BYTES (1 * 1024)
+#define PTO_AMD_FB_BYTES (2 * 1024)
 #endif
 #ifndef PTO_AMD_L0S_BYTES
-#define PTO_AMD_L0S_BYTES (1 * 1024)
+#define PTO_AMD_L0S_BYTES (4 * 1024)
 #endif
 
 // A PTO kernel entry is written `__global__ AICORE void f(...)`; here it is a device function run by pto::amd::launch.
@@ -152,9 +152,20 @@ struct GlobalTensor {
             i2 = r / sh[3];
             i3 = r % sh[3];
             i4 = c % sh[4];
+        } else if constexpr (Layout_ == Layout::MX_A_ZZ) {  // E8M0 scales of the A side: r = row, c = K-group
+            i0 = 0; i1 = r / 16; i2 = c / 2; i3 = r % 16; i4 = c % 2;
+        } else if constexpr (Layout_ == Layout::MX_B_NN) {  // B side: r = K-group, c = column
+            i0 = 0; i1 = c / 16; i2 = r / 2; i3 = c % 16; i4 = r % 2;
+        } else if constexpr (Layout_ == Layout::MX_A_ND) {
+            i0 = 0; i1 = 0; i2 = r; i3 = c / 2; i4 = c % 2;
+        } else if constexpr (Layout_ == Layout::MX_A_DN) {
+            i0 = 0; i1 = 0; i2 = c / 2; i3 = r; i4 = c % 2;
+        } else if constexpr (Layout_ == Layout::MX_B_ND) {
+            i0 = 0; i1 = 0; i2 = r / 2; i3 = c; i4 = r % 2;
+        } else if constexpr (Layout_ == Layout::MX_B_DN) {
+            i0 = 0; i1 = 0; i2 = c; i3 = r / 2; i4 = r % 2;
         } else {
-            static_assert(Layout_ == Layout::ND || Layout_ == Layout::DN || Layout_ == Layout::NZ,
-                          "GlobalTensor layout not supported by the gfx950 backend");
+            static_assert(Layout_ == Layout::ND, "GlobalTensor layout not supported by the gfx950 backend");
             i4 = c;
             i3 = r % sh[3];
             i2 = (r / sh[3]) % sh[2];
@@ -190,6 +201,36 @@ private:
     Shape shape_;
     Stride stride_;
 };
+
+// Shape / stride of a whole [rows, cols] logical matrix in a given layout (reference: common/pto_tile.hpp:664-1101).
+// BaseShape2D is the *stride* type, as in the reference.  For the MX layouts rows x cols is the logical scale matrix
+// ([M][K/32] on the A side, [K/32][N] on the B side).
+template <typename T, int64_t rows, int64_t cols, Layout L = Layout::ND>
+struct TileShape2D;
+template <typename T, int64_t rows, int64_t cols, Layout L = Layout::ND>
+struct BaseShape2D;
+#define PTO_AMD_SHAPE2D(LAYOUT, SHAPE, STRIDE)                                          \
+    template <typename T, int64_t rows, int64_t cols>                                 \
+    struct TileShape2D<T, rows, cols, LAYOUT> : SHAPE {                               \
+        using Parent = SHAPE;                                                         \
+        using Parent::Parent;                                                         \
+    };                                                                                \
+    template <typename T, int64_t rows, int64_t cols>                                 \
+    struct BaseShape2D<T, rows, cols, LAYOUT> : STRIDE {                              \
+        using Parent = STRIDE;                                                        \
+        using Parent::Parent;                                                         \
+    };
+#define PTO_AMD_C(...) __VA_ARGS__
+PTO_AMD_SHAPE2D(Layout::ND, PTO_AMD_C(Shape<1, 1, 1, rows, cols>), PTO_AMD_C(Stride<rows * cols, rows * cols, rows * cols, cols, 1>))
+PTO_AMD_SHAPE2D(Layout::DN, PTO_AMD_C(Shape<1, 1, 1, rows, cols>), PTO_AMD_C(Stride<rows * cols, rows * cols, rows * cols, 1, rows>))
+PTO_AMD_SHAPE2D(Layout::MX_A_ZZ, PTO_AMD_C(Shape<1, rows / 16, cols / 2, 16, 2>), PTO_AMD_C(Stride<rows * cols, cols * 16, 32, 2, 1>))
+PTO_AMD_SHAPE2D(Layout::MX_A_ND, PTO_AMD_C(Shape<1, 1, rows, cols / 2, 2>), PTO_AMD_C(Stride<rows * cols, rows * cols, cols, 2, 1>))
+PTO_AMD_SHAPE2D(Layout::MX_A_DN, PTO_AMD_C(Shape<1, 1, cols / 2, rows, 2>), PTO_AMD_C(Stride<rows * cols, rows * cols, 2 * rows, 2, 1>))
+PTO_AMD_SHAPE2D(Layout::MX_B_NN, PTO_AMD_C(Shape<1, cols / 16, rows / 2, 16, 2>), PTO_AMD_C(Stride<rows * cols, rows * 16, 32, 2, 1>))
+PTO_AMD_SHAPE2D(Layout::MX_B_ND, PTO_AMD_C(Shape<1, 1, rows / 2, cols, 2>), PTO_AMD_C(Stride<rows * cols, rows * cols, 2 * cols, 2, 1>))
+PTO_AMD_SHAPE2D(Layout::MX_B_DN, PTO_AMD_C(Shape<1, 1, cols, rows / 2, 2>), PTO_AMD_C(Stride<rows * cols, rows * cols, rows, 2, 1>))
+#undef PTO_AMD_SHAPE2D
+#undef PTO_AMD_C
 
 // ---- pipes and event ids (reference: common/cpu_stub.hpp:36-61): names only, ordering is by workgroup barriers
 using pipe_t = int;

@@ -201,6 +201,66 @@ PTO_INST void tmatmul(TileRes& c, TileLeftT& a, TileRightT& b)
     }
 }
 
+// Block-scaled contraction on v_mfma_scale_f32_32x32x64_f8f6f4: a k-step is two MX blocks of 32; lane (l32, lhi) feeds
+// bytes [16 lhi, 16 lhi + 16) of each block of its row / column and the E8M0 scale of block lhi.
+template <typename T>
+struct MxFormat;
+template <>
+struct MxFormat<float8_e4m3_t> {
+    static constexpr int code = 0;
+};
+template <>
+struct MxFormat<float8_e5m2_t> {
+    static constexpr int code = 1;
+};
+typedef int i32x8v __attribute__((ext_vector_type(8)));
+
+template <bool INIT, typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT>
+PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRightT& b, TileRightScaleT& bs)
+{
+    using TA = typename TileLeftT::DType;
+    using TB = typename TileRightT::DType;
+    static_assert(TileRes::Loc == TileType::Acc && TileLeftT::Loc == TileType::Left && TileRightT::Loc == TileType::Right &&
+                      TileLeftScaleT::Loc == TileType::ScaleLeft && TileRightScaleT::Loc == TileType::ScaleRight,
+                  "TMATMUL_MX takes (Acc, Left, ScaleLeft, Right, ScaleRight) tiles");
+    static_assert(std::is_same_v<typename TileRes::DType, float>, "TMATMUL_MX accumulates in float");
+    static_assert(TileLeftT::Cols % 64 == 0, "TMATMUL_MX: the static K of the Left tile must be a multiple of 64");
+    static_assert(TileLeftT::Cols == TileRightT::Rows && TileRes::Rows == TileLeftT::Rows && TileRes::Cols == TileRightT::Cols,
+                  "TMATMUL_MX: static tile shapes do not chain");
+    static_assert(TileLeftScaleT::Rows == TileLeftT::Rows && TileLeftScaleT::Cols * 32 == TileLeftT::Cols &&
+                      TileRightScaleT::Cols == TileRightT::Cols && TileRightScaleT::Rows * 32 == TileRightT::Rows,
+                  "TMATMUL_MX: one E8M0 scale per 32 K-elements");
+    const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kpad = min((a.GetValidCol() + 63) / 64 * 64, TileLeftT::Cols);
+    const uint8_t *pa = a.Storage(), *pb = b.Storage(), *psa = as.Storage(), *psb = bs.Storage();
+    constexpr int CB = TileRes::CB;
+#pragma unroll
+    for (int slot = 0; slot < TileRes::NBLK; ++slot) {
+        const int blk = slot * WAVES + wave;
+        if (blk < TileRes::RB * CB) {
+            const int bi = blk / CB, bj = blk - bi * CB;
+            const int arow = min(bi * 32 + l32, TileLeftT::Rows - 1);
+            const int bcol = min(bj * 32 + l32, TileRightT::Cols - 1);
+            typename TileRes::Vec16 acc = c.regs[slot];
+            if constexpr (INIT)
+                acc = typename TileRes::Vec16(0);
+            for (int k0 = 0; k0 < kpad; k0 += 64) {
+                const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 16 * lhi));
+                const uint4 a1 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 32 + 16 * lhi));
+                const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 16 * lhi, bcol));
+                const uint4 b1 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 + 16 * lhi, bcol));
+                const int g = k0 / 32 + lhi;
+                const int sa = psa[as.ByteOffset(arow, g)], sb = psb[bs.ByteOffset(g, bcol)];
+                const i32x8v av = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                const i32x8v bv = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, MxFormat<TA>::code, MxFormat<TB>::code, 0, sa, 0, sb);
+            }
+            c.regs[slot] = acc;
+        }
+    }
+}
+
 // visits every accumulator element this lane owns: f(slot, reg index, row, col)
 template <typename TileRes, typename F>
 PTO_INST void for_each_acc(TileRes& c, F&& f)
@@ -327,6 +387,48 @@ PTO_INST RecordEvent TMATMUL_BIAS(TileRes& cMatrix, TileLeftT& aMatrix, TileRigh
     });
     return {};
 }
+// ---- TMATMUL_MX / TGEMV_MX (fp8 E4M3 / E5M2 operands; reference: cpu/TMatmul.hpp:169-205,254-326) ------------------
+template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT,
+          typename = std::enable_if_t<TileLeftScaleT::Loc == TileType::ScaleLeft>>
+PTO_INST RecordEvent TMATMUL_MX(TileRes& cMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale, TileRightT& bMatrix, TileRightScaleT& bScale)
+{
+    amd::tmatmul_mx<true>(cMatrix, aMatrix, aScale, bMatrix, bScale);
+    return {};
+}
+template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT,
+          typename = std::enable_if_t<TileLeftScaleT::Loc == TileType::ScaleLeft>>
+PTO_INST RecordEvent TMATMUL_MX(TileRes& cOutMatrix, TileRes& cInMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale,
+                                TileRightT& bMatrix, TileRightScaleT& bScale)
+{
+    if (&cOutMatrix != &cInMatrix) {
+#pragma unroll
+        for (int s = 0; s < TileRes::NBLK; ++s)
+            cOutMatrix.regs[s] = cInMatrix.regs[s];
+    }
+    amd::tmatmul_mx<false>(cOutMatrix, aMatrix, aScale, bMatrix, bScale);
+    return {};
+}
+template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT, typename TileBias,
+          typename = std::enable_if_t<TileLeftScaleT::Loc == TileType::ScaleLeft && TileBias::Loc == TileType::Bias>>
+PTO_INST RecordEvent TMATMUL_MX(TileRes& cMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale, TileRightT& bMatrix,
+                                TileRightScaleT& bScale, TileBias& biasData)
+{
+    static_assert(std::is_same_v<typename TileBias::DType, float> && TileBias::Rows == 1, "TMATMUL_MX: bias is one row of float");
+    amd::tmatmul_mx<true>(cMatrix, aMatrix, aScale, bMatrix, bScale);
+    const uint8_t* pb = biasData.Storage();
+    const int vc = cMatrix.GetValidCol();
+    amd::for_each_acc(cMatrix, [&](int slot, int r, int, int col) {
+        if (col < vc)
+            cMatrix.regs[slot][r] += *reinterpret_cast<const float*>(pb + biasData.ByteOffset(0, col));
+    });
+    return {};
+}
+template <typename TileRes, typename... Rest>
+PTO_INST RecordEvent TGEMV_MX(TileRes& cMatrix, Rest&... rest)
+{
+    return TMATMUL_MX(cMatrix, rest...);
+}
+
 template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
 PTO_INST RecordEvent TGEMV(TileRes& c, TileLeftT& a, TileRightT& b, WaitEvents&...)
 {

@@ -25,20 +25,23 @@ __device__ __forceinline__ uint8_t* lds_arena()
 template <TileType L>
 struct Region {
     static constexpr bool in_lds = L != TileType::Acc && L != TileType::Ctrl;
-    static constexpr uint32_t base = L == TileType::Mat       ? 0u
-                                     : L == TileType::Left    ? PTO_AMD_L1_BYTES
-                                     : L == TileType::Right   ? PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES
-                                     : L == TileType::Vec     ? PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES
-                                     : L == TileType::Bias    ? PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES
-                                     : L == TileType::Scaling ? PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES + PTO_AMD_BIAS_BYTES
-                                                              : PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES + PTO_AMD_BIAS_BYTES + PTO_AMD_FB_BYTES;
+    static constexpr uint32_t L1 = 0, L0A = L1 + PTO_AMD_L1_BYTES, L0B = L0A + PTO_AMD_L0A_BYTES, UB = L0B + PTO_AMD_L0B_BYTES,
+                              BT = UB + PTO_AMD_UB_BYTES, FB = BT + PTO_AMD_BIAS_BYTES, L0S = FB + PTO_AMD_FB_BYTES;
+    static constexpr uint32_t base = L == TileType::Mat          ? L1
+                                     : L == TileType::Left       ? L0A
+                                     : L == TileType::Right      ? L0B
+                                     : L == TileType::Vec        ? UB
+                                     : L == TileType::Bias       ? BT
+                                     : L == TileType::Scaling    ? FB
+                                     : L == TileType::ScaleLeft  ? L0S
+                                                                 : L0S + PTO_AMD_L0S_BYTES / 2;  // ScaleRight
     static constexpr uint32_t size = L == TileType::Mat       ? PTO_AMD_L1_BYTES
                                      : L == TileType::Left    ? PTO_AMD_L0A_BYTES
                                      : L == TileType::Right   ? PTO_AMD_L0B_BYTES
                                      : L == TileType::Vec     ? PTO_AMD_UB_BYTES
                                      : L == TileType::Bias    ? PTO_AMD_BIAS_BYTES
                                      : L == TileType::Scaling ? PTO_AMD_FB_BYTES
-                                                              : PTO_AMD_L0S_BYTES;  // ScaleLeft and ScaleRight share it
+                                                              : PTO_AMD_L0S_BYTES / 2;
 };
 constexpr uint32_t LDS_TOTAL = PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES +
                                PTO_AMD_BIAS_BYTES + PTO_AMD_FB_BYTES + PTO_AMD_L0S_BYTES;
@@ -75,7 +78,8 @@ struct AccStorage {
     Vec16 regs[NBLK];
 };
 struct LdsStorage {
-    uint32_t lds_ = 0;  // byte offset of the tile in the arena
+    uint32_t lds_ = 0;   // byte offset of the tile in the arena
+    uint32_t addr_ = 0;  // the TASSIGN address (offset inside the tile's region)
 };
 
 }  // namespace amd
@@ -137,6 +141,14 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
             return (uint32_t)(row * row_bytes + kb);
         }
     }
+    // the tile's on-chip address as TASSIGN bound it (what the reference's data() pointer stands for)
+    PTO_INST uint64_t data() const
+    {
+        if constexpr (Loc_ == TileType::Acc)
+            return 0;
+        else
+            return this->addr_;
+    }
     PTO_INST uint8_t* Storage() const
     {
         static_assert(Loc_ != TileType::Acc, "accumulator tiles live in registers");
@@ -169,6 +181,10 @@ constexpr bool is_tile_data_v = is_tile<std::remove_cv_t<T>>::value;
 
 struct RecordEvent {};
 
+// address of the scale tile that belongs to a Left / Right tile at `addr` (reference: cpu/NPUMemoryModel.hpp:409-415:
+// the L0 scale buffers mirror L0A / L0B at one sixteenth of the offset)
+PTO_INST uint64_t GetScaleAddr(uint64_t addr) { return addr >> 4; }
+
 // TASSIGN: binds a tile to a byte address of its on-chip buffer (reference: cpu/TAssign.hpp:21-36,
 // common/pto_instr.hpp:104-121).  Accumulator tiles are register-resident: the address is accepted and ignored.
 template <typename T, typename AddrType>
@@ -183,6 +199,7 @@ PTO_INST void TASSIGN(T& obj, AddrType addr)
         }
         static_assert(T::Bytes <= R::size, "tile larger than its on-chip region (raise PTO_AMD_*_BYTES)");
         obj.lds_ = R::base + a;
+        obj.addr_ = a;
     }
 }
 template <std::size_t Addr, typename T>

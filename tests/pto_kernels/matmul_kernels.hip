@@ -40,7 +40,7 @@ __global__ AICORE void RunTMATMUL(__gm__ OutT* out, __gm__ AT* src0, __gm__ BT* 
     MatA aMat;
     MatB bMat;
     TASSIGN(aMat, 0x0);
-    TASSIGN(bMat, 0x10000);
+    TASSIGN(bMat, 0x8000);
     LeftT aTile;
     RightT bTile;
     AccT cTile;
@@ -91,7 +91,7 @@ __global__ AICORE void RunTMATMUL_SPLIT_K(__gm__ OutT* out, __gm__ AT* src0, __g
     MatA aMat;
     MatB bMat;
     TASSIGN(aMat, 0x0);
-    TASSIGN(bMat, 0x10000);
+    TASSIGN(bMat, 0x8000);
     TileLeft<AT, M, K> aTile;
     TileRight<BT, K, N> bTile;
     TileAcc<OutT, M, N> cTile;
@@ -110,6 +110,86 @@ __global__ AICORE void RunTMATMUL_SPLIT_K(__gm__ OutT* out, __gm__ AT* src0, __g
         else
             TMATMUL_ACC(cTile, cTile, aTile, bTile);
     }
+    TSTORE(outGlobal, cTile);
+}
+
+// Block-scaled single tile: C = sum_k A(i, k) B(k, j) 2^(sa(i, k/32) - 127) 2^(sb(k/32, j) - 127) (+ bias).  A is [M][K],
+// B is [K][N] row-major, one byte per element; the E8M0 scales sit in global memory in the layouts named by LA / LB
+// (logical [M][K/32] and [K/32][N]).  Structure after tests/cpu/st/testcase/tmatmul_mx/tmatmul_mx_kernel.cpp:66-200.
+template <typename AT, typename BT, int validM, int validK, int validN, Layout LA, Layout LB, bool isBias>
+__global__ AICORE void RunTMATMUL_MX(__gm__ float* out, __gm__ AT* src0, __gm__ BT* src1, __gm__ float8_e8m0_t* src2,
+                                     __gm__ float8_e8m0_t* src3, __gm__ float* src4)
+{
+    using ScaleType = float8_e8m0_t;
+    constexpr int M = CeilAlign<int>(validM, 16), N = CeilAlign<int>(validN, 32), K = CeilAlign<int>(validK, 64);
+    constexpr int kMX = K / 32, validKMX = validK / 32;
+    static_assert(validK % 64 == 0, "MX matmul needs K to be a multiple of 64");
+
+    using GlobalA = GlobalTensor<AT, TileShape2D<AT, validM, validK>, BaseShape2D<AT, validM, validK>>;
+    using GlobalB = GlobalTensor<BT, TileShape2D<BT, validK, validN>, BaseShape2D<BT, validK, validN>>;
+    using GlobalSA = GlobalTensor<ScaleType, TileShape2D<ScaleType, validM, validKMX, LA>, BaseShape2D<ScaleType, validM, validKMX, LA>, LA>;
+    using GlobalSB = GlobalTensor<ScaleType, TileShape2D<ScaleType, validKMX, validN, LB>, BaseShape2D<ScaleType, validKMX, validN, LB>, LB>;
+    using GlobalBias = GlobalTensor<float, TileShape2D<float, 1, validN>, BaseShape2D<float, 1, validN>>;
+    using GlobalOut = GlobalTensor<float, TileShape2D<float, validM, validN>, BaseShape2D<float, validM, validN>>;
+    GlobalA aGlobal(src0);
+    GlobalB bGlobal(src1);
+    GlobalSA saGlobal(src2);
+    GlobalSB sbGlobal(src3);
+    GlobalOut outGlobal(out);
+
+    using MatA = Tile<TileType::Mat, AT, M, K, BLayout::ColMajor, validM, validK, SLayout::RowMajor, 512>;
+    using MatB = Tile<TileType::Mat, BT, K, N, BLayout::ColMajor, validK, validN, SLayout::RowMajor, 512>;
+    using MatSA = Tile<TileType::Mat, ScaleType, M, kMX, BLayout::RowMajor, validM, validKMX, SLayout::RowMajor, 32>;
+    using MatSB = Tile<TileType::Mat, ScaleType, kMX, N, BLayout::ColMajor, validKMX, validN, SLayout::ColMajor, 32>;
+    using BiasMat = Tile<TileType::Mat, float, 1, N, BLayout::RowMajor, 1, validN>;
+    MatA aMat;
+    MatB bMat;
+    MatSA saMat;
+    MatSB sbMat;
+    BiasMat biasMat;
+    TASSIGN(aMat, 0x0);
+    TASSIGN(bMat, M * K);
+    TASSIGN(saMat, M * K + K * N);
+    TASSIGN(sbMat, M * K + K * N + M * kMX);
+    TASSIGN(biasMat, M * K + K * N + M * kMX + N * kMX);
+
+    TileLeft<AT, M, K, validM, validK> aTile;
+    TileRight<BT, K, N, validK, validN> bTile;
+    TileLeftScale<ScaleType, M, kMX, validM, validKMX> saTile;
+    TileRightScale<ScaleType, kMX, N, validKMX, validN> sbTile;
+    TileAcc<float, M, N, validM, validN> cTile;
+    Tile<TileType::Bias, float, 1, N, BLayout::RowMajor, 1, validN> biasTile;
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(cTile, 0x0);
+    TASSIGN(biasTile, 0x0);
+    TASSIGN(saTile, GetScaleAddr(aTile.data()));
+    TASSIGN(sbTile, GetScaleAddr(bTile.data()));
+
+    TLOAD(aMat, aGlobal);
+    TLOAD(bMat, bGlobal);
+    TLOAD<MatSA, GlobalSA>(saMat, saGlobal);
+    TLOAD<MatSB, GlobalSB>(sbMat, sbGlobal);
+    if constexpr (isBias) {
+        GlobalBias biasGlobal(src4);
+        TLOAD(biasMat, biasGlobal);
+    }
+    set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    TMOV(aTile, aMat);
+    TMOV(bTile, bMat);
+    TMOV(saTile, saMat);
+    TMOV(sbTile, sbMat);
+    if constexpr (isBias)
+        TMOV(biasTile, biasMat);
+    set_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
+    wait_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
+    if constexpr (isBias)
+        TMATMUL_MX(cTile, aTile, saTile, bTile, sbTile, biasTile);
+    else
+        TMATMUL_MX(cTile, aTile, saTile, bTile, sbTile);
+    set_flag(PIPE_M, PIPE_FIX, EVENT_ID0);
+    wait_flag(PIPE_M, PIPE_FIX, EVENT_ID0);
     TSTORE(outGlobal, cTile);
 }
 
@@ -187,6 +267,22 @@ extern "C" int pto_kernels_launch(int id, void* out, void* src0, void* src1, voi
     case 13: return run<&RunTMATMUL<float, half, half, float, 1, 64, 96, true>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)src2);
     case 100: return run<&RunTiledGemm<float, half, 512, 512, 512, 128, 128, 64, false>>(stream, 16, (float*)out, (half*)src0, (half*)src1);
     case 101: return run<&RunTiledGemm<bfloat16_t, bfloat16_t, 512, 512, 512, 128, 128, 64, true>>(stream, 16, (bfloat16_t*)out, (bfloat16_t*)src0, (bfloat16_t*)src1);
+    default: return -1;
+    }
+}
+
+// MX cases: 1: e4m3 x e4m3 32x128x48, scales MX_A_ZZ / MX_B_NN      2: e5m2 x e4m3 33x192x70, scales MX_A_ND / MX_B_DN, bias
+//           3: e4m3 x e5m2 16x64x32, scales MX_A_DN / MX_B_ND
+extern "C" int pto_kernels_launch_mx(int id, void* out, void* a, void* b, void* sa, void* sb, void* bias, void* stream)
+{
+    using S = float8_e8m0_t;
+    switch (id) {
+    case 1: return run<&RunTMATMUL_MX<float8_e4m3_t, float8_e4m3_t, 32, 128, 48, Layout::MX_A_ZZ, Layout::MX_B_NN, false>>(
+            stream, 1, (float*)out, (float8_e4m3_t*)a, (float8_e4m3_t*)b, (S*)sa, (S*)sb, (float*)nullptr);
+    case 2: return run<&RunTMATMUL_MX<float8_e5m2_t, float8_e4m3_t, 33, 192, 70, Layout::MX_A_ND, Layout::MX_B_DN, true>>(
+            stream, 1, (float*)out, (float8_e5m2_t*)a, (float8_e4m3_t*)b, (S*)sa, (S*)sb, (float*)bias);
+    case 3: return run<&RunTMATMUL_MX<float8_e4m3_t, float8_e5m2_t, 16, 64, 32, Layout::MX_A_DN, Layout::MX_B_ND, false>>(
+            stream, 1, (float*)out, (float8_e4m3_t*)a, (float8_e5m2_t*)b, (S*)sa, (S*)sb, (float*)nullptr);
     default: return -1;
     }
 }

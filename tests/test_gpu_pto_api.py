@@ -114,6 +114,48 @@ def test_single_tile_fp8(kernels, oracle):
     assert relerr(got, oracle.matmul_fp8(a, b)) <= 2e-2
 
 
+# MX case id -> (A type, B type, M, K, N, A-scale layout, B-scale layout, bias)
+MX_CASES = {1: (ob.E4M3, ob.E4M3, 32, 128, 48, ob.MX_A_ZZ, ob.MX_B_NN, False),
+            2: (ob.E5M2, ob.E4M3, 33, 192, 70, ob.MX_A_ND, ob.MX_B_DN, True),
+            3: (ob.E4M3, ob.E5M2, 16, 64, 32, ob.MX_A_DN, ob.MX_B_ND, False)}
+
+
+def _codes(r, typ, shape):
+    c = r.integers(0, 256, shape).astype(np.uint8)
+    if typ == ob.E4M3:
+        c[(c & 0x7F) == 0x7F] = 0x38  # NaN codes -> 1.0
+    else:
+        c[(c & 0x7F) >= 0x7C] = 0x3C  # inf / NaN codes -> 1.0
+    return c
+
+
+@pytest.mark.parametrize("case", sorted(MX_CASES))
+def test_tmatmul_mx_with_scale_tiles(kernels, oracle, case):
+    """TLOAD of the E8M0 scale matrices from their GM layouts, TMOV into the Left / Right scale tiles, TMATMUL_MX."""
+    ta, tb, m, k, n, la, lb, has_bias = MX_CASES[case]
+    r = np.random.default_rng(40 + case)
+    a, b = _codes(r, ta, (m, k)), _codes(r, tb, (k, n))
+    kg = k // 32
+    sa_log, sb_log = r.integers(120, 134, (m, kg)).astype(np.uint8), r.integers(120, 134, (kg, n)).astype(np.uint8)
+    sa, sb = np.zeros(m * kg, np.uint8), np.zeros(kg * n, np.uint8)
+    sa[oracle.mx_scale_offsets(la, m, kg)] = sa_log
+    sb[oracle.mx_scale_offsets(lb, kg, n)] = sb_log
+    bias = r.uniform(-1, 1, (1, n)).astype(np.float32) if has_bias else None
+    ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ta, tb, sa_layout=la, sb_layout=lb, b_dn=False, bias=bias)
+
+    kernels.pto_kernels_launch_mx.argtypes = [ctypes.c_int] + [ctypes.c_void_p] * 7
+    kernels.pto_kernels_launch_mx.restype = ctypes.c_int
+    d = [torch.from_numpy(x).to(DEV) for x in (a, b, sa, sb)]
+    dbias = torch.from_numpy(bias).to(DEV) if has_bias else None
+    out = torch.zeros((m, n), dtype=torch.float32, device=DEV)
+    rc = kernels.pto_kernels_launch_mx(case, out.data_ptr(), d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(),
+                                       dbias.data_ptr() if has_bias else None, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert kernels.pto_kernels_status() == 0
+    assert relerr(out.cpu().numpy(), ref) <= 2e-2
+
+
 def test_split_k_accumulates_in_the_accumulator_tile(kernels, oracle):
     """TMATMUL then four TMATMUL_ACC over five K-slabs of a 128 x 128 x 64 tile (reference case 3)."""
     r = np.random.default_rng(3)
