@@ -1,77 +1,3 @@
-// Device-side element types and conversions for the gfx950 backend.
-// Semantics follow the reference CPU simulator's types (include/pto/cpu/MXTypes.hpp:232-274 for the MX decode,
-// include/pto/cpu/TQuant.hpp:49-55 for bf16 rounding); the static_cast<half> of TSTORE is IEEE round-to-nearest-even.
+// Device-side scalar helpers shared with the PTO header layer live with it.
 #pragma once
-#include <hip/hip_runtime.h>
-#include <stdint.h>
-
-namespace ptoamd {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(4))) int i32x4;
-typedef __attribute__((ext_vector_type(8))) int i32x8;
-typedef __attribute__((ext_vector_type(16))) int i32x16;
-
-__device__ __forceinline__ uint32_t f2u(float f) { return __float_as_uint(f); }
-__device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
-
-// float -> bf16 bits, round to nearest even; NaN keeps a quiet payload
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
-{
-    const uint32_t b = f2u(f);
-    if ((b & 0x7FFFFFFFu) > 0x7F800000u)
-        return (uint16_t)((b >> 16) | 0x0040u);
-    return (uint16_t)((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
-}
-__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
-
-// float -> fp16 bits, round to nearest even (v_cvt_f16_f32 under the default rounding mode)
-__device__ __forceinline__ uint16_t f32_to_f16_bits(float f)
-{
-    const _Float16 h = (_Float16)f;
-    return __builtin_bit_cast(uint16_t, h);
-}
-__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
-
-// E8M0 -> 2^(e-127) as a double (e = 0 -> 2^-127, e = 255 -> 2^128, no NaN; MXTypes.hpp:254-259)
-__device__ __forceinline__ double e8m0_to_f64(uint32_t e)
-{
-    return __longlong_as_double((long long)((uint64_t)(e + 1023u - 127u) << 52));
-}
-// E8M0 -> float scale; 2^-127 is a float denormal, 2^128 overflows to +inf
-__device__ __forceinline__ float e8m0_to_f32(uint32_t e)
-{
-    return e == 0 ? u2f(0x00400000u) : u2f(e << 23);
-}
-
-__device__ __forceinline__ float e4m3_to_f32(uint32_t c)
-{
-    const uint32_t mag = c & 0x7Fu;
-    if (mag == 0x7Fu)
-        return u2f(0x7FC00000u | ((c & 0x80u) << 24));
-    const uint32_t e = mag >> 3, m = mag & 7u;
-    float v = e == 0 ? (float)m * 0.001953125f /* 2^-9 */ : u2f(((e + 120u) << 23) | (m << 20));
-    return (c & 0x80u) ? -v : v;
-}
-__device__ __forceinline__ float e5m2_to_f32(uint32_t c)
-{
-    // E5M2 is the upper byte of an IEEE half
-    return f16_bits_to_f32((uint16_t)(c << 8));
-}
-__device__ __forceinline__ float e2m1_to_f32(uint32_t c)
-{
-    const uint32_t mag = c & 7u;
-    const uint32_t e = mag >> 1, m = mag & 1u;
-    const float v = e == 0 ? 0.5f * (float)m : u2f(((e + 126u) << 23) | (m << 22));
-    return (c & 8u) ? -v : v;  // code 0x8 gives -0, which contributes nothing to a sum (the reference decodes +0)
-}
-__device__ __forceinline__ float e1m2_to_f32(uint32_t c)
-{
-    const float v = 0.25f * (float)(c & 7u);  // e = 0: m/4; e = 1: (1 + m/4) = (4 + m)/4
-    return (c & 8u) ? -v : v;
-}
-
-}  // namespace ptoamd
+#include "../include/pto/amd/device_types.hpp"

@@ -23,6 +23,9 @@ PTO_INST D convert(S v)
 
 // number of bytes one logical element occupies for plain (non-packed) types
 template <typename T>
+constexpr bool is_number = std::is_integral_v<T> || std::is_same_v<T, float> || std::is_same_v<T, double> ||
+                           std::is_same_v<T, _Float16> || std::is_same_v<T, __bf16>;
+template <typename T>
 constexpr bool is_packed4 = std::is_same_v<T, float4_e2m1x2_t> || std::is_same_v<T, float4_e1m2x2_t>;
 
 // ---- generic element movement between global memory and an LDS tile ------------------------------------------------
@@ -31,12 +34,17 @@ PTO_INST void tload_lds(TileData& dst, GlobalData& src)
 {
     using T = typename TileData::DType;
     static_assert(sizeof(T) == sizeof(typename GlobalData::DType), "TLOAD: tile and global element sizes differ");
-    static_assert(!is_packed4<T>, "TLOAD of packed fp4 tiles is not implemented on this backend yet");
     const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
     const auto* g = reinterpret_cast<const T*>(src.data());
     uint8_t* base = dst.Storage();
     __syncthreads();
-    if constexpr (GlobalData::layout == Layout::DN) {  // rows are the contiguous direction in memory
+    if constexpr (is_packed4<T>) {  // two codes per byte along a row: move bytes (element offsets are even)
+        static_assert(GlobalData::layout == Layout::ND, "packed fp4 tiles load from row-major global tensors");
+        for (int idx = threadIdx.x; idx < vr * (vc / 2); idx += PTO_AMD_THREADS) {
+            const int r = idx / (vc / 2), c = 2 * (idx - r * (vc / 2));
+            base[dst.ByteOffset(r, c)] = reinterpret_cast<const uint8_t*>(g)[src.Offset(r, c) / 2];
+        }
+    } else if constexpr (GlobalData::layout == Layout::DN) {  // rows are the contiguous direction in memory
         for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
             const int c = idx / vr, r = idx - c * vr;
             *reinterpret_cast<T*>(base + dst.ByteOffset(r, c)) = g[src.Offset(r, c)];
@@ -55,17 +63,29 @@ PTO_INST void tstore_lds(GlobalData& dst, TileData& src)
 {
     using T = typename TileData::DType;
     using G = typename GlobalData::DType;
-    static_assert(!is_packed4<T>, "TSTORE of packed fp4 tiles is not implemented on this backend yet");
     static_assert(atomic == AtomicType::AtomicNone, "TSTORE AtomicAdd from an LDS tile is not implemented on this backend");
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
     auto* g = reinterpret_cast<G*>(dst.data());
     const uint8_t* base = src.Storage();
-    for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
-        const int r = idx / vc, c = idx - r * vc;
-        T v = *reinterpret_cast<const T*>(base + src.ByteOffset(r, c));
-        if constexpr (relu == ReluPreMode::NormalRelu)
-            v = v > T(0) ? v : T(0);
-        g[dst.Offset(r, c)] = convert<G>(v);
+    if constexpr (is_packed4<T>) {
+        static_assert(GlobalData::layout == Layout::ND && sizeof(G) == 1, "packed fp4 tiles store to row-major global tensors");
+        for (int idx = threadIdx.x; idx < vr * (vc / 2); idx += PTO_AMD_THREADS) {
+            const int r = idx / (vc / 2), c = 2 * (idx - r * (vc / 2));
+            reinterpret_cast<uint8_t*>(g)[dst.Offset(r, c) / 2] = base[src.ByteOffset(r, c)];
+        }
+    } else {
+        for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
+            const int r = idx / vc, c = idx - r * vc;
+            T v = *reinterpret_cast<const T*>(base + src.ByteOffset(r, c));
+            if constexpr (is_number<T>) {
+                if constexpr (relu == ReluPreMode::NormalRelu)
+                    v = v > T(0) ? v : T(0);
+                g[dst.Offset(r, c)] = convert<G>(v);
+            } else {  // one-byte code types move as bytes
+                static_assert(sizeof(G) == sizeof(T), "TSTORE: code tiles store to a global tensor of the same element size");
+                reinterpret_cast<T*>(g)[dst.Offset(r, c)] = v;
+            }
+        }
     }
 }
 

@@ -1,0 +1,140 @@
+// TQUANT and TDEQUANT on LDS-resident tiles.  Reference semantics: cpu/TQuant.hpp:78-96,461-547 (INT8 forms, MX forms
+// with 32-element groups along a row), cpu/TDeQuant.hpp:18-37; wrapper signatures common/pto_instr.hpp:2978-3072.
+// The scalar arithmetic is quant_math.hpp's, shared with the streaming kernels behind the C ABI, so codes, exponents,
+// group maxima and scalings are bit-identical to the simulator's.
+#pragma once
+#include "quant_math.hpp"
+#include "tile.hpp"
+
+namespace pto {
+
+enum class QuantType { MXFP8 = 0, MXFP4_E2M1 = 1, INT8_SYM = 2, INT8_ASYM = 3 };
+enum class QuantScaleAlg { OCP = 0, NV = 1 };
+enum class MxQuantAlg { OcpMxFp8E4M3 = 0, NvMxFp8E4M3 = 1, OcpMxFp4E2M1 = 2, NvMxFp4E2M1 = 3 };
+enum class VecStoreMode { ND = 0, NZ = 1 };
+
+namespace amd {
+
+template <typename T>
+PTO_INST float to_float(T v)
+{
+    return static_cast<float>(v);
+}
+// parameter tiles are read with the row / column clamped to their valid extent (reference: cpu/TQuant.hpp:78-84)
+template <typename TilePara>
+PTO_INST float para(const TilePara& t, int r, int c)
+{
+    const int rr = min(r, max(t.GetValidRow(), 1) - 1), cc = min(c, max(t.GetValidCol(), 1) - 1);
+    return to_float(*reinterpret_cast<const typename TilePara::DType*>(t.Storage() + t.ByteOffset(rr, cc)));
+}
+
+template <bool ASYM, typename TileOut, typename TileSrc, typename TilePara>
+PTO_INST void tquant_int8(TileOut& dst, TileSrc& src, TilePara& scale, TilePara* offset)
+{
+    static_assert(std::is_same_v<typename TileSrc::DType, float>, "TQUANT INT8 takes a float source tile");
+    static_assert(sizeof(typename TileOut::DType) == 1, "TQUANT INT8 writes one byte per element");
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
+        const int r = idx / vc, c = idx - r * vc;
+        float v = __fmul_rn(*reinterpret_cast<const float*>(src.Storage() + src.ByteOffset(r, c)), para(scale, r, c));
+        if constexpr (ASYM)
+            v = __fadd_rn(v, para(*offset, r, c));
+        v = rintf(v);
+        const float lo = ASYM ? 0.0f : -128.0f, hi = ASYM ? 255.0f : 127.0f;
+        v = v < lo ? lo : (v > hi ? hi : v);
+        *reinterpret_cast<uint8_t*>(dst.Storage() + dst.ByteOffset(r, c)) = (uint8_t)(int)v;
+    }
+    __syncthreads();
+}
+
+// one thread per 32-element group along a row
+template <int ALG, typename TileOut, typename TileSrc, typename TileExp, typename TileMax, typename TileScaling>
+PTO_INST void tquant_mx(TileOut& dst, TileSrc& src, TileExp* exp, TileMax* mx, TileScaling* scaling)
+{
+    using S = typename TileSrc::DType;
+    constexpr bool SRC_BF16 = std::is_same_v<S, __bf16>;
+    constexpr bool FP4 = ALG == ptoamd::MX_OCP_FP4 || ALG == ptoamd::MX_NV_FP4;
+    static_assert(std::is_same_v<S, float> || std::is_same_v<S, _Float16> || SRC_BF16, "TQUANT MX: source is float, half or bf16");
+    const int vr = src.GetValidRow(), vc = src.GetValidCol(), groups_per_row = vc / 32;
+    __syncthreads();
+    for (int g = threadIdx.x; g < vr * groups_per_row; g += PTO_AMD_THREADS) {
+        const int r = g / groups_per_row, c0 = (g - r * groups_per_row) * 32;
+        uint32_t run = 0;
+        float first_nan = 0.0f;
+        bool seen_nan = false;
+        for (int i = 0; i < 32; ++i) {
+            const float v = to_float(*reinterpret_cast<const S*>(src.Storage() + src.ByteOffset(r, c0 + i)));
+            if (!seen_nan && v != v) {
+                first_nan = v;
+                seen_nan = true;
+            }
+            run = ptoamd::max_step<ALG>(run, v);
+        }
+        const float maxabs = ptoamd::max_value<ALG>(run, first_nan);
+        const uint32_t e = ptoamd::shared_exponent<ALG>(maxabs);
+        const float sc = ptoamd::group_scaling<ALG>(maxabs, e);
+        if (exp)
+            *reinterpret_cast<uint8_t*>(exp->Storage() + g) = (uint8_t)e;
+        if (mx)
+            reinterpret_cast<float*>(mx->Storage())[g] = maxabs;
+        if (scaling)
+            reinterpret_cast<float*>(scaling->Storage())[g] = sc;
+        for (int i = 0; i < 32; i += 2) {
+            const float v0 = to_float(*reinterpret_cast<const S*>(src.Storage() + src.ByteOffset(r, c0 + i)));
+            const float v1 = to_float(*reinterpret_cast<const S*>(src.Storage() + src.ByteOffset(r, c0 + i + 1)));
+            const uint32_t q0 = ptoamd::encode_mx<ALG, SRC_BF16>(v0, sc), q1 = ptoamd::encode_mx<ALG, SRC_BF16>(v1, sc);
+            if constexpr (FP4) {
+                *reinterpret_cast<uint8_t*>(dst.Storage() + dst.ByteOffset(r, c0 + i)) = (uint8_t)(q0 | (q1 << 4));
+            } else {
+                *reinterpret_cast<uint8_t*>(dst.Storage() + dst.ByteOffset(r, c0 + i)) = (uint8_t)q0;
+                *reinterpret_cast<uint8_t*>(dst.Storage() + dst.ByteOffset(r, c0 + i + 1)) = (uint8_t)q1;
+            }
+        }
+    }
+    __syncthreads();
+}
+
+}  // namespace amd
+
+// INT8: dst = clamp(nearbyint(src * scale[row] (+ offset[row]))); the "scale" operand multiplies
+template <auto quant_type, typename TileDataOut, typename TileDataSrc, typename TileDataPara,
+          typename = std::enable_if_t<quant_type == QuantType::INT8_SYM || quant_type == QuantType::INT8_ASYM>>
+PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataPara& scale, TileDataPara* offset = nullptr)
+{
+    amd::tquant_int8<quant_type == QuantType::INT8_ASYM>(dst, src, scale, offset);
+    return {};
+}
+
+// MX: dst codes (E4M3 bytes or packed E2M1 pairs), exp [rows][cols / 32] E8M0, max and scaling per group (flat)
+template <auto quant_type, typename TileDataOut, typename TileDataSrc, typename TileDataExp, typename TileDataMax,
+          typename TileDataScaling, auto scale_alg = QuantScaleAlg::OCP,
+          typename = std::enable_if_t<quant_type == QuantType::MXFP8 || quant_type == QuantType::MXFP4_E2M1>>
+PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataExp* exp, TileDataMax* max, TileDataScaling* scaling)
+{
+    constexpr int alg = (quant_type == QuantType::MXFP8 ? 0 : 2) + (scale_alg == QuantScaleAlg::NV ? 1 : 0);
+    amd::tquant_mx<alg>(dst, src, exp, max, scaling);
+    return {};
+}
+
+// dst(r, c) = (D(src(r, c)) - D(offset(r, pc))) * D(scale(r, pc)), pc = min(c, max(1, scale.validCol) - 1)
+template <typename TileDataDst, typename TileDataSrc, typename TileDataPara, typename... WaitEvents>
+PTO_INST RecordEvent TDEQUANT(TileDataDst& dst, TileDataSrc& src, TileDataPara& scale, TileDataPara& offset, WaitEvents&...)
+{
+    using D = typename TileDataDst::DType;
+    static_assert(std::is_same_v<D, float>, "TDEQUANT writes a float tile on this backend");
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
+        const int r = idx / vc, c = idx - r * vc;
+        const int pc = min(c, max(1, scale.GetValidCol()) - 1);
+        const float s = amd::to_float(*reinterpret_cast<const typename TileDataPara::DType*>(scale.Storage() + scale.ByteOffset(r, pc)));
+        const float o = amd::to_float(*reinterpret_cast<const typename TileDataPara::DType*>(offset.Storage() + offset.ByteOffset(r, pc)));
+        const float v = amd::to_float(*reinterpret_cast<const typename TileDataSrc::DType*>(src.Storage() + src.ByteOffset(r, c)));
+        *reinterpret_cast<float*>(dst.Storage() + dst.ByteOffset(r, c)) = __fmul_rn(__fsub_rn(v, o), s);
+    }
+    __syncthreads();
+    return {};
+}
+
+}  // namespace pto

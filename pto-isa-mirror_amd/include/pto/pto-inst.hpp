@@ -15,4 +15,5 @@
 #include "amd/base.hpp"
 #include "amd/tile.hpp"
 #include "amd/instr.hpp"
+#include "amd/quant.hpp"
 #include "amd/launch.hpp"

@@ -287,4 +287,107 @@ extern "C" int pto_kernels_launch_mx(int id, void* out, void* a, void* b, void* 
     }
 }
 
+// ---- TQUANT / TDEQUANT on Vec tiles ----------------------------------------------------------------------------------
+template <typename SrcT, typename DstT, int R, int C, QuantType QT, QuantScaleAlg ALG>
+__global__ AICORE void RunTQUANT_MX(__gm__ DstT* dst, __gm__ uint8_t* exp, __gm__ float* max, __gm__ float* scaling, __gm__ SrcT* src)
+{
+    constexpr int G = R * C / 32;
+    using SrcTile = Tile<TileType::Vec, SrcT, R, C, BLayout::RowMajor, R, C>;
+    using DstTile = Tile<TileType::Vec, DstT, R, C, BLayout::RowMajor, R, C>;
+    using ExpTile = Tile<TileType::Vec, uint8_t, 1, G, BLayout::RowMajor, 1, G>;
+    using FlatTile = Tile<TileType::Vec, float, 1, G, BLayout::RowMajor, 1, G>;
+    SrcTile srcTile;
+    DstTile dstTile;
+    ExpTile expTile;
+    FlatTile maxTile, scalingTile;
+    constexpr int a1 = CeilAlign<int>(SrcTile::Bytes, 32), a2 = a1 + CeilAlign<int>(DstTile::Bytes, 32),
+                  a3 = a2 + CeilAlign<int>(ExpTile::Bytes, 32), a4 = a3 + CeilAlign<int>(FlatTile::Bytes, 32);
+    TASSIGN(srcTile, 0x0);
+    TASSIGN(dstTile, a1);
+    TASSIGN(expTile, a2);
+    TASSIGN(maxTile, a3);
+    TASSIGN(scalingTile, a4);
+    GlobalTensor<SrcT, TileShape2D<SrcT, R, C>, BaseShape2D<SrcT, R, C>> srcGlobal(src);
+    GlobalTensor<DstT, TileShape2D<DstT, R, C>, BaseShape2D<DstT, R, C>> dstGlobal(dst);
+    GlobalTensor<uint8_t, TileShape2D<uint8_t, 1, G>, BaseShape2D<uint8_t, 1, G>> expGlobal(exp);
+    GlobalTensor<float, TileShape2D<float, 1, G>, BaseShape2D<float, 1, G>> maxGlobal(max), scalingGlobal(scaling);
+    TLOAD(srcTile, srcGlobal);
+    TQUANT<QT, DstTile, SrcTile, ExpTile, FlatTile, FlatTile, ALG>(dstTile, srcTile, &expTile, &maxTile, &scalingTile);
+    TSTORE(dstGlobal, dstTile);
+    TSTORE(expGlobal, expTile);
+    TSTORE(maxGlobal, maxTile);
+    TSTORE(scalingGlobal, scalingTile);
+}
+
+template <int R, int C, bool ASYM>
+__global__ AICORE void RunTQUANT_INT8(__gm__ uint8_t* dst, __gm__ float* src, __gm__ float* scale, __gm__ float* offset)
+{
+    using SrcTile = Tile<TileType::Vec, float, R, C, BLayout::RowMajor, R, C>;
+    using DstTile = Tile<TileType::Vec, uint8_t, R, C, BLayout::RowMajor, R, C>;
+    using ParaTile = Tile<TileType::Vec, float, R, 8, BLayout::RowMajor, R, 1>;  // one value per row
+    SrcTile srcTile;
+    DstTile dstTile;
+    ParaTile scaleTile, offsetTile;
+    TASSIGN(srcTile, 0x0);
+    TASSIGN(dstTile, SrcTile::Bytes);
+    TASSIGN(scaleTile, SrcTile::Bytes + DstTile::Bytes);
+    TASSIGN(offsetTile, SrcTile::Bytes + DstTile::Bytes + ParaTile::Bytes);
+    GlobalTensor<float, TileShape2D<float, R, C>, BaseShape2D<float, R, C>> srcGlobal(src);
+    GlobalTensor<uint8_t, TileShape2D<uint8_t, R, C>, BaseShape2D<uint8_t, R, C>> dstGlobal(dst);
+    GlobalTensor<float, TileShape2D<float, R, 1>, BaseShape2D<float, R, 1>> scaleGlobal(scale), offsetGlobal(offset);
+    TLOAD(srcTile, srcGlobal);
+    TLOAD(scaleTile, scaleGlobal);
+    if constexpr (ASYM) {
+        TLOAD(offsetTile, offsetGlobal);
+        TQUANT<QuantType::INT8_ASYM>(dstTile, srcTile, scaleTile, &offsetTile);
+    } else {
+        TQUANT<QuantType::INT8_SYM>(dstTile, srcTile, scaleTile);
+    }
+    TSTORE(dstGlobal, dstTile);
+}
+
+template <typename SrcT, int R, int C>
+__global__ AICORE void RunTDEQUANT(__gm__ float* dst, __gm__ SrcT* src, __gm__ float* scale, __gm__ float* offset)
+{
+    using SrcTile = Tile<TileType::Vec, SrcT, R, C, BLayout::RowMajor, R, C>;
+    using DstTile = Tile<TileType::Vec, float, R, C, BLayout::RowMajor, R, C>;
+    using ParaTile = Tile<TileType::Vec, float, R, 8, BLayout::RowMajor, R, 1>;
+    SrcTile srcTile;
+    DstTile dstTile;
+    ParaTile scaleTile, offsetTile;
+    TASSIGN(dstTile, 0x0);
+    TASSIGN(srcTile, DstTile::Bytes);
+    TASSIGN(scaleTile, DstTile::Bytes + CeilAlign<int>(SrcTile::Bytes, 32));
+    TASSIGN(offsetTile, DstTile::Bytes + CeilAlign<int>(SrcTile::Bytes, 32) + ParaTile::Bytes);
+    GlobalTensor<SrcT, TileShape2D<SrcT, R, C>, BaseShape2D<SrcT, R, C>> srcGlobal(src);
+    GlobalTensor<float, TileShape2D<float, R, C>, BaseShape2D<float, R, C>> dstGlobal(dst);
+    GlobalTensor<float, TileShape2D<float, R, 1>, BaseShape2D<float, R, 1>> scaleGlobal(scale), offsetGlobal(offset);
+    TLOAD(srcTile, srcGlobal);
+    TLOAD(scaleTile, scaleGlobal);
+    TLOAD(offsetTile, offsetGlobal);
+    TDEQUANT(dstTile, srcTile, scaleTile, offsetTile);
+    TSTORE(dstGlobal, dstTile);
+}
+
+// quant cases: 1-4: f32 16x64 -> OCP-FP8, NV-FP8, OCP-FP4, NV-FP4     5: bf16 8x128 -> OCP-FP4     6: half 8x128 -> OCP-FP8
+//              10: INT8 sym 16x64   11: INT8 asym 16x64    20: TDEQUANT int8 16x64    21: TDEQUANT int32 8x32
+extern "C" int pto_kernels_launch_quant(int id, void* dst, void* exp, void* max, void* scaling, void* src, void* scale, void* offset, void* stream)
+{
+    using F8 = float8_e4m3_t;
+    using F4 = float4_e2m1x2_t;
+    switch (id) {
+    case 1: return run<&RunTQUANT_MX<float, F8, 16, 64, QuantType::MXFP8, QuantScaleAlg::OCP>>(stream, 1, (F8*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (float*)src);
+    case 2: return run<&RunTQUANT_MX<float, F8, 16, 64, QuantType::MXFP8, QuantScaleAlg::NV>>(stream, 1, (F8*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (float*)src);
+    case 3: return run<&RunTQUANT_MX<float, F4, 16, 64, QuantType::MXFP4_E2M1, QuantScaleAlg::OCP>>(stream, 1, (F4*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (float*)src);
+    case 4: return run<&RunTQUANT_MX<float, F4, 16, 64, QuantType::MXFP4_E2M1, QuantScaleAlg::NV>>(stream, 1, (F4*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (float*)src);
+    case 5: return run<&RunTQUANT_MX<bfloat16_t, F4, 8, 128, QuantType::MXFP4_E2M1, QuantScaleAlg::OCP>>(stream, 1, (F4*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (bfloat16_t*)src);
+    case 6: return run<&RunTQUANT_MX<half, F8, 8, 128, QuantType::MXFP8, QuantScaleAlg::OCP>>(stream, 1, (F8*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (half*)src);
+    case 10: return run<&RunTQUANT_INT8<16, 64, false>>(stream, 1, (uint8_t*)dst, (float*)src, (float*)scale, (float*)offset);
+    case 11: return run<&RunTQUANT_INT8<16, 64, true>>(stream, 1, (uint8_t*)dst, (float*)src, (float*)scale, (float*)offset);
+    case 20: return run<&RunTDEQUANT<int8_t, 16, 64>>(stream, 1, (float*)dst, (int8_t*)src, (float*)scale, (float*)offset);
+    case 21: return run<&RunTDEQUANT<int32_t, 8, 32>>(stream, 1, (float*)dst, (int32_t*)src, (float*)scale, (float*)offset);
+    default: return -1;
+    }
+}
+
 extern "C" int pto_kernels_status() { return pto::amd::device_status(); }

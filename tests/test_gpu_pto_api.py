@@ -199,3 +199,65 @@ def test_host_demo_program():
     res = subprocess.run([DEMO], capture_output=True, text=True, timeout=120)
     assert res.returncode == 0, res.stdout + res.stderr
     assert "max_abs_diff=" in res.stdout and "status=0" in res.stdout
+
+
+# ------------------------------------------------------------------------------------------- TQUANT / TDEQUANT tiles
+def _eq_f32(a, b):
+    return np.array_equal(a.view(np.uint32) & 0xFFBFFFFF, b.view(np.uint32) & 0xFFBFFFFF)  # NaN quiet bit aside
+
+
+def _quant_launch(lib, case, dst, exp, mx, sc, src, scale=None, offset=None):
+    lib.pto_kernels_launch_quant.argtypes = [ctypes.c_int] + [ctypes.c_void_p] * 8
+    lib.pto_kernels_launch_quant.restype = ctypes.c_int
+    p = lambda t: t.data_ptr() if t is not None else None
+    rc = lib.pto_kernels_launch_quant(case, p(dst), p(exp), p(mx), p(sc), p(src), p(scale), p(offset),
+                                      torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert lib.pto_kernels_status() == 0
+
+
+# case -> (rows, cols, algorithm id, source dtype, oracle source kind)
+QUANT_MX = {1: (16, 64, ob.OCP_FP8, torch.float32, ob.SRC_F32), 2: (16, 64, ob.NV_FP8, torch.float32, ob.SRC_F32),
+            3: (16, 64, ob.OCP_FP4, torch.float32, ob.SRC_F32), 4: (16, 64, ob.NV_FP4, torch.float32, ob.SRC_F32),
+            5: (8, 128, ob.OCP_FP4, torch.bfloat16, ob.SRC_BF16), 6: (8, 128, ob.OCP_FP8, torch.float16, ob.SRC_F16)}
+
+
+@pytest.mark.parametrize("case", sorted(QUANT_MX))
+def test_tquant_mx_tile_instruction_bit_exact(kernels, oracle, case):
+    rows, cols, alg, dtype, kind = QUANT_MX[case]
+    r = np.random.default_rng(case)
+    x = (r.standard_normal((rows, cols)) * 10 ** r.uniform(-3, 3, (rows, 1))).astype(np.float32)
+    x[0, :32] = 0                      # an all-zero group
+    x[1, 3] = np.inf                   # the reference tests' edge inputs: infinity, NaN, the E4M3 boundary
+    x[2, 40] = np.nan
+    x[3, 0], x[3, 1] = 448.0, np.nextafter(np.float32(448.0), np.float32(np.inf))
+    src = torch.from_numpy(x).to(dtype)
+    fp4 = alg in (ob.OCP_FP4, ob.NV_FP4)
+    g = rows * cols // 32
+    dst = torch.zeros(rows * cols // (2 if fp4 else 1), dtype=torch.uint8, device=DEV)
+    exp = torch.zeros(g, dtype=torch.uint8, device=DEV)
+    mx, sc = torch.zeros(g, dtype=torch.float32, device=DEV), torch.zeros(g, dtype=torch.float32, device=DEV)
+    _quant_launch(kernels, case, dst, exp, mx, sc, src.to(DEV))
+    rc, re, rm, rs = oracle.tquant_mx(src.float().numpy(), alg, 1, kind)
+    assert np.array_equal(exp.cpu().numpy(), re.ravel())
+    assert np.array_equal(dst.cpu().numpy(), rc.ravel())
+    assert _eq_f32(mx.cpu().numpy(), rm.ravel()) and _eq_f32(sc.cpu().numpy(), rs.ravel())
+
+
+def test_tquant_int8_and_tdequant_tile_instructions_bit_exact(kernels, oracle):
+    r = np.random.default_rng(21)
+    src = (r.standard_normal((16, 64)) * 60).astype(np.float32)
+    scale, off = r.uniform(0.2, 3, 16).astype(np.float32), r.uniform(0, 200, 16).astype(np.float32)
+    d = lambda a: torch.from_numpy(a).to(DEV)
+    for case, offset in ((10, None), (11, off)):
+        dst = torch.zeros((16, 64), dtype=torch.uint8, device=DEV)
+        _quant_launch(kernels, case, dst, None, None, None, d(src), d(scale), d(off))
+        ref = oracle.tquant_int8(src, scale, offset)
+        assert np.array_equal(dst.cpu().numpy(), ref.view(np.uint8))
+    for case, shape, dt in ((20, (16, 64), np.int8), (21, (8, 32), np.int32)):
+        q = r.integers(-120, 120, shape).astype(dt) if dt == np.int8 else r.integers(-10 ** 6, 10 ** 6, shape).astype(dt)
+        s, o = r.uniform(0.01, 2, shape[0]).astype(np.float32), r.uniform(-5, 5, shape[0]).astype(np.float32)
+        out = torch.zeros(shape, dtype=torch.float32, device=DEV)
+        _quant_launch(kernels, case, out, None, None, None, d(q), d(s), d(o))
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), oracle.tdequant(q, s, o).view(np.uint32))
