@@ -6,6 +6,7 @@
 // Ordering: every instruction that writes LDS ends with a workgroup barrier, and starts with one (earlier readers of
 // the bytes it overwrites are done); instructions that only read LDS need no barrier of their own.
 #pragma once
+#include "device_types.hpp"
 #include "tile.hpp"
 
 namespace pto {
@@ -322,6 +323,62 @@ PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
     });
 }
 
+// Fix-pipe quantisation of one accumulator element (reference: cpu/common.hpp:117-185).  Scalar words carry an fp32
+// scale in the low 32 bits; vector (per-column) words a 19-bit (1, 8, 10) float at bits 13..31.  Bits 37..45 hold the
+// offset and bit 46 the signedness of 8-bit targets.
+template <bool VECTOR>
+PTO_INST float quant_word_scale(uint64_t word)
+{
+    if constexpr (!VECTOR) {
+        return ptoamd::u2f((uint32_t)(word & 0xFFFFFFFFu));
+    } else {
+        const uint32_t m1 = (uint32_t)((word >> 13) & 0x7FFFFu);
+        const uint32_t s = (m1 >> 18) & 1u, e = (m1 >> 10) & 0xFFu, mant = m1 & 0x3FFu;
+        if (e == 0 && mant == 0)
+            return 0.0f;
+        const float mv = 1.0f + (float)mant / 1024.0f;
+        return __fmul_rn(__fmul_rn(s ? -1.0f : 1.0f, mv), ptoamd::e8m0_to_f32(e));
+    }
+}
+template <bool VECTOR, typename G, typename Reg>
+PTO_INST float quantize_element(Reg acc, uint64_t word)
+{
+    constexpr bool src_is_int = std::is_integral_v<Reg>;
+    static_assert(std::is_same_v<G, int8_t> || std::is_same_v<G, uint8_t> || std::is_same_v<G, _Float16> || std::is_same_v<G, __bf16>,
+                  "TSTORE with quantisation targets int8, uint8, half or bfloat16");
+    float r = __fmul_rn((float)acc, quant_word_scale<VECTOR>(word));
+    if constexpr (sizeof(G) == 1) {
+        const float offset = (float)(uint32_t)((word >> 37) & 0x1FFu);
+        const bool sign = (word >> 46) & 1u;
+        const float rounded = rintf(__fadd_rn(r, offset));
+        const float lo = sign ? -128.0f : 0.0f, hi = sign ? 127.0f : 255.0f;
+        r = rounded < lo ? lo : (rounded > hi ? hi : rounded);
+    } else if constexpr (std::is_same_v<G, _Float16>) {
+        if (src_is_int || (r == r && fabsf(r) != __builtin_inff()))
+            r = r < -65504.0f ? -65504.0f : (r > 65504.0f ? 65504.0f : r);
+    } else {
+        if (r == r && fabsf(r) != __builtin_inff())
+            r = r < -3.402823466e38f ? -3.402823466e38f : (r > 3.402823466e38f ? 3.402823466e38f : r);
+    }
+    return r;
+}
+
+template <bool VECTOR, typename TileRes, typename GlobalData, ReluPreMode relu, typename WordOf>
+PTO_INST void tstore_acc_quant(GlobalData& dst, TileRes& src, WordOf&& word_of)
+{
+    using G = typename GlobalData::DType;
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    auto* g = reinterpret_cast<G*>(dst.data());
+    for_each_acc(src, [&](int slot, int r, int row, int col) {
+        if (row < vr && col < vc) {
+            float v = quantize_element<VECTOR, G>(src.regs[slot][r], word_of(col));
+            if constexpr (relu == ReluPreMode::NormalRelu)
+                v = v > 0 ? v : 0;
+            g[dst.Offset(row, col)] = static_cast<G>(v);
+        }
+    });
+}
+
 }  // namespace amd
 
 // ---- TLOAD ---------------------------------------------------------------------------------------------------------
@@ -342,6 +399,29 @@ PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, WaitEvents&...)
         amd::tstore_acc<TileData, GlobalData, atomicType, reluPreMode>(dst, src);
     else
         amd::tstore_lds<TileData, GlobalData, atomicType, reluPreMode>(dst, src);
+    return {};
+}
+
+// TSTORE with fix-pipe quantisation: one scalar word for the whole tile, or one word per column from a Scaling tile
+// (reference: common/pto_instr.hpp:439-490, cpu/TStore.hpp:118-181)
+template <typename TileData, typename GlobalData, AtomicType atomicType = AtomicType::AtomicNone,
+          ReluPreMode reluPreMode = ReluPreMode::NoRelu>
+PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, uint64_t preQuantScalar)
+{
+    static_assert(TileData::Loc == TileType::Acc && atomicType == AtomicType::AtomicNone, "quantising TSTORE drains an accumulator tile");
+    amd::tstore_acc_quant<false, TileData, GlobalData, reluPreMode>(dst, src, [&](int) { return preQuantScalar; });
+    return {};
+}
+template <typename TileData, typename GlobalData, typename FpTileData, AtomicType atomicType = AtomicType::AtomicNone,
+          ReluPreMode reluPreMode = ReluPreMode::NoRelu,
+          typename = std::enable_if_t<is_tile_data_v<FpTileData> && FpTileData::Loc == TileType::Scaling>>
+PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, FpTileData& fp)
+{
+    static_assert(TileData::Loc == TileType::Acc && atomicType == AtomicType::AtomicNone, "quantising TSTORE drains an accumulator tile");
+    static_assert(sizeof(typename FpTileData::DType) == 8, "the Scaling tile holds one 64-bit quantisation word per column");
+    const uint8_t* words = fp.Storage();
+    amd::tstore_acc_quant<true, TileData, GlobalData, reluPreMode>(
+        dst, src, [&](int col) { return *reinterpret_cast<const uint64_t*>(words + fp.ByteOffset(0, col)); });
     return {};
 }
 

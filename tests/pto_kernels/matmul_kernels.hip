@@ -287,6 +287,42 @@ extern "C" int pto_kernels_launch_mx(int id, void* out, void* a, void* b, void* 
     }
 }
 
+// matmul, then TSTORE through the fix-pipe quantiser: a scalar word, or one word per column from a Scaling tile
+template <typename OutT, typename AccT, typename InT, int validM, int validK, int validN, bool VECTOR, bool RELU>
+__global__ AICORE void RunTMATMUL_QUANT(__gm__ OutT* out, __gm__ InT* src0, __gm__ InT* src1, __gm__ uint64_t* words)
+{
+    constexpr int blockAlign = (sizeof(InT) == 1) ? 32 : 16;
+    constexpr int M = CeilAlign<int>(validM, 16), N = CeilAlign<int>(validN, blockAlign), K = CeilAlign<int>(validK, blockAlign);
+    GlobalTensor<InT, TileShape2D<InT, validM, validK>, BaseShape2D<InT, validM, validK>> aGlobal(src0);
+    GlobalTensor<InT, TileShape2D<InT, validK, validN>, BaseShape2D<InT, validK, validN>> bGlobal(src1);
+    GlobalTensor<OutT, TileShape2D<OutT, validM, validN>, BaseShape2D<OutT, validM, validN>> outGlobal(out);
+    GlobalTensor<uint64_t, TileShape2D<uint64_t, 1, validN>, BaseShape2D<uint64_t, 1, validN>> wordsGlobal(words);
+    Tile<TileType::Mat, InT, M, K, BLayout::ColMajor, validM, validK, SLayout::RowMajor, 512> aMat;
+    Tile<TileType::Mat, InT, K, N, BLayout::ColMajor, validK, validN, SLayout::RowMajor, 512> bMat;
+    TileLeft<InT, M, K, validM, validK> aTile;
+    TileRight<InT, K, N, validK, validN> bTile;
+    TileAcc<AccT, M, N, validM, validN> cTile;
+    Tile<TileType::Scaling, uint64_t, 1, N, BLayout::RowMajor, 1, validN> fpTile;
+    TASSIGN(aMat, 0x0);
+    TASSIGN(bMat, 0x8000);
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(cTile, 0x0);
+    TASSIGN(fpTile, 0x0);
+    TLOAD(aMat, aGlobal);
+    TLOAD(bMat, bGlobal);
+    TMOV(aTile, aMat);
+    TMOV(bTile, bMat);
+    TMATMUL(cTile, aTile, bTile);
+    constexpr ReluPreMode relu = RELU ? ReluPreMode::NormalRelu : ReluPreMode::NoRelu;
+    if constexpr (VECTOR) {
+        TLOAD(fpTile, wordsGlobal);
+        TSTORE<decltype(cTile), decltype(outGlobal), decltype(fpTile), AtomicType::AtomicNone, relu>(outGlobal, cTile, fpTile);
+    } else {
+        TSTORE<decltype(cTile), decltype(outGlobal), AtomicType::AtomicNone, relu>(outGlobal, cTile, words[0]);
+    }
+}
+
 // ---- TQUANT / TDEQUANT on Vec tiles ----------------------------------------------------------------------------------
 template <typename SrcT, typename DstT, int R, int C, QuantType QT, QuantScaleAlg ALG>
 __global__ AICORE void RunTQUANT_MX(__gm__ DstT* dst, __gm__ uint8_t* exp, __gm__ float* max, __gm__ float* scaling, __gm__ SrcT* src)
@@ -386,6 +422,19 @@ extern "C" int pto_kernels_launch_quant(int id, void* dst, void* exp, void* max,
     case 11: return run<&RunTQUANT_INT8<16, 64, true>>(stream, 1, (uint8_t*)dst, (float*)src, (float*)scale, (float*)offset);
     case 20: return run<&RunTDEQUANT<int8_t, 16, 64>>(stream, 1, (float*)dst, (int8_t*)src, (float*)scale, (float*)offset);
     case 21: return run<&RunTDEQUANT<int32_t, 8, 32>>(stream, 1, (float*)dst, (int32_t*)src, (float*)scale, (float*)offset);
+    default: return -1;
+    }
+}
+
+// store-quant cases: 1: f16 -> f32 acc -> int8, scalar word     2: f16 -> f32 acc -> uint8, per-column words, relu
+//                    3: int8 -> i32 acc -> f16 (dequant), per-column words     4: int8 -> i32 acc -> int8 (requant), scalar
+extern "C" int pto_kernels_launch_store_quant(int id, void* out, void* a, void* b, void* words, void* stream)
+{
+    switch (id) {
+    case 1: return run<&RunTMATMUL_QUANT<int8_t, float, half, 40, 50, 60, false, false>>(stream, 1, (int8_t*)out, (half*)a, (half*)b, (uint64_t*)words);
+    case 2: return run<&RunTMATMUL_QUANT<uint8_t, float, half, 33, 64, 70, true, true>>(stream, 1, (uint8_t*)out, (half*)a, (half*)b, (uint64_t*)words);
+    case 3: return run<&RunTMATMUL_QUANT<half, int32_t, int8_t, 24, 96, 40, true, false>>(stream, 1, (half*)out, (int8_t*)a, (int8_t*)b, (uint64_t*)words);
+    case 4: return run<&RunTMATMUL_QUANT<int8_t, int32_t, int8_t, 24, 96, 40, false, false>>(stream, 1, (int8_t*)out, (int8_t*)a, (int8_t*)b, (uint64_t*)words);
     default: return -1;
     }
 }

@@ -261,3 +261,52 @@ def test_tquant_int8_and_tdequant_tile_instructions_bit_exact(kernels, oracle):
         out = torch.zeros(shape, dtype=torch.float32, device=DEV)
         _quant_launch(kernels, case, out, None, None, None, d(q), d(s), d(o))
         assert np.array_equal(out.cpu().numpy().view(np.uint32), oracle.tdequant(q, s, o).view(np.uint32))
+
+
+# ------------------------------------------------------------------------------------------- TSTORE with quantisation
+def _word(scale, offset=0, signed=True, vector=False):
+    bits = int(np.float32(scale).view(np.uint32))
+    if vector:
+        bits &= 0xFFFFE000  # 19-bit (1, 8, 10) float at bits 13..31
+    return np.uint64(bits | (offset << 37) | (int(signed) << 46))
+
+
+# case -> (input kind, M, K, N, per-column words, relu, oracle destination kind, numpy output dtype, signed 8-bit target)
+STORE_QUANT = {1: ("f16", 40, 50, 60, False, False, ob.ST_I8, np.int8, True),
+               2: ("f16", 33, 64, 70, True, True, ob.ST_U8, np.uint8, False),
+               3: ("i8", 24, 96, 40, True, False, ob.ST_F16, np.uint16, True),
+               4: ("i8", 24, 96, 40, False, False, ob.ST_I8, np.int8, True)}
+
+
+@pytest.mark.parametrize("case", sorted(STORE_QUANT))
+def test_tstore_fix_pipe_quantisation(kernels, oracle, case):
+    """Accumulators are exact here (integer-valued inputs), so the quantised stores must match the simulator bit for bit."""
+    kind, m, k, n, vector, relu, dst_kind, out_dt, signed = STORE_QUANT[case]
+    r = np.random.default_rng(60 + case)
+    if kind == "f16":
+        a, b = r.integers(-4, 5, (m, k)).astype(np.float32), r.integers(-4, 5, (k, n)).astype(np.float32)
+        acc = oracle.matmul_f16(f16_bits(a), f16_bits(b))
+        da, db = f16_bits(a), f16_bits(b)
+    else:
+        da, db = r.integers(-128, 128, (m, k)).astype(np.int8), r.integers(-128, 128, (k, n)).astype(np.int8)
+        acc = oracle.matmul_i8(da, db)
+    span = float(np.abs(acc).max())
+    scales = r.uniform(0.5, 1.5, n) * (100.0 / span if dst_kind != ob.ST_F16 else 1.0 / 64)
+    words = np.array([_word(s, offset=(3 if dst_kind != ob.ST_F16 else 0), signed=signed, vector=vector) for s in scales], np.uint64)
+    if not vector:
+        words = words[:1]
+    ref = oracle.store_quant(acc, dst_kind, words, per_column=vector, relu=relu)
+
+    kernels.pto_kernels_launch_store_quant.argtypes = [ctypes.c_int] + [ctypes.c_void_p] * 5
+    kernels.pto_kernels_launch_store_quant.restype = ctypes.c_int
+    t = [torch.from_numpy(np.ascontiguousarray(x)).to(DEV) for x in (da, db)]
+    dw = torch.from_numpy(words.view(np.int64)).to(DEV)
+    out = torch.zeros(m * n * np.dtype(out_dt).itemsize, dtype=torch.uint8, device=DEV)
+    rc = kernels.pto_kernels_launch_store_quant(case, out.data_ptr(), t[0].data_ptr(), t[1].data_ptr(), dw.data_ptr(),
+                                                torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert kernels.pto_kernels_status() == 0
+    got = out.cpu().numpy().view(out_dt).reshape(m, n)
+    assert np.array_equal(got, ref.view(out_dt))
+    assert len(np.unique(got)) > 8  # the case exercises the quantiser, not a saturated constant
