@@ -1,6 +1,6 @@
 """Throughput of the PTO tile-matmul hot path on one MI355X, with roofline fraction and a CPU baseline.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra] [--only N] [--calibrate-copy]
 
 A "step" is one TLOAD -> TMATMUL_ACC -> TSTORE pass over one synthetic batch.  The headline workload is
 BASELINE.json configs[1] (bf16 GEMM, M = N = K = 4096, A row-major, B column-major, N(0,1) * 0.02, fp32 accumulate,
@@ -155,6 +155,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-config measurements after the headline")
+    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4], default=None,
+                    help="measure just BASELINE.json configs[N] (a per_config entry) and print it: for profiling one kernel")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -173,6 +175,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     gen = torch.Generator(device=DEV).manual_seed(1)
+    if args.only is not None:
+        fn = {0: config1, 2: config3, 3: config4, 4: config5}[args.only]
+        print(json.dumps(fn(pa, ev, gen, args.steps, args.warmup)))
+        return
 
     m = n = k = 4096
     a = randn_bf16((m, k), gen, 0.02)
