@@ -12,6 +12,7 @@
 // (kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:115-150).
 #pragma once
 #include "device_types.hpp"
+#include "lds_dma.hpp"
 
 namespace ptoamd {
 
@@ -143,64 +144,57 @@ struct TileCfg {
 };
 
 // ---- TSTORE: drains one wave's accumulator blocks through the fix-pipe epilogue ------------------------------------
-// KIND (OutKind) and FULL (no bounds checks: the wave's tile lies inside the matrix) are compile-time so that each form
-// is a short, fully unrolled store sequence; a run-time switch inside the 16-register loop keeps the compiler from
-// unrolling it and pushes the accumulators into scratch memory.  The TMATMUL_ACC input is folded in here: C = Cin + A.B.
+// The output kind and FULL (no bounds checks: the wave's tile lies inside the matrix) are run-time properties, but the
+// dispatch on them sits *inside* the compile-time loop over 32x32 blocks: each variant then touches the 16 registers
+// of one block only.  A dispatch around the whole loop keeps every accumulator live across the branch, which with 128
+// or 256 accumulator registers per lane pushes them through scratch memory.  The TMATMUL_ACC input is folded in here:
+// C = Cin + A.B.
 template <int KIND, bool FULL, class Cfg, class Acc>
-__device__ __forceinline__ void tstore_blocks(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0,
-                                              int l32, int lhi)
+__device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi)
 {
     using Elem = typename Cfg::Op::Elem;
     const Elem* cin = reinterpret_cast<const Elem*>(p.c_in);
+    const int gj = col_b + l32;
+    float cs = 1.0f;
+    if (KIND == OUT_W8A8_BF16)
+        cs = (FULL || gj < p.n) ? p.col_scale[gj] : 0.0f;
 #pragma unroll
-    for (int i = 0; i < Cfg::MB; ++i)
-#pragma unroll
-        for (int j = 0; j < Cfg::NB; ++j) {
-            // keep the address arithmetic of one 32x32 block from being hoisted over the others (register pressure)
-            __builtin_amdgcn_sched_barrier(0);
-            const int gj = col0 + j * 32 + l32;
-            float cs = 1.0f;
-            if (KIND == OUT_W8A8_BF16)
-                cs = (FULL || gj < p.n) ? p.col_scale[gj] : 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int gi = row0 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-                if (FULL || (gi < p.m && gj < p.n)) {
-                    const long o = (long)gi * p.ldc + gj;
-                    auto v = acc[i][j][r];
-                    if (cin != nullptr)
-                        v += cin[o];
-                    if (p.relu)
-                        v = v > 0 ? v : 0;
-                    if (KIND == OUT_F32) {
-                        reinterpret_cast<float*>(p.c)[o] = (float)v;
-                    } else if (KIND == OUT_F16) {
-                        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits((float)v);
-                    } else if (KIND == OUT_BF16) {
-                        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits((float)v);
-                    } else if (KIND == OUT_I32) {
-                        reinterpret_cast<int32_t*>(p.c)[o] = (int32_t)v;
-                    } else {  // W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16, each step rounded to f32
-                        if (p.acc_out != nullptr)
-                            p.acc_out[o] = (int32_t)v;
-                        const float t = __fmul_rn((float)v, p.row_scale[gi]);
-                        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(__fmul_rn(t, cs));
-                    }
-                }
+    for (int r = 0; r < 16; ++r) {
+        const int gi = row_b + 8 * (r >> 2) + 4 * lhi + (r & 3);
+        if (FULL || (gi < p.m && gj < p.n)) {
+            const long o = (long)gi * p.ldc + gj;
+            auto v = acc[r];
+            if (cin != nullptr)
+                v += cin[o];
+            if (p.relu)
+                v = v > 0 ? v : 0;
+            if (KIND == OUT_F32) {
+                reinterpret_cast<float*>(p.c)[o] = (float)v;
+            } else if (KIND == OUT_F16) {
+                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits((float)v);
+            } else if (KIND == OUT_BF16) {
+                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits((float)v);
+            } else if (KIND == OUT_I32) {
+                reinterpret_cast<int32_t*>(p.c)[o] = (int32_t)v;
+            } else {  // W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16, each step rounded to f32
+                if (p.acc_out != nullptr)
+                    p.acc_out[o] = (int32_t)v;
+                const float t = __fmul_rn((float)v, p.row_scale[gi]);
+                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(__fmul_rn(t, cs));
             }
         }
+    }
 }
 
 template <bool FULL, class Cfg, class Acc>
-__device__ __forceinline__ void tstore_kind(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0,
-                                            int l32, int lhi)
+__device__ __forceinline__ void tstore_block_kind(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi)
 {
     switch (p.out_kind) {
-        case OUT_F32: tstore_blocks<OUT_F32, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
-        case OUT_F16: tstore_blocks<OUT_F16, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
-        case OUT_BF16: tstore_blocks<OUT_BF16, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
-        case OUT_I32: tstore_blocks<OUT_I32, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
-        default: tstore_blocks<OUT_W8A8_BF16, FULL, Cfg>(p, acc, row0, col0, l32, lhi); break;
+        case OUT_F32: tstore_block<OUT_F32, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
+        case OUT_F16: tstore_block<OUT_F16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
+        case OUT_BF16: tstore_block<OUT_BF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
+        case OUT_I32: tstore_block<OUT_I32, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
+        default: tstore_block<OUT_W8A8_BF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
     }
 }
 
@@ -208,10 +202,17 @@ template <class Cfg, class Acc>
 __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0, int l32,
                                        int lhi)
 {
-    if (row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n)
-        tstore_kind<true, Cfg>(p, acc, row0, col0, l32, lhi);
-    else
-        tstore_kind<false, Cfg>(p, acc, row0, col0, l32, lhi);
+    const bool full = row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n;
+    static_for<Cfg::MB * Cfg::NB>([&](auto bc) {
+        constexpr int i = decltype(bc)::value / Cfg::NB, j = decltype(bc)::value % Cfg::NB;
+        // keep the address arithmetic of one 32x32 block from being hoisted over the others (register pressure)
+        __builtin_amdgcn_sched_barrier(0);
+        const Acc block = acc[i][j];
+        if (full)
+            tstore_block_kind<true, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi);
+        else
+            tstore_block_kind<false, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi);
+    });
 }
 
 template <class Cfg>
