@@ -376,8 +376,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
                     uint32_t xa = 127u, xb = 127u;
                     if (has_scales) {
                         const int g = 2 * s + lhi;  // MX group of this lane inside the slab
-                        xa = (sca[i][g >> 2] >> ((g & 3) * 8)) & 0xFFu;
-                        xb = (scb[j][g >> 2] >> ((g & 3) * 8)) & 0xFFu;
+                        xa = (sca[i][s >> 1] >> ((g & 3) * 8)) & 0xFFu;  // (2 s + lhi) >> 2 == s >> 1
+                        xb = (scb[j][s >> 1] >> ((g & 3) * 8)) & 0xFFu;
                     }
                     Op::mma(acc[i][j], fa[i], fb[j], xa, xb);
                 }

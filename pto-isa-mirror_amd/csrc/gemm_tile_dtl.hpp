@@ -180,9 +180,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
             constexpr int i = x / NB, j = x % NB;
             uint32_t xa = 127u, xb = 127u;
             if (has_scales) {
+                // MX group 2 s + lhi of the slab: its dword is (2 s + lhi) >> 2 == s >> 1 for either lane half, which
+                // keeps the register-array index a compile-time constant
                 const int g = 2 * s + lhi;
-                xa = (sca[i][g >> 2] >> ((g & 3) * 8)) & 0xFFu;
-                xb = (scb[j][g >> 2] >> ((g & 3) * 8)) & 0xFFu;
+                xa = (sca[i][s >> 1] >> ((g & 3) * 8)) & 0xFFu;
+                xb = (scb[j][s >> 1] >> ((g & 3) * 8)) & 0xFFu;
             }
             Op::mma(acc[i][j], fa[set][i], fb[set][j], xa, xb);
             if (reads) {

@@ -347,6 +347,23 @@ def test_config4_mxfp8_full_size(pa, oracle):
     assert torch.equal(f2, f * 2)
 
 
+def test_mxfp4_gemm_large_takes_the_256_tile(pa, oracle):
+    """MXFP4 x MXFP4 at a grid that fills the chip: 2048 x 4096 x 2048, operands quantised by TQUANT<MXFP4> (OCP)."""
+    m, n, k = 2048, 4096, 2048
+    gen = torch.Generator(device=DEV).manual_seed(44)
+    a, sa = pa.tquant_mx(torch.randn((m, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
+    b, sb = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
+    out = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E2M1, pa.E2M1, pa.F32)
+    assert pa.last_kernel() == "tile256x256w8_dtl_fp4_e2m1"
+    rows, cols = np.array([0, 31, 32, 255, 256, 1027, 2047]), np.arange(0, n, 131)
+    ref = oracle.matmul_mx(host(sel(a, rows)), host(sel(b, cols)), host(sel(sa, rows)), host(sel(sb, cols)), len(rows), k, len(cols),
+                           ob.E2M1, ob.E2M1)
+    assert relerr(host(out)[np.ix_(rows, cols)], ref) <= 2e-2
+    with tile_env(PTOAMD_TILE=5):
+        other = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E2M1, pa.E2M1, pa.F32)
+    assert relerr(host(other), host(out)) <= 1e-5
+
+
 # ------------------------------------------------------------------------------------------- decode GEMV
 def _gemv_reference(oracle, a_bits, w, sw, n, k):
     tab = oracle.mx_decode_table(ob.E2M1)
