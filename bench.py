@@ -163,7 +163,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every box of this build has one MI355X and the path needs no second "
-                 "(C tiles are independent; see DESIGN.md on sharding). Run with --gpus 1.")
+                 "(output tiles are independent, so M or N shards need no exchange). Run with --gpus 1.")
 
     pa = ge.load_package()
     pa.init(0)
