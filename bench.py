@@ -130,13 +130,31 @@ def config5(pa, ev, gen, steps, warmup):
 
 
 def cpu_baseline():
-    """The CPU-simulator-shaped port (oracle/pto_oracle.c: per-element fractal addressing, per-TMATMUL thread
-    fan-out) on a bounded slab of the headline workload: 256 output rows x 4096 columns x K = 4096."""
-    from oracle.binding import Oracle, ST_BF16
+    """The reference CPU simulator itself where its compiled form is present (oracle/_ref, built from the reference's
+    headers: TLOAD / TMOV / TMATMUL_ACC / TSTORE on 256 x 256 output tiles, K walked by 512), else the plain-C port of
+    it (oracle/pto_oracle.c: per-element fractal addressing, per-TMATMUL thread fan-out).  Bounded slab of the headline
+    workload: 256 output rows x N x K = 4096."""
+    from oracle.binding import Oracle, RefLib, ST_BF16
 
-    orc = Oracle()
     rng = np.random.default_rng(0)
-    m, n, k = 256, 4096, 4096
+    k = 4096
+    threads = min(os.cpu_count() or 1, 16)
+    if RefLib.available():
+        # the simulator's bfloat16_t degrades to _Float16 without <stdfloat>: same loops and fp32 fma on fp16 inputs
+        ref = RefLib()
+        m, n, cols = 256, 256, 32
+        a = (rng.standard_normal((m, k)) * 0.02).astype(np.float16).view(np.uint16)
+        b = (rng.standard_normal((cols * n, k)) * 0.02).astype(np.float16).view(np.uint16)
+        t0 = time.perf_counter()
+        for j in range(cols):
+            ref.gemm("f16", a, b[j * n:(j + 1) * n], b_dn=True, kstep=512)
+        dt = time.perf_counter() - t0
+        flop = 2.0 * m * n * cols * k
+        return {"value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "reference",
+                "sample": f"{cols} output tiles of 256 x 256 (rows 0-255, columns 0-{cols * n - 1}) x K=4096, fp16 inputs "
+                          f"({flop / 1e9:.1f} GFLOP) in {dt:.1f} s; full 4096^3 extrapolates to {dt * 256 / cols:.0f} s"}
+    orc = Oracle()
+    m, n = 256, 4096
     a = ((rng.standard_normal((m, k)) * 0.02).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
     b = ((rng.standard_normal((n, k)) * 0.02).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
     t0 = time.perf_counter()

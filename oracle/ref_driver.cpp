@@ -21,7 +21,7 @@ using namespace pto;
 namespace {
 
 constexpr int TM = 256;  // max rows of A / C handled by one call
-constexpr int TK = 512;  // max contraction length handled by one call
+constexpr int TK = 512;  // max contraction length of one TMATMUL (longer K is walked in slabs)
 constexpr int TN = 256;  // max cols of B / C handled by one call
 
 using DynShape = Shape<1, 1, 1, DYNAMIC, DYNAMIC>;
@@ -48,10 +48,12 @@ template <typename OutT, typename InT, typename AccT>
 int RunGemm(OutT* out, InT* a, InT* b, const AccT* cin, int m, int k, int n, int lda, int ldb, int ldc, int b_dn,
             int kstep, int relu)
 {
-    if (m < 1 || m > TM || k < 1 || k > TK || n < 1 || n > TN)
+    if (m < 1 || m > TM || k < 1 || n < 1 || n > TN)
         return -1;
     if (kstep <= 0 || kstep > k)
         kstep = k;
+    if (kstep > TK)  // any K, walked in slabs of at most TK through TMATMUL_ACC
+        return -1;
     using MatA = Tile<TileType::Mat, InT, TM, TK, BLayout::ColMajor, DYNAMIC, DYNAMIC, SLayout::RowMajor, 512>;
     using MatB = Tile<TileType::Mat, InT, TK, TN, BLayout::ColMajor, DYNAMIC, DYNAMIC, SLayout::RowMajor, 512>;
     using MatBzn = Tile<TileType::Mat, InT, TK, TN, BLayout::RowMajor, DYNAMIC, DYNAMIC, SLayout::ColMajor, 512>;
