@@ -142,7 +142,7 @@ def cpu_baseline():
     if RefLib.available():
         # the simulator's bfloat16_t degrades to _Float16 without <stdfloat>: same loops and fp32 fma on fp16 inputs
         ref = RefLib()
-        m, n, cols = 256, 256, 32
+        m, n, cols = 256, 256, 96
         a = (rng.standard_normal((m, k)) * 0.02).astype(np.float16).view(np.uint16)
         b = (rng.standard_normal((cols * n, k)) * 0.02).astype(np.float16).view(np.uint16)
         t0 = time.perf_counter()
