@@ -223,6 +223,9 @@ struct BaseShape2D;
 #define PTO_AMD_C(...) __VA_ARGS__
 PTO_AMD_SHAPE2D(Layout::ND, PTO_AMD_C(Shape<1, 1, 1, rows, cols>), PTO_AMD_C(Stride<rows * cols, rows * cols, rows * cols, cols, 1>))
 PTO_AMD_SHAPE2D(Layout::DN, PTO_AMD_C(Shape<1, 1, 1, rows, cols>), PTO_AMD_C(Stride<rows * cols, rows * cols, rows * cols, 1, rows>))
+// NZ: column blocks of C0 = 32 bytes' worth of elements, rows contiguous inside a block (reference: pto_tile.hpp:709-725,797-815)
+PTO_AMD_SHAPE2D(Layout::NZ, PTO_AMD_C(Shape<1, cols / (32 / (int64_t)sizeof(T)), rows / 16, 16, 32 / (int64_t)sizeof(T)>),
+                PTO_AMD_C(Stride<rows * cols, rows * (32 / (int64_t)sizeof(T)), 16 * (32 / (int64_t)sizeof(T)), 32 / (int64_t)sizeof(T), 1>))
 PTO_AMD_SHAPE2D(Layout::MX_A_ZZ, PTO_AMD_C(Shape<1, rows / 16, cols / 2, 16, 2>), PTO_AMD_C(Stride<rows * cols, cols * 16, 32, 2, 1>))
 PTO_AMD_SHAPE2D(Layout::MX_A_ND, PTO_AMD_C(Shape<1, 1, rows, cols / 2, 2>), PTO_AMD_C(Stride<rows * cols, rows * cols, cols, 2, 1>))
 PTO_AMD_SHAPE2D(Layout::MX_A_DN, PTO_AMD_C(Shape<1, 1, cols / 2, rows, 2>), PTO_AMD_C(Stride<rows * cols, rows * cols, 2 * rows, 2, 1>))

@@ -429,9 +429,24 @@ PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, FpTileData& fp)
 template <typename DstTileData, typename SrcTileData, typename... WaitEvents>
 PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, WaitEvents&...)
 {
-    static_assert(DstTileData::Loc != TileType::Acc && SrcTileData::Loc != TileType::Acc,
-                  "TMOV from / to accumulator tiles is not implemented on this backend yet");
-    amd::textract_lds(dst, src, 0, 0);
+    static_assert(DstTileData::Loc != TileType::Acc, "TMOV into an accumulator tile is not implemented on this backend");
+    if constexpr (SrcTileData::Loc == TileType::Acc) {
+        // Acc -> Vec / Mat: the fix-pipe move of an accumulator into an on-chip buffer (reference: cpu/TMov.hpp:21-35),
+        // element type converted like TSTORE's static_cast
+        static_assert(DstTileData::Loc == TileType::Vec || DstTileData::Loc == TileType::Mat,
+                      "an accumulator tile moves to a Vec or Mat tile");
+        using D = typename DstTileData::DType;
+        const int vr = src.GetValidRow(), vc = src.GetValidCol();
+        uint8_t* d = dst.Storage();
+        __syncthreads();
+        amd::for_each_acc(src, [&](int slot, int r, int row, int col) {
+            if (row < vr && col < vc)
+                *reinterpret_cast<D*>(d + dst.ByteOffset(row, col)) = amd::convert<D>(src.regs[slot][r]);
+        });
+        __syncthreads();
+    } else {
+        amd::textract_lds(dst, src, 0, 0);
+    }
     return {};
 }
 template <typename DstTileData, typename SrcTileData, typename... WaitEvents>

@@ -193,6 +193,35 @@ __global__ AICORE void RunTMATMUL_MX(__gm__ float* out, __gm__ AT* src0, __gm__ 
     TSTORE(outGlobal, cTile);
 }
 
+// A in the NZ global layout (column blocks of 16 halves, rows contiguous inside a block), result moved Acc -> Vec tile
+// (converted to half) and stored from there
+template <int M, int K, int N>
+__global__ AICORE void RunTMATMUL_NZ_VEC(__gm__ half* out, __gm__ half* src0, __gm__ half* src1)
+{
+    GlobalTensor<half, TileShape2D<half, M, K, Layout::NZ>, BaseShape2D<half, M, K, Layout::NZ>, Layout::NZ> aGlobal(src0);
+    GlobalTensor<half, TileShape2D<half, K, N>, BaseShape2D<half, K, N>> bGlobal(src1);
+    GlobalTensor<half, TileShape2D<half, M, N>, BaseShape2D<half, M, N>> outGlobal(out);
+    Tile<TileType::Mat, half, M, K, BLayout::ColMajor, M, K, SLayout::RowMajor, 512> aMat;
+    Tile<TileType::Mat, half, K, N, BLayout::ColMajor, K, N, SLayout::RowMajor, 512> bMat;
+    TileLeft<half, M, K> aTile;
+    TileRight<half, K, N> bTile;
+    TileAcc<float, M, N> cTile;
+    Tile<TileType::Vec, half, M, N, BLayout::RowMajor, M, N> vTile;
+    TASSIGN(aMat, 0x0);
+    TASSIGN(bMat, 0x8000);
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(cTile, 0x0);
+    TASSIGN(vTile, 0x0);
+    TLOAD(aMat, aGlobal);
+    TLOAD(bMat, bGlobal);
+    TMOV(aTile, aMat);
+    TMOV(bTile, bMat);
+    TMATMUL(cTile, aTile, bTile);
+    TMOV(vTile, cTile);
+    TSTORE(outGlobal, vTile);
+}
+
 // The tiled GEMM of the CPU-simulator demo at full problem size: C[M, N] = A[M, K] . B[K, N], one core per BM x BN
 // output tile, K walked in BK slabs through TLOAD -> TMOV -> TMATMUL / TMATMUL_ACC, then TSTORE of the tile.
 template <typename OutT, typename InT, int M, int K, int N, int BM, int BN, int BK, bool B_IS_DN>
@@ -265,6 +294,7 @@ extern "C" int pto_kernels_launch(int id, void* out, void* src0, void* src1, voi
     case 11: return run<&RunTMATMUL<float, half, half, float, 26, 100, 94, true>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)src2);
     case 12: return run<&RunTMATMUL<int32_t, int8_t, int8_t, int32_t, 8, 7, 6, true>>(stream, 1, (int32_t*)out, (int8_t*)src0, (int8_t*)src1, (int32_t*)src2);
     case 13: return run<&RunTMATMUL<float, half, half, float, 1, 64, 96, true>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)src2);
+    case 20: return run<&RunTMATMUL_NZ_VEC<32, 64, 48>>(stream, 1, (half*)out, (half*)src0, (half*)src1);
     case 100: return run<&RunTiledGemm<float, half, 512, 512, 512, 128, 128, 64, false>>(stream, 16, (float*)out, (half*)src0, (half*)src1);
     case 101: return run<&RunTiledGemm<bfloat16_t, bfloat16_t, 512, 512, 512, 128, 128, 64, true>>(stream, 16, (bfloat16_t*)out, (bfloat16_t*)src0, (bfloat16_t*)src1);
     default: return -1;

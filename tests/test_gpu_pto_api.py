@@ -156,6 +156,24 @@ def test_tmatmul_mx_with_scale_tiles(kernels, oracle, case):
     assert relerr(out.cpu().numpy(), ref) <= 2e-2
 
 
+def test_nz_global_layout_and_acc_to_vec_move(kernels, oracle):
+    """TLOAD from an NZ GlobalTensor; TMOV Acc -> Vec (f32 -> f16, round to nearest even); TSTORE of the Vec tile."""
+    m, k, n, c0 = 32, 64, 48, 16
+    r = np.random.default_rng(20)
+    a, b = r.uniform(-1, 1, (m, k)).astype(np.float32), r.uniform(-1, 1, (k, n)).astype(np.float32)
+    ab, bb = f16_bits(a), f16_bits(b)
+    a_nz = np.ascontiguousarray(ab.reshape(m, k // c0, c0).transpose(1, 0, 2))  # [k / C0][m][C0]
+    out = run(kernels, 20, ((m, n), torch.float16), a_nz, bb)
+    got = out.cpu().numpy()
+    ref32 = oracle.matmul_f16(ab, bb)
+    assert relerr(got.astype(np.float32), ref32) <= 1e-2
+    with_int = r.integers(1, 5, (m, k)).astype(np.float32), r.integers(1, 5, (k, n)).astype(np.float32)
+    ab, bb = f16_bits(with_int[0]), f16_bits(with_int[1])
+    a_nz = np.ascontiguousarray(ab.reshape(m, k // c0, c0).transpose(1, 0, 2))
+    got = run(kernels, 20, ((m, n), torch.float16), a_nz, bb).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), oracle.store_f32(oracle.matmul_f16(ab, bb), ob.ST_F16))
+
+
 def test_split_k_accumulates_in_the_accumulator_tile(kernels, oracle):
     """TMATMUL then four TMATMUL_ACC over five K-slabs of a 128 x 128 x 64 tile (reference case 3)."""
     r = np.random.default_rng(3)
