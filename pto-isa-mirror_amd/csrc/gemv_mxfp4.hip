@@ -8,9 +8,9 @@
 //     k-slice s (1024 k) of every strip and keeps its activation fragments for that slice in registers for the whole
 //     kernel (128 VGPRs, loaded once).  Weights and scales stream global -> LDS by LDS-DMA into a per-wave
 //     double-buffered region (512 contiguous bytes per row, two rows per instruction, no VGPRs, no barriers: a wave
-//     reads back only what it wrote), are re-read as MFMA operand fragments (4 bytes = 8 fp4 per lane and MFMA; row
-//     pairs padded and odd rows half-swapped on the global side, so the reads are conflict-free), dequantised in
-//     registers and multiplied on
+//     reads back only what it wrote), are re-read as MFMA operand fragments (16 bytes = one MX group per lane, feeding
+//     four MFMAs; row pairs padded and odd rows half-swapped on the global side, so the reads are conflict-free),
+//     dequantised in registers and multiplied on
 //     v_mfma_f32_16x16x32_bf16.  The 8 k-slice partials of a strip are summed through LDS in a fixed order.
 //   * streaming (k % 512 == 0 otherwise): a wave owns 16 rows over the full K, register prefetch four chunks deep,
 //     activations staged per chunk through LDS.
@@ -192,13 +192,14 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
     const int ks = p.k / SK_SLICE, sb = p.k / 32;
     uint8_t* my = smem + wave * SK_WAVE_LDS;
     const uint32_t my_lds = lds_address(my);
-    // LDS byte of (row l16, chunk t, byte 4 q) is wread0 + 16 t for chunks with (t & 8) == 0, wread1 + 16 t for the others
-    // (odd rows keep their 128-byte halves swapped: 64 lanes reading one chunk index hit 64 different banks)
-    const int wrow = (l16 >> 1) * SK_PAIR + (l16 & 1) * 512 + 4 * q;
-    const int wread0 = wrow + 128 * (l16 & 1), wread1 = wrow - 128 * (l16 & 1);
-    // activation stages use the same row layout with 16-byte pieces: (row l16, step tt of the quarter, piece q)
-    const int arow = (l16 >> 1) * SK_PAIR + (l16 & 1) * 512 + 16 * q;
-    const int aread0 = arow + 128 * (l16 & 1), aread1 = arow - 128 * (l16 & 1);
+    // k-assignment inside a 1024-k slice: MFMA step (j, t), j < 8, t < 4, multiplies k = 32 (4 j + q) + 8 t .. + 7 in lane
+    // quarter q, so a lane's 16-byte weight read (one MX group = chunk 4 j + q of the row) feeds the four steps t.
+    // Rows sit in LDS as pairs (2 x 512 bytes + 16 pad) with the 128-byte halves of odd rows swapped (chunk ^ 8):
+    //   weights      chunk 4 j + q of row l16 is at (j & 2 ? wread1 : wread0) + 64 j
+    //   activations  piece 16 jj + 4 q + t of a quarter (jj < 2) is at aread + 16 (16 jj + t)
+    const int lrow = (l16 >> 1) * SK_PAIR + (l16 & 1) * 512;
+    const int wread0 = lrow + 16 * q + 128 * (l16 & 1), wread1 = lrow + 16 * q - 128 * (l16 & 1);
+    const int aread = lrow + (((4 * q) ^ (8 * (l16 & 1))) << 4);
     const int mine = s_end > s_begin + rg ? (s_end - s_begin - rg + rgs - 1) / rgs : 0;  // strips of this row group
     const int most = (s_end - s_begin + rgs - 1) / rgs;                                   // ... of row group 0
 
@@ -247,10 +248,10 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
                            p.m - 1, my_lds + (j & 1) * SK_STAGE, ln);
             };
 
-            // Activation fragments of this k-slice, in the MFMA's own k order: step t multiplies k = 32 t .. 32 t + 31 of
-            // the slice and lane (m = l16, quarter q) holds A[m][32 t + 8 q .. + 7].  Loading them straight from global
-            // memory would make 64 separate 16-byte requests per instruction (the row index is the fast lane index);
-            // instead the four quarters run through the same LDS-DMA pipeline as the weight strips, ahead of them.
+            // Activation fragments of this k-slice: areg[4 j + t] holds A[m = l16][32 (4 j + q) + 8 t .. + 7].  Loading
+            // them straight from global memory would make 64 separate 16-byte requests per instruction (the row index
+            // is the fast lane index); instead the four quarters (256 k each) run through the same LDS-DMA pipeline as
+            // the weight strips, ahead of them.
             uint4 areg[32];
             issue_a(0);
             issue_a(1);
@@ -263,8 +264,8 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
                 asm volatile("" ::: "memory");
                 const uint8_t* buf = my + (j & 1) * SK_STAGE;
 #pragma unroll
-                for (int tt = 0; tt < 8; ++tt)
-                    areg[8 * j + tt] = *reinterpret_cast<const uint4*>(buf + ((tt & 2) ? aread1 : aread0) + 64 * tt);
+                for (int x = 0; x < 8; ++x)  // x = 4 jj + t: the fragment of step (2 j + jj, t)
+                    areg[8 * j + x] = *reinterpret_cast<const uint4*>(buf + aread + 16 * (16 * (x >> 2) + (x & 3)));
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 if (j + 2 < 4)
                     issue_a(j + 2);
@@ -286,11 +287,11 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
                     const uint32_t sc[8] = {sc0.x, sc0.y, sc0.z, sc0.w, sc1.x, sc1.y, sc1.z, sc1.w};
                     static_for<2>([&](auto hc) {
                         constexpr int h = decltype(hc)::value;
-                        uint32_t wv[16];
+                        uint4 wv[4];
 #pragma unroll
-                        for (int j = 0; j < 16; ++j) {  // step t = 16 h + j: MX group t of the slice, 8 fp4 at byte 4 q
-                            const int t = 16 * h + j;
-                            wv[j] = *reinterpret_cast<const uint32_t*>(buf + ((t & 8) ? wread1 : wread0) + t * 16);
+                        for (int jj = 0; jj < 4; ++jj) {  // MX group 4 j + q of the slice, j = 4 h + jj
+                            const int j = 4 * h + jj;
+                            wv[jj] = *reinterpret_cast<const uint4*>(buf + ((j & 2) ? wread1 : wread0) + 64 * j);
                         }
                         if (h == 1) {
                             // the buffer is refilled only after every read of it has returned
@@ -299,12 +300,16 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
                                 issue(i + 2);
                         }
 #pragma unroll
-                        for (int j = 0; j < 16; ++j) {
-                            const int t = 16 * h + j;
-                            const float scale = e8m0_to_f32((sc[t >> 2] >> (8 * (t & 3))) & 0xFFu);
-                            const uint4 w8 = dequant8<HW_CVT>(wv[j], scale);
-                            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, areg[t]),
-                                                                            __builtin_bit_cast(bf16x8, w8), acc[i], 0, 0, 0);
+                        for (int jj = 0; jj < 4; ++jj) {
+                            const int j = 4 * h + jj;
+                            const float scale = e8m0_to_f32((sc[j] >> (8 * q)) & 0xFFu);  // scale byte 4 j + q
+                            const uint32_t xs[4] = {wv[jj].x, wv[jj].y, wv[jj].z, wv[jj].w};
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) {
+                                const uint4 w8 = dequant8<HW_CVT>(xs[t], scale);
+                                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, areg[4 * j + t]),
+                                                                                __builtin_bit_cast(bf16x8, w8), acc[i], 0, 0, 0);
+                            }
                         }
                     });
                 }
