@@ -97,12 +97,34 @@ PTO_INST void textract_lds(DstTile& dst, SrcTile& src, int row0, int col0)
 {
     using T = typename DstTile::DType;
     static_assert(std::is_same_v<T, typename SrcTile::DType>, "TMOV / TEXTRACT: element types differ");
-    static_assert(!is_packed4<T>, "TMOV of packed fp4 tiles is not implemented on this backend yet");
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
     const uint8_t* s = src.Storage();
     uint8_t* d = dst.Storage();
     __syncthreads();
-    if constexpr (DstTile::Loc == TileType::Right) {  // stored transposed: walk k (rows) fastest
+    if constexpr (is_packed4<T>) {
+        // two fp4 codes per byte: one thread builds one destination byte from the two source nibbles it needs (the
+        // pairing direction of source and destination may differ: a Right tile pairs along k, a Mat tile along a row)
+        auto code = [&](int r, int c) -> uint32_t {
+            const int sr = r + row0, sc = c + col0;
+            if (sr < vr && sc < vc && r < dst.GetValidRow() && c < dst.GetValidCol())
+                return (s[src.ByteOffset(sr, sc)] >> (4 * SrcTile::Nibble(sr, sc))) & 0xFu;
+            return 0u;
+        };
+        constexpr bool along_rows = DstTile::Loc == TileType::Right;
+        static_assert(along_rows ? DstTile::Rows % 2 == 0 : DstTile::Cols % 2 == 0, "packed fp4 tiles hold element pairs");
+        for (int idx = threadIdx.x; idx < DstTile::Rows * DstTile::Cols / 2; idx += PTO_AMD_THREADS) {
+            int r, c;
+            uint32_t lo, hi;
+            if constexpr (along_rows) {
+                c = idx / (DstTile::Rows / 2), r = 2 * (idx - c * (DstTile::Rows / 2));
+                lo = code(r, c), hi = code(r + 1, c);
+            } else {
+                r = idx / (DstTile::Cols / 2), c = 2 * (idx - r * (DstTile::Cols / 2));
+                lo = code(r, c), hi = code(r, c + 1);
+            }
+            d[dst.ByteOffset(r, c)] = (uint8_t)(lo | (hi << 4));
+        }
+    } else if constexpr (DstTile::Loc == TileType::Right) {  // stored transposed: walk k (rows) fastest
         for (int idx = threadIdx.x; idx < DstTile::Rows * DstTile::Cols; idx += PTO_AMD_THREADS) {
             const int c = idx / DstTile::Rows, r = idx - c * DstTile::Rows;
             const int sr = r + row0, sc = c + col0;
@@ -234,6 +256,10 @@ template <>
 struct MxFormat<float8_e5m2_t> {
     static constexpr int code = 1;
 };
+template <>
+struct MxFormat<float4_e2m1x2_t> {
+    static constexpr int code = 4;  // the scaled MFMA has no E1M2 format
+};
 typedef int i32x8v __attribute__((ext_vector_type(8)));
 
 template <bool INIT, typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT>
@@ -245,6 +271,7 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
                       TileLeftScaleT::Loc == TileType::ScaleLeft && TileRightScaleT::Loc == TileType::ScaleRight,
                   "TMATMUL_MX takes (Acc, Left, ScaleLeft, Right, ScaleRight) tiles");
     static_assert(std::is_same_v<typename TileRes::DType, float>, "TMATMUL_MX accumulates in float");
+    static_assert(is_packed4<TA> == is_packed4<TB>, "TMATMUL_MX: both operands fp8 or both fp4");
     static_assert(TileLeftT::Cols % 64 == 0, "TMATMUL_MX: the static K of the Left tile must be a multiple of 64");
     static_assert(TileLeftT::Cols == TileRightT::Rows && TileRes::Rows == TileLeftT::Rows && TileRes::Cols == TileRightT::Cols,
                   "TMATMUL_MX: static tile shapes do not chain");
@@ -267,14 +294,22 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
             if constexpr (INIT)
                 acc = typename TileRes::Vec16(0);
             for (int k0 = 0; k0 < kpad; k0 += 64) {
-                const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 16 * lhi));
-                const uint4 a1 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 32 + 16 * lhi));
-                const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 16 * lhi, bcol));
-                const uint4 b1 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 + 16 * lhi, bcol));
                 const int g = k0 / 32 + lhi;
                 const int sa = psa[as.ByteOffset(arow, g)], sb = psb[bs.ByteOffset(g, bcol)];
-                const i32x8v av = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
-                const i32x8v bv = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                i32x8v av = {0, 0, 0, 0, 0, 0, 0, 0}, bv = {0, 0, 0, 0, 0, 0, 0, 0};
+                if constexpr (is_packed4<TA>) {  // fp4: the lane's 16 bytes are the whole MX block lhi
+                    const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 32 * lhi));
+                    const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 * lhi, bcol));
+                    av = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, 0, 0, 0, 0};
+                    bv = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, 0, 0, 0, 0};
+                } else {  // fp8: bytes [16 lhi, 16 lhi + 16) of each of the two blocks
+                    const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 16 * lhi));
+                    const uint4 a1 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 32 + 16 * lhi));
+                    const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 16 * lhi, bcol));
+                    const uint4 b1 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 + 16 * lhi, bcol));
+                    av = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                    bv = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                }
                 acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, MxFormat<TA>::code, MxFormat<TB>::code, 0, sa, 0, sb);
             }
             c.regs[slot] = acc;
@@ -502,7 +537,7 @@ PTO_INST RecordEvent TMATMUL_BIAS(TileRes& cMatrix, TileLeftT& aMatrix, TileRigh
     });
     return {};
 }
-// ---- TMATMUL_MX / TGEMV_MX (fp8 E4M3 / E5M2 operands; reference: cpu/TMatmul.hpp:169-205,254-326) ------------------
+// ---- TMATMUL_MX / TGEMV_MX (fp8 E4M3 / E5M2 or fp4 E2M1 operands; reference: cpu/TMatmul.hpp:169-205,254-326) ------------------
 template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT,
           typename = std::enable_if_t<TileLeftScaleT::Loc == TileType::ScaleLeft>>
 PTO_INST RecordEvent TMATMUL_MX(TileRes& cMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale, TileRightT& bMatrix, TileRightScaleT& bScale)

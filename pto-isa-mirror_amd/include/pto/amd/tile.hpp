@@ -125,6 +125,9 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
         else
             return (uint32_t)(((int64_t)r * Cols_ + c) * b2 / 2);
     }
+    // which nibble of that byte holds element (r, c) of a packed fp4 tile: pairs run along k for Left / Right tiles,
+    // along a row otherwise
+    PTO_INST static int Nibble(int r, int c) { return Loc_ == TileType::Right ? (r & 1) : (c & 1); }
     // [row][KC] with k contiguous; 16-byte chunk index XORed with the row when the row holds a power-of-two number of
     // chunks (<= 8 of its low bits), so 32 rows read at one k land in different banks
     template <int KC>

@@ -302,7 +302,8 @@ extern "C" int pto_kernels_launch(int id, void* out, void* src0, void* src1, voi
 }
 
 // MX cases: 1: e4m3 x e4m3 32x128x48, scales MX_A_ZZ / MX_B_NN      2: e5m2 x e4m3 33x192x70, scales MX_A_ND / MX_B_DN, bias
-//           3: e4m3 x e5m2 16x64x32, scales MX_A_DN / MX_B_ND
+//           3: e4m3 x e5m2 16x64x32, scales MX_A_DN / MX_B_ND      4: e2m1 x e2m1 (packed fp4) 40x128x60, ND / DN scales
+//           5: e2m1 x e2m1 32x256x64, scales MX_A_ZZ / MX_B_NN, bias
 extern "C" int pto_kernels_launch_mx(int id, void* out, void* a, void* b, void* sa, void* sb, void* bias, void* stream)
 {
     using S = float8_e8m0_t;
@@ -313,6 +314,10 @@ extern "C" int pto_kernels_launch_mx(int id, void* out, void* a, void* b, void* 
             stream, 1, (float*)out, (float8_e5m2_t*)a, (float8_e4m3_t*)b, (S*)sa, (S*)sb, (float*)bias);
     case 3: return run<&RunTMATMUL_MX<float8_e4m3_t, float8_e5m2_t, 16, 64, 32, Layout::MX_A_DN, Layout::MX_B_ND, false>>(
             stream, 1, (float*)out, (float8_e4m3_t*)a, (float8_e5m2_t*)b, (S*)sa, (S*)sb, (float*)nullptr);
+    case 4: return run<&RunTMATMUL_MX<float4_e2m1x2_t, float4_e2m1x2_t, 40, 128, 60, Layout::MX_A_ND, Layout::MX_B_DN, false>>(
+            stream, 1, (float*)out, (float4_e2m1x2_t*)a, (float4_e2m1x2_t*)b, (S*)sa, (S*)sb, (float*)nullptr);
+    case 5: return run<&RunTMATMUL_MX<float4_e2m1x2_t, float4_e2m1x2_t, 32, 256, 64, Layout::MX_A_ZZ, Layout::MX_B_NN, true>>(
+            stream, 1, (float*)out, (float4_e2m1x2_t*)a, (float4_e2m1x2_t*)b, (S*)sa, (S*)sb, (float*)bias);
     default: return -1;
     }
 }

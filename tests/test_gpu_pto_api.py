@@ -117,10 +117,14 @@ def test_single_tile_fp8(kernels, oracle):
 # MX case id -> (A type, B type, M, K, N, A-scale layout, B-scale layout, bias)
 MX_CASES = {1: (ob.E4M3, ob.E4M3, 32, 128, 48, ob.MX_A_ZZ, ob.MX_B_NN, False),
             2: (ob.E5M2, ob.E4M3, 33, 192, 70, ob.MX_A_ND, ob.MX_B_DN, True),
-            3: (ob.E4M3, ob.E5M2, 16, 64, 32, ob.MX_A_DN, ob.MX_B_ND, False)}
+            3: (ob.E4M3, ob.E5M2, 16, 64, 32, ob.MX_A_DN, ob.MX_B_ND, False),
+            4: (ob.E2M1, ob.E2M1, 40, 128, 60, ob.MX_A_ND, ob.MX_B_DN, False),   # packed fp4, two codes per byte
+            5: (ob.E2M1, ob.E2M1, 32, 256, 64, ob.MX_A_ZZ, ob.MX_B_NN, True)}
 
 
 def _codes(r, typ, shape):
+    if typ == ob.E2M1:  # every nibble is a finite value; pairs run along the last axis
+        return r.integers(0, 256, (shape[0], shape[1] // 2)).astype(np.uint8)
     c = r.integers(0, 256, shape).astype(np.uint8)
     if typ == ob.E4M3:
         c[(c & 0x7F) == 0x7F] = 0x38  # NaN codes -> 1.0
