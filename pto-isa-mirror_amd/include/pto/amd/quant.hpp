@@ -95,6 +95,50 @@ PTO_INST void tquant_mx(TileOut& dst, TileSrc& src, TileExp* exp, TileMax* mx, T
     __syncthreads();
 }
 
+// groups of 32 along a column (grouping axis 0, the DN form): one thread per (group, column pair); exp / max / scaling
+// are [rows / 32][cols]
+template <int ALG, typename TileOut, typename TileSrc, typename TileExp, typename TileMax, typename TileScaling>
+PTO_INST void tquant_mx_cols(TileOut& dst, TileSrc& src, TileExp* exp, TileMax* mx, TileScaling* scaling)
+{
+    using S = typename TileSrc::DType;
+    constexpr bool SRC_BF16 = std::is_same_v<S, __bf16>;
+    constexpr bool FP4 = ALG == ptoamd::MX_OCP_FP4 || ALG == ptoamd::MX_NV_FP4;
+    const int vr = src.GetValidRow(), vc = src.GetValidCol(), groups = vr / 32, pairs = vc / 2;
+    auto at = [&](int r, int c) { return to_float(*reinterpret_cast<const S*>(src.Storage() + src.ByteOffset(r, c))); };
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < groups * pairs; idx += PTO_AMD_THREADS) {
+        const int g = idx / pairs, c0 = 2 * (idx - g * pairs);
+        float sc[2];
+        for (int j = 0; j < 2; ++j) {
+            uint32_t run = 0;
+            for (int r = 0; r < 32; ++r)
+                run = ptoamd::max_step<ALG>(run, at(g * 32 + r, c0 + j));
+            const float maxabs = ptoamd::max_value<ALG>(run, ptoamd::u2f(0x7FC00000u));
+            const uint32_t e = ptoamd::shared_exponent<ALG>(maxabs);
+            sc[j] = ptoamd::group_scaling<ALG>(maxabs, e);
+            const int gi = g * vc + c0 + j;
+            if (exp)
+                *reinterpret_cast<uint8_t*>(exp->Storage() + gi) = (uint8_t)e;
+            if (mx)
+                reinterpret_cast<float*>(mx->Storage())[gi] = maxabs;
+            if (scaling)
+                reinterpret_cast<float*>(scaling->Storage())[gi] = sc[j];
+        }
+        for (int r = 0; r < 32; ++r) {
+            const int row = g * 32 + r;
+            const uint32_t q0 = ptoamd::encode_mx<ALG, SRC_BF16>(at(row, c0), sc[0]);
+            const uint32_t q1 = ptoamd::encode_mx<ALG, SRC_BF16>(at(row, c0 + 1), sc[1]);
+            if constexpr (FP4) {
+                *reinterpret_cast<uint8_t*>(dst.Storage() + dst.ByteOffset(row, c0)) = (uint8_t)(q0 | (q1 << 4));
+            } else {
+                *reinterpret_cast<uint8_t*>(dst.Storage() + dst.ByteOffset(row, c0)) = (uint8_t)q0;
+                *reinterpret_cast<uint8_t*>(dst.Storage() + dst.ByteOffset(row, c0 + 1)) = (uint8_t)q1;
+            }
+        }
+    }
+    __syncthreads();
+}
+
 }  // namespace amd
 
 // INT8: dst = clamp(nearbyint(src * scale[row] (+ offset[row]))); the "scale" operand multiplies
@@ -114,6 +158,23 @@ PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataExp* exp
 {
     constexpr int alg = (quant_type == QuantType::MXFP8 ? 0 : 2) + (scale_alg == QuantScaleAlg::NV ? 1 : 0);
     amd::tquant_mx<alg>(dst, src, exp, max, scaling);
+    return {};
+}
+
+// MX with an explicit grouping axis (1: along a row, 0: along a column) and the unified algorithm tag
+// (reference: common/pto_instr.hpp:3006-3019, cpu/TQuant.hpp:524-547)
+template <int grp_axis, auto mx_alg, typename TileDataOut, typename TileDataSrc, typename TileDataExp, typename TileDataMax,
+          typename TileDataScaling>
+PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataExp* exp, TileDataMax* max, TileDataScaling* scaling)
+{
+    static_assert(grp_axis == 0 || grp_axis == 1, "TQUANT: the grouping axis is 0 or 1");
+    static_assert(std::is_same_v<decltype(mx_alg), MxQuantAlg>, "TQUANT<grp_axis, mx_alg>: mx_alg is an MxQuantAlg");
+    constexpr int alg = static_cast<int>(mx_alg);
+    static_assert(alg >= 0 && alg <= 3, "TQUANT: the HiFloat4 algorithm is not implemented on this backend");
+    if constexpr (grp_axis == 1)
+        amd::tquant_mx<alg>(dst, src, exp, max, scaling);
+    else
+        amd::tquant_mx_cols<alg>(dst, src, exp, max, scaling);
     return {};
 }
 

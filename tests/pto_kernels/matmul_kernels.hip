@@ -390,6 +390,39 @@ __global__ AICORE void RunTQUANT_MX(__gm__ DstT* dst, __gm__ uint8_t* exp, __gm_
     TSTORE(scalingGlobal, scalingTile);
 }
 
+// column-grouped form: 32 consecutive rows of one column share an exponent; exp / max / scaling are [R / 32][C]
+template <typename DstT, int R, int C, MxQuantAlg ALG>
+__global__ AICORE void RunTQUANT_MX_DN(__gm__ DstT* dst, __gm__ uint8_t* exp, __gm__ float* max, __gm__ float* scaling, __gm__ float* src)
+{
+    constexpr int G = R / 32 * C;
+    using SrcTile = Tile<TileType::Vec, float, R, C, BLayout::RowMajor, R, C>;
+    using DstTile = Tile<TileType::Vec, DstT, R, C, BLayout::RowMajor, R, C>;
+    using ExpTile = Tile<TileType::Vec, uint8_t, R / 32, C, BLayout::RowMajor, R / 32, C>;
+    using FlatTile = Tile<TileType::Vec, float, R / 32, C, BLayout::RowMajor, R / 32, C>;
+    SrcTile srcTile;
+    DstTile dstTile;
+    ExpTile expTile;
+    FlatTile maxTile, scalingTile;
+    constexpr int a1 = CeilAlign<int>(SrcTile::Bytes, 32), a2 = a1 + CeilAlign<int>(DstTile::Bytes, 32),
+                  a3 = a2 + CeilAlign<int>(ExpTile::Bytes, 32), a4 = a3 + CeilAlign<int>(FlatTile::Bytes, 32);
+    static_assert(G > 0, "at least one group");
+    TASSIGN(srcTile, 0x0);
+    TASSIGN(dstTile, a1);
+    TASSIGN(expTile, a2);
+    TASSIGN(maxTile, a3);
+    TASSIGN(scalingTile, a4);
+    GlobalTensor<float, TileShape2D<float, R, C>, BaseShape2D<float, R, C>> srcGlobal(src);
+    GlobalTensor<DstT, TileShape2D<DstT, R, C>, BaseShape2D<DstT, R, C>> dstGlobal(dst);
+    GlobalTensor<uint8_t, TileShape2D<uint8_t, R / 32, C>, BaseShape2D<uint8_t, R / 32, C>> expGlobal(exp);
+    GlobalTensor<float, TileShape2D<float, R / 32, C>, BaseShape2D<float, R / 32, C>> maxGlobal(max), scalingGlobal(scaling);
+    TLOAD(srcTile, srcGlobal);
+    TQUANT<0, ALG>(dstTile, srcTile, &expTile, &maxTile, &scalingTile);
+    TSTORE(dstGlobal, dstTile);
+    TSTORE(expGlobal, expTile);
+    TSTORE(maxGlobal, maxTile);
+    TSTORE(scalingGlobal, scalingTile);
+}
+
 template <int R, int C, bool ASYM>
 __global__ AICORE void RunTQUANT_INT8(__gm__ uint8_t* dst, __gm__ float* src, __gm__ float* scale, __gm__ float* offset)
 {
@@ -441,6 +474,7 @@ __global__ AICORE void RunTDEQUANT(__gm__ float* dst, __gm__ SrcT* src, __gm__ f
 }
 
 // quant cases: 1-4: f32 16x64 -> OCP-FP8, NV-FP8, OCP-FP4, NV-FP4     5: bf16 8x128 -> OCP-FP4     6: half 8x128 -> OCP-FP8
+//              7, 8: f32 64x16 grouped along columns -> OCP-FP8, NV-FP4
 //              10: INT8 sym 16x64   11: INT8 asym 16x64    20: TDEQUANT int8 16x64    21: TDEQUANT int32 8x32
 extern "C" int pto_kernels_launch_quant(int id, void* dst, void* exp, void* max, void* scaling, void* src, void* scale, void* offset, void* stream)
 {
@@ -453,6 +487,8 @@ extern "C" int pto_kernels_launch_quant(int id, void* dst, void* exp, void* max,
     case 4: return run<&RunTQUANT_MX<float, F4, 16, 64, QuantType::MXFP4_E2M1, QuantScaleAlg::NV>>(stream, 1, (F4*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (float*)src);
     case 5: return run<&RunTQUANT_MX<bfloat16_t, F4, 8, 128, QuantType::MXFP4_E2M1, QuantScaleAlg::OCP>>(stream, 1, (F4*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (bfloat16_t*)src);
     case 6: return run<&RunTQUANT_MX<half, F8, 8, 128, QuantType::MXFP8, QuantScaleAlg::OCP>>(stream, 1, (F8*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (half*)src);
+    case 7: return run<&RunTQUANT_MX_DN<F8, 64, 16, MxQuantAlg::OcpMxFp8E4M3>>(stream, 1, (F8*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (float*)src);
+    case 8: return run<&RunTQUANT_MX_DN<F4, 64, 16, MxQuantAlg::NvMxFp4E2M1>>(stream, 1, (F4*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (float*)src);
     case 10: return run<&RunTQUANT_INT8<16, 64, false>>(stream, 1, (uint8_t*)dst, (float*)src, (float*)scale, (float*)offset);
     case 11: return run<&RunTQUANT_INT8<16, 64, true>>(stream, 1, (uint8_t*)dst, (float*)src, (float*)scale, (float*)offset);
     case 20: return run<&RunTDEQUANT<int8_t, 16, 64>>(stream, 1, (float*)dst, (int8_t*)src, (float*)scale, (float*)offset);

@@ -267,6 +267,26 @@ def test_tquant_mx_tile_instruction_bit_exact(kernels, oracle, case):
     assert _eq_f32(mx.cpu().numpy(), rm.ravel()) and _eq_f32(sc.cpu().numpy(), rs.ravel())
 
 
+@pytest.mark.parametrize("case,alg", [(7, ob.OCP_FP8), (8, ob.NV_FP4)])
+def test_tquant_mx_column_groups_bit_exact(kernels, oracle, case, alg):
+    """TQUANT<0, alg>: 32 consecutive rows of a column share the exponent (the reference's tquant_dn form)."""
+    rows, cols = 64, 16
+    r = np.random.default_rng(case)
+    x = (r.standard_normal((rows, cols)) * 10 ** r.uniform(-3, 3, (1, cols))).astype(np.float32)
+    x[:32, 0] = 0
+    x[5, 1] = np.inf
+    fp4 = alg in (ob.OCP_FP4, ob.NV_FP4)
+    g = rows // 32 * cols
+    dst = torch.zeros(rows * cols // (2 if fp4 else 1), dtype=torch.uint8, device=DEV)
+    exp = torch.zeros(g, dtype=torch.uint8, device=DEV)
+    mx, sc = torch.zeros(g, dtype=torch.float32, device=DEV), torch.zeros(g, dtype=torch.float32, device=DEV)
+    _quant_launch(kernels, case, dst, exp, mx, sc, torch.from_numpy(x).to(DEV))
+    rc, re, rm, rs = oracle.tquant_mx(x, alg, 0, ob.SRC_F32)
+    assert np.array_equal(exp.cpu().numpy(), re.ravel())
+    assert np.array_equal(dst.cpu().numpy(), rc.ravel())
+    assert _eq_f32(mx.cpu().numpy(), rm.ravel()) and _eq_f32(sc.cpu().numpy(), rs.ravel())
+
+
 def test_tquant_int8_and_tdequant_tile_instructions_bit_exact(kernels, oracle):
     r = np.random.default_rng(21)
     src = (r.standard_normal((16, 64)) * 60).astype(np.float32)
