@@ -198,11 +198,99 @@ __device__ __forceinline__ void tstore_block_kind(const TileGemmParams& p, const
     }
 }
 
+// ---- TSTORE of 16-bit outputs through LDS ---------------------------------------------------------------------------
+// An accumulator register holds one column of the block per lane, so storing it directly writes 2 bytes per lane
+// (64-byte row pieces, 16 store instructions per block) and the store unit's per-lane rate, not HBM, bounds the
+// epilogue.  Here a wave converts one 32-row band of its tile into a private, padded LDS region with the same fix-pipe
+// arithmetic, reads it back as 16-byte row chunks and writes whole 128-byte (or longer) row pieces.  LDS operations of
+// one wave execute in order, so the region is reused for the next band without a barrier.
+template <class Cfg>
+struct StagedStore {
+    static constexpr int ROW_BYTES = Cfg::WTN * 2 + 16;        // the pad keeps lanes 32-63 (rows + 4) off lanes 0-31's banks
+    static constexpr int WAVE_BYTES = 32 * ROW_BYTES;
+    static constexpr int CHUNKS = Cfg::WTN / 8;                // 16-byte chunks per row
+    static constexpr int ITERS = 32 * CHUNKS / 64;             // chunks per lane per band
+    static_assert(Cfg::THREADS / 64 * WAVE_BYTES <= Cfg::LDS_BYTES, "staging regions fit in the operand ring");
+    static_assert((32 * CHUNKS) % 64 == 0, "a band is a whole number of 64-lane reads");
+};
+
+template <int KIND, class Cfg, class Acc>
+__device__ __forceinline__ void tstage_block(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi,
+                                             uint8_t* lane_base)
+{
+    using Elem = typename Cfg::Op::Elem;
+    const Elem* cin = reinterpret_cast<const Elem*>(p.c_in);
+    const int gj = col_b + l32;
+    float cs = 1.0f;
+    if (KIND == OUT_W8A8_BF16)
+        cs = p.col_scale[gj];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int lr = 8 * (r >> 2) + 4 * lhi + (r & 3);
+        const int gi = row_b + lr;
+        auto v = acc[r];
+        if (cin != nullptr)
+            v += cin[(long)gi * p.ldc + gj];
+        if (p.relu)
+            v = v > 0 ? v : 0;
+        uint16_t bits;
+        if (KIND == OUT_F16) {
+            bits = f32_to_f16_bits((float)v);
+        } else if (KIND == OUT_BF16) {
+            bits = f32_to_bf16_bits((float)v);
+        } else {
+            const float t = __fmul_rn((float)v, p.row_scale[gi]);
+            bits = f32_to_bf16_bits(__fmul_rn(t, cs));
+        }
+        *reinterpret_cast<uint16_t*>(lane_base + lr * StagedStore<Cfg>::ROW_BYTES) = bits;
+    }
+}
+
+// `stage` is the calling wave's private LDS region of StagedStore<Cfg>::WAVE_BYTES bytes; the wave's tile lies inside
+// the matrix and rows of C start on 16-byte boundaries (checked by the caller)
+template <class Cfg, class Acc>
+__device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0,
+                                              int l32, int lhi, uint8_t* stage)
+{
+    using S = StagedStore<Cfg>;
+    const int lane = lhi * 32 + l32;
+    static_for<Cfg::MB>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        static_for<Cfg::NB>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            __builtin_amdgcn_sched_barrier(0);
+            const Acc block = acc[i][j];
+            uint8_t* lane_base = stage + (j * 32 + l32) * 2;
+            switch (p.out_kind) {
+                case OUT_F16: tstage_block<OUT_F16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base); break;
+                case OUT_BF16: tstage_block<OUT_BF16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base); break;
+                default: tstage_block<OUT_W8A8_BF16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base); break;
+            }
+        });
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int it = 0; it < S::ITERS; ++it) {
+            const int q = it * 64 + lane, row = q / S::CHUNKS, ch = q % S::CHUNKS;
+            const uint4 v = *reinterpret_cast<const uint4*>(stage + row * S::ROW_BYTES + ch * 16);
+            typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
+            nt_u32x4* dst = reinterpret_cast<nt_u32x4*>(reinterpret_cast<uint8_t*>(p.c) + ((long)(row0 + i * 32 + row) * p.ldc + col0 + ch * 8) * 2);
+            const nt_u32x4 vv = {v.x, v.y, v.z, v.w};
+            __builtin_nontemporal_store(vv, dst);  // C is not read again by this kernel: keep it out of the L2's way
+        }
+    });
+}
+
+// `stage`: the wave's private LDS region for the staged form, free of other uses from here on; nullptr = direct stores
 template <class Cfg, class Acc>
 __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0, int l32,
-                                       int lhi)
+                                       int lhi, uint8_t* stage = nullptr)
 {
     const bool full = row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n;
+    const bool two_byte = p.out_kind == OUT_F16 || p.out_kind == OUT_BF16 || (p.out_kind == OUT_W8A8_BF16 && p.acc_out == nullptr);
+    if (stage != nullptr && full && two_byte && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0) {
+        tstore_staged<Cfg>(p, acc, row0, col0, l32, lhi, stage);
+        return;
+    }
     static_for<Cfg::MB * Cfg::NB>([&](auto bc) {
         constexpr int i = decltype(bc)::value / Cfg::NB, j = decltype(bc)::value % Cfg::NB;
         // keep the address arithmetic of one 32x32 block from being hoisted over the others (register pressure)
@@ -387,8 +475,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
         __syncthreads();
     }
 
-    // ---- TSTORE: drain the accumulators through the epilogue
-    tstore<Cfg>(p, acc, m0 + wm * Cfg::WTM, n0 + wn * Cfg::WTN, l32, lhi);
+    // ---- TSTORE: drain the accumulators through the epilogue (the ring is free after the loop's last barrier)
+    tstore<Cfg>(p, acc, m0 + wm * Cfg::WTM, n0 + wn * Cfg::WTN, l32, lhi, smem + wave * StagedStore<Cfg>::WAVE_BYTES);
 }
 
 // One launcher per (tile shape, operand type); defined in gemm_tile_<op>.hip, called from gemm.hip.

@@ -252,8 +252,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     }
     slab(kt, false, false);
 
-    // ---- TSTORE
-    tstore<Cfg>(p, acc, m0 + wm * Cfg::WTM, n0 + wn * Cfg::WTN, l32, lhi);
+    // ---- TSTORE.  No wave reads the ring after the last slab's barrier (its fragment reads were issued before it) and
+    // no DMA is in flight, so each wave may reuse a piece of it for the staged store without another barrier.
+    tstore<Cfg>(p, acc, m0 + wm * Cfg::WTM, n0 + wn * Cfg::WTN, l32, lhi, smem + wave * StagedStore<Cfg>::WAVE_BYTES);
 }
 
 }  // namespace ptoamd
