@@ -205,9 +205,9 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // LDS and need K to be a whole number of 128-byte slabs.  Measured on MI355X: the 8-wave 256x256 DMA tile (4) is the
 // fastest for bf16 / f16 / int8 once the grid fills the chip; the block-scaled operand types keep more registers live
 // per MFMA: fp8 (32-byte fragments) runs best on the 128x128 DMA tile (5), two workgroups per CU; fp4 fits tile 4.
-static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false)
+static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, bool scale_dma_ok = true)
 {
-    const bool dtl_ok = (k_bytes % 128) == 0;
+    const bool dtl_ok = (k_bytes % 128) == 0 && scale_dma_ok;
     const char* env = getenv("PTOAMD_TILE");
     if (env && env[0] >= '0' && env[0] <= '6') {
         const int t = env[0] - '0';
@@ -479,7 +479,10 @@ int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type
         op = b_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E4E5;
     else
         op = b_type == PTOAMD_E5M2 ? TOP_FP8_E5E5 : TOP_FP8_E5E4;
-    const int tile = pick_tile(m, n, k_bytes, true, a4);
+    // the DMA tiles fetch scales as 16-byte chunks per row: 4 slabs of fp8, 2 of fp4
+    const long k_slabs = k_bytes / 128;
+    const bool scale_dma_ok = (kg % 16) == 0 && aligned16(sa_nd) && aligned16(sb_dn) && (k_slabs % (a4 ? 2 : 4)) == 0;
+    const int tile = pick_tile(m, n, k_bytes, true, a4, scale_dma_ok);
     PTOAMD_HIP_CHECK(launch_gemm_tile(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;

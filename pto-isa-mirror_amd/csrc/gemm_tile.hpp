@@ -137,7 +137,10 @@ struct TileCfg {
     static constexpr int SLAB = 128;                              // bytes of K per slab row
     static constexpr int KSTEPS = SLAB / (2 * Op::FRAG_BYTES);
     static constexpr int A_BYTES = BM * SLAB, B_BYTES = BN * SLAB, STAGE_BYTES = A_BYTES + B_BYTES;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+    // the direct-to-LDS kernel of a block-scaled operand type keeps two buffers of 16 scale bytes per tile row behind
+    // the operand ring
+    static constexpr int SCALE_BYTES = Op::SCALED ? 2 * (BM + BN) * 16 : 0;
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES + SCALE_BYTES;
     static constexpr int LA = BM * 8 / THREADS, LB = BN * 8 / THREADS;  // 16-byte chunks per thread per slab
     static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "wave tiles are made of 32x32 blocks");
     static_assert((BM * 8) % THREADS == 0 && (BN * 8) % THREADS == 0, "slab chunks must divide over the workgroup");

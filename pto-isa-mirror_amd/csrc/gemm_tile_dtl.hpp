@@ -101,30 +101,50 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
             tload_piece(kt, buf, q);
     };
 
-    // ---- MX block scales
-    constexpr int SW = Op::SCALED ? Op::GROUPS_PER_SLAB / 4 : 1;
+    // ---- MX block scales.  A lane needs the E8M0 bytes of its own rows, 4 (fp8) or 8 (fp4) per row per slab; fetched
+    // per lane from global memory they are 64 separate small requests per load instruction and keep the CU's address
+    // unit busier than the operand DMAs do.  Instead the 16 scale bytes of every row of the tile -- SPG slabs' worth --
+    // are DMAed into one of two LDS scale buffers, one instruction per 64 rows, and each wave reads the dwords of its
+    // rows from there.  Chunk g + 1 is requested in the last k-step of slab g * SPG and read from the last k-step of
+    // slab (g + 1) * SPG - 1 on, i.e. at least one slab barrier (with its vmcnt(0)) later.
+    constexpr int GPS = Op::SCALED ? Op::GROUPS_PER_SLAB : 4;  // scale bytes per row per slab
+    constexpr int SW = GPS / 4, SPG = 16 / GPS;
+    constexpr int SROWS = BM + BN, NSI = SROWS / 64, NW = NT / 64, NSW = (NSI + NW - 1) / NW;
+    static_assert(SROWS % 64 == 0 && BM % 64 == 0, "one scale DMA covers 64 rows of one operand");
     uint32_t sca[MB][SW], scb[NB][SW], sca_n[MB][SW], scb_n[NB][SW];
-    const uint8_t* gsa[MB];
-    const uint8_t* gsb[NB];
     const bool has_scales = Op::SCALED && p.sa != nullptr;
+    const uint8_t* sc_src[NSW];
+    const uint32_t lds_scales = lds_address(smem) + 2 * Cfg::STAGE_BYTES;
     if (has_scales) {
 #pragma unroll
-        for (int i = 0; i < MB; ++i)
-            gsa[i] = p.sa + (long)min(m0 + wm * Cfg::WTM + i * 32 + l32, p.m - 1) * p.scale_ld;
-#pragma unroll
-        for (int j = 0; j < NB; ++j)
-            gsb[j] = p.sb + (long)min(n0 + wn * Cfg::WTN + j * 32 + l32, p.n - 1) * p.scale_ld;
+        for (int w = 0; w < NSW; ++w) {
+            const int r = (wave + w * NW) * 64 + lane;  // row of [A rows | B rows]; past the end for idle waves (unused)
+            sc_src[w] = r < BM ? p.sa + (long)min(m0 + r, p.m - 1) * p.scale_ld
+                               : p.sb + (long)min(n0 + max(r - BM, 0), p.n - 1) * p.scale_ld;
+        }
     }
-    auto load_scales = [&](int kt) {
+    auto tload_scales = [&](int g) {
         if (has_scales) {
+#pragma unroll
+            for (int w = 0; w < NSW; ++w) {
+                const int i = wave + w * NW;
+                if (i < NSI)
+                    lds_dma16(sc_src[w] + (long)g * 16, lds_scales + (g & 1) * (SROWS * 16) + i * 1024);
+            }
+        }
+    };
+    // slab kt's scales of this lane's rows, LDS -> sca_n / scb_n
+    auto read_scales = [&](int kt) {
+        if (has_scales) {
+            const uint8_t* base = smem + 2 * Cfg::STAGE_BYTES + ((kt / SPG) & 1) * (SROWS * 16) + (kt % SPG) * GPS;
 #pragma unroll
             for (int w = 0; w < SW; ++w) {
 #pragma unroll
                 for (int i = 0; i < MB; ++i)
-                    sca_n[i][w] = *reinterpret_cast<const uint32_t*>(gsa[i] + (long)kt * (SW * 4) + w * 4);
+                    sca_n[i][w] = *reinterpret_cast<const uint32_t*>(base + (wm * Cfg::WTM + i * 32 + l32) * 16 + w * 4);
 #pragma unroll
                 for (int j = 0; j < NB; ++j)
-                    scb_n[j][w] = *reinterpret_cast<const uint32_t*>(gsb[j] + (long)kt * (SW * 4) + w * 4);
+                    scb_n[j][w] = *reinterpret_cast<const uint32_t*>(base + (BM + wn * Cfg::WTN + j * 32 + l32) * 16 + w * 4);
             }
         }
     };
@@ -209,7 +229,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
 
     // ---- prologue: slabs 0 and 1 in flight, first fragments in registers
     tload(0, 0);
-    load_scales(0);
+    tload_scales(0);
     if (k_slabs > 1)
         tload(1, 1);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMAs have landed
@@ -217,6 +237,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
 #pragma unroll
     for (int q = 0; q < NREAD; ++q)
         textract_piece(0, 0, 0, q);
+    read_scales(0);
 
     // One slab.  `more` = slab kt+1 exists (read its first fragments in the last k-step), `dma` = slab kt+2 exists
     // (start its DMA into the buffer this slab frees); both are literal at the call sites so the branches fold.
@@ -232,8 +253,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
                 for (int j = 0; j < NB; ++j)
                     scb[j][w] = scb_n[j][w];
             }
-            if (more)
-                load_scales(kt + 1);
         }
 #pragma unroll
         for (int s = 0; s < KS - 1; ++s)
@@ -241,6 +260,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         // every wave is done reading slab kt, and its DMAs of slab kt+1 (issued one slab ago) have landed
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
+        if (more)
+            read_scales(kt + 1);
+        if (kt % SPG == 0 && (kt / SPG + 1) * SPG < k_slabs)
+            tload_scales(kt / SPG + 1);
         kstep(KS - 1, more, cur ^ 1, 0, dma, kt + 2, cur);
     };
     int kt = 0;
