@@ -158,20 +158,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 acc[i][j][r] = 0;
-    // ---- fragment addressing: byte offset of (row, chunk 0) and the row's swizzle, per 32-row block
-    int fa_off[MB], fb_off[NB], fa_swz[MB], fb_swz[NB];
-#pragma unroll
-    for (int i = 0; i < MB; ++i) {
-        const int r = wm * Cfg::WTM + i * 32 + l32;
-        fa_off[i] = r * 128;
-        fa_swz[i] = swizzle_chunk(r, 0);
-    }
-#pragma unroll
-    for (int j = 0; j < NB; ++j) {
-        const int r = wn * Cfg::WTN + j * 32 + l32;
-        fb_off[j] = Cfg::A_BYTES + r * 128;
-        fb_swz[j] = swizzle_chunk(r, 0);
-    }
+    // ---- fragment addressing.  A lane reads row l32 of every 32-row block of its wave tile; blocks are 32 * 128 bytes
+    // apart and the swizzle depends on row % 16 only, so one lane-constant per operand serves all blocks: the byte
+    // offset of (row, chunk lhi ^ swizzle).  Chunk c = c0 + lhi with c0 even, and (c0 + lhi) ^ swz = c0 ^ (lhi ^ swz),
+    // so the address of chunk c is that constant XOR (c0 << 4): one VALU op per k-step piece, shared by the blocks.
+    static_assert(Cfg::WTM % 32 == 0 && Cfg::WTN % 32 == 0, "wave tiles start on 32-row boundaries");
+    const uint32_t fa_lane = (wm * Cfg::WTM + l32) * 128 + ((lhi ^ swizzle_chunk(l32, 0)) << 4);
+    const uint32_t fb_lane = Cfg::A_BYTES + (wn * Cfg::WTN + l32) * 128 + ((lhi ^ swizzle_chunk(l32, 0)) << 4);
     // Two fragment register sets (next k-step's reads overlap this k-step's MFMAs) unless 32-byte fragments of a
     // large wave tile would not fit the register file next to the accumulators; then one set is refilled piecewise,
     // each block right after the last MFMA that reads it, and the second wave of the SIMD covers the LDS latency.
@@ -184,10 +177,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         const uint8_t* base = smem + buf * Cfg::STAGE_BYTES;
         if (q < NB * FR) {
             const int j = q / FR, f = q % FR;
-            fb[set][j][f] = *reinterpret_cast<const uint4*>(base + fb_off[j] + ((frag_chunk<FR>(s, lhi, f) ^ fb_swz[j]) << 4));
+            fb[set][j][f] = *reinterpret_cast<const uint4*>(base + (fb_lane ^ (frag_chunk<FR>(s, 0, f) << 4)) + j * (32 * 128));
         } else {
             const int i = (q - NB * FR) / FR, f = (q - NB * FR) % FR;
-            fa[set][i][f] = *reinterpret_cast<const uint4*>(base + fa_off[i] + ((frag_chunk<FR>(s, lhi, f) ^ fa_swz[i]) << 4));
+            fa[set][i][f] = *reinterpret_cast<const uint4*>(base + (fa_lane ^ (frag_chunk<FR>(s, 0, f) << 4)) + i * (32 * 128));
         }
     };
     // One k-step: the MFMAs of step s (register set s & 1), with the fragment reads of the next step (register set
