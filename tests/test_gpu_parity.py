@@ -295,6 +295,38 @@ def test_mx_block_scales_select_the_right_group(pa, oracle):
         assert relerr(got, ref) <= 2e-2, g
 
 
+@pytest.mark.parametrize("tile", [3, 4, 5, 6])
+@pytest.mark.parametrize("typ", [ob.E4M3, ob.E2M1])
+def test_mx_scale_chunks_across_slabs(pa, oracle, typ, tile):
+    """The DMA tiles fetch scales as 16-byte chunks per row (4 fp8 slabs / 2 fp4 slabs) into two alternating LDS
+    buffers: a large exponent in the groups either side of every chunk boundary catches a stale or misplaced chunk."""
+    r = np.random.default_rng(40 + tile)
+    m, n, k = 160, 96, 2048  # 64 scale groups per row = 4 chunks
+    a, b, _, _ = _mx_inputs(r, typ, m, n, k)
+    for g in (0, 15, 16, 17, 31, 32, 47, 48, 63):
+        sa = np.full((m, k // 32), 121, np.uint8)
+        sb = np.full((n, k // 32), 122, np.uint8)
+        sa[:, g] = 133
+        sb[1::2, g] = 130
+        sa[m - 1, (g + 5) % 64] = 129  # a row-specific byte: rows must not be swapped either
+        ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, typ, typ)
+        with tile_env(PTOAMD_TILE=tile):
+            got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[typ], PA_T[typ], pa.F32))
+            assert "_dtl_" in pa.last_kernel(), pa.last_kernel()
+        assert relerr(got, ref) <= 2e-2, (g, pa.last_kernel())
+
+
+def test_mx_scale_rows_that_are_not_16_byte_multiples_take_the_register_tiles(pa, oracle):
+    r = np.random.default_rng(41)
+    m, n, k = 130, 70, 640  # 20 scale bytes per row, 5 fp8 slabs
+    a, b, sa, sb = _mx_inputs(r, ob.E4M3, m, n, k)
+    ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ob.E4M3, ob.E4M3)
+    with tile_env(PTOAMD_TILE=5):
+        got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, pa.E4M3, pa.E4M3, pa.F32))
+        assert pa.last_kernel().startswith("tile") and "_dtl_" not in pa.last_kernel(), pa.last_kernel()
+    assert relerr(got, ref) <= 2e-2
+
+
 def test_mx_golden_and_scale_layouts(pa, golden):
     g = golden
     m, k, n = 48, 192, 80
