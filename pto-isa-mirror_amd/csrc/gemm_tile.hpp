@@ -52,6 +52,11 @@ struct OpBF16 {
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]),
                                                     c, 0, 0, 0);
     }
+    template <int SEL>
+    __device__ static __forceinline__ void mma_sel(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        mma(c, a, b, sa, sb);
+    }
 };
 struct OpF16 {
     using Acc = f32x16;
@@ -64,6 +69,11 @@ struct OpF16 {
         c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c,
                                                    0, 0, 0);
     }
+    template <int SEL>
+    __device__ static __forceinline__ void mma_sel(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        mma(c, a, b, sa, sb);
+    }
 };
 struct OpI8 {
     using Acc = i32x16;
@@ -75,6 +85,11 @@ struct OpI8 {
     {
         c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a[0]), __builtin_bit_cast(i32x4, b[0]), c,
                                                   0, 0, 0);
+    }
+    template <int SEL>
+    __device__ static __forceinline__ void mma_sel(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        mma(c, a, b, sa, sb);
     }
 };
 // fp8 (E4M3 = format 0, E5M2 = format 1) through the block-scaled MFMA; each lane's 32 bytes are one MX group.
@@ -95,6 +110,17 @@ struct OpFP8 {
         bv.s4 = b[1].x; bv.s5 = b[1].y; bv.s6 = b[1].z; bv.s7 = b[1].w;
         c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, AFMT, BFMT, 0, (int)sa, 0, (int)sb);
     }
+    // the scales are byte SEL of the dwords sa / sb (the instruction's own byte select: no VALU extraction)
+    template <int SEL>
+    __device__ static __forceinline__ void mma_sel(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        i32x8 av, bv;
+        av.s0 = a[0].x; av.s1 = a[0].y; av.s2 = a[0].z; av.s3 = a[0].w;
+        av.s4 = a[1].x; av.s5 = a[1].y; av.s6 = a[1].z; av.s7 = a[1].w;
+        bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
+        bv.s4 = b[1].x; bv.s5 = b[1].y; bv.s6 = b[1].z; bv.s7 = b[1].w;
+        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, AFMT, BFMT, SEL, (int)sa, SEL, (int)sb);
+    }
 };
 // fp4 E2M1 (format 4): 32 elements = 16 bytes per lane = one MX group
 struct OpFP4 {
@@ -109,6 +135,14 @@ struct OpFP4 {
         av.s0 = a[0].x; av.s1 = a[0].y; av.s2 = a[0].z; av.s3 = a[0].w;
         bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
         c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 4, 4, 0, (int)sa, 0, (int)sb);
+    }
+    template <int SEL>
+    __device__ static __forceinline__ void mma_sel(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        i32x8 av = {0, 0, 0, 0, 0, 0, 0, 0}, bv = {0, 0, 0, 0, 0, 0, 0, 0};
+        av.s0 = a[0].x; av.s1 = a[0].y; av.s2 = a[0].z; av.s3 = a[0].w;
+        bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
+        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 4, 4, SEL, (int)sa, SEL, (int)sb);
     }
 };
 

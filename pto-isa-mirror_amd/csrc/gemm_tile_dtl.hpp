@@ -57,7 +57,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     static_assert((NT / 8) % 16 == 0, "the swizzle of a lane's row must not depend on the piece index");
     extern __shared__ __align__(16) uint8_t smem[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps the tile bookkeeping in scalar registers
     const int wm = wave % Cfg::WAVES_M, wn = wave / Cfg::WAVES_M;
     const int l32 = lane & 31, lhi = lane >> 5;
 
@@ -113,6 +114,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     static_assert(SROWS % 64 == 0 && BM % 64 == 0, "one scale DMA covers 64 rows of one operand");
     uint32_t sca[MB][SW], scb[NB][SW], sca_n[MB][SW], scb_n[NB][SW];
     const bool has_scales = Op::SCALED && p.sa != nullptr;
+#pragma unroll
+    for (int w = 0; w < SW; ++w) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+            sca_n[i][w] = 0x7F7F7F7Fu;
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+            scb_n[j][w] = 0x7F7F7F7Fu;
+    }
     const uint8_t* sc_src[NSW];
     const uint32_t lds_scales = lds_address(smem) + 2 * Cfg::STAGE_BYTES;
     if (has_scales) {
@@ -168,7 +178,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // Two fragment register sets (next k-step's reads overlap this k-step's MFMAs) unless 32-byte fragments of a
     // large wave tile would not fit the register file next to the accumulators; then one set is refilled piecewise,
     // each block right after the last MFMA that reads it, and the second wave of the SIMD covers the LDS latency.
-    constexpr int SETS = (FR == 2 && MB * NB >= 8) ? 1 : 2;
+    constexpr int SETS = ((FR == 2 && MB * NB >= 8) || NT > 512) ? 1 : 2;  // 16 waves: 128 registers per lane
     uint4 fa[SETS][MB][FR], fb[SETS][NB][FR];
     constexpr int NREAD = (MB + NB) * FR, NMMA = MB * NB, NDMA = LA + LB;
     // fragment read number q of k-step s of ring buffer buf into register set `set`; B fragments come first because the
@@ -191,20 +201,21 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         static_for<NMMA>([&](auto xc) {
             constexpr int x = decltype(xc)::value;
             constexpr int i = x / NB, j = x % NB;
-            uint32_t xa = 127u, xb = 127u;
-            if (has_scales) {
-                // MX group 2 s + lhi of the slab: its dword is (2 s + lhi) >> 2 == s >> 1 for either lane half, which
-                // keeps the register-array index a compile-time constant
-                const int g = 2 * s + lhi;
-                xa = (sca[i][s >> 1] >> ((g & 3) * 8)) & 0xFFu;
-                xb = (scb[j][s >> 1] >> ((g & 3) * 8)) & 0xFFu;
-            }
-            Op::mma(acc[i][j], fa[set][i], fb[set][j], xa, xb);
+            // MX group 2 s + lhi of the slab lives in dword s >> 1 (either lane half) at byte 2 (s & 1) + lhi; the
+            // dwords were shifted right by 8 lhi when the slab started, so both halves select byte 2 (s & 1) and the
+            // instruction's own byte select does the extraction.  Without scale arrays every byte is E8M0 127.
+            if (s & 1)
+                Op::template mma_sel<2>(acc[i][j], fa[set][i], fb[set][j], sca[i][s >> 1], scb[j][s >> 1]);
+            else
+                Op::template mma_sel<0>(acc[i][j], fa[set][i], fb[set][j], sca[i][s >> 1], scb[j][s >> 1]);
             if (reads) {
                 if constexpr (SETS == 2) {
                     constexpr int q0 = x * NREAD / NMMA, q1 = (x + 1) * NREAD / NMMA;
                     static_for<q1 - q0>([&](auto qc) { textract_piece(nset, rbuf, rs, q0 + decltype(qc)::value); });
                 } else {
+                    // keep the refill behind the MFMA that frees the registers: hoisted above it, the reads would need a
+                    // second set of fragment registers after all
+                    __builtin_amdgcn_sched_barrier(0);
                     if constexpr (j == NB - 1)  // row i of A is free once its last MFMA has issued
                         static_for<FR>([&](auto fc) { textract_piece(0, rbuf, rs, NB * FR + i * FR + decltype(fc)::value); });
                     if constexpr (x == NMMA - 1)  // B is free after the last MFMA
@@ -236,15 +247,15 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // (start its DMA into the buffer this slab frees); both are literal at the call sites so the branches fold.
     auto slab = [&](int kt, bool more, bool dma) {
         const int cur = kt & 1;
-        if (has_scales) {
+        if (Op::SCALED) {
 #pragma unroll
             for (int w = 0; w < SW; ++w) {
 #pragma unroll
                 for (int i = 0; i < MB; ++i)
-                    sca[i][w] = sca_n[i][w];
+                    sca[i][w] = sca_n[i][w] >> (8 * lhi);
 #pragma unroll
                 for (int j = 0; j < NB; ++j)
-                    scb[j][w] = scb_n[j][w];
+                    scb[j][w] = scb_n[j][w] >> (8 * lhi);
             }
         }
 #pragma unroll
