@@ -203,8 +203,8 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // PTOAMD_FORCE_GENERIC=1 sends everything to the order-exact kernel (used by the parity tests).
 // Tiles 0-2 stage slabs through registers (any K that is a multiple of 16 bytes); tiles 3-6 DMA slabs straight into
 // LDS and need K to be a whole number of 128-byte slabs.  Measured on MI355X: the 8-wave 256x256 DMA tile (4) is the
-// fastest for bf16 / f16 / int8 once the grid fills the chip; the block-scaled operand types keep more registers live
-// per MFMA: fp8 (32-byte fragments) runs best on the 128x128 DMA tile (5), two workgroups per CU; fp4 fits tile 4.
+// fastest for every operand type once the grid fills the chip (the block-scaled types included: their scales come
+// through LDS, which leaves the 32-byte fp8 fragments just enough registers); smaller grids take the 128x128 DMA tile.
 static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, bool scale_dma_ok = true)
 {
     const bool dtl_ok = (k_bytes % 128) == 0 && scale_dma_ok;
@@ -217,8 +217,8 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
     }
     const long t256 = (long)((m + 255) / 256) * ((n + 255) / 256);
     const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128);
-    if (scaled && fp4 && dtl_ok && t256 >= 128)
-        return 4;  // 16-byte fragments: the 8-wave 256x256 tile fits the register file (2.5 vs 2.3 PFLOP/s at 4096x8192x8192)
+    if (scaled && dtl_ok && t256 >= 128)
+        return 4;  // half the copy-in bytes per MFMA of the 128x128 tile: fp8 2.03 vs 1.84, fp4 2.5 vs 2.3 PFLOP/s
     if (scaled)
         return t128 >= 96 ? (dtl_ok ? 5 : 1) : 2;
     if (t256 >= 128)

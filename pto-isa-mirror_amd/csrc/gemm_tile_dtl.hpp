@@ -92,9 +92,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     auto tload_piece = [&](int kt, int buf, int q) {
         const uint32_t dst = lds_wave_base + buf * Cfg::STAGE_BYTES;
         if (q < LA)
-            lds_dma16(p.a + goff_a[q] + (long)kt * 128, dst + q * (NT * 16));
+            lds_dma16_off(p.a + (long)kt * 128, goff_a[q], dst + q * (NT * 16));
         else
-            lds_dma16(p.b + goff_b[q - LA] + (long)kt * 128, dst + Cfg::A_BYTES + (q - LA) * (NT * 16));
+            lds_dma16_off(p.b + (long)kt * 128, goff_b[q - LA], dst + Cfg::A_BYTES + (q - LA) * (NT * 16));
     };
     auto tload = [&](int kt, int buf) {
 #pragma unroll
@@ -112,6 +112,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     constexpr int SW = GPS / 4, SPG = 16 / GPS;
     constexpr int SROWS = BM + BN, NSI = SROWS / 64, NW = NT / 64, NSW = (NSI + NW - 1) / NW;
     static_assert(SROWS % 64 == 0 && BM % 64 == 0, "one scale DMA covers 64 rows of one operand");
+    // The scale dwords of slab kt + 1 are read one k-step ahead, except where 32-byte fragments of a large wave tile
+    // leave no registers for the second copy: there they are read when the slab starts and the SIMD's other wave
+    // covers the LDS latency.
+    constexpr bool SC_AHEAD = !(Op::FRAG_BYTES == 32 && MB * NB >= 8);
     uint32_t sca[MB][SW], scb[NB][SW], sca_n[MB][SW], scb_n[NB][SW];
     const bool has_scales = Op::SCALED && p.sa != nullptr;
 #pragma unroll
@@ -248,6 +252,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     auto slab = [&](int kt, bool more, bool dma) {
         const int cur = kt & 1;
         if (Op::SCALED) {
+            if constexpr (!SC_AHEAD)
+                read_scales(kt);
 #pragma unroll
             for (int w = 0; w < SW; ++w) {
 #pragma unroll
@@ -264,7 +270,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         // every wave is done reading slab kt, and its DMAs of slab kt+1 (issued one slab ago) have landed
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
-        if (more)
+        if (SC_AHEAD && more)
             read_scales(kt + 1);
         if (kt % SPG == 0 && (kt / SPG + 1) * SPG < k_slabs)
             tload_scales(kt / SPG + 1);

@@ -364,7 +364,7 @@ def test_config4_mxfp8_full_size(pa, oracle):
     a, sa = pa.tquant_mx(xa, pa.OCP_MXFP8, want_aux=False)
     b, sb = pa.tquant_mx(xb, pa.OCP_MXFP8, want_aux=False)
     out = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E4M3, pa.E4M3, pa.BF16)
-    assert pa.last_kernel() == "tile128x128_dtl_fp8_e4m3_e4m3"
+    assert pa.last_kernel() == "tile256x256w8_dtl_fp8_e4m3_e4m3"
     rows = np.array([0, 255, 256, 2049, 4095])
     cols = np.arange(0, n, 449)
     ref = oracle.matmul_mx(host(sel(a, rows)), host(sel(b, cols)), host(sel(sa, rows)), host(sel(sb, cols)), len(rows), k, len(cols),
