@@ -228,6 +228,44 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
     return 2;
 }
 
+// Launch on the chosen tile.  When the 256x256 grid is some whole rounds of the 256 CUs plus a mostly empty last one,
+// the columns of that last round run as 128x128 tiles (two workgroups per CU) in a second launch on the same stream:
+// a tile of the tail then costs about a quarter of a 256x256 tile's time instead of a whole round.
+// PTOAMD_TILE (an explicit tile) and PTOAMD_NO_TAIL_SPLIT=1 switch the split off.
+static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStream_t stream)
+{
+    if (tile == 4 && getenv("PTOAMD_TILE") == nullptr && getenv("PTOAMD_NO_TAIL_SPLIT") == nullptr) {
+        const int tiles_m = (p.m + 255) / 256, tiles_n = (p.n + 255) / 256;
+        int whole = tiles_n;  // tile columns that make whole rounds
+        while (whole > 0 && ((long)tiles_m * whole) % 256 != 0)
+            --whole;
+        const long tail_tiles = (long)tiles_m * (tiles_n - whole);
+        if (whole > 0 && whole < tiles_n && tail_tiles <= 160) {
+            const int n1 = whole * 256;
+            TileGemmParams head = p;
+            head.n = n1;
+            const hipError_t e = launch_gemm_tile(4, op, head, stream);
+            if (e != hipSuccess)
+                return e;
+            TileGemmParams tail = p;
+            const size_t esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : 2;
+            tail.n = p.n - n1;
+            tail.b = p.b + (long)n1 * p.ldb_bytes;
+            tail.c = static_cast<uint8_t*>(p.c) + (size_t)n1 * esz;
+            if (p.c_in)
+                tail.c_in = static_cast<const uint8_t*>(p.c_in) + (size_t)n1 * 4;
+            if (p.acc_out)
+                tail.acc_out = p.acc_out + n1;
+            if (p.sb)
+                tail.sb = p.sb + (long)n1 * p.scale_ld;
+            if (p.col_scale)
+                tail.col_scale = p.col_scale + n1;
+            return launch_gemm_tile(5, op, tail, stream);
+        }
+    }
+    return launch_gemm_tile(tile, op, p, stream);
+}
+
 static bool force_generic()
 {
     const char* env = getenv("PTOAMD_FORCE_GENERIC");
@@ -358,7 +396,7 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
                    : ab_type == PTOAMD_I8 ? TOP_I8
                    : ab_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E5E5;
     const int tile = pick_tile(m, n, k_bytes, false);
-    PTOAMD_HIP_CHECK(launch_gemm_tile(tile, op, p, stream));
+    PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;
 }
@@ -401,7 +439,7 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
     p.m = m; p.n = n; p.k_bytes = k; p.lda_bytes = lda; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
     p.out_kind = OUT_W8A8_BF16; p.group_m = 4;
     const int tile = pick_tile(m, n, k, false);
-    PTOAMD_HIP_CHECK(launch_gemm_tile(tile, TOP_I8, p, stream));
+    PTOAMD_HIP_CHECK(launch_tiles(tile, TOP_I8, p, stream));
     set_last_kernel(tile_kernel_name(tile, TOP_I8));
     return PTOAMD_OK;
 }
@@ -483,7 +521,7 @@ int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type
     const long k_slabs = k_bytes / 128;
     const bool scale_dma_ok = (kg % 16) == 0 && aligned16(sa_nd) && aligned16(sb_dn) && (k_slabs % (a4 ? 2 : 4)) == 0;
     const int tile = pick_tile(m, n, k_bytes, true, a4, scale_dma_ok);
-    PTOAMD_HIP_CHECK(launch_gemm_tile(tile, op, p, stream));
+    PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;
 }

@@ -243,6 +243,39 @@ def test_config3_w8a8_full_size(pa, oracle):
     assert torch.equal(acc[:64].to(torch.int64).sum(1), want)
 
 
+def test_tail_round_runs_as_a_second_launch(pa, oracle):
+    """16 x 17 tiles of 256 x 256 are one whole round of the chip plus 16 tiles: the last tile column runs as 128 x 128
+    tiles in a second launch.  Every pointer that moves with the column offset (B, C, per-column scales, raw
+    accumulators, MX scales) is checked on both sides of the seam, with a ragged last tile."""
+    r = np.random.default_rng(77)
+    m, n, k = 4096, 17 * 256 - 40, 128
+    rows = np.array([0, 255, 256, 2049, 4095])
+    cols = np.concatenate([np.arange(0, n, 331), np.arange(4090, 4110), [n - 1]])
+    a8 = r.integers(-127, 128, (m, k)).astype(np.int8)
+    b8 = r.integers(-127, 128, (n, k)).astype(np.int8)
+    sa = (r.random(m) * 0.01 + 0.001).astype(np.float32)
+    sb = (r.random(n) * 0.01 + 0.001).astype(np.float32)
+    out, acc = pa.gemm_w8a8(dev(a8), dev(b8), dev(sa), dev(sb), want_acc=True)
+    assert pa.last_kernel() == "tile256x256w8_dtl_i8"
+    ref_acc, ref_out = _w8a8_reference(oracle, a8[rows], b8[cols], sa[rows], sb[cols])
+    assert np.array_equal(host(acc)[np.ix_(rows, cols)], ref_acc)
+    assert np.array_equal(host(out)[np.ix_(rows, cols)], ref_out)
+    out2 = pa.gemm_w8a8(dev(a8), dev(b8), dev(sa), dev(sb))  # staged 16-bit epilogue (no raw accumulators)
+    out2 = out2[0] if isinstance(out2, tuple) else out2
+    assert np.array_equal(host(out2), host(out))
+    with tile_env(PTOAMD_NO_TAIL_SPLIT="1"):
+        one = pa.gemm_w8a8(dev(a8), dev(b8), dev(sa), dev(sb))
+        one = one[0] if isinstance(one, tuple) else one
+    assert np.array_equal(host(one), host(out))
+    # MX: B scales move with the columns too
+    km = 512
+    a, b, xa, xb = _mx_inputs(r, ob.E4M3, m, n, km)
+    got = pa.gemm_mx(dev(a), dev(b), dev(xa), dev(xb), m, n, km, pa.E4M3, pa.E4M3, pa.F32)
+    assert pa.last_kernel() == "tile256x256w8_dtl_fp8_e4m3_e4m3"
+    ref = oracle.matmul_mx(a[rows], b[cols], xa[rows], xb[cols], len(rows), km, len(cols), ob.E4M3, ob.E4M3)
+    assert relerr(host(got)[np.ix_(rows, cols)], ref) <= 2e-2
+
+
 # ------------------------------------------------------------------------------------------- TMATMUL_MX
 def _mx_inputs(r, typ, m, n, k, spread=8):
     packed = typ in (ob.E2M1, ob.E1M2)
