@@ -161,6 +161,32 @@ PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataExp* exp
     return {};
 }
 
+// MXFP8, NZ store mode: as above, and the exponents once more in exp_zz in the order of 16-row x 2-group boxes (the
+// layout of an MX matmul's left scale tile): box (row / 16, group / 2), then row % 16, then group % 2
+// (reference: cpu/TQuant.hpp:254-278, 585-611)
+template <auto quant_type, auto store_mode, typename TileDataOut, typename TileDataSrc, typename TileDataExp,
+          typename TileDataMax, typename TileDataScaling,
+          typename = std::enable_if_t<std::is_same_v<decltype(store_mode), VecStoreMode>>>
+PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataExp* exp, TileDataMax* max, TileDataScaling* scaling,
+                            TileDataExp* exp_zz)
+{
+    static_assert(quant_type == QuantType::MXFP8, "TQUANT: the NZ store mode is defined for MXFP8");
+    static_assert(store_mode == VecStoreMode::NZ, "TQUANT: this overload is the NZ store mode");
+    amd::tquant_mx<0>(dst, src, exp, max, scaling);
+    const int rows = src.GetValidRow(), groups = src.GetValidCol() / 32;
+    if (exp == nullptr || exp_zz == nullptr || rows % 16 != 0 || groups % 2 != 0) {
+        amd::report(2);  // the reorder needs whole 16 x 2 boxes
+        return {};
+    }
+    for (int i = threadIdx.x; i < rows * groups; i += PTO_AMD_THREADS) {
+        const int r = i / groups, g = i - r * groups;
+        const int zz = ((r / 16) * (groups / 2) + g / 2) * 32 + (r % 16) * 2 + g % 2;
+        *reinterpret_cast<uint8_t*>(exp_zz->Storage() + zz) = *reinterpret_cast<const uint8_t*>(exp->Storage() + i);
+    }
+    __syncthreads();
+    return {};
+}
+
 // MX with an explicit grouping axis (1: along a row, 0: along a column) and the unified algorithm tag
 // (reference: common/pto_instr.hpp:3006-3019, cpu/TQuant.hpp:524-547)
 template <int grp_axis, auto mx_alg, typename TileDataOut, typename TileDataSrc, typename TileDataExp, typename TileDataMax,

@@ -48,7 +48,8 @@ constexpr uint32_t LDS_TOTAL = PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0
 static_assert(LDS_TOTAL <= 160 * 1024, "the on-chip regions must fit the 160 KiB LDS of a CU");
 
 // Sticky status word of the kernels of this translation unit: 0, or the first constraint a core violated
-// (1: TASSIGN address outside its region).  pto::amd::device_status() reads it on the host.
+// (1: TASSIGN address outside its region, 2: TQUANT NZ mode on a tile that is not whole 16-row x 2-group boxes).
+// pto::amd::device_status() reads it on the host.
 static __device__ int g_status = 0;
 __device__ __forceinline__ void report(int code)
 {

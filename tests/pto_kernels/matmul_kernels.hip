@@ -390,6 +390,41 @@ __global__ AICORE void RunTQUANT_MX(__gm__ DstT* dst, __gm__ uint8_t* exp, __gm_
     TSTORE(scalingGlobal, scalingTile);
 }
 
+// NZ store mode: the exponents are written twice, row-major in exp and in 16 x 2 boxes in exp_zz (stored to `max`'s
+// buffer reinterpreted as bytes: the launcher has no separate pointer for it)
+template <typename SrcT, int R, int C>
+__global__ AICORE void RunTQUANT_MX_NZ(__gm__ float8_e4m3_t* dst, __gm__ uint8_t* exp, __gm__ uint8_t* exp_zz, __gm__ float* scaling, __gm__ SrcT* src)
+{
+    constexpr int G = R * C / 32;
+    using SrcTile = Tile<TileType::Vec, SrcT, R, C, BLayout::RowMajor, R, C>;
+    using DstTile = Tile<TileType::Vec, float8_e4m3_t, R, C, BLayout::RowMajor, R, C>;
+    using ExpTile = Tile<TileType::Vec, uint8_t, 1, G, BLayout::RowMajor, 1, G>;
+    using FlatTile = Tile<TileType::Vec, float, 1, G, BLayout::RowMajor, 1, G>;
+    SrcTile srcTile;
+    DstTile dstTile;
+    ExpTile expTile, zzTile;
+    FlatTile maxTile, scalingTile;
+    constexpr int a1 = CeilAlign<int>(SrcTile::Bytes, 32), a2 = a1 + CeilAlign<int>(DstTile::Bytes, 32),
+                  a3 = a2 + CeilAlign<int>(ExpTile::Bytes, 32), a4 = a3 + CeilAlign<int>(ExpTile::Bytes, 32),
+                  a5 = a4 + CeilAlign<int>(FlatTile::Bytes, 32);
+    TASSIGN(srcTile, 0x0);
+    TASSIGN(dstTile, a1);
+    TASSIGN(expTile, a2);
+    TASSIGN(zzTile, a3);
+    TASSIGN(maxTile, a4);
+    TASSIGN(scalingTile, a5);
+    GlobalTensor<SrcT, TileShape2D<SrcT, R, C>, BaseShape2D<SrcT, R, C>> srcGlobal(src);
+    GlobalTensor<float8_e4m3_t, TileShape2D<float8_e4m3_t, R, C>, BaseShape2D<float8_e4m3_t, R, C>> dstGlobal(dst);
+    GlobalTensor<uint8_t, TileShape2D<uint8_t, 1, G>, BaseShape2D<uint8_t, 1, G>> expGlobal(exp), zzGlobal(exp_zz);
+    GlobalTensor<float, TileShape2D<float, 1, G>, BaseShape2D<float, 1, G>> scalingGlobal(scaling);
+    TLOAD(srcTile, srcGlobal);
+    TQUANT<QuantType::MXFP8, VecStoreMode::NZ>(dstTile, srcTile, &expTile, &maxTile, &scalingTile, &zzTile);
+    TSTORE(dstGlobal, dstTile);
+    TSTORE(expGlobal, expTile);
+    TSTORE(zzGlobal, zzTile);
+    TSTORE(scalingGlobal, scalingTile);
+}
+
 // column-grouped form: 32 consecutive rows of one column share an exponent; exp / max / scaling are [R / 32][C]
 template <typename DstT, int R, int C, MxQuantAlg ALG>
 __global__ AICORE void RunTQUANT_MX_DN(__gm__ DstT* dst, __gm__ uint8_t* exp, __gm__ float* max, __gm__ float* scaling, __gm__ float* src)
@@ -474,7 +509,7 @@ __global__ AICORE void RunTDEQUANT(__gm__ float* dst, __gm__ SrcT* src, __gm__ f
 }
 
 // quant cases: 1-4: f32 16x64 -> OCP-FP8, NV-FP8, OCP-FP4, NV-FP4     5: bf16 8x128 -> OCP-FP4     6: half 8x128 -> OCP-FP8
-//              7, 8: f32 64x16 grouped along columns -> OCP-FP8, NV-FP4
+//              7, 8: f32 64x16 grouped along columns -> OCP-FP8, NV-FP4     9: half 16x128 -> OCP-FP8, NZ store mode
 //              10: INT8 sym 16x64   11: INT8 asym 16x64    20: TDEQUANT int8 16x64    21: TDEQUANT int32 8x32
 extern "C" int pto_kernels_launch_quant(int id, void* dst, void* exp, void* max, void* scaling, void* src, void* scale, void* offset, void* stream)
 {
@@ -489,6 +524,7 @@ extern "C" int pto_kernels_launch_quant(int id, void* dst, void* exp, void* max,
     case 6: return run<&RunTQUANT_MX<half, F8, 8, 128, QuantType::MXFP8, QuantScaleAlg::OCP>>(stream, 1, (F8*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (half*)src);
     case 7: return run<&RunTQUANT_MX_DN<F8, 64, 16, MxQuantAlg::OcpMxFp8E4M3>>(stream, 1, (F8*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (float*)src);
     case 8: return run<&RunTQUANT_MX_DN<F4, 64, 16, MxQuantAlg::NvMxFp4E2M1>>(stream, 1, (F4*)dst, (uint8_t*)exp, (float*)max, (float*)scaling, (float*)src);
+    case 9: return run<&RunTQUANT_MX_NZ<half, 16, 128>>(stream, 1, (F8*)dst, (uint8_t*)exp, (uint8_t*)max, (float*)scaling, (half*)src);
     case 10: return run<&RunTQUANT_INT8<16, 64, false>>(stream, 1, (uint8_t*)dst, (float*)src, (float*)scale, (float*)offset);
     case 11: return run<&RunTQUANT_INT8<16, 64, true>>(stream, 1, (uint8_t*)dst, (float*)src, (float*)scale, (float*)offset);
     case 20: return run<&RunTDEQUANT<int8_t, 16, 64>>(stream, 1, (float*)dst, (int8_t*)src, (float*)scale, (float*)offset);

@@ -287,6 +287,28 @@ def test_tquant_mx_column_groups_bit_exact(kernels, oracle, case, alg):
     assert _eq_f32(mx.cpu().numpy(), rm.ravel()) and _eq_f32(sc.cpu().numpy(), rs.ravel())
 
 
+def test_tquant_mx_nz_store_mode_reorders_exponents(kernels, oracle):
+    """TQUANT<MXFP8, VecStoreMode::NZ>: codes and row-major exponents as in ND mode, plus the exponents in 16-row x
+    2-group boxes (reference: cpu/TQuant.hpp:254-278 ReorderExponentZZ)."""
+    rows, cols = 16, 128
+    r = np.random.default_rng(9)
+    x = (r.standard_normal((rows, cols)) * 10 ** r.uniform(-2, 2, (rows, cols // 32)).repeat(32, axis=1)).astype(np.float16)
+    g = rows * cols // 32
+    dst = torch.zeros(rows * cols, dtype=torch.uint8, device=DEV)
+    exp = torch.zeros(g, dtype=torch.uint8, device=DEV)
+    zz = torch.zeros(g, dtype=torch.float32, device=DEV)  # the launcher's `max` slot carries exp_zz's bytes here
+    sc = torch.zeros(g, dtype=torch.float32, device=DEV)
+    _quant_launch(kernels, 9, dst, exp, zz, sc, torch.from_numpy(x).to(DEV))
+    rc, re, _, rs = oracle.tquant_mx(x.astype(np.float32), ob.OCP_FP8, 1, ob.SRC_F16)
+    assert np.array_equal(dst.cpu().numpy(), rc.ravel())
+    assert np.array_equal(exp.cpu().numpy(), re.ravel())
+    assert _eq_f32(sc.cpu().numpy(), rs.ravel())
+    gc = cols // 32
+    want = re.reshape(rows // 16, 16, gc // 2, 2).transpose(0, 2, 1, 3).ravel()
+    assert len(set(re.ravel().tolist())) > 4  # the permutation is visible in the data
+    assert np.array_equal(zz.cpu().numpy().view(np.uint8)[:g], want)
+
+
 def test_tquant_int8_and_tdequant_tile_instructions_bit_exact(kernels, oracle):
     r = np.random.default_rng(21)
     src = (r.standard_normal((16, 64)) * 60).astype(np.float32)
