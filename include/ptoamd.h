@@ -118,6 +118,15 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
                 int lda, int ldb, int ldc, int b_layout, int relu, void* stream);
 
 /*
+ * The same pipeline with TMATMUL_BIAS: C = A * B (+ Cin) + bias, the bias row added to every row of C after the K loop
+ * and before TSTORE's relu / conversion.
+ * reference: include/pto/cpu/TMatmul.hpp:219-230 (TMATMUL_BIAS_IMPL), common/pto_instr.hpp (TMATMUL_BIAS).
+ *   bias    : [N] of the accumulator type (f32 for float inputs, i32 for int8); NULL = ptoamd_gemm
+ */
+int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
+                     int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream);
+
+/*
  * W8A8: int8 x int8 -> int32 accumulate, then the dequantising drain fused in registers:
  *   out(i, j) = bf16( (float(acc(i, j)) * scale_a[i]) * scale_b[j] )
  * i.e. TMATMUL (cpu/TMatmul.hpp:106) -> TDEQUANT with offset 0 (cpu/TDeQuant.hpp:31-34) -> per-column multiply

@@ -39,7 +39,7 @@ EXPORTS = [
     "ptoamd_malloc_host", "ptoamd_free_host", "ptoamd_memcpy", "ptoamd_memcpy_async", "ptoamd_memset",
     "ptoamd_stream_create", "ptoamd_stream_destroy", "ptoamd_stream_synchronize", "ptoamd_event_create",
     "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
-    "ptoamd_gemm", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
+    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
     "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_mx_scale_relayout", "ptoamd_last_kernel",
 ]
 
@@ -76,13 +76,20 @@ def _stream(stream):
 _TORCH_OUT = {F32: torch.float32, F16: torch.float16, BF16: torch.bfloat16, I32: torch.int32}
 
 
-def gemm(a, b, ab_type, c_type=F32, b_layout=B_DN, c_in=None, relu=False, m=None, n=None, k=None, stream=None, out=None):
-    """TLOAD -> TMATMUL / TMATMUL_ACC -> TSTORE.  a: [m, k]; b: [n, k] (B_DN) or [k, n] (B_ND), raw-typed tensors."""
+def gemm(a, b, ab_type, c_type=F32, b_layout=B_DN, c_in=None, relu=False, m=None, n=None, k=None, stream=None, out=None,
+         bias=None):
+    """TLOAD -> TMATMUL / TMATMUL_ACC / TMATMUL_BIAS -> TSTORE.  a: [m, k]; b: [n, k] (B_DN) or [k, n] (B_ND), raw-typed
+    tensors; bias: [n] of the accumulator type."""
     m = a.shape[0] if m is None else m
     k = a.shape[1] if k is None else k
     n = (b.shape[0] if b_layout == B_DN else b.shape[1]) if n is None else n
     if out is None:
         out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
+    if bias is not None:
+        _check(_lib.ptoamd_gemm_bias(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), _ptr(bias), m, n, k,
+                                     a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu), _stream(stream)),
+               "ptoamd_gemm_bias")
+        return out
     _check(_lib.ptoamd_gemm(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), m, n, k, a.stride(0), b.stride(0),
                             out.stride(0), b_layout, int(relu), _stream(stream)), "ptoamd_gemm")
     return out

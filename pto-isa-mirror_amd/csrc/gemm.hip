@@ -93,6 +93,7 @@ struct GenericParams {
     const void* b;
     void* c;
     const void* c_in;
+    const void* bias;  // [n] of the accumulator type, added after the K loop (TMATMUL_BIAS)
     int32_t* acc_out;
     const uint8_t* sa;
     const uint8_t* sb;
@@ -145,6 +146,8 @@ __global__ void gemm_generic_kernel(const GenericParams p)
         const int8_t* b = reinterpret_cast<const int8_t*>(p.b) + (long)gj * p.sbn;
         for (int kk = 0; kk < p.k; ++kk)
             acc += (uint32_t)((int32_t)a[kk] * (int32_t)b[(long)kk * p.sbk]);
+        if (p.bias)
+            acc += (uint32_t) reinterpret_cast<const int32_t*>(p.bias)[gj];
         int32_t v = (int32_t)acc;
         if (p.relu)
             v = v > 0 ? v : 0;
@@ -175,6 +178,8 @@ __global__ void gemm_generic_kernel(const GenericParams p)
             acc = (float)((double)acc + av * bv * sf);  // double add, then one rounding to float per k
         }
     }
+    if (p.bias)
+        acc = __fadd_rn(acc, reinterpret_cast<const float*>(p.bias)[gj]);
     store_out(p, o, acc, gi, gj);
 }
 
@@ -254,6 +259,8 @@ static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStr
             tail.c = static_cast<uint8_t*>(p.c) + (size_t)n1 * esz;
             if (p.c_in)
                 tail.c_in = static_cast<const uint8_t*>(p.c_in) + (size_t)n1 * 4;
+            if (p.bias)
+                tail.bias = static_cast<const uint8_t*>(p.bias) + (size_t)n1 * 4;
             if (p.acc_out)
                 tail.acc_out = p.acc_out + n1;
             if (p.sb)
@@ -338,6 +345,12 @@ int ptoamd_mx_scale_relayout(uint8_t* dst, int dst_layout, const uint8_t* src, i
 int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, int m, int n, int k,
                 int lda, int ldb, int ldc, int b_layout, int relu, void* stream_)
 {
+    return ptoamd_gemm_bias(c, c_type, a, b, ab_type, c_in, nullptr, m, n, k, lda, ldb, ldc, b_layout, relu, stream_);
+}
+
+int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
+                     int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream_)
+{
     hipStream_t stream = as_stream(stream_);
     PTOAMD_REQUIRE(c && a && b, PTOAMD_E_INVALID, "ptoamd_gemm: null operand");
     PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemm: m, n, k must be positive (%d, %d, %d)", m, n, k);
@@ -365,7 +378,7 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
                          (b_layout == PTOAMD_B_DN ? (ldb_b % 16) == 0 : true);
     if (!tile_ok) {
         GenericParams g{};
-        g.a = a; g.b = b; g.c = c; g.c_in = c_in;
+        g.a = a; g.b = b; g.c = c; g.c_in = c_in; g.bias = bias;
         g.m = m; g.n = n; g.k = k; g.lda = lda; g.ldc = ldc;
         g.sbk = b_layout == PTOAMD_B_DN ? 1 : ldb;
         g.sbn = b_layout == PTOAMD_B_DN ? ldb : 1;
@@ -387,7 +400,7 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
     TileGemmParams p{};
     p.a = reinterpret_cast<const uint8_t*>(a);
     p.b = b_kmajor;
-    p.c = c; p.c_in = c_in;
+    p.c = c; p.c_in = c_in; p.bias = bias;
     p.m = m; p.n = n; p.k_bytes = (int)k_bytes;
     p.lda_bytes = lda_b; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
     p.relu = relu; p.out_kind = out_kind; p.group_m = 4;

@@ -21,6 +21,7 @@ struct TileGemmParams {
     const uint8_t* b;       // [n][ldb_bytes]
     void* c;                // [m][ldc] of the output type
     const void* c_in;       // optional accumulator input, [m][ldc] f32 / i32
+    const void* bias;       // optional TMATMUL_BIAS row, [n] f32 / i32, added to every row after the K loop
     int32_t* acc_out;       // optional raw int32 accumulators (W8A8), [m][ldc]
     const uint8_t* sa;      // MX: [m][k/32] E8M0
     const uint8_t* sb;      // MX: [n][k/32] E8M0
@@ -195,6 +196,7 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
     float cs = 1.0f;
     if (KIND == OUT_W8A8_BF16)
         cs = (FULL || gj < p.n) ? p.col_scale[gj] : 0.0f;
+    const Elem bias_j = (p.bias != nullptr && (FULL || gj < p.n)) ? reinterpret_cast<const Elem*>(p.bias)[gj] : Elem(0);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int gi = row_b + 8 * (r >> 2) + 4 * lhi + (r & 3);
@@ -203,6 +205,7 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
             auto v = acc[r];
             if (cin != nullptr)
                 v += cin[o];
+            v += bias_j;
             if (p.relu)
                 v = v > 0 ? v : 0;
             if (KIND == OUT_F32) {
@@ -261,6 +264,7 @@ __device__ __forceinline__ void tstage_block(const TileGemmParams& p, const Acc&
     float cs = 1.0f;
     if (KIND == OUT_W8A8_BF16)
         cs = p.col_scale[gj];
+    const Elem bias_j = p.bias != nullptr ? reinterpret_cast<const Elem*>(p.bias)[gj] : Elem(0);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int lr = 8 * (r >> 2) + 4 * lhi + (r & 3);
@@ -268,6 +272,7 @@ __device__ __forceinline__ void tstage_block(const TileGemmParams& p, const Acc&
         auto v = acc[r];
         if (cin != nullptr)
             v += cin[(long)gi * p.ldc + gj];
+        v += bias_j;
         if (p.relu)
             v = v > 0 ? v : 0;
         uint16_t bits;

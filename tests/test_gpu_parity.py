@@ -243,6 +243,36 @@ def test_config3_w8a8_full_size(pa, oracle):
     assert torch.equal(acc[:64].to(torch.int64).sum(1), want)
 
 
+@pytest.mark.parametrize("tile", [2, 4, 5])
+def test_tmatmul_bias(pa, oracle, tile):
+    """TMATMUL_BIAS: the bias row is added to every row after the K loop, before relu and the TSTORE conversion
+    (reference: cpu/TMatmul.hpp:219-230); with TMATMUL_ACC input as well; int8 with an int32 bias bit-exact."""
+    r = np.random.default_rng(60 + tile)
+    m, n, k = 200, 328, 256
+    a = bf16_bits(r.standard_normal((m, k)) * 0.05)
+    b = bf16_bits(r.standard_normal((n, k)) * 0.05)
+    bias = (r.standard_normal(n) * 0.5).astype(np.float32)
+    cin = r.standard_normal((m, n)).astype(np.float32)
+    ref = oracle.matmul_bf16(a, b, cin=cin, bias=bias, b_dn=True)
+    with tile_env(PTOAMD_TILE=tile):
+        got = host(pa.gemm(dev(a), dev(b), pa.BF16, pa.F32, pa.B_DN, c_in=dev(cin), bias=dev(bias)))
+        assert pa.last_kernel().startswith("tile")
+        got16 = host(pa.gemm(dev(a), dev(b), pa.BF16, pa.BF16, pa.B_DN, bias=dev(bias), relu=True))
+    assert relerr(got, ref) <= 1e-2
+    ref16 = np.maximum(oracle.matmul_bf16(a, b, bias=bias, b_dn=True), 0)
+    assert relerr(bf16_to_f32(got16), ref16) <= 1e-2
+    assert (bf16_to_f32(got16) >= 0).all() and (ref16 == 0).any()
+    with tile_env(PTOAMD_FORCE_GENERIC=1):
+        exact = host(pa.gemm(dev(a), dev(b), pa.BF16, pa.F32, pa.B_DN, c_in=dev(cin), bias=dev(bias)))
+    assert np.array_equal(exact.view(np.uint32), ref.view(np.uint32))
+    a8 = r.integers(-128, 128, (m, k)).astype(np.int8)
+    b8 = r.integers(-128, 128, (n, k)).astype(np.int8)
+    bias32 = r.integers(-2 ** 30, 2 ** 30, n).astype(np.int32)
+    with tile_env(PTOAMD_TILE=tile):
+        acc = host(pa.gemm(dev(a8), dev(b8), pa.I8, pa.I32, pa.B_DN, bias=dev(bias32)))
+    assert np.array_equal(acc, oracle.matmul_i8(a8, b8, bias=bias32, b_dn=True))
+
+
 def test_tail_round_runs_as_a_second_launch(pa, oracle):
     """16 x 17 tiles of 256 x 256 are one whole round of the chip plus 16 tiles: the last tile column runs as 128 x 128
     tiles in a second launch.  Every pointer that moves with the column offset (B, C, per-column scales, raw
