@@ -297,6 +297,15 @@ def test_tail_round_runs_as_a_second_launch(pa, oracle):
         one = pa.gemm_w8a8(dev(a8), dev(b8), dev(sa), dev(sb))
         one = one[0] if isinstance(one, tuple) else one
     assert np.array_equal(host(one), host(out))
+    # TMATMUL_ACC input and the bias row move with the columns as well (f32 output: 4-byte column offset)
+    ab = bf16_bits(r.standard_normal((m, k)) * 0.05)
+    bb = bf16_bits(r.standard_normal((n, k)) * 0.05)
+    cin = r.standard_normal((m, n)).astype(np.float32)
+    bias = r.standard_normal(n).astype(np.float32)
+    got = host(pa.gemm(dev(ab), dev(bb), pa.BF16, pa.F32, pa.B_DN, c_in=dev(cin), bias=dev(bias)))
+    assert pa.last_kernel() == "tile256x256w8_dtl_bf16"
+    ref = oracle.matmul_bf16(ab[rows], bb[cols], cin=np.ascontiguousarray(cin[np.ix_(rows, cols)]), bias=bias[cols], b_dn=True)
+    assert relerr(got[np.ix_(rows, cols)], ref) <= 1e-2
     # MX: B scales move with the columns too
     km = 512
     a, b, xa, xb = _mx_inputs(r, ob.E4M3, m, n, km)
