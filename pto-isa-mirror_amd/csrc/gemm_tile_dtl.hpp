@@ -46,6 +46,30 @@ __device__ __forceinline__ void sched_kstep()
     SchedKStep<0, NM, ND, NV>::run();
 }
 
+// DMA issue plan.  A slab's copy-in can start only when the barrier before the last k-step of slab kt has freed the
+// buffer, and must have landed by the same barrier of slab kt + 1.  Issuing all of it in that one k-step makes a burst
+// the CU's 64 B/clk global -> LDS path cannot absorb (64 one-KiB DMAs need ~1000 clocks, twice the k-step), and the
+// MFMAs queued behind the stalled DMA instructions wait.  So a share of the pieces is held back for the first k-step
+// of the following slab: measured on the bf16 4096^3 GEMM, (8) 112.7 us, (6, 2) and (4, 4) 110.7 us (int8 alike),
+// anything issued later than that first k-step loses again (the data has less time to land), and so does any split
+// for the 32-byte-fragment types whose slab has only two k-steps (fp8: 109 -> 112 us), which keep the single phase.  Shares are eighths of the slab's pieces
+// per phase: phase 0 = the last k-step of the slab that frees the buffer, phase f > 0 = k-step f - 1 of the next slab.
+#ifndef PTOAMD_DMA_PHASES
+#define PTOAMD_DMA_PHASES 4, 4
+#endif
+template <int NDMA, int KS>
+__host__ __device__ constexpr int dma_phase_begin(int phase)
+{
+    constexpr int share[] = {PTOAMD_DMA_PHASES};
+    constexpr int n = sizeof(share) / sizeof(share[0]);
+    int eighths = 0;
+    for (int f = 0; f < phase && f < n; ++f)
+        eighths += share[f];
+    if (phase >= n || phase >= KS || (KS < 4 && phase >= 1))  // two k-steps per slab: phase 1 would be the k-step before the barrier
+        eighths = 8;
+    return eighths * NDMA / 8;
+}
+
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileGemmParams p)
 {
@@ -199,7 +223,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     };
     // One k-step: the MFMAs of step s (register set s & 1), with the fragment reads of the next step (register set
     // (s + 1) & 1, from buffer rbuf step rs) and, in a slab's last step, the DMAs of slab dkt spread between them.
-    auto kstep = [&](int s, bool reads, int rbuf, int rs, bool dmas, int dkt, int dbuf) {
+    auto kstep = [&](auto phase, int s, bool reads, int rbuf, int rs, bool dmas, int dkt, int dbuf) {
+        constexpr int DQ0 = dma_phase_begin<NDMA, KS>(decltype(phase)::value), DN = dma_phase_begin<NDMA, KS>(decltype(phase)::value + 1) - DQ0;
         const int set = SETS == 2 ? (s & 1) : 0;
         const int nset = SETS == 2 ? (set ^ 1) : 0;
         static_for<NMMA>([&](auto xc) {
@@ -227,7 +252,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
                 }
             }
             if (dmas) {
-                constexpr int q0 = x * NDMA / NMMA, q1 = (x + 1) * NDMA / NMMA;
+                constexpr int q0 = DQ0 + x * DN / NMMA, q1 = DQ0 + (x + 1) * DN / NMMA;
                 static_for<q1 - q0>([&](auto qc) { tload_piece(dkt, dbuf, q0 + decltype(qc)::value); });
             }
         });
@@ -239,7 +264,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     tload(0, 0);
     tload_scales(0);
     if (k_slabs > 1)
-        tload(1, 1);
+        static_for<dma_phase_begin<NDMA, KS>(1)>([&](auto qc) { tload_piece(1, 1, decltype(qc)::value); });
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMAs have landed
     __syncthreads();
 #pragma unroll
@@ -264,9 +289,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
                     scb[j][w] = scb_n[j][w] >> (8 * lhi);
             }
         }
-#pragma unroll
-        for (int s = 0; s < KS - 1; ++s)
-            kstep(s, true, cur, s + 1, false, 0, 0);
+        static_for<KS - 1>([&](auto sc) {
+            constexpr int s = decltype(sc)::value;
+            kstep(std::integral_constant<int, s + 1>{}, s, true, cur, s + 1, more, kt + 1, cur ^ 1);
+        });
         // every wave is done reading slab kt, and its DMAs of slab kt+1 (issued one slab ago) have landed
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
@@ -274,7 +300,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
             read_scales(kt + 1);
         if (kt % SPG == 0 && (kt / SPG + 1) * SPG < k_slabs)
             tload_scales(kt / SPG + 1);
-        kstep(KS - 1, more, cur ^ 1, 0, dma, kt + 2, cur);
+        kstep(std::integral_constant<int, 0>{}, KS - 1, more, cur ^ 1, 0, dma, kt + 2, cur);
     };
     int kt = 0;
     for (; kt + 2 < k_slabs; ++kt)
