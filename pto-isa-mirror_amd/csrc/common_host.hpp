@@ -10,6 +10,8 @@ namespace ptoamd {
 
 void set_error(const char* fmt, ...);
 void set_last_kernel(const char* name);
+// sets hipFuncAttributeMaxDynamicSharedMemorySize once per (kernel, current device); thread-safe
+hipError_t ensure_dynamic_lds(const void* kernel, int bytes);
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 

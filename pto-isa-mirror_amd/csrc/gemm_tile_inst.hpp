@@ -1,6 +1,7 @@
 // Instantiates gemm_tile_kernel for one operand type at the three tile shapes.  Included by gemm_tile_<op>.hip with
 // PTOAMD_TILE_OP (the traits type) and PTOAMD_TILE_FN (the launcher's name) defined, so the operand types compile in
 // parallel translation units.
+#include "common_host.hpp"
 #include "gemm_tile_dtl.hpp"
 
 namespace ptoamd {
@@ -8,14 +9,9 @@ namespace ptoamd {
 template <class Cfg>
 static hipError_t launch_cfg(const TileGemmParams& p, hipStream_t stream)
 {
-    static bool attr_set = false;  // one kernel symbol per instantiation; the attribute persists per device
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<Cfg>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-        if (e != hipSuccess)
-            return e;
-        attr_set = true;
-    }
+    const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_kernel<Cfg>), Cfg::LDS_BYTES);
+    if (e != hipSuccess)
+        return e;
     const int tiles = ((p.m + Cfg::BM - 1) / Cfg::BM) * ((p.n + Cfg::BN - 1) / Cfg::BN);
     hipLaunchKernelGGL(gemm_tile_kernel<Cfg>, dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
     return hipGetLastError();
@@ -24,14 +20,9 @@ static hipError_t launch_cfg(const TileGemmParams& p, hipStream_t stream)
 template <class Cfg>
 static hipError_t launch_dtl(const TileGemmParams& p, hipStream_t stream)
 {
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_dtl_kernel<Cfg>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-        if (e != hipSuccess)
-            return e;
-        attr_set = true;
-    }
+    const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_dtl_kernel<Cfg>), Cfg::LDS_BYTES);
+    if (e != hipSuccess)
+        return e;
     const int tiles = ((p.m + Cfg::BM - 1) / Cfg::BM) * ((p.n + Cfg::BN - 1) / Cfg::BN);
     hipLaunchKernelGGL(gemm_tile_dtl_kernel<Cfg>, dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
     return hipGetLastError();

@@ -348,6 +348,212 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
     }
 }
 
+// ---- split-K kernel with loader waves (k % 4096 == 0) ----------------------------------------------------------
+// Same arithmetic and k-assignment as the split-K kernel above.  Two things hold that kernel back: its 512-byte row
+// pieces (an LDS-DMA that covers 1 KiB of one row streams about a fifth faster, non-temporal another 13 %: a weight byte
+// is read once and stays out of the memory-side cache), and that a wave which both computes and issues its own DMAs
+// sits in the issue whenever the CU's memory queue is full, its matrix pipe idle, while the queue runs dry during its
+// MFMAs.  Here the roles are split: waves 4-7 only load, waves 0-3 only compute.
+//   K       is walked in chunks of 4096: compute wave c owns k-slice c (1024 k) of the chunk and keeps its activation
+//           fragments in registers; it loads them itself at a chunk's start (its own DMA counter sees nothing else),
+//           through three private 4 KiB buffers, one MFMA j-step (16 rows x 256 bytes, chunk c of row r at c ^ r) each,
+//           while the loaders run up to three stages ahead.
+//   stage   one strip of 16 weight rows x one chunk: 32 pieces of 1 KiB (row r, half h at (2 r + h) KiB; 16-byte chunk c
+//           of a piece at position c ^ r, applied on the global side, so that the 16 rows a 16-lane group reads at one
+//           chunk index fall into 16 different bank groups), then 16 x 128 scale bytes.  A ring of three stages.
+//   sync    two workgroup barriers per stage: (A) every loader's pieces of stage t have landed, (B) every compute wave
+//           has its fragments of stage t in registers, so the loaders refill the slot with stage t + 3.
+constexpr int WD_CHUNK = 4096;                       // k per chunk
+constexpr int WD_WBYTES = 16 * (WD_CHUNK / 2);       // 32 KiB
+constexpr int WD_SBYTES = 16 * (WD_CHUNK / 32);      // 2 KiB
+constexpr int WD_STAGE = WD_WBYTES + WD_SBYTES;
+constexpr int WD_RING = 3;
+constexpr int WD_ABYTES = 3 * 4096;                  // activation staging of one compute wave (also its partial sums)
+constexpr int WD_LDS = WD_RING * WD_STAGE + 4 * WD_ABYTES;   // 150 KiB
+constexpr int WD_VM_PER_STAGE = 10;                  // LDS-DMA instructions per loader wave per stage: 8 weight + 2 scale
+static_assert(SK_RMAX * 64 * 16 <= WD_ABYTES, "a compute wave's partial sums fit its staging region");
+static_assert(WD_LDS <= 160 * 1024, "LDS capacity");
+
+// s_waitcnt vmcnt(n) alone, n < 64 (the count is split over bits 3:0 and 15:14 of the immediate)
+#define PTOAMD_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+
+__device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+template <bool HW_CVT>
+__global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvParams p, int strips_per_wg)
+{
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool loader = wave >= 4;
+    const int wc = wave & 3;                          // compute: k-slice of the chunk; loader: which quarter of a stage
+    const int l16 = lane & 15, q = lane >> 4;
+    const int s_begin = blockIdx.x * strips_per_wg, s_end = min(s_begin + strips_per_wg, p.n_groups);
+    const int nsteps = s_end - s_begin, kchunks = p.k / WD_CHUNK, sb = p.k / 32;
+    const uint32_t lds0 = lds_address(smem);
+    uint8_t* mine = smem + WD_RING * WD_STAGE + wc * WD_ABYTES;      // compute wave's private region
+    const uint32_t mine_lds = lds0 + WD_RING * WD_STAGE + wc * WD_ABYTES;
+    // fragment read addresses of a compute lane inside a stage: weight chunk 4 j + q of its slice is at wread ^ (64 j)
+    const int wread = (l16 * 2 + (wc >> 1)) * 1024 + 512 * (wc & 1) + ((q ^ l16) << 4);
+    const int sread = WD_WBYTES + l16 * 128 + wc * 32;
+    const int aread = l16 * 256 + (((4 * q) ^ l16) << 4);   // activation fragment t of a j-step is at aread ^ (16 t)
+
+    // ---- loader side: stage number x of this workgroup (batch b0, chunk kc, strip i of the batch) -> ring slot x % 3
+    int nx_b0 = 0, nx_kc = 0, nx_i = 0, issued = 0;   // the next stage to issue
+    auto issue_next = [&]() {
+        if (nx_b0 >= nsteps)
+            return;
+        const int strip = s_begin + nx_b0 + nx_i;
+        const uint32_t dst = lds0 + (issued % WD_RING) * WD_STAGE;
+        const int rlim = min(15, p.n - 1 - strip * 16);
+        const uint8_t* wbase = p.w + (long)strip * 16 * p.ldw_bytes + (long)nx_kc * (WD_CHUNK / 2);
+#pragma unroll
+        for (int d = 0; d < 8; ++d) {   // piece u = 4 d + wc: row u / 2, half u % 2
+            const int u = 4 * d + wc, r = u >> 1;
+            lds_dma16_off_nt(wbase + (u & 1) * 1024, (uint32_t)(min(r, rlim) * (int)p.ldw_bytes) + (uint32_t)((lane ^ r) << 4),
+                             dst + u * 1024);
+        }
+        const uint8_t* sbase = p.sw + (long)strip * 16 * sb + (long)nx_kc * (WD_CHUNK / 32);
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {   // 64 dwords = two scale rows of the stage per instruction
+            const int e = (wc * 2 + d) * 64 + lane;
+            lds_dma4_off_nt(sbase, (uint32_t)(min(e >> 5, rlim) * sb + (e & 31) * 4), dst + WD_WBYTES + (wc * 2 + d) * 256);
+        }
+        ++issued;
+        if (++nx_i == min(SK_RMAX, nsteps - nx_b0)) {
+            nx_i = 0;
+            if (++nx_kc == kchunks) {
+                nx_kc = 0;
+                nx_b0 += SK_RMAX;
+            }
+        }
+    };
+    if (loader) {
+        issue_next();
+        issue_next();
+        issue_next();
+    }
+
+    uint4 areg[32];
+    int consumed = 0;   // stages taken so far
+    for (int b0 = 0; b0 < nsteps; b0 += SK_RMAX) {
+        const int cnt = min(SK_RMAX, nsteps - b0);
+        f32x4 acc[SK_RMAX];
+#pragma unroll
+        for (int i = 0; i < SK_RMAX; ++i)
+            acc[i] = f32x4{0, 0, 0, 0};
+
+        for (int kc = 0; kc < kchunks; ++kc) {
+            if (!loader && !(kchunks == 1 && b0 > 0)) {
+                // activation fragments of k-slice 4 kc + wc: areg[4 e + t] = A[l16][1024 (4 kc + wc) + 128 e + 32 q + 8 t .. + 7];
+                // rows past m - 1 re-read row m - 1 (their output rows are never stored)
+                const uint8_t* abase = reinterpret_cast<const uint8_t*>(p.a) + (long)(kc * 4 + wc) * 2048;
+                auto issue_a = [&](int e) {
+                    int ln = lane;
+                    asm volatile("" : "+v"(ln));
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const int row = 4 * d + (ln >> 4), pos = ln & 15;
+                        lds_dma16_off(abase + e * 256, (uint32_t)(min(row, p.m - 1) * (int)p.lda * 2 + ((pos ^ row) << 4)),
+                                      mine_lds + (e % 3) * 4096 + d * 1024);
+                    }
+                };
+                issue_a(0);
+                issue_a(1);
+                issue_a(2);
+                static_for<8>([&](auto ec) {
+                    constexpr int e = decltype(ec)::value;
+                    PTOAMD_WAIT_VM(4 * (e + 2 < 8 ? 2 : 7 - e));   // all but the j-steps issued after e
+                    asm volatile("" ::: "memory");
+                    const uint8_t* buf = mine + (e % 3) * 4096;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        areg[4 * e + t] = *reinterpret_cast<const uint4*>(buf + (aread ^ (16 * t)));
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    if (e + 3 < 8)
+                        issue_a(e + 3);
+                });
+            }
+
+            static_for<SK_RMAX>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                if (i < cnt) {
+                    if (loader) {   // own pieces of this stage have landed once only the stages issued after it are outstanding
+                        const int ahead = issued - consumed - 1;
+                        if (ahead >= 2)
+                            PTOAMD_WAIT_VM(2 * WD_VM_PER_STAGE);
+                        else if (ahead == 1)
+                            PTOAMD_WAIT_VM(WD_VM_PER_STAGE);
+                        else
+                            PTOAMD_WAIT_VM(0);
+                    }
+                    wg_barrier();   // (A)
+                    const uint8_t* buf = smem + (consumed % WD_RING) * WD_STAGE;
+                    uint4 sc0, sc1, wv[8];
+                    if (!loader) {
+                        sc0 = *reinterpret_cast<const uint4*>(buf + sread);
+                        sc1 = *reinterpret_cast<const uint4*>(buf + sread + 16);
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            wv[j] = *reinterpret_cast<const uint4*>(buf + (wread ^ (64 * j)));
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    }
+                    wg_barrier();   // (B)
+                    ++consumed;
+                    if (loader) {
+                        issue_next();
+                    } else {
+                        const uint32_t sc[8] = {sc0.x, sc0.y, sc0.z, sc0.w, sc1.x, sc1.y, sc1.z, sc1.w};
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const float scale = e8m0_to_f32((sc[j] >> (8 * q)) & 0xFFu);  // scale byte 4 j + q of the slice
+                            const uint32_t xs[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) {
+                                const uint4 w8 = dequant8<HW_CVT>(xs[t], scale);
+                                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, areg[4 * j + t]),
+                                                                                __builtin_bit_cast(bf16x8, w8), acc[i], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+            });
+        }
+
+        // sum the four k-slice partials of each strip in slice order; every compute wave parks its accumulators in its
+        // own region, then all 512 threads take one output lane each
+        if (!loader) {
+            f32x4* part = reinterpret_cast<f32x4*>(mine);
+#pragma unroll
+            for (int i = 0; i < SK_RMAX; ++i)
+                part[i * 64 + lane] = acc[i];
+        }
+        __syncthreads();
+        {
+            const int i = tid >> 6, strip = s_begin + b0 + i;
+            if (i < cnt) {
+                f32x4 sum = {0, 0, 0, 0};
+                for (int s = 0; s < 4; ++s) {
+                    const f32x4 v = reinterpret_cast<const f32x4*>(smem + WD_RING * WD_STAGE + s * WD_ABYTES)[i * 64 + lane];
+                    sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
+                }
+                const int gj = strip * 16 + l16;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int gi = 4 * q + r;
+                    if (gi < p.m && gj < p.n) {
+                        if (p.out_bf16)
+                            reinterpret_cast<uint16_t*>(p.out)[(long)gi * p.ldc + gj] = f32_to_bf16_bits(sum[r]);
+                        else
+                            reinterpret_cast<float*>(p.out)[(long)gi * p.ldc + gj] = sum[r];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // Generic form for shapes the streaming kernel does not take: one thread per output, k ascending, fp32 fma
 // (the same order as the reference TMATMUL on the dequantised bf16 weights).
 __global__ void gemv_mxfp4_generic_kernel(const GemvParams p)
@@ -406,9 +612,25 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
     const char* sw_cvt = getenv("PTOAMD_GEMV_SW_CVT");
     const bool swc = sw_cvt && sw_cvt[0] == '1';
     const char* no_sk = getenv("PTOAMD_GEMV_NO_SPLITK");
+    const char* no_wide = getenv("PTOAMD_GEMV_NO_WIDE");
+    const bool sk_ok = k % SK_SLICE == 0 && (reinterpret_cast<uintptr_t>(sw) & 3u) == 0 && !(no_sk && no_sk[0] == '1');
+    // loader-wave form: K in chunks of 4096; rows are addressed with 32-bit lane offsets
+    if (sk_ok && k % WD_CHUNK == 0 && (long)lda * 2 * 16 < (1L << 31) && p.ldw_bytes * 16 < (1L << 31) && !(no_wide && no_wide[0] == '1')) {
+        const int spw = (p.n_groups + cus - 1) / cus;    // strips per workgroup
+        const int grid = (p.n_groups + spw - 1) / spw;
+        const void* fn = swc ? reinterpret_cast<const void*>(gemv_mxfp4_splitk_wide_kernel<false>)
+                             : reinterpret_cast<const void*>(gemv_mxfp4_splitk_wide_kernel<true>);
+        PTOAMD_HIP_CHECK(ensure_dynamic_lds(fn, WD_LDS));
+        if (swc)
+            hipLaunchKernelGGL(gemv_mxfp4_splitk_wide_kernel<false>, dim3(grid), dim3(512), WD_LDS, stream, p, spw);
+        else
+            hipLaunchKernelGGL(gemv_mxfp4_splitk_wide_kernel<true>, dim3(grid), dim3(512), WD_LDS, stream, p, spw);
+        PTOAMD_HIP_CHECK(hipGetLastError());
+        set_last_kernel(swc ? "gemv_mxfp4_splitk_wide_swcvt" : "gemv_mxfp4_splitk_wide");
+        return PTOAMD_OK;
+    }
     // (row pitches are multiplied as 24-bit integers in the kernel's address arithmetic)
-    if (k % SK_SLICE == 0 && (reinterpret_cast<uintptr_t>(sw) & 3u) == 0 && (long)lda * 2 < (1L << 24) && p.ldw_bytes < (1L << 24) &&
-        !(no_sk && no_sk[0] == '1')) {
+    if (sk_ok && (long)lda * 2 < (1L << 24) && p.ldw_bytes < (1L << 24)) {
         const int ks = k / SK_SLICE;
         int ksw_log2 = 0;
         while (ksw_log2 < 3 && (2 << ksw_log2) <= ks)
@@ -417,14 +639,9 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
         int spw = (p.n_groups + cus - 1) / cus;          // strips per workgroup, a multiple of the row-group count
         spw = (spw + rgs - 1) / rgs * rgs;
         const int grid = (p.n_groups + spw - 1) / spw;
-        static bool attr_set[2] = {false, false};
-        if (!attr_set[swc]) {
-            PTOAMD_HIP_CHECK(swc ? hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mxfp4_splitk_kernel<false>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS)
-                                 : hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mxfp4_splitk_kernel<true>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS));
-            attr_set[swc] = true;
-        }
+        const void* fn = swc ? reinterpret_cast<const void*>(gemv_mxfp4_splitk_kernel<false>)
+                             : reinterpret_cast<const void*>(gemv_mxfp4_splitk_kernel<true>);
+        PTOAMD_HIP_CHECK(ensure_dynamic_lds(fn, SK_LDS));
         if (swc)
             hipLaunchKernelGGL(gemv_mxfp4_splitk_kernel<false>, dim3(grid), dim3(SK_WAVES * 64), SK_LDS, stream, p, ksw_log2, spw);
         else

@@ -59,6 +59,22 @@ __device__ __forceinline__ void lds_dma16_off(const uint8_t* base_ptr, uint32_t 
     const uint64_t gs = uniform_u64(g);
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(gs), "s"(base) : "memory", "m0");
 }
+// Non-temporal forms for data that is read once (a weight stream): the lines are not kept in the memory-side cache, and
+// a streaming read runs about 13 % faster on this part (6.5 against 5.75 TB/s for 1 KiB-per-instruction row reads).
+__device__ __forceinline__ void lds_dma16_off_nt(const uint8_t* base_ptr, uint32_t lane_off, uint32_t lds_base)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    const uint64_t g = (uint64_t)(uintptr_t)base_ptr;
+    const uint64_t gs = uniform_u64(g);
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 nt" : : "v"(lane_off), "s"(gs), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void lds_dma4_off_nt(const uint8_t* base_ptr, uint32_t lane_off, uint32_t lds_base)
+{
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);
+    const uint64_t g = (uint64_t)(uintptr_t)base_ptr;
+    const uint64_t gs = uniform_u64(g);
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1 nt" : : "v"(lane_off), "s"(gs), "s"(base) : "memory", "m0");
+}
 __device__ __forceinline__ void lds_dma4_off(const uint8_t* base_ptr, uint32_t lane_off, uint32_t lds_base)
 {
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds_base);

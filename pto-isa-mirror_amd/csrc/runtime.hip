@@ -2,6 +2,10 @@
 // (include/pto/common/cpu_stub.hpp:73-120, 524-555), on the HIP runtime.
 #include <string.h>
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 #include "common_host.hpp"
 
 namespace ptoamd {
@@ -19,6 +23,26 @@ void set_last_kernel(const char* name)
 {
     strncpy(g_kernel, name, sizeof g_kernel - 1);
     g_kernel[sizeof g_kernel - 1] = 0;
+}
+
+// hipFuncAttributeMaxDynamicSharedMemorySize is a property of (kernel, device): it is set once per pair, under a lock,
+// so that launches from several host threads or on several devices of one process all see it.
+hipError_t ensure_dynamic_lds(const void* kernel, int bytes)
+{
+    static std::mutex mu;
+    static std::set<std::pair<int, const void*>> done;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return e;
+    std::lock_guard<std::mutex> lock(mu);
+    const auto key = std::make_pair(dev, kernel);
+    if (done.count(key))
+        return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess)
+        done.insert(key);
+    return e;
 }
 }  // namespace ptoamd
 

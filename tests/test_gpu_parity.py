@@ -506,18 +506,25 @@ def _check_gemv(pa, oracle, m, n, k, kernel):
     return got
 
 
-# k a multiple of 1024: 1, 2, 3, 4, 8, 12 and 16 k-slices (1, 2, 2, 4, 8, 8, 8 waves per strip), ragged n and m,
-# more strips per workgroup than one accumulator batch holds (n = 40000: 2500 strips over 256 workgroups, 10 each)
+# k a multiple of 1024: 1, 2, 3, 4, 8, 12 and 16 k-slices, ragged n and m, more strips per workgroup than one accumulator
+# batch holds (n = 40000: 2500 strips over 256 workgroups, 10 each).  K a multiple of 4096 takes the loader-wave form
+# (1, 2, 3 and 4 chunks of 4096), otherwise every wave loads for itself.
 @pytest.mark.parametrize("m,n,k", [(16, 256, 1024), (16, 1000, 8192), (5, 48, 2048), (1, 16, 1024), (7, 333, 3072),
                                    (16, 4096, 4096), (2, 40000, 1024), (16, 520, 12288), (3, 36, 16384),
-                                   (16, 40000, 8192)])
+                                   (16, 40000, 8192), (16, 28672 + 5, 8192), (9, 100, 6144)])
 def test_gemv_mxfp4_splitk(pa, oracle, m, n, k):
-    got = _check_gemv(pa, oracle, m, n, k, "gemv_mxfp4_splitk")
+    wide = k % 4096 == 0
+    got = _check_gemv(pa, oracle, m, n, k, "gemv_mxfp4_splitk_wide" if wide else "gemv_mxfp4_splitk")
+    a, w, sw = _gemv_case(m, n, k)
     with tile_env(PTOAMD_GEMV_NO_SPLITK=1):  # the streaming kernel agrees to rounding
-        a, w, sw = _gemv_case(m, n, k)
         other = host(pa.gemv_mxfp4(dev(a).view(torch.bfloat16), dev(w), dev(sw), n, k, pa.F32))
         assert pa.last_kernel() == "gemv_mxfp4_stream"
     assert relerr(other, got) <= 1e-5
+    if wide:  # every wave loading for itself: other partial sums once K is more than one chunk, same result to rounding
+        with tile_env(PTOAMD_GEMV_NO_WIDE=1):
+            narrow = host(pa.gemv_mxfp4(dev(a).view(torch.bfloat16), dev(w), dev(sw), n, k, pa.F32))
+            assert pa.last_kernel() == "gemv_mxfp4_splitk"
+        assert relerr(narrow, got) <= 1e-5
 
 
 @pytest.mark.parametrize("m,n,k", [(16, 256, 512), (5, 1000, 1536), (1, 16, 2560), (16, 2049, 512)])
@@ -544,7 +551,7 @@ def test_config5_mxfp4_decode_full_size(pa, oracle):
     xw = torch.randn((n, k), generator=gen, device=DEV)
     w, sw = pa.tquant_mx(xw, pa.OCP_MXFP4, want_aux=False)
     out = pa.gemv_mxfp4(a, w, sw, n, k, pa.F32)
-    assert pa.last_kernel() == "gemv_mxfp4_splitk"
+    assert pa.last_kernel() == "gemv_mxfp4_splitk_wide"
     cols = np.arange(0, n, 97)
     ref = _gemv_reference(oracle, host(a), host(sel(w, cols)), host(sel(sw, cols)), len(cols), k)
     assert relerr(host(out)[:, cols], ref) <= 2e-2
