@@ -348,29 +348,30 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
     }
 }
 
-// ---- split-K kernel with loader waves (k % 4096 == 0) ----------------------------------------------------------
+// ---- split-K kernel with loader waves (k % 2048 == 0) ----------------------------------------------------------
 // Same arithmetic and k-assignment as the split-K kernel above.  Two things hold that kernel back: its 512-byte row
 // pieces (an LDS-DMA that covers 1 KiB of one row streams about a fifth faster, non-temporal another 13 %: a weight byte
 // is read once and stays out of the memory-side cache), and that a wave which both computes and issues its own DMAs
 // sits in the issue whenever the CU's memory queue is full, its matrix pipe idle, while the queue runs dry during its
 // MFMAs.  Here the roles are split: waves 4-7 only load, waves 0-3 only compute.
-//   K       is walked in chunks of 4096: compute wave c owns k-slice c (1024 k) of the chunk and keeps its activation
-//           fragments in registers; it loads them itself at a chunk's start (its own DMA counter sees nothing else),
-//           through three private 4 KiB buffers, one MFMA j-step (16 rows x 256 bytes, chunk c of row r at c ^ r) each,
-//           while the loaders run up to three stages ahead.
-//   stage   one strip of 16 weight rows x one chunk: 32 pieces of 1 KiB (row r, half h at (2 r + h) KiB; 16-byte chunk c
-//           of a piece at position c ^ r, applied on the global side, so that the 16 rows a 16-lane group reads at one
-//           chunk index fall into 16 different bank groups), then 16 x 128 scale bytes.  A ring of three stages.
+//   K       is walked in chunks of 2048 (workgroup b starts at chunk b % chunks: with every workgroup on the same
+//           quarter of the rows at the same time, part of the memory channels sits idle).  Compute wave c owns k-slice c
+//           (512 k) of the chunk and keeps its activation fragments in registers.  It loads them itself -- its own DMA
+//           counter sees nothing else -- through three private 4 KiB buffers, one MFMA j-step (16 rows x 256 bytes,
+//           chunk c of row r at c ^ r) at a time, and it loads the next chunk's while it works on this one.
+//   stage   one strip of 16 weight rows x one chunk: row r is one piece of 1 KiB at r KiB (16-byte chunk c at position
+//           c ^ r, applied on the global side, so that the 16 rows a 16-lane group reads at one chunk index fall into
+//           16 different bank groups), then 16 x 64 scale bytes.  A ring of six stages: the loaders run up to six ahead.
 //   sync    two workgroup barriers per stage: (A) every loader's pieces of stage t have landed, (B) every compute wave
-//           has its fragments of stage t in registers, so the loaders refill the slot with stage t + 3.
-constexpr int WD_CHUNK = 4096;                       // k per chunk
-constexpr int WD_WBYTES = 16 * (WD_CHUNK / 2);       // 32 KiB
-constexpr int WD_SBYTES = 16 * (WD_CHUNK / 32);      // 2 KiB
+//           has its fragments of stage t in registers, so the loaders refill the slot with stage t + 6.
+constexpr int WD_CHUNK = 2048;                       // k per chunk
+constexpr int WD_WBYTES = 16 * (WD_CHUNK / 2);       // 16 KiB
+constexpr int WD_SBYTES = 16 * (WD_CHUNK / 32);      // 1 KiB
 constexpr int WD_STAGE = WD_WBYTES + WD_SBYTES;
-constexpr int WD_RING = 3;
+constexpr int WD_RING = 6;
 constexpr int WD_ABYTES = 3 * 4096;                  // activation staging of one compute wave (also its partial sums)
 constexpr int WD_LDS = WD_RING * WD_STAGE + 4 * WD_ABYTES;   // 150 KiB
-constexpr int WD_VM_PER_STAGE = 10;                  // LDS-DMA instructions per loader wave per stage: 8 weight + 2 scale
+constexpr int WD_VM_PER_STAGE = 5;                   // LDS-DMA instructions per loader wave per stage: 4 weight + 1 scale
 static_assert(SK_RMAX * 64 * 16 <= WD_ABYTES, "a compute wave's partial sums fit its staging region");
 static_assert(WD_LDS <= 160 * 1024, "LDS capacity");
 
@@ -390,35 +391,34 @@ __global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvP
     const int l16 = lane & 15, q = lane >> 4;
     const int s_begin = blockIdx.x * strips_per_wg, s_end = min(s_begin + strips_per_wg, p.n_groups);
     const int nsteps = s_end - s_begin, kchunks = p.k / WD_CHUNK, sb = p.k / 32;
+    const int kc_first = blockIdx.x % kchunks;        // chunk number x of this workgroup is chunk (kc_first + x) % kchunks of K
     const uint32_t lds0 = lds_address(smem);
     uint8_t* mine = smem + WD_RING * WD_STAGE + wc * WD_ABYTES;      // compute wave's private region
     const uint32_t mine_lds = lds0 + WD_RING * WD_STAGE + wc * WD_ABYTES;
     // fragment read addresses of a compute lane inside a stage: weight chunk 4 j + q of its slice is at wread ^ (64 j)
-    const int wread = (l16 * 2 + (wc >> 1)) * 1024 + 512 * (wc & 1) + ((q ^ l16) << 4);
-    const int sread = WD_WBYTES + l16 * 128 + wc * 32;
+    const int wread = l16 * 1024 + 256 * wc + ((q ^ l16) << 4);
+    const int sread = WD_WBYTES + l16 * 64 + wc * 16;
     const int aread = l16 * 256 + (((4 * q) ^ l16) << 4);   // activation fragment t of a j-step is at aread ^ (16 t)
 
-    // ---- loader side: stage number x of this workgroup (batch b0, chunk kc, strip i of the batch) -> ring slot x % 3
+    // ---- loader side: stage number x of this workgroup (batch b0, chunk kc, strip i of the batch) -> ring slot x % 6
     int nx_b0 = 0, nx_kc = 0, nx_i = 0, issued = 0;   // the next stage to issue
     auto issue_next = [&]() {
         if (nx_b0 >= nsteps)
             return;
         const int strip = s_begin + nx_b0 + nx_i;
+        const int kc = (kc_first + nx_kc) % kchunks;
         const uint32_t dst = lds0 + (issued % WD_RING) * WD_STAGE;
         const int rlim = min(15, p.n - 1 - strip * 16);
-        const uint8_t* wbase = p.w + (long)strip * 16 * p.ldw_bytes + (long)nx_kc * (WD_CHUNK / 2);
+        const uint8_t* wbase = p.w + (long)strip * 16 * p.ldw_bytes + (long)kc * (WD_CHUNK / 2);
 #pragma unroll
-        for (int d = 0; d < 8; ++d) {   // piece u = 4 d + wc: row u / 2, half u % 2
-            const int u = 4 * d + wc, r = u >> 1;
-            lds_dma16_off_nt(wbase + (u & 1) * 1024, (uint32_t)(min(r, rlim) * (int)p.ldw_bytes) + (uint32_t)((lane ^ r) << 4),
-                             dst + u * 1024);
+        for (int d = 0; d < 4; ++d) {
+            const int r = 4 * d + wc;
+            lds_dma16_off_nt(wbase, (uint32_t)(min(r, rlim) * (int)p.ldw_bytes) + (uint32_t)((lane ^ r) << 4), dst + r * 1024);
         }
-        const uint8_t* sbase = p.sw + (long)strip * 16 * sb + (long)nx_kc * (WD_CHUNK / 32);
-#pragma unroll
-        for (int d = 0; d < 2; ++d) {   // 64 dwords = two scale rows of the stage per instruction
-            const int e = (wc * 2 + d) * 64 + lane;
-            lds_dma4_off_nt(sbase, (uint32_t)(min(e >> 5, rlim) * sb + (e & 31) * 4), dst + WD_WBYTES + (wc * 2 + d) * 256);
-        }
+        // 64 dwords = the scales of four rows
+        const int e = wc * 64 + lane;
+        lds_dma4_off_nt(p.sw + (long)strip * 16 * sb + (long)kc * (WD_CHUNK / 32), (uint32_t)(min(e >> 4, rlim) * sb + (e & 15) * 4),
+                        dst + WD_WBYTES + wc * 256);
         ++issued;
         if (++nx_i == min(SK_RMAX, nsteps - nx_b0)) {
             nx_i = 0;
@@ -429,12 +429,49 @@ __global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvP
         }
     };
     if (loader) {
-        issue_next();
-        issue_next();
-        issue_next();
+#pragma unroll 1
+        for (int x = 0; x < WD_RING; ++x)
+            issue_next();
     }
 
-    uint4 areg[32];
+    // ---- compute side: activation fragments of this wave's k-slice of a chunk, areg[4 e + t] =
+    // A[l16][2048 kc + 512 wc + 128 e + 32 q + 8 t .. + 7]; rows past m - 1 re-read row m - 1 (their outputs are never stored).
+    // anext collects the next chunk's while the current chunk is being multiplied.
+    uint4 areg[16], anext[16];
+    const uint8_t* abase = nullptr;
+    auto issue_a = [&](int e) {
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const int row = 4 * d + (ln >> 4), pos = ln & 15;
+            lds_dma16_off(abase + e * 256, (uint32_t)(min(row, p.m - 1) * (int)p.lda * 2 + ((pos ^ row) << 4)),
+                          mine_lds + (e % 3) * 4096 + d * 1024);
+        }
+    };
+    auto prefetch_begin = [&](int kc) {
+        abase = reinterpret_cast<const uint8_t*>(p.a) + (long)(kc * 4 + wc) * 1024;
+        issue_a(0);
+        issue_a(1);
+        issue_a(2);
+    };
+    auto prefetch_step = [&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        PTOAMD_WAIT_VM(4 * (e < 2 ? 2 : 3 - e));   // all but the j-steps issued after e
+        asm volatile("" ::: "memory");
+        const uint8_t* buf = mine + (e % 3) * 4096;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            anext[4 * e + t] = *reinterpret_cast<const uint4*>(buf + (aread ^ (16 * t)));
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (e == 0)
+            issue_a(3);
+    };
+    if (!loader) {
+        prefetch_begin(kc_first);
+        static_for<4>([&](auto ec) { prefetch_step(ec); });
+    }
+
     int consumed = 0;   // stages taken so far
     for (int b0 = 0; b0 < nsteps; b0 += SK_RMAX) {
         const int cnt = min(SK_RMAX, nsteps - b0);
@@ -443,58 +480,39 @@ __global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvP
         for (int i = 0; i < SK_RMAX; ++i)
             acc[i] = f32x4{0, 0, 0, 0};
 
-        for (int kc = 0; kc < kchunks; ++kc) {
-            if (!loader && !(kchunks == 1 && b0 > 0)) {
-                // activation fragments of k-slice 4 kc + wc: areg[4 e + t] = A[l16][1024 (4 kc + wc) + 128 e + 32 q + 8 t .. + 7];
-                // rows past m - 1 re-read row m - 1 (their output rows are never stored)
-                const uint8_t* abase = reinterpret_cast<const uint8_t*>(p.a) + (long)(kc * 4 + wc) * 2048;
-                auto issue_a = [&](int e) {
-                    int ln = lane;
-                    asm volatile("" : "+v"(ln));
+        for (int kcx = 0; kcx < kchunks; ++kcx) {
+            // the chunk after this one, if the workgroup has one and its activations differ
+            const bool more = kchunks > 1 && (kcx + 1 < kchunks || b0 + SK_RMAX < nsteps);
+            if (!loader) {
+                if (kchunks > 1 || (b0 == 0 && kcx == 0)) {
 #pragma unroll
-                    for (int d = 0; d < 4; ++d) {
-                        const int row = 4 * d + (ln >> 4), pos = ln & 15;
-                        lds_dma16_off(abase + e * 256, (uint32_t)(min(row, p.m - 1) * (int)p.lda * 2 + ((pos ^ row) << 4)),
-                                      mine_lds + (e % 3) * 4096 + d * 1024);
-                    }
-                };
-                issue_a(0);
-                issue_a(1);
-                issue_a(2);
-                static_for<8>([&](auto ec) {
-                    constexpr int e = decltype(ec)::value;
-                    PTOAMD_WAIT_VM(4 * (e + 2 < 8 ? 2 : 7 - e));   // all but the j-steps issued after e
-                    asm volatile("" ::: "memory");
-                    const uint8_t* buf = mine + (e % 3) * 4096;
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        areg[4 * e + t] = *reinterpret_cast<const uint4*>(buf + (aread ^ (16 * t)));
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    if (e + 3 < 8)
-                        issue_a(e + 3);
-                });
+                    for (int x = 0; x < 16; ++x)
+                        areg[x] = anext[x];
+                }
+                if (more)
+                    prefetch_begin((kc_first + kcx + 1) % kchunks);
             }
 
             static_for<SK_RMAX>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
                 if (i < cnt) {
                     if (loader) {   // own pieces of this stage have landed once only the stages issued after it are outstanding
-                        const int ahead = issued - consumed - 1;
-                        if (ahead >= 2)
-                            PTOAMD_WAIT_VM(2 * WD_VM_PER_STAGE);
-                        else if (ahead == 1)
-                            PTOAMD_WAIT_VM(WD_VM_PER_STAGE);
-                        else
-                            PTOAMD_WAIT_VM(0);
+                        switch (issued - consumed - 1) {
+                            case 0: PTOAMD_WAIT_VM(0); break;
+                            case 1: PTOAMD_WAIT_VM(WD_VM_PER_STAGE); break;
+                            case 2: PTOAMD_WAIT_VM(2 * WD_VM_PER_STAGE); break;
+                            case 3: PTOAMD_WAIT_VM(3 * WD_VM_PER_STAGE); break;
+                            case 4: PTOAMD_WAIT_VM(4 * WD_VM_PER_STAGE); break;
+                            default: PTOAMD_WAIT_VM(5 * WD_VM_PER_STAGE); break;
+                        }
                     }
                     wg_barrier();   // (A)
                     const uint8_t* buf = smem + (consumed % WD_RING) * WD_STAGE;
-                    uint4 sc0, sc1, wv[8];
+                    uint4 sc4, wv[4];
                     if (!loader) {
-                        sc0 = *reinterpret_cast<const uint4*>(buf + sread);
-                        sc1 = *reinterpret_cast<const uint4*>(buf + sread + 16);
+                        sc4 = *reinterpret_cast<const uint4*>(buf + sread);
 #pragma unroll
-                        for (int j = 0; j < 8; ++j)
+                        for (int j = 0; j < 4; ++j)
                             wv[j] = *reinterpret_cast<const uint4*>(buf + (wread ^ (64 * j)));
                         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                     }
@@ -503,9 +521,9 @@ __global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvP
                     if (loader) {
                         issue_next();
                     } else {
-                        const uint32_t sc[8] = {sc0.x, sc0.y, sc0.z, sc0.w, sc1.x, sc1.y, sc1.z, sc1.w};
+                        const uint32_t sc[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) {
+                        for (int j = 0; j < 4; ++j) {
                             const float scale = e8m0_to_f32((sc[j] >> (8 * q)) & 0xFFu);  // scale byte 4 j + q of the slice
                             const uint32_t xs[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
 #pragma unroll
@@ -515,9 +533,16 @@ __global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvP
                                                                                 __builtin_bit_cast(bf16x8, w8), acc[i], 0, 0, 0);
                             }
                         }
+                        if (i < 4 && more)
+                            prefetch_step(std::integral_constant<int, (i < 4 ? i : 0)>{});
                     }
                 }
             });
+            if (!loader && more)   // a batch of fewer than four strips: the rest of the next chunk's activations
+                static_for<4>([&](auto ec) {
+                    if (decltype(ec)::value >= cnt)
+                        prefetch_step(ec);
+                });
         }
 
         // sum the four k-slice partials of each strip in slice order; every compute wave parks its accumulators in its
@@ -614,7 +639,7 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
     const char* no_sk = getenv("PTOAMD_GEMV_NO_SPLITK");
     const char* no_wide = getenv("PTOAMD_GEMV_NO_WIDE");
     const bool sk_ok = k % SK_SLICE == 0 && (reinterpret_cast<uintptr_t>(sw) & 3u) == 0 && !(no_sk && no_sk[0] == '1');
-    // loader-wave form: K in chunks of 4096; rows are addressed with 32-bit lane offsets
+    // loader-wave form: K in chunks of 2048; rows are addressed with 32-bit lane offsets
     if (sk_ok && k % WD_CHUNK == 0 && (long)lda * 2 * 16 < (1L << 31) && p.ldw_bytes * 16 < (1L << 31) && !(no_wide && no_wide[0] == '1')) {
         const int spw = (p.n_groups + cus - 1) / cus;    // strips per workgroup
         const int grid = (p.n_groups + spw - 1) / spw;

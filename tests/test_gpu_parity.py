@@ -507,13 +507,13 @@ def _check_gemv(pa, oracle, m, n, k, kernel):
 
 
 # k a multiple of 1024: 1, 2, 3, 4, 8, 12 and 16 k-slices, ragged n and m, more strips per workgroup than one accumulator
-# batch holds (n = 40000: 2500 strips over 256 workgroups, 10 each).  K a multiple of 4096 takes the loader-wave form
-# (1, 2, 3 and 4 chunks of 4096), otherwise every wave loads for itself.
+# batch holds (n = 40000: 2500 strips over 256 workgroups, 10 each).  K a multiple of 2048 takes the loader-wave form
+# (1, 2, 3, 4, 6 and 8 chunks of 2048), otherwise every wave loads for itself.
 @pytest.mark.parametrize("m,n,k", [(16, 256, 1024), (16, 1000, 8192), (5, 48, 2048), (1, 16, 1024), (7, 333, 3072),
                                    (16, 4096, 4096), (2, 40000, 1024), (16, 520, 12288), (3, 36, 16384),
                                    (16, 40000, 8192), (16, 28672 + 5, 8192), (9, 100, 6144)])
 def test_gemv_mxfp4_splitk(pa, oracle, m, n, k):
-    wide = k % 4096 == 0
+    wide = k % 2048 == 0
     got = _check_gemv(pa, oracle, m, n, k, "gemv_mxfp4_splitk_wide" if wide else "gemv_mxfp4_splitk")
     a, w, sw = _gemv_case(m, n, k)
     with tile_env(PTOAMD_GEMV_NO_SPLITK=1):  # the streaming kernel agrees to rounding
