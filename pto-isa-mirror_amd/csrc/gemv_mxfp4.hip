@@ -412,7 +412,7 @@ __global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvP
         const uint8_t* wbase = p.w + (long)strip * 16 * p.ldw_bytes + (long)kc * (WD_CHUNK / 2);
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-            const int r = 4 * d + wc;
+            const int r = 4 * wc + d;   // a loader takes four neighbouring rows (slightly faster than every fourth)
             lds_dma16_off_nt(wbase, (uint32_t)(min(r, rlim) * (int)p.ldw_bytes) + (uint32_t)((lane ^ r) << 4), dst + r * 1024);
         }
         // 64 dwords = the scales of four rows
