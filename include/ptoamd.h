@@ -151,6 +151,19 @@ int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type
                    int ldb, int ldc, int b_layout, void* stream);
 
 /*
+ * ptoamd_gemm_mx with a caller-provided device workspace for what the kernels need beyond inputs and outputs: the MFMA
+ * kernels stream scales as [M][K/32] (MX_A_ND) and [N][K/32] (MX_B_DN), and scales that arrive in another GM layout
+ * (the TLOAD + TMOV of a scale tile, cpu/TLoad.hpp:287-321 with the MX_* maps of cpu/tile_offsets.hpp:233-268) are
+ * re-laid into the workspace first.  ptoamd_gemm_mx takes that memory from a stream-ordered allocation per call; this
+ * form allocates nothing.  workspace: 256-byte aligned, at least ptoamd_gemm_mx_workspace_bytes(...) bytes (0 for the
+ * two natural layouts: workspace may then be NULL).
+ */
+int ptoamd_gemm_mx_ws(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
+                      const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n, int k, int lda,
+                      int ldb, int ldc, int b_layout, void* workspace, size_t workspace_bytes, void* stream);
+size_t ptoamd_gemm_mx_workspace_bytes(int m, int n, int k, int sa_layout, int sb_layout);
+
+/*
  * Decode-shaped weight-only MXFP4 GEMV/GEMM (m <= 16):
  *   out(i, j) = sum_k bf16 A(i, k) * ( e2m1 W(j, k) * 2^(sw(j, k/32) - 127) )      fp32 accumulate
  * The dequantised weight is exact in bf16, so this is TMATMUL on bf16 operands (cpu/TMatmul.hpp:77-113) fed by the

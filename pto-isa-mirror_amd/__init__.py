@@ -33,13 +33,15 @@ if not os.path.exists(LIB_PATH):
 _lib = C.CDLL(LIB_PATH)
 _lib.ptoamd_last_error.restype = C.c_char_p
 _lib.ptoamd_last_kernel.restype = C.c_char_p
+_lib.ptoamd_gemm_mx_workspace_bytes.restype = C.c_size_t
 
 EXPORTS = [
     "ptoamd_init", "ptoamd_finalize", "ptoamd_last_error", "ptoamd_device_info", "ptoamd_malloc", "ptoamd_free",
     "ptoamd_malloc_host", "ptoamd_free_host", "ptoamd_memcpy", "ptoamd_memcpy_async", "ptoamd_memset",
     "ptoamd_stream_create", "ptoamd_stream_destroy", "ptoamd_stream_synchronize", "ptoamd_event_create",
     "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
-    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
+    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_ws",
+    "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
     "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_mx_scale_relayout", "ptoamd_last_kernel",
 ]
 
@@ -107,13 +109,24 @@ def gemm_w8a8(a, b, scale_a, scale_b, b_layout=B_DN, want_acc=False, stream=None
     return (out, acc) if want_acc else out
 
 
+def gemm_mx_workspace_bytes(m, n, k, sa_layout=MX_A_ND, sb_layout=MX_B_DN):
+    return int(_lib.ptoamd_gemm_mx_workspace_bytes(m, n, k, sa_layout, sb_layout))
+
+
 def gemm_mx(a, b, sa, sb, m, n, k, a_type, b_type, c_type=F32, sa_layout=MX_A_ND, sb_layout=MX_B_DN, b_layout=B_DN,
-            c_in=None, stream=None, out=None):
-    """TMATMUL_MX.  a / b hold element codes (uint8; fp4 packed two per byte); sa / sb hold E8M0 bytes."""
+            c_in=None, stream=None, out=None, workspace=None):
+    """TMATMUL_MX.  a / b hold element codes (uint8; fp4 packed two per byte); sa / sb hold E8M0 bytes.  workspace: a
+    uint8 device tensor of gemm_mx_workspace_bytes(...) bytes selects the form that allocates nothing."""
     if out is None:
         out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
     lda = k
     ldb = k if b_layout == B_DN else n
+    if workspace is not None:
+        _check(_lib.ptoamd_gemm_mx_ws(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
+                                      sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _ptr(workspace),
+                                      C.c_size_t(workspace.numel() * workspace.element_size()), _stream(stream)),
+               "ptoamd_gemm_mx_ws")
+        return out
     _check(_lib.ptoamd_gemm_mx(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
                                sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),
            "ptoamd_gemm_mx")

@@ -457,30 +457,34 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
     return PTOAMD_OK;
 }
 
-int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
-                   const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n, int k, int lda,
-                   int ldb, int ldc, int b_layout, void* stream_)
+// Shared body of the TMATMUL_MX entry points.  The MFMA kernels stream scales as [M][K/32] and [N][K/32]; other GM layouts
+// are re-laid first, into `ws` (ws_bytes; the caller's workspace or the library's static array) when one is given, else
+// into a stream-ordered allocation.
+static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, const void* b, int a_type, int b_type,
+                          const uint8_t* sa, const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n,
+                          int k, int lda, int ldb, int ldc, int b_layout, uint8_t* ws, size_t ws_bytes, bool may_allocate,
+                          void* stream_)
 {
     hipStream_t stream = as_stream(stream_);
-    PTOAMD_REQUIRE(c && a && b && sa && sb, PTOAMD_E_INVALID, "ptoamd_gemm_mx: null operand");
-    PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemm_mx: m, n, k must be positive");
-    PTOAMD_REQUIRE(k % 64 == 0, PTOAMD_E_INVALID, "ptoamd_gemm_mx: k = %d must be a multiple of 64", k);
-    PTOAMD_REQUIRE(b_layout == PTOAMD_B_ND || b_layout == PTOAMD_B_DN, PTOAMD_E_INVALID, "ptoamd_gemm_mx: unknown b_layout");
+    PTOAMD_REQUIRE(c && a && b && sa && sb, PTOAMD_E_INVALID, "%s: null operand", who);
+    PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "%s: m, n, k must be positive", who);
+    PTOAMD_REQUIRE(k % 64 == 0, PTOAMD_E_INVALID, "%s: k = %d must be a multiple of 64", who, k);
+    PTOAMD_REQUIRE(b_layout == PTOAMD_B_ND || b_layout == PTOAMD_B_DN, PTOAMD_E_INVALID, "%s: unknown b_layout", who);
     PTOAMD_REQUIRE(sa_layout >= PTOAMD_MX_A_ZZ && sa_layout <= PTOAMD_MX_A_DN && sb_layout >= PTOAMD_MX_B_NN &&
                        sb_layout <= PTOAMD_MX_B_DN,
-                   PTOAMD_E_INVALID, "ptoamd_gemm_mx: sa_layout must be an MX_A_* and sb_layout an MX_B_* layout");
+                   PTOAMD_E_INVALID, "%s: sa_layout must be an MX_A_* and sb_layout an MX_B_* layout", who);
     const bool a8 = a_type == PTOAMD_E4M3 || a_type == PTOAMD_E5M2, b8 = b_type == PTOAMD_E4M3 || b_type == PTOAMD_E5M2;
     const bool a4 = a_type == PTOAMD_E2M1 || a_type == PTOAMD_E1M2, b4 = b_type == PTOAMD_E2M1 || b_type == PTOAMD_E1M2;
     PTOAMD_REQUIRE((a8 && b8) || (a4 && b4), PTOAMD_E_UNSUPPORTED,
-                   "ptoamd_gemm_mx: operands must both be fp8 (e4m3/e5m2) or both fp4 (e2m1/e1m2)");
+                   "%s: operands must both be fp8 (e4m3/e5m2) or both fp4 (e2m1/e1m2)", who);
     PTOAMD_REQUIRE(c_type == PTOAMD_F32 || c_type == PTOAMD_F16 || c_type == PTOAMD_BF16, PTOAMD_E_UNSUPPORTED,
-                   "ptoamd_gemm_mx: the accumulator stores as f32, f16 or bf16");
+                   "%s: the accumulator stores as f32, f16 or bf16", who);
     PTOAMD_REQUIRE(lda >= k && ldc >= n && ldb >= (b_layout == PTOAMD_B_DN ? k : n), PTOAMD_E_INVALID,
-                   "ptoamd_gemm_mx: leading dimension smaller than the row length");
-    PTOAMD_REQUIRE(sa_layout != PTOAMD_MX_A_ZZ || m % 16 == 0, PTOAMD_E_INVALID, "ptoamd_gemm_mx: MX_A_ZZ needs m %% 16 == 0");
-    PTOAMD_REQUIRE(sb_layout != PTOAMD_MX_B_NN || n % 16 == 0, PTOAMD_E_INVALID, "ptoamd_gemm_mx: MX_B_NN needs n %% 16 == 0");
+                   "%s: leading dimension smaller than the row length", who);
+    PTOAMD_REQUIRE(sa_layout != PTOAMD_MX_A_ZZ || m % 16 == 0, PTOAMD_E_INVALID, "%s: MX_A_ZZ needs m %% 16 == 0", who);
+    PTOAMD_REQUIRE(sb_layout != PTOAMD_MX_B_NN || n % 16 == 0, PTOAMD_E_INVALID, "%s: MX_B_NN needs n %% 16 == 0", who);
     if (a4)
-        PTOAMD_REQUIRE(lda % 2 == 0 && ldb % 2 == 0, PTOAMD_E_ALIGNMENT, "ptoamd_gemm_mx: fp4 leading dimensions must be even");
+        PTOAMD_REQUIRE(lda % 2 == 0 && ldb % 2 == 0, PTOAMD_E_ALIGNMENT, "%s: fp4 leading dimensions must be even", who);
     const int out_kind = c_type == PTOAMD_F32 ? OUT_F32 : (c_type == PTOAMD_F16 ? OUT_F16 : OUT_BF16);
     const int bits = a8 ? 8 : 4;
     const long k_bytes = (long)k * bits / 8, lda_b = (long)lda * bits / 8, ldb_b = (long)ldb * bits / 8;
@@ -501,22 +505,36 @@ int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type
     StreamTemp ta(stream), tb(stream);
     const uint8_t* sa_nd = sa;
     const uint8_t* sb_dn = sb;
+    // workspace layout: [M][K/32] scales of A, rounded up to 256 bytes, then [N][K/32] scales of B
+    const size_t need_a = sa_layout != PTOAMD_MX_A_ND ? (((size_t)m * kg + 255) & ~(size_t)255) : 0;
+    const size_t need_b = sb_layout != PTOAMD_MX_B_DN ? (size_t)n * kg : 0;
+    if (ws != nullptr || !may_allocate)
+        PTOAMD_REQUIRE(need_a + need_b <= ws_bytes && (need_a + need_b == 0 || ws != nullptr), PTOAMD_E_INVALID,
+                       "%s: the scale layouts need %zu bytes of workspace, %zu available", who, need_a + need_b, ws_bytes);
     if (sa_layout != PTOAMD_MX_A_ND) {  // the kernel streams scales as [M][K/32] and [N][K/32]
-        PTOAMD_HIP_CHECK(ta.alloc((size_t)m * kg));
-        const int rc = ptoamd_mx_scale_relayout(reinterpret_cast<uint8_t*>(ta.ptr), PTOAMD_MX_A_ND, sa, sa_layout, m, kg, stream_);
+        uint8_t* dst = ws;
+        if (dst == nullptr) {
+            PTOAMD_HIP_CHECK(ta.alloc((size_t)m * kg));
+            dst = reinterpret_cast<uint8_t*>(ta.ptr);
+        }
+        const int rc = ptoamd_mx_scale_relayout(dst, PTOAMD_MX_A_ND, sa, sa_layout, m, kg, stream_);
         if (rc != PTOAMD_OK)
             return rc;
-        sa_nd = reinterpret_cast<const uint8_t*>(ta.ptr);
+        sa_nd = dst;
     }
     if (sb_layout != PTOAMD_MX_B_DN) {
-        PTOAMD_HIP_CHECK(tb.alloc((size_t)n * kg));
-        const int rc = ptoamd_mx_scale_relayout(reinterpret_cast<uint8_t*>(tb.ptr), PTOAMD_MX_B_DN, sb, sb_layout, kg, n, stream_);
+        uint8_t* dst = ws != nullptr ? ws + need_a : nullptr;
+        if (dst == nullptr) {
+            PTOAMD_HIP_CHECK(tb.alloc((size_t)n * kg));
+            dst = reinterpret_cast<uint8_t*>(tb.ptr);
+        }
+        const int rc = ptoamd_mx_scale_relayout(dst, PTOAMD_MX_B_DN, sb, sb_layout, kg, n, stream_);
         if (rc != PTOAMD_OK)
             return rc;
-        sb_dn = reinterpret_cast<const uint8_t*>(tb.ptr);
+        sb_dn = dst;
     }
     PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(sa_nd) & 3u) == 0 && (reinterpret_cast<uintptr_t>(sb_dn) & 3u) == 0,
-                   PTOAMD_E_ALIGNMENT, "ptoamd_gemm_mx: scale arrays must be 4-byte aligned");
+                   PTOAMD_E_ALIGNMENT, "%s: scale arrays must be 4-byte aligned", who);
     TileGemmParams p{};
     p.a = reinterpret_cast<const uint8_t*>(a);
     p.b = reinterpret_cast<const uint8_t*>(b);
@@ -537,6 +555,34 @@ int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;
+}
+
+int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
+                   const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n, int k, int lda,
+                   int ldb, int ldc, int b_layout, void* stream_)
+{
+    return gemm_mx_common("ptoamd_gemm_mx", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k, lda, ldb,
+                          ldc, b_layout, nullptr, 0, true, stream_);
+}
+
+int ptoamd_gemm_mx_ws(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
+                      const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n, int k, int lda,
+                      int ldb, int ldc, int b_layout, void* workspace, size_t workspace_bytes, void* stream_)
+{
+    PTOAMD_REQUIRE(workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, PTOAMD_E_ALIGNMENT,
+                   "ptoamd_gemm_mx_ws: the workspace must be 256-byte aligned");
+    return gemm_mx_common("ptoamd_gemm_mx_ws", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k, lda,
+                          ldb, ldc, b_layout, reinterpret_cast<uint8_t*>(workspace), workspace ? workspace_bytes : 0, false, stream_);
+}
+
+size_t ptoamd_gemm_mx_workspace_bytes(int m, int n, int k, int sa_layout, int sb_layout)
+{
+    if (m <= 0 || n <= 0 || k <= 0)
+        return 0;
+    const size_t kg = (size_t)k / 32;
+    const size_t need_a = sa_layout != PTOAMD_MX_A_ND ? (((size_t)m * kg + 255) & ~(size_t)255) : 0;
+    const size_t need_b = sb_layout != PTOAMD_MX_B_DN ? (size_t)n * kg : 0;
+    return need_a + need_b;
 }
 
 }  // extern "C"

@@ -54,3 +54,6 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert rc == -1 and b"multiple of 64" in lib.ptoamd_last_error()
     rc = lib.ptoamd_gemv_mxfp4(buf, 0, buf, buf, buf, 17, 32, 256, 256, 256, 32, None)
     assert rc == -2
+    lib.ptoamd_gemm_mx_workspace_bytes.restype = ctypes.c_size_t
+    assert lib.ptoamd_gemm_mx_workspace_bytes(64, 48, 256, 0, 3) == 64 * 8 + 48 * 8  # ZZ / NN: both scale arrays re-laid
+    assert lib.ptoamd_gemm_mx_workspace_bytes(64, 48, 256, 1, 5) == 0                # the natural layouts need none

@@ -415,6 +415,36 @@ def test_mx_golden_and_scale_layouts(pa, golden):
         assert np.array_equal(got.view(np.uint32), g[f"mx_{tname}_out_fmt0"].view(np.uint32))
 
 
+def test_gemm_mx_workspace_form(pa, oracle):
+    """ptoamd_gemm_mx_ws: scales in the boxed ZZ / NN layouts are re-laid into the caller's workspace; same kernels, same
+    bits as the allocating form, and no workspace is needed for the two natural layouts."""
+    r = np.random.default_rng(77)
+    m, n, k = 256, 384, 1024
+    a, b, sa, sb = _mx_inputs(r, ob.E4M3, m, n, k)
+    ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ob.E4M3, ob.E4M3)
+    da, db = dev(a), dev(b)
+    sa_zz = pa.mx_scale_relayout(dev(sa), pa.MX_A_ND, pa.MX_A_ZZ, m, k // 32)
+    sb_nn = pa.mx_scale_relayout(dev(sb), pa.MX_B_DN, pa.MX_B_NN, k // 32, n)
+    need = pa.gemm_mx_workspace_bytes(m, n, k, pa.MX_A_ZZ, pa.MX_B_NN)
+    assert need == m * (k // 32) + n * (k // 32)
+    assert pa.gemm_mx_workspace_bytes(m, n, k, pa.MX_A_ND, pa.MX_B_DN) == 0
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    with tile_env(PTOAMD_TILE=5):
+        got = host(pa.gemm_mx(da, db, sa_zz, sb_nn, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sa_layout=pa.MX_A_ZZ,
+                              sb_layout=pa.MX_B_NN, workspace=ws))
+        assert "_dtl_" in pa.last_kernel(), pa.last_kernel()
+        alloc = host(pa.gemm_mx(da, db, sa_zz, sb_nn, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sa_layout=pa.MX_A_ZZ,
+                                sb_layout=pa.MX_B_NN))
+    assert np.array_equal(got.view(np.uint32), alloc.view(np.uint32))
+    assert relerr(got, ref) <= 2e-2
+    with tile_env(PTOAMD_TILE=5):
+        nat = host(pa.gemm_mx(da, db, dev(sa), dev(sb), m, n, k, pa.E4M3, pa.E4M3, pa.F32, workspace=ws[:0]))
+    assert np.array_equal(nat.view(np.uint32), got.view(np.uint32))
+    with pytest.raises(pa.PtoAmdError, match="workspace"):
+        pa.gemm_mx(da, db, sa_zz, sb_nn, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sa_layout=pa.MX_A_ZZ, sb_layout=pa.MX_B_NN,
+                   workspace=ws[:need - 256])
+
+
 def test_mx_scale_relayout_matches_reference_offsets(pa, golden):
     for lid, layout in enumerate((pa.MX_A_ZZ, pa.MX_A_ND, pa.MX_A_DN, pa.MX_B_NN, pa.MX_B_ND, pa.MX_B_DN)):
         rows, cols = (32, 8) if lid < 3 else (8, 32)
