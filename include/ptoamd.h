@@ -164,6 +164,20 @@ int ptoamd_gemm_mx_ws(void* c, int c_type, const void* a, const void* b, int a_t
 size_t ptoamd_gemm_mx_workspace_bytes(int m, int n, int k, int sa_layout, int sb_layout);
 
 /*
+ * ptoamd_gemm_mx_ws with the workspace inside the library: a static device array of PTOAMD_STATIC_SCRATCH_BYTES, one
+ * copy per GPU, held until the process ends.  It has no counterpart in the reference; it is for callers that cannot
+ * allocate device memory around a call: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  The call allocates nothing (no hipMalloc / hipFree, no stream-ordered allocation).  Scale sets whose
+ * re-laid form (ptoamd_gemm_mx_workspace_bytes) exceeds the array are rejected with PTOAMD_E_UNSUPPORTED.  All calls on
+ * one GPU share the one array: calls that overlap in time on the same GPU (two streams, two threads) race on it --
+ * serialise them, or give each stream its own workspace through ptoamd_gemm_mx_ws.
+ */
+#define PTOAMD_STATIC_SCRATCH_BYTES (4 * 1024 * 1024)
+int ptoamd_gemm_mx_static(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
+                          const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n, int k, int lda,
+                          int ldb, int ldc, int b_layout, void* stream);
+
+/*
  * Decode-shaped weight-only MXFP4 GEMV/GEMM (m <= 16):
  *   out(i, j) = sum_k bf16 A(i, k) * ( e2m1 W(j, k) * 2^(sw(j, k/32) - 127) )      fp32 accumulate
  * The dequantised weight is exact in bf16, so this is TMATMUL on bf16 operands (cpu/TMatmul.hpp:77-113) fed by the

@@ -41,7 +41,7 @@ EXPORTS = [
     "ptoamd_stream_create", "ptoamd_stream_destroy", "ptoamd_stream_synchronize", "ptoamd_event_create",
     "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
     "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_ws",
-    "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
+    "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
     "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_mx_scale_relayout", "ptoamd_last_kernel",
 ]
 
@@ -107,6 +107,22 @@ def gemm_w8a8(a, b, scale_a, scale_b, b_layout=B_DN, want_acc=False, stream=None
     _check(_lib.ptoamd_gemm_w8a8(_ptr(out), _ptr(acc), _ptr(a), _ptr(b), _ptr(scale_a), _ptr(scale_b), m, n, k,
                                  a.stride(0), b.stride(0), out.stride(0), b_layout, _stream(stream)), "ptoamd_gemm_w8a8")
     return (out, acc) if want_acc else out
+
+
+STATIC_SCRATCH_BYTES = 4 * 1024 * 1024
+
+
+def gemm_mx_static(a, b, sa, sb, m, n, k, a_type, b_type, out, sa_layout=MX_A_ND, sb_layout=MX_B_DN, b_layout=B_DN, c_in=None,
+                   stream=None):
+    """TMATMUL_MX into a caller-provided `out`, re-laying scales in the library's static device array: nothing is
+    allocated, here or in the library.  Calls that overlap in time on one GPU race on that array."""
+    c_type = {v: key for key, v in _TORCH_OUT.items()}[out.dtype]
+    lda = k
+    ldb = k if b_layout == B_DN else n
+    _check(_lib.ptoamd_gemm_mx_static(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
+                                      sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),
+           "ptoamd_gemm_mx_static")
+    return out
 
 
 def gemm_mx_workspace_bytes(m, n, k, sa_layout=MX_A_ND, sb_layout=MX_B_DN):

@@ -7,6 +7,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+
 namespace ptoamd {
 
 hipError_t launch_gemm_tile_bf16(int, const TileGemmParams&, hipStream_t);
@@ -313,6 +315,33 @@ static int transpose_b(void* dst, const void* src, int k, int n, long ldb, hipSt
     return PTOAMD_OK;
 }
 
+// ---- the library's own scratch memory ---------------------------------------------------------------------------
+// ptoamd_gemm_mx_static re-lays scales into this array instead of a caller workspace or an allocation.  Each GPU the
+// library runs on holds its own copy at its own address until the process ends.  In host code the name `scratch` is
+// only a handle for hipGetSymbolAddress: the device address it yields (once per device, with that device current) is
+// what kernels and copies are given.
+static __device__ __align__(256) uint8_t scratch[PTOAMD_STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+static uint8_t* g_scratch_ptr[MAX_DEVICES];   // device address of `scratch`, per device; written once under g_scratch_mu
+static std::mutex g_scratch_mu;
+
+static int static_scratch(uint8_t** ptr)
+{
+    int dev = 0;
+    PTOAMD_HIP_CHECK(hipGetDevice(&dev));
+    PTOAMD_REQUIRE(dev >= 0 && dev < MAX_DEVICES, PTOAMD_E_UNSUPPORTED, "ptoamd_gemm_mx_static: device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        PTOAMD_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        PTOAMD_REQUIRE(p != nullptr, PTOAMD_E_HIP, "ptoamd_gemm_mx_static: the scratch array has no device address");
+        g_scratch_ptr[dev] = reinterpret_cast<uint8_t*>(p);
+    }
+    *ptr = g_scratch_ptr[dev];
+    return PTOAMD_OK;
+}
+
 }  // namespace ptoamd
 
 using namespace ptoamd;
@@ -573,6 +602,22 @@ int ptoamd_gemm_mx_ws(void* c, int c_type, const void* a, const void* b, int a_t
                    "ptoamd_gemm_mx_ws: the workspace must be 256-byte aligned");
     return gemm_mx_common("ptoamd_gemm_mx_ws", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k, lda,
                           ldb, ldc, b_layout, reinterpret_cast<uint8_t*>(workspace), workspace ? workspace_bytes : 0, false, stream_);
+}
+
+int ptoamd_gemm_mx_static(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
+                          const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n, int k, int lda,
+                          int ldb, int ldc, int b_layout, void* stream_)
+{
+    const size_t need = ptoamd_gemm_mx_workspace_bytes(m, n, k, sa_layout, sb_layout);
+    PTOAMD_REQUIRE(need <= (size_t)PTOAMD_STATIC_SCRATCH_BYTES, PTOAMD_E_UNSUPPORTED,
+                   "ptoamd_gemm_mx_static: re-laying these scales needs %zu bytes, the static scratch holds %d "
+                   "(use ptoamd_gemm_mx_ws with a workspace of that size)", need, PTOAMD_STATIC_SCRATCH_BYTES);
+    uint8_t* ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != PTOAMD_OK)
+        return rc;
+    return gemm_mx_common("ptoamd_gemm_mx_static", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k,
+                          lda, ldb, ldc, b_layout, ws, PTOAMD_STATIC_SCRATCH_BYTES, false, stream_);
 }
 
 size_t ptoamd_gemm_mx_workspace_bytes(int m, int n, int k, int sa_layout, int sb_layout)
