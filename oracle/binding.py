@@ -59,6 +59,10 @@ class Oracle:
         L.pto_group_scaling.restype = C.c_float
         L.pto_group_scaling.argtypes = [C.c_int, C.c_float, C.c_uint]
         L.pto_tile_offset.restype = C.c_int64
+        L.pto_global_offset.restype = C.c_int64
+        L.pto_global_offset.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]
+        L.pto_layout_2d.restype = C.c_int
+        L.pto_layout_2d.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
         L.pto_sim_gemm_tiled.restype = C.c_int
         L.pto_sim_gemm_mx_tiled.restype = C.c_int
 
@@ -91,6 +95,24 @@ class Oracle:
     def mx_scale_offsets(self, layout, rows, cols):
         return np.array([[self.lib.pto_mx_scale_offset(layout, rows, cols, r, c) for c in range(cols)]
                          for r in range(rows)], np.int64)
+
+    def global_offsets(self, layout, shape, stride, rows, cols):
+        """Element offsets of the rows x cols logical view of a 5-D GlobalTensor (ND, DN or NZ)."""
+        sh = np.ascontiguousarray(shape, np.int64)
+        st = np.ascontiguousarray(stride, np.int64)
+        return np.array([[self.lib.pto_global_offset(layout, r, c, _p(sh), _p(st)) for c in range(cols)]
+                         for r in range(rows)], np.int64)
+
+    def layout_2d(self, layout, rows, cols, c0=8):
+        sh, st = np.zeros(5, np.int64), np.zeros(5, np.int64)
+        assert self.lib.pto_layout_2d(layout, rows, cols, c0, _p(sh), _p(st)) == 0
+        return sh, st
+
+    def reorder_exp_zz(self, exp):
+        exp = np.ascontiguousarray(exp, np.uint8)
+        out = np.empty(exp.size, np.uint8)
+        self.lib.pto_reorder_exp_zz(_p(out), _p(exp), exp.shape[0], exp.shape[1])
+        return out
 
     # -- matmul ------------------------------------------------------------------------------
     def _mm(self, fn, out_dt, in_dt, a, b, cin, bias, b_dn):
@@ -251,6 +273,8 @@ class RefLib:
         L.ref_extract_m1.argtypes = [C.c_uint64, C.c_int]
         L.ref_tile_offset.restype = C.c_int64
         L.ref_mx_scale_offset.restype = C.c_int64
+        L.ref_global_offset.restype = C.c_int64
+        L.ref_global_offset.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
 
     def gemm(self, kind, a, b, cin=None, b_dn=False, kstep=0):
         fn, in_dt, out_dt = {
@@ -295,6 +319,24 @@ class RefLib:
         acc = np.ascontiguousarray(acc)
         rc = getattr(self.lib, "ref_store_" + key)(_p(out), _p(acc), m, n, _p(words), int(per_column), int(relu))
         assert rc == 0, rc
+        return out
+
+    def global_offsets(self, which, rows, cols):
+        """(offsets[rows][cols], shape[5], stride[5]) of ref_global_offset's tensor `which`."""
+        sh, st = np.zeros(5, np.int64), np.zeros(5, np.int64)
+        out = np.array([[self.lib.ref_global_offset(which, r, c, _p(sh), _p(st)) for c in range(cols)]
+                        for r in range(rows)], np.int64)
+        return out, sh, st
+
+    def layout_2d(self, layout, rows, cols):
+        sh, st = np.zeros(5, np.int64), np.zeros(5, np.int64)
+        assert self.lib.ref_layout_2d(layout, rows, cols, _p(sh), _p(st)) == 0
+        return sh, st
+
+    def reorder_exp_zz(self, exp):
+        exp = np.ascontiguousarray(exp, np.uint8)
+        out = np.empty(exp.size, np.uint8)
+        self.lib.ref_reorder_exp_zz(_p(out), _p(exp), exp.shape[0], exp.shape[1])
         return out
 
     def shape(self, shape_id):

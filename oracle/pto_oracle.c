@@ -11,8 +11,10 @@
  *                                          boundary cases.
  *   pto_mx_decode / encode_*               compiled reference (oracle/_ref) over all codes / dense value sweeps,
  *                                          frozen in tests/golden; E4M3 decode also against the OCP value table.
- *   pto_tile_offset / pto_global_offset    compiled reference over whole tiles, frozen in tests/golden; bijection
- *                                          property.
+ *   pto_tile_offset / pto_global_offset    compiled reference over whole tiles and over 5-D ND / DN / NZ tensors with
+ *   / pto_layout_2d                        every outer dimension above 1 and padded strides, frozen in tests/golden;
+ *                                          bijection property; ND / DN equal numpy's strided views.
+ *   pto_reorder_exp_zz                     compiled reference, frozen in tests/golden; equals the MX_A_ZZ offset map.
  *   pto_matmul_*                           compiled reference bit for bit; exact integer identities on the
  *                                          reference tests' own input distribution (randint(1,5)); the
  *                                          accIn = 1e8 K-order case of tmatmul_layout; int64 reference mod 2^32.
@@ -549,17 +551,6 @@ void pto_store_f32(void* out, int dst_kind, const float* acc, int m, int n, int 
             if (relu)
                 v = v > 0 ? v : 0;
             put_converted(out, dst_kind, (size_t)i * ldout + j, v);
-        }
-}
-
-void pto_store_i32(int32_t* out, const int32_t* acc, int m, int n, int ldacc, int ldout, int relu)
-{
-    for (int i = 0; i < m; ++i)
-        for (int j = 0; j < n; ++j) {
-            int32_t v = acc[(size_t)i * ldacc + j];
-            if (relu)
-                v = v > 0 ? v : 0;
-            out[(size_t)i * ldout + j] = v;
         }
 }
 

@@ -84,7 +84,6 @@ void pto_matmul_mx(float* out, const uint8_t* a, const uint8_t* b, const uint8_t
 enum pto_store_dst { PTO_ST_F32 = 0, PTO_ST_F16 = 1, PTO_ST_BF16 = 2, PTO_ST_I32 = 3, PTO_ST_I8 = 4, PTO_ST_U8 = 5 };
 /* no-quant path: optional relu then static_cast */
 void pto_store_f32(void* out, int dst_kind, const float* acc, int m, int n, int ldacc, int ldout, int relu);
-void pto_store_i32(int32_t* out, const int32_t* acc, int m, int n, int ldacc, int ldout, int relu);
 /* quant path: words[j] per column when per_column, else words[0] */
 float pto_quant_word_scale(uint64_t word, int vector_mode);
 void pto_store_quant_f32(void* out, int dst_kind, const float* acc, int m, int n, const uint64_t* words,

@@ -609,4 +609,70 @@ int64_t ref_mx_scale_offset(int layout, int rows, int cols, int r, int c)
 #undef W
 }
 
+// GM element offset of logical (r, c) of a 5-D GlobalTensor with static shape and padded strides.
+// which: 0 ND Shape<2,3,4,8,16>, 1 DN Shape<2,3,4,8,16>, 2 NZ Shape<1,4,3,16,8> (the three global layouts TLOAD takes
+// for matrix operands).  shape_out / stride_out receive what the tensor reports.  Logical extents as the
+// simulator's TLOAD walks them (cpu/TLoad.hpp): ND rows = s0*s1*s2*s3, cols = s4; DN rows = s3,
+// cols = s0*s1*s2*s4; NZ rows = s2*s3, cols = s0*s1*s4.
+int64_t ref_global_offset(int which, int r, int c, int64_t* shape_out, int64_t* stride_out)
+{
+#define G(L, SH, ST)                                                                                         \
+    {                                                                                                        \
+        GlobalTensor<float, SH, ST, L> g(nullptr);                                                           \
+        std::vector<int64_t> sh, st;                                                                         \
+        for (int d = 0; d < 5; ++d) {                                                                        \
+            sh.push_back(g.GetShape(d));                                                                     \
+            st.push_back(g.GetStride(d));                                                                    \
+            if (shape_out) shape_out[d] = sh[d];                                                             \
+            if (stride_out) stride_out[d] = st[d];                                                           \
+        }                                                                                                    \
+        return (int64_t)MapTileIndicesToGlobalOffset<decltype(g)>(r, c, sh, st);                             \
+    }
+    using S0 = Shape<2, 3, 4, 8, 16>;
+    using S2 = Shape<1, 4, 3, 16, 8>;
+    using T0 = Stride<3 * 4 * 8 * 20 + 12, 4 * 8 * 20 + 4, 8 * 20, 20, 1>;   // row pitch 20 > 16, gaps between batches
+    using T1 = Stride<3 * 4 * 16 * 10 + 6, 4 * 16 * 10 + 2, 16 * 10, 1, 10>; // column pitch 10 > 8
+    using T2 = Stride<4 * 3 * 128 + 64, 3 * 128 + 16, 128, 8, 1>;
+    switch (which) {
+        case 0: G(Layout::ND, S0, T0)
+        case 1: G(Layout::DN, S0, T1)
+        case 2: G(Layout::NZ, S2, T2)
+        default: return -1;
+    }
+#undef G
+}
+
+// Shape and stride the whole-matrix helpers TileShape2D / BaseShape2D give a [rows, cols] float matrix.
+// layout: 0 ND, 1 DN, 2 NZ
+int ref_layout_2d(int layout, int rows, int cols, int64_t* shape_out, int64_t* stride_out)
+{
+#define W(L)                                                                                                 \
+    {                                                                                                        \
+        using S = TileShape2D<float, DYNAMIC, DYNAMIC, L>;                                                   \
+        using B = BaseShape2D<float, DYNAMIC, DYNAMIC, L>;                                                   \
+        GlobalTensor<float, S, B, L> g(nullptr, S(rows, cols), B(rows, cols));                               \
+        for (int d = 0; d < 5; ++d) {                                                                        \
+            shape_out[d] = g.GetShape(d);                                                                    \
+            stride_out[d] = g.GetStride(d);                                                                  \
+        }                                                                                                    \
+        return 0;                                                                                            \
+    }
+    switch (layout) {
+        case 0: W(Layout::ND)
+        case 1: W(Layout::DN)
+        case 2: W(Layout::NZ)
+        default: return -1;
+    }
+#undef W
+}
+
+// TQuant.hpp ReorderExponentZZ on a [rows][group_cols] exponent matrix
+void ref_reorder_exp_zz(uint8_t* dst, const uint8_t* exp, int rows, int group_cols)
+{
+    std::vector<uint8_t> in(exp, exp + (size_t)rows * group_cols);
+    auto out = pto::cpu_quant::ReorderExponentZZ(in, rows, group_cols);
+    std::copy(out.begin(), out.end(), dst);
+}
+
 }  // extern "C"
+

@@ -167,6 +167,17 @@ def main():
         g[f"dq_src_{nm}"] = q
         g[f"dq_out_{nm}"] = ref.tdequant(3, q, scale, off)
 
+    # --- 5-D global tensors, whole-matrix shape helpers, ZZ exponent reorder (appended: earlier draws unchanged) ---
+    for which, (rows, cols) in enumerate(((2 * 3 * 4 * 8, 16), (8, 2 * 3 * 4 * 16), (48, 32))):
+        offs, sh, st = ref.global_offsets(which, rows, cols)
+        g[f"global_offset_{which}"], g[f"global_shape_{which}"], g[f"global_stride_{which}"] = offs, sh, st
+    for lay in range(3):
+        for rows, cols in ((32, 64), (48, 16)):
+            sh, st = ref.layout_2d(lay, rows, cols)
+            g[f"layout2d_{lay}_{rows}x{cols}"] = np.stack([sh, st])
+    e = r.integers(0, 256, (48, 6)).astype(np.uint8)
+    g["zz_exp"], g["zz_reordered"] = e, ref.reorder_exp_zz(e)
+
     out = os.path.join(ROOT, "tests", "golden", "pto_golden.npz")
     np.savez_compressed(out, **g)
     print(f"wrote {out}: {len(g)} arrays, {os.path.getsize(out)} bytes")

@@ -127,6 +127,48 @@ def test_mx_scale_layout_fixtures(oracle, golden):
 
 
 # ---------------------------------------------------------------- TMATMUL
+GLOBAL_CASES = {0: (ob.ND, 2 * 3 * 4 * 8, 16), 1: (ob.DN, 8, 2 * 3 * 4 * 16), 2: (ob.NZ, 48, 32)}
+
+
+@pytest.mark.parametrize("which", sorted(GLOBAL_CASES))
+def test_global_offset_fixtures(oracle, golden, which):
+    """5-D GlobalTensors with every outer dimension above 1 and padded strides, as the compiled reference maps them."""
+    layout, rows, cols = GLOBAL_CASES[which]
+    sh, st = golden[f"global_shape_{which}"], golden[f"global_stride_{which}"]
+    got = oracle.global_offsets(layout, sh, st, rows, cols)
+    assert np.array_equal(golden[f"global_offset_{which}"], got)
+    assert len(np.unique(got)) == got.size
+
+
+def test_global_offset_nd_is_numpy_strides(oracle):
+    """ND: the logical row runs over dims 0..3 in C order, so the map is numpy's own strided view."""
+    sh, st = np.array([2, 3, 4, 8, 16]), np.array([2000, 650, 160, 20, 1])
+    buf = np.arange(2 * 2000)
+    view = np.lib.stride_tricks.as_strided(buf, sh, st * buf.itemsize).reshape(-1, 16)
+    assert np.array_equal(view, oracle.global_offsets(ob.ND, sh, st, 2 * 3 * 4 * 8, 16))
+    # DN: rows are dim 3, columns run over dims 0, 1, 2, 4
+    st = np.array([2000, 650, 160, 1, 10])
+    view = np.lib.stride_tricks.as_strided(buf, sh, st * buf.itemsize).transpose(3, 0, 1, 2, 4).reshape(8, -1)
+    assert np.array_equal(view, oracle.global_offsets(ob.DN, sh, st, 8, 2 * 3 * 4 * 16))
+
+
+def test_layout_2d_fixtures(oracle, golden):
+    for lay in (ob.ND, ob.DN, ob.NZ):
+        for rows, cols in ((32, 64), (48, 16)):
+            sh, st = oracle.layout_2d(lay, rows, cols, c0=8)  # 32-byte C0 of float
+            assert np.array_equal(golden[f"layout2d_{lay}_{rows}x{cols}"], np.stack([sh, st])), (lay, rows, cols)
+            offs = oracle.global_offsets(lay, sh, st, rows, cols)
+            assert sorted(offs.ravel().tolist()) == list(range(rows * cols))
+
+
+def test_reorder_exp_zz_fixture_and_layout_identity(oracle, golden):
+    assert np.array_equal(golden["zz_reordered"], oracle.reorder_exp_zz(golden["zz_exp"]))
+    # the reordered stream is the MX_A_ZZ global layout of the same [rows][groups] matrix
+    e = golden["zz_exp"]
+    offs = oracle.mx_scale_offsets(ob.MX_A_ZZ, *e.shape)
+    assert np.array_equal(oracle.reorder_exp_zz(e)[offs], e)
+
+
 def test_matmul_reference_test_distribution_is_exact(oracle, golden):
     """tests/cpu/st/testcase/tmatmul/gen_data.py draws randint(1,5): every partial sum is an exact integer."""
     for name in ("case1", "case3_splitk", "gemv"):
@@ -334,6 +376,19 @@ def test_tquant_fixtures(oracle, golden):
     for nm in ("i8", "i16", "i32"):
         got = oracle.tdequant(g[f"dq_src_{nm}"], g["q8_scale"], g["q8_off"])
         assert np.array_equal(bits(g[f"dq_out_{nm}"]), bits(got))
+
+
+@pytest.mark.parametrize("alg", [ob.OCP_FP8, ob.NV_FP8, ob.OCP_FP4, ob.NV_FP4])
+def test_tquant_bf16_source_equals_f32_source_on_bf16_values(oracle, alg):
+    """The bf16 source path may differ from fp32 only through rounding to bf16 (group maximum taken on bf16 bits,
+    scaled value re-rounded): on inputs that already are bf16 values, scaled by a power of two, nothing rounds."""
+    r = np.random.default_rng(31)
+    src = (r.standard_normal((32, 256)) * 10.0 ** r.uniform(-2, 2, (32, 1))).astype(np.float32)
+    src = (src.view(np.uint32) & 0xFFFF0000).view(np.float32)
+    a = oracle.tquant_mx(src, alg, 1, ob.SRC_F32)
+    b = oracle.tquant_mx(src, alg, 1, ob.SRC_BF16)
+    for x, y in zip(a, b):
+        assert np.array_equal(bits(x) if x.dtype == np.float32 else x, bits(y) if y.dtype == np.float32 else y)
 
 
 def test_tquant_round_trip_error_bound(oracle):

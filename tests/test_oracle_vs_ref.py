@@ -159,6 +159,25 @@ def test_mx_scale_layouts(oracle, reflib, layout, ref_id):
     assert sorted(got.ravel().tolist()) == list(range(rows * cols))
 
 
+@pytest.mark.parametrize("which,layout,rows,cols", [(0, ob.ND, 192, 16), (1, ob.DN, 8, 384), (2, ob.NZ, 48, 32)])
+def test_global_offsets_5d(oracle, reflib, which, layout, rows, cols):
+    ref, sh, st = reflib.global_offsets(which, rows, cols)
+    assert np.array_equal(ref, oracle.global_offsets(layout, sh, st, rows, cols))
+
+
+@pytest.mark.parametrize("layout", [ob.ND, ob.DN, ob.NZ])
+@pytest.mark.parametrize("rows,cols", [(32, 64), (48, 16), (16, 8)])
+def test_layout_2d(oracle, reflib, layout, rows, cols):
+    want = reflib.layout_2d(layout, rows, cols)
+    got = oracle.layout_2d(layout, rows, cols, c0=8)
+    assert np.array_equal(want[0], got[0]) and np.array_equal(want[1], got[1])
+
+
+def test_reorder_exp_zz(oracle, reflib):
+    e = np.random.default_rng(3).integers(0, 256, (64, 10)).astype(np.uint8)
+    assert np.array_equal(reflib.reorder_exp_zz(e), oracle.reorder_exp_zz(e))
+
+
 def _word_scalar(scale, offset=0, sign=1):
     return int(np.float32(scale).view(np.uint32)) | (offset << 37) | (sign << 46)
 
