@@ -34,9 +34,15 @@
 #endif
 
 // A PTO kernel entry is written `__global__ AICORE void f(...)`; here it is a device function run by pto::amd::launch.
+// (PTO_AMD_CHECK_REFERENCE_SOURCE: a device-only syntax pass over an unmodified reference kernel file, whose
+// CPU-simulator launch functions call the core programs directly; the cores are then also callable from host code.)
 #undef __global__
 #define __global__
+#ifdef PTO_AMD_CHECK_REFERENCE_SOURCE
+#define AICORE __host__ __device__
+#else
 #define AICORE __device__
+#endif
 #define __aicore__
 #define __gm__
 #define __ubuf__
@@ -52,6 +58,7 @@
 #define PTO_INTERNAL __device__ __forceinline__
 
 using half = _Float16;
+using aclFloat16 = _Float16;
 using bfloat16_t = __bf16;
 
 namespace pto {

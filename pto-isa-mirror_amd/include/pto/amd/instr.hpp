@@ -258,9 +258,36 @@ struct MxFormat<float8_e5m2_t> {
 };
 template <>
 struct MxFormat<float4_e2m1x2_t> {
-    static constexpr int code = 4;  // the scaled MFMA has no E1M2 format
+    static constexpr int code = 4;
+};
+template <>
+struct MxFormat<float4_e1m2x2_t> {
+    static constexpr int code = 0;  // the scaled MFMA has no E1M2 format: such operands are widened to E4M3 first
 };
 typedef int i32x8v __attribute__((ext_vector_type(8)));
+
+// Packed fp4 codes -> E4M3 bytes, exactly: every E2M1 value (0 .. 6) and every E1M2 value (0 .. 1.75) is an E4M3 number.
+// The scaled MFMA has no E1M2 format, so E1M2 operands (and an E2M1 operand paired with one) run as fp8.
+template <typename T>
+PTO_INST uint2 fp4x8_to_e4m3(uint32_t packed)
+{
+    // E4M3 codes of the eight magnitudes, one byte each, low magnitude in the low byte
+    constexpr uint32_t lo = std::is_same_v<T, float4_e1m2x2_t> ? 0x34302800u : 0x3C383000u;   // E1M2: 0, .25, .5, .75 | E2M1: 0, .5, 1, 1.5
+    constexpr uint32_t hi = std::is_same_v<T, float4_e1m2x2_t> ? 0x3E3C3A38u : 0x4C484440u;   // E1M2: 1, 1.25, 1.5, 1.75 | E2M1: 2, 3, 4, 6
+    uint2 out;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const uint32_t x = (packed >> (16 * half)) & 0xFFFFu;   // four codes
+        const uint32_t spread = (x & 0xFu) | ((x & 0xF0u) << 4) | ((x & 0xF00u) << 8) | ((x & 0xF000u) << 12);   // one code per byte
+        const uint32_t mag = __builtin_amdgcn_perm(hi, lo, spread & 0x07070707u);   // byte i of the result = table[code i & 7]
+        const uint32_t v = mag | ((spread & 0x08080808u) << 4);
+        if (half == 0)
+            out.x = v;
+        else
+            out.y = v;
+    }
+    return out;
+}
 
 template <bool INIT, typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT>
 PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRightT& b, TileRightScaleT& bs)
@@ -273,14 +300,19 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
     static_assert(std::is_same_v<typename TileRes::DType, float>, "TMATMUL_MX accumulates in float");
     static_assert(is_packed4<TA> == is_packed4<TB>, "TMATMUL_MX: both operands fp8 or both fp4");
     static_assert(TileLeftT::Cols % 64 == 0, "TMATMUL_MX: the static K of the Left tile must be a multiple of 64");
-    static_assert(TileLeftT::Cols == TileRightT::Rows && TileRes::Rows == TileLeftT::Rows && TileRes::Cols == TileRightT::Cols,
+    // a one-row Left tile (TGEMV_MX) may be declared wider than the Right tile is tall, and meets a 16-row accumulator
+    constexpr bool gemv = TileLeftT::Rows == 1;
+    static_assert((TileLeftT::Cols == TileRightT::Rows || (gemv && TileLeftT::Cols >= TileRightT::Rows)) &&
+                      (TileRes::Rows == TileLeftT::Rows || gemv) && TileRes::Cols == TileRightT::Cols,
                   "TMATMUL_MX: static tile shapes do not chain");
-    static_assert(TileLeftScaleT::Rows == TileLeftT::Rows && TileLeftScaleT::Cols * 32 == TileLeftT::Cols &&
-                      TileRightScaleT::Cols == TileRightT::Cols && TileRightScaleT::Rows * 32 == TileRightT::Rows,
+    // (scale tiles may be declared larger than the K / 32 groups they hold)
+    static_assert(TileLeftScaleT::Rows == TileLeftT::Rows && TileLeftScaleT::Cols * 32 >= TileRightT::Rows &&
+                      TileRightScaleT::Cols == TileRightT::Cols && TileRightScaleT::Rows * 32 >= TileRightT::Rows,
                   "TMATMUL_MX: one E8M0 scale per 32 K-elements");
+    constexpr bool via_fp8 = std::is_same_v<TA, float4_e1m2x2_t> || std::is_same_v<TB, float4_e1m2x2_t>;
     const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int kpad = min((a.GetValidCol() + 63) / 64 * 64, TileLeftT::Cols);
+    const int kpad = min((a.GetValidCol() + 63) / 64 * 64, TileRightT::Rows);
     const uint8_t *pa = a.Storage(), *pb = b.Storage(), *psa = as.Storage(), *psb = bs.Storage();
     constexpr int CB = TileRes::CB;
 #pragma unroll
@@ -297,20 +329,32 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
                 const int g = k0 / 32 + lhi;
                 const int sa = psa[as.ByteOffset(arow, g)], sb = psb[bs.ByteOffset(g, bcol)];
                 i32x8v av = {0, 0, 0, 0, 0, 0, 0, 0}, bv = {0, 0, 0, 0, 0, 0, 0, 0};
-                if constexpr (is_packed4<TA>) {  // fp4: the lane's 16 bytes are the whole MX block lhi
-                    const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 32 * lhi));
-                    const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 * lhi, bcol));
-                    av = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, 0, 0, 0, 0};
-                    bv = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, 0, 0, 0, 0};
-                } else {  // fp8: bytes [16 lhi, 16 lhi + 16) of each of the two blocks
-                    const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 16 * lhi));
-                    const uint4 a1 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 32 + 16 * lhi));
-                    const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 16 * lhi, bcol));
-                    const uint4 b1 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 + 16 * lhi, bcol));
-                    av = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
-                    bv = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                if constexpr (via_fp8) {  // fp4 codes widened to E4M3 bytes, then fed like fp8: 16 elements of each block per lane
+                    const uint2 a0 = *reinterpret_cast<const uint2*>(pa + a.ByteOffset(arow, k0 + 16 * lhi));
+                    const uint2 a1 = *reinterpret_cast<const uint2*>(pa + a.ByteOffset(arow, k0 + 32 + 16 * lhi));
+                    const uint2 b0 = *reinterpret_cast<const uint2*>(pb + b.ByteOffset(k0 + 16 * lhi, bcol));
+                    const uint2 b1 = *reinterpret_cast<const uint2*>(pb + b.ByteOffset(k0 + 32 + 16 * lhi, bcol));
+                    const uint2 ea[4] = {fp4x8_to_e4m3<TA>(a0.x), fp4x8_to_e4m3<TA>(a0.y), fp4x8_to_e4m3<TA>(a1.x), fp4x8_to_e4m3<TA>(a1.y)};
+                    const uint2 eb[4] = {fp4x8_to_e4m3<TB>(b0.x), fp4x8_to_e4m3<TB>(b0.y), fp4x8_to_e4m3<TB>(b1.x), fp4x8_to_e4m3<TB>(b1.y)};
+                    av = i32x8v{(int)ea[0].x, (int)ea[0].y, (int)ea[1].x, (int)ea[1].y, (int)ea[2].x, (int)ea[2].y, (int)ea[3].x, (int)ea[3].y};
+                    bv = i32x8v{(int)eb[0].x, (int)eb[0].y, (int)eb[1].x, (int)eb[1].y, (int)eb[2].x, (int)eb[2].y, (int)eb[3].x, (int)eb[3].y};
+                    acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 0, 0, 0, sa, 0, sb);
+                } else {
+                    if constexpr (is_packed4<TA>) {  // fp4: the lane's 16 bytes are the whole MX block lhi
+                        const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 32 * lhi));
+                        const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 * lhi, bcol));
+                        av = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, 0, 0, 0, 0};
+                        bv = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, 0, 0, 0, 0};
+                    } else {  // fp8: bytes [16 lhi, 16 lhi + 16) of each of the two blocks
+                        const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 16 * lhi));
+                        const uint4 a1 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 32 + 16 * lhi));
+                        const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 16 * lhi, bcol));
+                        const uint4 b1 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 + 16 * lhi, bcol));
+                        av = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                        bv = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                    }
+                    acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, MxFormat<TA>::code, MxFormat<TB>::code, 0, sa, 0, sb);
                 }
-                acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, MxFormat<TA>::code, MxFormat<TB>::code, 0, sa, 0, sb);
             }
             c.regs[slot] = acc;
         }
@@ -379,10 +423,16 @@ template <bool VECTOR, typename G, typename Reg>
 PTO_INST float quantize_element(Reg acc, uint64_t word)
 {
     constexpr bool src_is_int = std::is_integral_v<Reg>;
-    static_assert(std::is_same_v<G, int8_t> || std::is_same_v<G, uint8_t> || std::is_same_v<G, _Float16> || std::is_same_v<G, __bf16>,
-                  "TSTORE with quantisation targets int8, uint8, half or bfloat16");
+    static_assert(std::is_same_v<G, int8_t> || std::is_same_v<G, uint8_t> || std::is_same_v<G, _Float16> || std::is_same_v<G, __bf16> ||
+                      (std::is_same_v<G, int16_t> && src_is_int),
+                  "fix-pipe quantisation targets int8, uint8, half or bfloat16 (and int16 from an int32 accumulator)");
     float r = __fmul_rn((float)acc, quant_word_scale<VECTOR>(word));
-    if constexpr (sizeof(G) == 1) {
+    if constexpr (std::is_same_v<G, int16_t>) {
+        // shift mode (cpu/common.hpp:174-180): arithmetic shift right by bits 32..35 of the word plus one; the
+        // reference narrows to int16 before it clamps, so the value wraps
+        const int shift = (int)((word >> 32) & 0xFu) + 1;
+        r = (float)(int16_t)((int32_t)acc >> shift);
+    } else if constexpr (sizeof(G) == 1) {
         const float offset = (float)(uint32_t)((word >> 37) & 0x1FFu);
         const bool sign = (word >> 46) & 1u;
         const float rounded = rintf(__fadd_rn(r, offset));
@@ -460,36 +510,133 @@ PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, FpTileData& fp)
     return {};
 }
 
+template <typename TileData, typename GlobalData, typename FpTileData, AtomicType atomicType = AtomicType::AtomicNone,
+          ReluPreMode reluPreMode = ReluPreMode::NoRelu, typename... WaitEvents,
+          std::enable_if_t<is_tile_data_v<FpTileData> && all_events_v<WaitEvents...>, int> = 0>
+PTO_INST RecordEvent TSTORE_FP(GlobalData& dst, TileData& src, FpTileData& fp, WaitEvents&...)
+{
+    return TSTORE<TileData, GlobalData, FpTileData, atomicType, reluPreMode>(dst, src, fp);
+}
+
 // ---- TMOV / TEXTRACT -----------------------------------------------------------------------------------------------
-template <typename DstTileData, typename SrcTileData, typename... WaitEvents>
+namespace amd {
+// Accumulator -> on-chip buffer tile, the fix-pipe move: dst(r, c) = f(src(r + row0, c + col0)) over dst's valid region
+// (reference: cpu/TExtract.hpp:21-46).  QUANT 0: optional relu, then the element conversion of TSTORE; 1 / 2: fix-pipe
+// quantisation with one word for the tile / one word per source column (cpu/common.hpp:139-185), relu after it.
+template <int QUANT, ReluPreMode relu, typename DstTile, typename SrcTile, typename WordOf>
+PTO_INST void tmov_acc(DstTile& dst, SrcTile& src, int row0, int col0, WordOf&& word_of)
+{
+    static_assert(DstTile::Loc == TileType::Vec || DstTile::Loc == TileType::Mat, "an accumulator tile moves to a Vec or Mat tile");
+    using D = typename DstTile::DType;
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    uint8_t* d = dst.Storage();
+    __syncthreads();
+    for_each_acc(src, [&](int slot, int r, int row, int col) {
+        const int dr = row - row0, dc = col - col0;
+        if (dr >= 0 && dc >= 0 && dr < vr && dc < vc && row < src.GetValidRow() && col < src.GetValidCol()) {
+            if constexpr (QUANT == 0) {
+                auto v = src.regs[slot][r];
+                if constexpr (relu == ReluPreMode::NormalRelu)
+                    v = v > 0 ? v : 0;
+                *reinterpret_cast<D*>(d + dst.ByteOffset(dr, dc)) = convert<D>(v);
+            } else {
+                float v = quantize_element<QUANT == 2, D>(src.regs[slot][r], word_of(col));
+                if constexpr (relu == ReluPreMode::NormalRelu)
+                    v = v > 0 ? v : 0;
+                *reinterpret_cast<D*>(d + dst.ByteOffset(dr, dc)) = static_cast<D>(v);
+            }
+        }
+    });
+    __syncthreads();
+}
+// relu over the valid region of an LDS tile (TMOV's relu form between buffer tiles, cpu/TMov.hpp:37-54)
+template <typename TileData>
+PTO_INST void trelu_lds(TileData& t)
+{
+    using T = typename TileData::DType;
+    static_assert(is_number<T>, "relu needs a numeric element type");
+    const int vr = t.GetValidRow(), vc = t.GetValidCol();
+    uint8_t* d = t.Storage();
+    for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
+        const int r = idx / vc, c = idx - r * vc;
+        T* e = reinterpret_cast<T*>(d + t.ByteOffset(r, c));
+        if (*e < T(0))
+            *e = T(0);
+    }
+    __syncthreads();
+}
+}  // namespace amd
+
+template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode, typename... WaitEvents,
+          std::enable_if_t<all_events_v<WaitEvents...>, int> = 0>
 PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, WaitEvents&...)
 {
     static_assert(DstTileData::Loc != TileType::Acc, "TMOV into an accumulator tile is not implemented on this backend");
     if constexpr (SrcTileData::Loc == TileType::Acc) {
-        // Acc -> Vec / Mat: the fix-pipe move of an accumulator into an on-chip buffer (reference: cpu/TMov.hpp:21-35),
-        // element type converted like TSTORE's static_cast
-        static_assert(DstTileData::Loc == TileType::Vec || DstTileData::Loc == TileType::Mat,
-                      "an accumulator tile moves to a Vec or Mat tile");
-        using D = typename DstTileData::DType;
-        const int vr = src.GetValidRow(), vc = src.GetValidCol();
-        uint8_t* d = dst.Storage();
-        __syncthreads();
-        amd::for_each_acc(src, [&](int slot, int r, int row, int col) {
-            if (row < vr && col < vc)
-                *reinterpret_cast<D*>(d + dst.ByteOffset(row, col)) = amd::convert<D>(src.regs[slot][r]);
-        });
-        __syncthreads();
+        amd::tmov_acc<0, reluMode>(dst, src, 0, 0, [](int) { return (uint64_t)0; });
     } else {
         amd::textract_lds(dst, src, 0, 0);
+        if constexpr (reluMode == ReluPreMode::NormalRelu)
+            amd::trelu_lds(dst);
     }
     return {};
 }
-template <typename DstTileData, typename SrcTileData, typename... WaitEvents>
+template <typename DstTileData, typename SrcTileData, typename... WaitEvents, std::enable_if_t<all_events_v<WaitEvents...>, int> = 0>
+PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, WaitEvents&...)
+{
+    return TMOV<DstTileData, SrcTileData, ReluPreMode::NoRelu>(dst, src);
+}
+// fix-pipe quantising forms: one scalar word, or one word per column from a Scaling tile
+template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode = ReluPreMode::NoRelu, typename... WaitEvents,
+          std::enable_if_t<all_events_v<WaitEvents...>, int> = 0>
+PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, uint64_t preQuantScalar, WaitEvents&...)
+{
+    static_assert(SrcTileData::Loc == TileType::Acc, "the quantising TMOV drains an accumulator tile");
+    amd::tmov_acc<1, reluMode>(dst, src, 0, 0, [&](int) { return preQuantScalar; });
+    return {};
+}
+template <typename DstTileData, typename SrcTileData, typename FpTileData, ReluPreMode reluMode = ReluPreMode::NoRelu, typename... WaitEvents,
+          std::enable_if_t<is_tile_data_v<FpTileData> && FpTileData::Loc == TileType::Scaling && all_events_v<WaitEvents...>, int> = 0>
+PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, FpTileData& fp, WaitEvents&...)
+{
+    static_assert(SrcTileData::Loc == TileType::Acc, "the quantising TMOV drains an accumulator tile");
+    static_assert(sizeof(typename FpTileData::DType) == 8, "the Scaling tile holds one 64-bit quantisation word per column");
+    const uint8_t* words = fp.Storage();
+    amd::tmov_acc<2, reluMode>(dst, src, 0, 0, [&](int col) { return *reinterpret_cast<const uint64_t*>(words + fp.ByteOffset(0, col)); });
+    return {};
+}
+
+template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode = ReluPreMode::NoRelu, typename... WaitEvents,
+          std::enable_if_t<all_events_v<WaitEvents...>, int> = 0>
 PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, uint16_t indexRow = 0, uint16_t indexCol = 0, WaitEvents&...)
 {
-    static_assert(DstTileData::Loc != TileType::Acc && SrcTileData::Loc != TileType::Acc,
-                  "TEXTRACT from / to accumulator tiles is not implemented on this backend yet");
-    amd::textract_lds(dst, src, indexRow, indexCol);
+    static_assert(DstTileData::Loc != TileType::Acc, "TEXTRACT into an accumulator tile is not implemented on this backend");
+    if constexpr (SrcTileData::Loc == TileType::Acc) {
+        amd::tmov_acc<0, reluMode>(dst, src, indexRow, indexCol, [](int) { return (uint64_t)0; });
+    } else {
+        amd::textract_lds(dst, src, indexRow, indexCol);
+        if constexpr (reluMode == ReluPreMode::NormalRelu)
+            amd::trelu_lds(dst);
+    }
+    return {};
+}
+template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode = ReluPreMode::NoRelu, typename... WaitEvents,
+          std::enable_if_t<all_events_v<WaitEvents...>, int> = 0>
+PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, uint64_t preQuantScalar, uint16_t indexRow, uint16_t indexCol, WaitEvents&...)
+{
+    static_assert(SrcTileData::Loc == TileType::Acc, "the quantising TEXTRACT drains an accumulator tile");
+    amd::tmov_acc<1, reluMode>(dst, src, indexRow, indexCol, [&](int) { return preQuantScalar; });
+    return {};
+}
+template <typename DstTileData, typename SrcTileData, typename FpTileData, ReluPreMode reluMode = ReluPreMode::NoRelu, typename... WaitEvents,
+          std::enable_if_t<is_tile_data_v<FpTileData> && FpTileData::Loc == TileType::Scaling && all_events_v<WaitEvents...>, int> = 0>
+PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, FpTileData& fp, uint16_t indexRow, uint16_t indexCol, WaitEvents&...)
+{
+    static_assert(SrcTileData::Loc == TileType::Acc, "the quantising TEXTRACT drains an accumulator tile");
+    static_assert(sizeof(typename FpTileData::DType) == 8, "the Scaling tile holds one 64-bit quantisation word per column");
+    const uint8_t* words = fp.Storage();
+    amd::tmov_acc<2, reluMode>(dst, src, indexRow, indexCol,
+                               [&](int col) { return *reinterpret_cast<const uint64_t*>(words + fp.ByteOffset(0, col)); });
     return {};
 }
 

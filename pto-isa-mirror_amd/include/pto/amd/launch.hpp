@@ -2,6 +2,8 @@
 // PTO_AMD_THREADS threads) with the core's LDS arena; get_block_idx() / get_block_num() name them, like the `<<<>>>`
 // launch of the reference's NPU tests and LaunchKernelMultiCore of its CPU simulator (common/cpu_stub.hpp:367-427).
 #pragma once
+#include <atomic>
+
 #include "tile.hpp"
 
 namespace pto {
@@ -18,13 +20,18 @@ template <auto Kernel, typename... Args>
 inline int launch(int blocks, void* stream, Args... args)
 {
     auto* entry = core_entry<Kernel, Args...>;
-    static bool configured = false;
-    if (!configured) {
+    // the attribute belongs to (kernel, device): remember per device which ones have it (devices past 63 set it every time)
+    static std::atomic<uint64_t> configured{0};
+    int dev = 0;
+    if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess)
+        return (int)e;
+    const uint64_t bit = dev < 64 ? (1ull << dev) : 0;
+    if (!(configured.load(std::memory_order_acquire) & bit)) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(entry),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
         if (e != hipSuccess)
             return (int)e;
-        configured = true;
+        configured.fetch_or(bit, std::memory_order_release);
     }
     hipLaunchKernelGGL(entry, dim3(blocks), dim3(PTO_AMD_THREADS), LDS_TOTAL, static_cast<hipStream_t>(stream), args...);
     return (int)hipGetLastError();
@@ -37,6 +44,13 @@ inline int device_status()
     if (hipMemcpyFromSymbol(&v, HIP_SYMBOL(g_status), sizeof(int)) != hipSuccess)
         return -1;
     return v;
+}
+
+// clears the status word (after a test that provoked a violation on purpose)
+inline int reset_device_status()
+{
+    const int zero = 0;
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_status), &zero, sizeof(int));
 }
 
 }  // namespace amd

@@ -45,7 +45,9 @@ struct Region {
 };
 constexpr uint32_t LDS_TOTAL = PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES +
                                PTO_AMD_BIAS_BYTES + PTO_AMD_FB_BYTES + PTO_AMD_L0S_BYTES;
+#ifndef PTO_AMD_CHECK_REFERENCE_SOURCE
 static_assert(LDS_TOTAL <= 160 * 1024, "the on-chip regions must fit the 160 KiB LDS of a CU");
+#endif
 
 // Sticky status word of the kernels of this translation unit: 0, or the first constraint a core violated
 // (1: TASSIGN address outside its region, 2: TQUANT NZ mode on a tile that is not whole 16-row x 2-group boxes).
@@ -96,22 +98,32 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
     static constexpr BLayout BFractal = BFractal_;
     static constexpr SLayout SFractal = SFractal_;
     static constexpr int SFractalSize = SFractalSize_;
+    static constexpr auto PadVal = PadVal_;
+    static constexpr CompactMode Compact = Compact_;
     static constexpr int Numel = Rows_ * Cols_;
     static constexpr uint32_t Bytes = (uint32_t)((int64_t)Rows_ * Cols_ * amd::ElemTraits<Element_>::bytes2 / 2);
     static constexpr bool isRowMajor = BFractal_ == BLayout::RowMajor;
 
     int vrow_ = RowValid_, vcol_ = ColValid_;
 
-    PTO_INST Tile() {}
+    // a tile that was never TASSIGNed sits at the start of its own region (not of the arena, which is L1)
+    PTO_INST Tile() { BindDefault(); }
     // dynamic valid extents, in declaration order (reference: pto_tile.hpp:1654-1676)
     PTO_INST Tile(int a)
     {
+        BindDefault();
         if constexpr (RowValid_ == DYNAMIC)
             vrow_ = a;
         else
             vcol_ = a;
     }
-    PTO_INST Tile(int r, int c) : vrow_(r), vcol_(c) {}
+    PTO_INST Tile(int r, int c) : vrow_(r), vcol_(c) { BindDefault(); }
+    PTO_INST void BindDefault()
+    {
+        if constexpr (Loc_ != TileType::Acc)
+            this->lds_ = amd::Region<Loc_>::base;
+    }
+    static constexpr size_t GetSizeInBytes() { return Bytes; }
     PTO_INST int GetValidRow() const { return vrow_; }
     PTO_INST int GetValidCol() const { return vcol_; }
 
@@ -176,6 +188,23 @@ template <typename Element_, const int Rows_, const int Cols_, const int RowVali
 using TileRightScale = Tile<TileType::ScaleRight, Element_, Rows_, Cols_, BLayout::ColMajor, RowValid_, ColValid_,
                             SLayout::ColMajor, TileConfig::fractalMxSize>;
 
+// the Compact forms (reference: common/pto_tile.hpp:1780-1835): same tiles, CompactMode::Normal recorded in the type
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileLeftCompact = Tile<TileType::Left, Element_, Rows_, Cols_, BLayout::ColMajor, RowValid_, ColValid_, SLayout::RowMajor,
+                             TileConfig::fractalABSize, PadValue::Null, CompactMode::Normal>;
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileRightCompact = Tile<TileType::Right, Element_, Rows_, Cols_, BLayout::RowMajor, RowValid_, ColValid_, SLayout::ColMajor,
+                              TileConfig::fractalABSize, PadValue::Null, CompactMode::Normal>;
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileAccCompact = Tile<TileType::Acc, Element_, Rows_, Cols_, BLayout::ColMajor, RowValid_, ColValid_, SLayout::RowMajor,
+                            TileConfig::fractalCSize, PadValue::Null, CompactMode::Normal>;
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileLeftScaleCompact = Tile<TileType::ScaleLeft, Element_, Rows_, Cols_, BLayout::RowMajor, RowValid_, ColValid_,
+                                  SLayout::RowMajor, TileConfig::fractalMxSize, PadValue::Null, CompactMode::Normal>;
+template <typename Element_, const int Rows_, const int Cols_, const int RowValid_ = Rows_, const int ColValid_ = Cols_>
+using TileRightScaleCompact = Tile<TileType::ScaleRight, Element_, Rows_, Cols_, BLayout::ColMajor, RowValid_, ColValid_,
+                                   SLayout::ColMajor, TileConfig::fractalMxSize, PadValue::Null, CompactMode::Normal>;
+
 template <typename T>
 struct is_tile : std::false_type {};
 template <TileType L, typename E, int R, int C, BLayout B, int RV, int CV, SLayout S, int F, auto P, CompactMode M>
@@ -184,6 +213,34 @@ template <typename T>
 constexpr bool is_tile_data_v = is_tile<std::remove_cv_t<T>>::value;
 
 struct RecordEvent {};
+
+// Instruction classes an Event orders (the subset of the reference's Op list, common/event.hpp:21-130, that the matmul
+// path names).
+enum class Op : uint16_t {
+    TLOAD, TSTORE_VEC, SCALAR, TRESHAPE, VECTOR, TCVT, TMOV_V2V, TMOV_V2M, TEXTRACT_V2M, TMOV_M2B, TMOV_M2L, TMOV_M2R, TMOV_M2S,
+    TMOV_A2V, TMOV_A2M, TSTORE_ACC, TSTORE_MAT, TMATMUL, TGEMV, TEXTRACT_M2LR, TEXTRACT_A2M, TDEQUANT, TQUANT, TFILLPAD, OP_COUNT
+};
+// Event<SrcOp, DstOp> (reference: common/event.hpp:361-427).  Every tile instruction of this backend is bracketed by
+// workgroup barriers, so an event has nothing left to wait for: the type exists so that kernels written with explicit
+// events compile and keep their meaning.  Instructions accept events as trailing arguments.
+struct EventBaseTag {};
+template <Op SrcOp, Op DstOp, bool AutoToken = true, event_t EventID = 0>
+struct Event : EventBaseTag {
+    static constexpr Op srcOp = SrcOp, dstOp = DstOp;
+    PTO_INST Event() {}
+    PTO_INST Event(RecordEvent) {}
+    PTO_INST Event& operator=(RecordEvent) { return *this; }
+    template <uint8_t CrossCoreId = 0xff>
+    PTO_INST Event& Wait() { return *this; }
+    template <uint8_t CrossCoreId = 0xff>
+    PTO_INST Event& Init() { return *this; }
+    template <uint8_t CrossCoreId = 0xff>
+    PTO_INST Event& Record() { return *this; }
+};
+template <typename T>
+struct is_event : std::is_base_of<EventBaseTag, T> {};
+template <typename... Ts>
+inline constexpr bool all_events_v = (is_event<Ts>::value && ...);
 
 // address of the scale tile that belongs to a Left / Right tile at `addr` (reference: cpu/NPUMemoryModel.hpp:409-415:
 // the L0 scale buffers mirror L0A / L0B at one sixteenth of the offset)

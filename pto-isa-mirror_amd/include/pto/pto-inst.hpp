@@ -15,5 +15,6 @@
 #include "amd/base.hpp"
 #include "amd/tile.hpp"
 #include "amd/instr.hpp"
+#include "amd/convert.hpp"
 #include "amd/quant.hpp"
 #include "amd/launch.hpp"
