@@ -7,6 +7,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <mutex>
 
 namespace ptoamd {
@@ -212,6 +213,14 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // LDS and need K to be a whole number of 128-byte slabs.  Measured on MI355X: the 8-wave 256x256 DMA tile (4) is the
 // fastest for every operand type once the grid fills the chip (the block-scaled types included: their scales come
 // through LDS, which leaves the 32-byte fp8 fragments just enough registers); smaller grids take the 128x128 DMA tile.
+// The DMA tiles address an operand as a wave-uniform 64-bit base plus a 32-bit per-lane byte offset: the last row's offset
+// plus the K extent must fit 32 bits, or the tile has to take the register-staged form (64-bit addresses per lane).
+static bool dma_offsets_fit(int m, int n, long lda_bytes, long ldb_bytes, long k_bytes)
+{
+    const long last = std::max((long)(m - 1) * lda_bytes, (long)(n - 1) * ldb_bytes) + k_bytes;
+    return last <= (long)UINT32_MAX;
+}
+
 static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, bool scale_dma_ok = true)
 {
     const bool dtl_ok = (k_bytes % 128) == 0 && scale_dma_ok;
@@ -437,7 +446,7 @@ int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_t
                    : ab_type == PTOAMD_F16 ? TOP_F16
                    : ab_type == PTOAMD_I8 ? TOP_I8
                    : ab_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E5E5;
-    const int tile = pick_tile(m, n, k_bytes, false);
+    const int tile = pick_tile(m, n, k_bytes, false, false, dma_offsets_fit(m, n, lda_b, ldb_kmajor, k_bytes));
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;
@@ -480,7 +489,7 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
     p.c = out_bf16; p.acc_out = acc_out; p.row_scale = scale_a; p.col_scale = scale_b;
     p.m = m; p.n = n; p.k_bytes = k; p.lda_bytes = lda; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
     p.out_kind = OUT_W8A8_BF16; p.group_m = 4;
-    const int tile = pick_tile(m, n, k, false);
+    const int tile = pick_tile(m, n, k, false, false, dma_offsets_fit(m, n, lda, ldb_kmajor, k));
     PTOAMD_HIP_CHECK(launch_tiles(tile, TOP_I8, p, stream));
     set_last_kernel(tile_kernel_name(tile, TOP_I8));
     return PTOAMD_OK;
@@ -580,7 +589,7 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
     // the DMA tiles fetch scales as 16-byte chunks per row: 4 slabs of fp8, 2 of fp4
     const long k_slabs = k_bytes / 128;
     const bool scale_dma_ok = (kg % 16) == 0 && aligned16(sa_nd) && aligned16(sb_dn) && (k_slabs % (a4 ? 2 : 4)) == 0;
-    const int tile = pick_tile(m, n, k_bytes, true, a4, scale_dma_ok);
+    const int tile = pick_tile(m, n, k_bytes, true, a4, scale_dma_ok && dma_offsets_fit(m, n, lda_b, ldb_b, k_bytes));
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;

@@ -11,6 +11,7 @@
 // the other buffer; one __syncthreads per slab replaces the MTE2/MTE1/M event chain of the reference kernels
 // (kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:115-150).
 #pragma once
+#include <type_traits>
 #include "device_types.hpp"
 #include "lds_dma.hpp"
 
@@ -187,54 +188,90 @@ struct TileCfg {
 // of one block only.  A dispatch around the whole loop keeps every accumulator live across the branch, which with 128
 // or 256 accumulator registers per lane pushes them through scratch memory.  The TMATMUL_ACC input is folded in here:
 // C = Cin + A.B.
-template <int KIND, bool FULL, class Cfg, class Acc>
-__device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi)
+// The optional terms (accumulator input, bias row, relu) are applied in passes over the block's 16 registers, one
+// wave-uniform branch per term and block; tested per element they turn the epilogue into thousands of basic blocks,
+// hundreds of KiB of code, and the instruction fetch -- not the stores -- sets its duration.
+template <bool FULL, class Cfg, class Acc>
+__device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int row_b, int gj, int lhi)
 {
     using Elem = typename Cfg::Op::Elem;
     const Elem* cin = reinterpret_cast<const Elem*>(p.c_in);
+    if (cin != nullptr) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int gi = row_b + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            if (FULL || (gi < p.m && gj < p.n))
+                v[r] += cin[(long)gi * p.ldc + gj];
+        }
+    }
+    if (p.bias != nullptr) {
+        const Elem bias_j = (FULL || gj < p.n) ? reinterpret_cast<const Elem*>(p.bias)[gj] : Elem(0);
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            v[r] += bias_j;
+    }
+    if (p.relu) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            v[r] = v[r] > 0 ? v[r] : 0;
+    }
+    return v;
+}
+
+template <int KIND, bool FULL, class Cfg, class Acc>
+__device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi)
+{
     const int gj = col_b + l32;
     float cs = 1.0f;
     if (KIND == OUT_W8A8_BF16)
         cs = (FULL || gj < p.n) ? p.col_scale[gj] : 0.0f;
-    const Elem bias_j = (p.bias != nullptr && (FULL || gj < p.n)) ? reinterpret_cast<const Elem*>(p.bias)[gj] : Elem(0);
+    const Acc v = tstore_terms<FULL, Cfg>(p, acc, row_b, gj, lhi);
+    const bool raw = KIND == OUT_W8A8_BF16 && p.acc_out != nullptr;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int gi = row_b + 8 * (r >> 2) + 4 * lhi + (r & 3);
         if (FULL || (gi < p.m && gj < p.n)) {
             const long o = (long)gi * p.ldc + gj;
-            auto v = acc[r];
-            if (cin != nullptr)
-                v += cin[o];
-            v += bias_j;
-            if (p.relu)
-                v = v > 0 ? v : 0;
             if (KIND == OUT_F32) {
-                reinterpret_cast<float*>(p.c)[o] = (float)v;
+                reinterpret_cast<float*>(p.c)[o] = (float)v[r];
             } else if (KIND == OUT_F16) {
-                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits((float)v);
+                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits((float)v[r]);
             } else if (KIND == OUT_BF16) {
-                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits((float)v);
+                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits((float)v[r]);
             } else if (KIND == OUT_I32) {
-                reinterpret_cast<int32_t*>(p.c)[o] = (int32_t)v;
+                reinterpret_cast<int32_t*>(p.c)[o] = (int32_t)v[r];
             } else {  // W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16, each step rounded to f32
-                if (p.acc_out != nullptr)
-                    p.acc_out[o] = (int32_t)v;
-                const float t = __fmul_rn((float)v, p.row_scale[gi]);
+                const float t = __fmul_rn((float)v[r], p.row_scale[gi]);
                 reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(__fmul_rn(t, cs));
             }
         }
     }
+    if (raw) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int gi = row_b + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            if (FULL || (gi < p.m && gj < p.n))
+                p.acc_out[(long)gi * p.ldc + gj] = (int32_t)v[r];
+        }
+    }
 }
 
+// float accumulators drain to f32 / f16 / bf16, int32 accumulators to int32 or (W8A8) scaled bf16: only those forms are
+// compiled for an operand type (the host rejects the other combinations)
 template <bool FULL, class Cfg, class Acc>
 __device__ __forceinline__ void tstore_block_kind(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi)
 {
-    switch (p.out_kind) {
-        case OUT_F32: tstore_block<OUT_F32, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
-        case OUT_F16: tstore_block<OUT_F16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
-        case OUT_BF16: tstore_block<OUT_BF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
-        case OUT_I32: tstore_block<OUT_I32, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
-        default: tstore_block<OUT_W8A8_BF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
+    if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
+        if (p.out_kind == OUT_I32)
+            tstore_block<OUT_I32, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
+        else
+            tstore_block<OUT_W8A8_BF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
+    } else {
+        switch (p.out_kind) {
+            case OUT_F32: tstore_block<OUT_F32, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
+            case OUT_F16: tstore_block<OUT_F16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
+            default: tstore_block<OUT_BF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi); break;
+        }
     }
 }
 
@@ -258,30 +295,21 @@ template <int KIND, class Cfg, class Acc>
 __device__ __forceinline__ void tstage_block(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi,
                                              uint8_t* lane_base)
 {
-    using Elem = typename Cfg::Op::Elem;
-    const Elem* cin = reinterpret_cast<const Elem*>(p.c_in);
     const int gj = col_b + l32;
     float cs = 1.0f;
     if (KIND == OUT_W8A8_BF16)
         cs = p.col_scale[gj];
-    const Elem bias_j = p.bias != nullptr ? reinterpret_cast<const Elem*>(p.bias)[gj] : Elem(0);
+    const Acc v = tstore_terms<true, Cfg>(p, acc, row_b, gj, lhi);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int lr = 8 * (r >> 2) + 4 * lhi + (r & 3);
-        const int gi = row_b + lr;
-        auto v = acc[r];
-        if (cin != nullptr)
-            v += cin[(long)gi * p.ldc + gj];
-        v += bias_j;
-        if (p.relu)
-            v = v > 0 ? v : 0;
         uint16_t bits;
         if (KIND == OUT_F16) {
-            bits = f32_to_f16_bits((float)v);
+            bits = f32_to_f16_bits((float)v[r]);
         } else if (KIND == OUT_BF16) {
-            bits = f32_to_bf16_bits((float)v);
+            bits = f32_to_bf16_bits((float)v[r]);
         } else {
-            const float t = __fmul_rn((float)v, p.row_scale[gi]);
+            const float t = __fmul_rn((float)v[r], p.row_scale[row_b + lr]);
             bits = f32_to_bf16_bits(__fmul_rn(t, cs));
         }
         *reinterpret_cast<uint16_t*>(lane_base + lr * StagedStore<Cfg>::ROW_BYTES) = bits;
@@ -303,10 +331,13 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
             __builtin_amdgcn_sched_barrier(0);
             const Acc block = acc[i][j];
             uint8_t* lane_base = stage + (j * 32 + l32) * 2;
-            switch (p.out_kind) {
-                case OUT_F16: tstage_block<OUT_F16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base); break;
-                case OUT_BF16: tstage_block<OUT_BF16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base); break;
-                default: tstage_block<OUT_W8A8_BF16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base); break;
+            if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
+                tstage_block<OUT_W8A8_BF16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base);
+            } else {
+                if (p.out_kind == OUT_F16)
+                    tstage_block<OUT_F16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base);
+                else
+                    tstage_block<OUT_BF16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base);
             }
         });
         __builtin_amdgcn_sched_barrier(0);
@@ -317,7 +348,11 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
             typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
             nt_u32x4* dst = reinterpret_cast<nt_u32x4*>(reinterpret_cast<uint8_t*>(p.c) + ((long)(row0 + i * 32 + row) * p.ldc + col0 + ch * 8) * 2);
             const nt_u32x4 vv = {v.x, v.y, v.z, v.w};
+#ifdef PTOAMD_PLAIN_C_STORES
+            *dst = vv;
+#else
             __builtin_nontemporal_store(vv, dst);  // C is not read again by this kernel: keep it out of the L2's way
+#endif
         }
     });
 }
