@@ -41,6 +41,10 @@ struct TileGemmParams {
 enum OutKind { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2, OUT_I32 = 3, OUT_W8A8_BF16 = 4 };
 
 // ---- MFMA operand traits ------------------------------------------------------------------------------------
+// Every mma() hands the matrix instruction B's fragment as its first operand and A's as its second, so a 32x32
+// accumulator block comes out transposed: lane (l32, lhi) holds row l32 of the block and register r its column
+// 8 (r / 4) + 4 lhi + r % 4 -- four consecutive columns per register quad, which the epilogue packs into one 8- or
+// 16-byte piece of an output row.  The sums themselves are the same (products commute, k runs in the same order).
 // FRAG_BYTES: operand bytes one lane feeds one MFMA; a k-step spans 2 * FRAG_BYTES of a slab row (lanes 0-31 take
 // the first half, lanes 32-63 the second), so a 128-byte slab is 128 / (2 * FRAG_BYTES) k-steps.
 struct OpBF16 {
@@ -51,7 +55,7 @@ struct OpBF16 {
     static constexpr int GROUPS_PER_SLAB = 0;
     __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t, uint32_t)
     {
-        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[0]), __builtin_bit_cast(bf16x8, b[0]),
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, b[0]), __builtin_bit_cast(bf16x8, a[0]),
                                                     c, 0, 0, 0);
     }
     template <int SEL>
@@ -68,7 +72,7 @@ struct OpF16 {
     static constexpr int GROUPS_PER_SLAB = 0;
     __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t, uint32_t)
     {
-        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b[0]), c,
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, b[0]), __builtin_bit_cast(f16x8, a[0]), c,
                                                    0, 0, 0);
     }
     template <int SEL>
@@ -85,7 +89,7 @@ struct OpI8 {
     static constexpr int GROUPS_PER_SLAB = 0;
     __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t, uint32_t)
     {
-        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a[0]), __builtin_bit_cast(i32x4, b[0]), c,
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, b[0]), __builtin_bit_cast(i32x4, a[0]), c,
                                                   0, 0, 0);
     }
     template <int SEL>
@@ -110,7 +114,7 @@ struct OpFP8 {
         av.s4 = a[1].x; av.s5 = a[1].y; av.s6 = a[1].z; av.s7 = a[1].w;
         bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
         bv.s4 = b[1].x; bv.s5 = b[1].y; bv.s6 = b[1].z; bv.s7 = b[1].w;
-        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, AFMT, BFMT, 0, (int)sa, 0, (int)sb);
+        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, BFMT, AFMT, 0, (int)sb, 0, (int)sa);
     }
     // the scales are byte SEL of the dwords sa / sb (the instruction's own byte select: no VALU extraction)
     template <int SEL>
@@ -121,7 +125,7 @@ struct OpFP8 {
         av.s4 = a[1].x; av.s5 = a[1].y; av.s6 = a[1].z; av.s7 = a[1].w;
         bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
         bv.s4 = b[1].x; bv.s5 = b[1].y; bv.s6 = b[1].z; bv.s7 = b[1].w;
-        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, AFMT, BFMT, SEL, (int)sa, SEL, (int)sb);
+        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, BFMT, AFMT, SEL, (int)sb, SEL, (int)sa);
     }
 };
 // fp4 E2M1 (format 4): 32 elements = 16 bytes per lane = one MX group
@@ -136,7 +140,7 @@ struct OpFP4 {
         i32x8 av = {0, 0, 0, 0, 0, 0, 0, 0}, bv = {0, 0, 0, 0, 0, 0, 0, 0};
         av.s0 = a[0].x; av.s1 = a[0].y; av.s2 = a[0].z; av.s3 = a[0].w;
         bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
-        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 4, 4, 0, (int)sa, 0, (int)sb);
+        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, 4, 4, 0, (int)sb, 0, (int)sa);
     }
     template <int SEL>
     __device__ static __forceinline__ void mma_sel(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
@@ -144,7 +148,7 @@ struct OpFP4 {
         i32x8 av = {0, 0, 0, 0, 0, 0, 0, 0}, bv = {0, 0, 0, 0, 0, 0, 0, 0};
         av.s0 = a[0].x; av.s1 = a[0].y; av.s2 = a[0].z; av.s3 = a[0].w;
         bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
-        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 4, 4, SEL, (int)sa, SEL, (int)sb);
+        c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, 4, 4, SEL, (int)sb, SEL, (int)sa);
     }
 };
 
@@ -188,27 +192,33 @@ struct TileCfg {
 // of one block only.  A dispatch around the whole loop keeps every accumulator live across the branch, which with 128
 // or 256 accumulator registers per lane pushes them through scratch memory.  The TMATMUL_ACC input is folded in here:
 // C = Cin + A.B.
+// column (inside its 32x32 block) of accumulator register r of a lane in half lhi
+__device__ __forceinline__ constexpr int acc_col(int r, int lhi) { return 8 * (r >> 2) + 4 * lhi + (r & 3); }
+
 // The optional terms (accumulator input, bias row, relu) are applied in passes over the block's 16 registers, one
 // wave-uniform branch per term and block; tested per element they turn the epilogue into thousands of basic blocks,
 // hundreds of KiB of code, and the instruction fetch -- not the stores -- sets its duration.
+// gi: the lane's row of C; col_b: first column of the block.
 template <bool FULL, class Cfg, class Acc>
-__device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int row_b, int gj, int lhi)
+__device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int gi, int col_b, int lhi)
 {
     using Elem = typename Cfg::Op::Elem;
     const Elem* cin = reinterpret_cast<const Elem*>(p.c_in);
     if (cin != nullptr) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int gi = row_b + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            const int gj = col_b + acc_col(r, lhi);
             if (FULL || (gi < p.m && gj < p.n))
                 v[r] += cin[(long)gi * p.ldc + gj];
         }
     }
     if (p.bias != nullptr) {
-        const Elem bias_j = (FULL || gj < p.n) ? reinterpret_cast<const Elem*>(p.bias)[gj] : Elem(0);
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-            v[r] += bias_j;
+        for (int r = 0; r < 16; ++r) {
+            const int gj = col_b + acc_col(r, lhi);
+            if (FULL || gj < p.n)
+                v[r] += reinterpret_cast<const Elem*>(p.bias)[gj];
+        }
     }
     if (p.relu) {
 #pragma unroll
@@ -218,40 +228,46 @@ __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int 
     return v;
 }
 
+// bits of one output element (2-byte kinds in the low half); W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16, each
+// step rounded to f32
+template <int KIND, class V>
+__device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs)
+{
+    if (KIND == OUT_F32)
+        return __builtin_bit_cast(uint32_t, (float)v);
+    if (KIND == OUT_I32)
+        return (uint32_t)(int32_t)v;
+    if (KIND == OUT_F16)
+        return f32_to_f16_bits((float)v);
+    if (KIND == OUT_BF16)
+        return f32_to_bf16_bits((float)v);
+    return f32_to_bf16_bits(__fmul_rn(__fmul_rn((float)v, rs), cs));
+}
+template <int KIND>
+constexpr int out_bytes = (KIND == OUT_F32 || KIND == OUT_I32) ? 4 : 2;
+
+// Element-wise form: any alignment, any edge.  A lane's elements are 4-column runs of one row, so this form is slow
+// (short scattered stores); whole, aligned wave tiles take the staged form below.
 template <int KIND, bool FULL, class Cfg, class Acc>
 __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi)
 {
-    const int gj = col_b + l32;
-    float cs = 1.0f;
-    if (KIND == OUT_W8A8_BF16)
-        cs = (FULL || gj < p.n) ? p.col_scale[gj] : 0.0f;
-    const Acc v = tstore_terms<FULL, Cfg>(p, acc, row_b, gj, lhi);
+    const int gi = row_b + l32;
+    const float rs = (KIND == OUT_W8A8_BF16 && (FULL || gi < p.m)) ? p.row_scale[gi] : 1.0f;
+    const Acc v = tstore_terms<FULL, Cfg>(p, acc, gi, col_b, lhi);
     const bool raw = KIND == OUT_W8A8_BF16 && p.acc_out != nullptr;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int gi = row_b + 8 * (r >> 2) + 4 * lhi + (r & 3);
+        const int gj = col_b + acc_col(r, lhi);
         if (FULL || (gi < p.m && gj < p.n)) {
             const long o = (long)gi * p.ldc + gj;
-            if (KIND == OUT_F32) {
-                reinterpret_cast<float*>(p.c)[o] = (float)v[r];
-            } else if (KIND == OUT_F16) {
-                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits((float)v[r]);
-            } else if (KIND == OUT_BF16) {
-                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits((float)v[r]);
-            } else if (KIND == OUT_I32) {
-                reinterpret_cast<int32_t*>(p.c)[o] = (int32_t)v[r];
-            } else {  // W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16, each step rounded to f32
-                const float t = __fmul_rn((float)v[r], p.row_scale[gi]);
-                reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(__fmul_rn(t, cs));
-            }
-        }
-    }
-    if (raw) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int gi = row_b + 8 * (r >> 2) + 4 * lhi + (r & 3);
-            if (FULL || (gi < p.m && gj < p.n))
-                p.acc_out[(long)gi * p.ldc + gj] = (int32_t)v[r];
+            const float cs = KIND == OUT_W8A8_BF16 ? p.col_scale[gj] : 1.0f;
+            const uint32_t bits = tstore_bits<KIND>(v[r], rs, cs);
+            if (out_bytes<KIND> == 4)
+                reinterpret_cast<uint32_t*>(p.c)[o] = bits;
+            else
+                reinterpret_cast<uint16_t*>(p.c)[o] = (uint16_t)bits;
+            if (raw)
+                p.acc_out[o] = (int32_t)v[r];
         }
     }
 }
@@ -275,97 +291,96 @@ __device__ __forceinline__ void tstore_block_kind(const TileGemmParams& p, const
     }
 }
 
-// ---- TSTORE of 16-bit outputs through LDS ---------------------------------------------------------------------------
-// An accumulator register holds one column of the block per lane, so storing it directly writes 2 bytes per lane
-// (64-byte row pieces, 16 store instructions per block) and the store unit's per-lane rate, not HBM, bounds the
-// epilogue.  Here a wave converts one 32-row band of its tile into a private, padded LDS region with the same fix-pipe
-// arithmetic, reads it back as 16-byte row chunks and writes whole 128-byte (or longer) row pieces.  LDS operations of
-// one wave execute in order, so the region is reused for the next band without a barrier.
+// ---- TSTORE through LDS ------------------------------------------------------------------------------------------------
+// A wave converts one 32-row band of its tile into a private, padded LDS region -- a lane writes its four consecutive
+// columns of a register quad as one 8-byte (16-bit outputs) or 16-byte (32-bit outputs) piece -- reads the band back as
+// 16-byte row chunks and stores whole row pieces of the wave tile's width.  LDS operations of one wave execute in
+// order, so the region is reused for the next band without a barrier.
 template <class Cfg>
 struct StagedStore {
-    static constexpr int ROW_BYTES = Cfg::WTN * 2 + 16;        // the pad keeps lanes 32-63 (rows + 4) off lanes 0-31's banks
-    static constexpr int WAVE_BYTES = 32 * ROW_BYTES;
-    static constexpr int CHUNKS = Cfg::WTN / 8;                // 16-byte chunks per row
-    static constexpr int ITERS = 32 * CHUNKS / 64;             // chunks per lane per band
+    // sized for 4-byte outputs; the 16 pad bytes per row keep the 32 rows a band's lanes write off each other's banks
+    static constexpr int WAVE_BYTES = 32 * (Cfg::WTN * 4 + 16);
     static_assert(Cfg::THREADS / 64 * WAVE_BYTES <= Cfg::LDS_BYTES, "staging regions fit in the operand ring");
-    static_assert((32 * CHUNKS) % 64 == 0, "a band is a whole number of 64-lane reads");
+    static_assert((32 * Cfg::WTN * 2 / 16) % 64 == 0, "a band is a whole number of 64-lane reads");
 };
 
-template <int KIND, class Cfg, class Acc>
-__device__ __forceinline__ void tstage_block(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi,
-                                             uint8_t* lane_base)
-{
-    const int gj = col_b + l32;
-    float cs = 1.0f;
-    if (KIND == OUT_W8A8_BF16)
-        cs = p.col_scale[gj];
-    const Acc v = tstore_terms<true, Cfg>(p, acc, row_b, gj, lhi);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int lr = 8 * (r >> 2) + 4 * lhi + (r & 3);
-        uint16_t bits;
-        if (KIND == OUT_F16) {
-            bits = f32_to_f16_bits((float)v[r]);
-        } else if (KIND == OUT_BF16) {
-            bits = f32_to_bf16_bits((float)v[r]);
-        } else {
-            const float t = __fmul_rn((float)v[r], p.row_scale[row_b + lr]);
-            bits = f32_to_bf16_bits(__fmul_rn(t, cs));
-        }
-        *reinterpret_cast<uint16_t*>(lane_base + lr * StagedStore<Cfg>::ROW_BYTES) = bits;
-    }
-}
-
 // `stage` is the calling wave's private LDS region of StagedStore<Cfg>::WAVE_BYTES bytes; the wave's tile lies inside
-// the matrix and rows of C start on 16-byte boundaries (checked by the caller)
-template <class Cfg, class Acc>
+// the matrix and its rows of C start on 16-byte boundaries (checked by the caller)
+template <int KIND, class Cfg, class Acc>
 __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0,
                                               int l32, int lhi, uint8_t* stage)
 {
-    using S = StagedStore<Cfg>;
+    constexpr int ESZ = out_bytes<KIND>;
+    constexpr int ROW_BYTES = Cfg::WTN * ESZ + 16, CHUNKS = Cfg::WTN * ESZ / 16, ITERS = 32 * CHUNKS / 64;
     const int lane = lhi * 32 + l32;
     static_for<Cfg::MB>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
+        const int gi = row0 + i * 32 + l32;
+        const float rs = KIND == OUT_W8A8_BF16 ? p.row_scale[gi] : 1.0f;
         static_for<Cfg::NB>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             __builtin_amdgcn_sched_barrier(0);
-            const Acc block = acc[i][j];
-            uint8_t* lane_base = stage + (j * 32 + l32) * 2;
-            if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
-                tstage_block<OUT_W8A8_BF16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base);
-            } else {
-                if (p.out_kind == OUT_F16)
-                    tstage_block<OUT_F16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base);
-                else
-                    tstage_block<OUT_BF16, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi, lane_base);
+            const int col_b = col0 + j * 32;
+            const Acc v = tstore_terms<true, Cfg>(p, acc[i][j], gi, col_b, lhi);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint8_t* dst = stage + l32 * ROW_BYTES + (j * 32 + 8 * g + 4 * lhi) * ESZ;
+                if constexpr (KIND == OUT_BF16 || KIND == OUT_W8A8_BF16) {  // packed conversion: one instruction per pair
+                    float f[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        f[e] = (float)v[4 * g + e];
+                        if (KIND == OUT_W8A8_BF16)
+                            f[e] = __fmul_rn(__fmul_rn(f[e], rs), p.col_scale[col_b + 8 * g + 4 * lhi + e]);
+                    }
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(f32x2_to_bf16x2_bits(f[0], f[1]), f32x2_to_bf16x2_bits(f[2], f[3]));
+                } else {
+                    uint32_t bits[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f);
+                    if (ESZ == 4)
+                        *reinterpret_cast<uint4*>(dst) = make_uint4(bits[0], bits[1], bits[2], bits[3]);
+                    else
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16));
+                }
             }
         });
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int it = 0; it < S::ITERS; ++it) {
-            const int q = it * 64 + lane, row = q / S::CHUNKS, ch = q % S::CHUNKS;
-            const uint4 v = *reinterpret_cast<const uint4*>(stage + row * S::ROW_BYTES + ch * 16);
+        for (int it = 0; it < ITERS; ++it) {
+            const int q = it * 64 + lane, row = q / CHUNKS, ch = q % CHUNKS;
+            const uint4 v = *reinterpret_cast<const uint4*>(stage + row * ROW_BYTES + ch * 16);
             typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
-            nt_u32x4* dst = reinterpret_cast<nt_u32x4*>(reinterpret_cast<uint8_t*>(p.c) + ((long)(row0 + i * 32 + row) * p.ldc + col0 + ch * 8) * 2);
+            nt_u32x4* dst = reinterpret_cast<nt_u32x4*>(reinterpret_cast<uint8_t*>(p.c) +
+                                                        ((long)(row0 + i * 32 + row) * p.ldc + col0) * ESZ + ch * 16);
             const nt_u32x4 vv = {v.x, v.y, v.z, v.w};
-#ifdef PTOAMD_PLAIN_C_STORES
-            *dst = vv;
-#else
             __builtin_nontemporal_store(vv, dst);  // C is not read again by this kernel: keep it out of the L2's way
-#endif
         }
     });
 }
 
-// `stage`: the wave's private LDS region for the staged form, free of other uses from here on; nullptr = direct stores
+// `stage`: the wave's private LDS region for the staged form, free of other uses from here on; nullptr = element-wise
 template <class Cfg, class Acc>
 __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0, int l32,
                                        int lhi, uint8_t* stage = nullptr)
 {
     const bool full = row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n;
-    const bool two_byte = p.out_kind == OUT_F16 || p.out_kind == OUT_BF16 || (p.out_kind == OUT_W8A8_BF16 && p.acc_out == nullptr);
-    if (stage != nullptr && full && two_byte && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0) {
-        tstore_staged<Cfg>(p, acc, row0, col0, l32, lhi, stage);
+    const int esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : 2;
+    const bool aligned = (((long)p.ldc * esz) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
+    if (stage != nullptr && full && aligned && !(p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr)) {
+        if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
+            if (p.out_kind == OUT_I32)
+                tstore_staged<OUT_I32, Cfg>(p, acc, row0, col0, l32, lhi, stage);
+            else
+                tstore_staged<OUT_W8A8_BF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
+        } else {
+            switch (p.out_kind) {
+                case OUT_F32: tstore_staged<OUT_F32, Cfg>(p, acc, row0, col0, l32, lhi, stage); break;
+                case OUT_F16: tstore_staged<OUT_F16, Cfg>(p, acc, row0, col0, l32, lhi, stage); break;
+                default: tstore_staged<OUT_BF16, Cfg>(p, acc, row0, col0, l32, lhi, stage); break;
+            }
+        }
         return;
     }
     static_for<Cfg::MB * Cfg::NB>([&](auto bc) {

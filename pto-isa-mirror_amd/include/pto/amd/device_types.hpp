@@ -27,6 +27,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
     return (uint16_t)((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
 }
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+// two floats -> two bf16 in one dword (a in the low half): v_cvt_pk_bf16_f32, round to nearest even, NaNs stay quiet NaNs
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float a, float b)
+{
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 
 // float -> fp16 bits, round to nearest even (v_cvt_f16_f32 under the default rounding mode)
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f)

@@ -120,6 +120,37 @@ def test_bf16_gemm_every_tile_shape(pa, oracle, tile, m, n, k):
     assert np.array_equal(got16, oracle.store_f32(got32, ob.ST_BF16))
 
 
+@pytest.mark.parametrize("tile", [2, 4, 5])
+def test_bf16_store_of_special_values(pa, oracle, tile):
+    """The staged TSTORE converts pairs with the packed hardware conversion: infinities, overflow to infinity, NaN,
+    zeros of both signs and values that round up into the next binade come out as the oracle's conversion gives them."""
+    m, n, k = 256, 256, 128
+    r = np.random.default_rng(17)
+    a = r.standard_normal((m, k)).astype(np.float32)
+    b = r.standard_normal((n, k)).astype(np.float32)
+    a[0, 0] = np.inf                       # +-inf rows
+    a[1, 0] = np.nan                       # NaN row
+    a[2, :] = 3.0e19                       # with the columns below: overflow to inf in the fp32 accumulator
+    b[0, :] = 3.0e19
+    a[3, :] = 0.0                          # exact zeros
+    a[4, :], b[1, :] = 1.0, 0.0
+    a[4, 0], b[1, 0] = 1.0, 1.0 + 2.0 ** -7  # 1 + 2^-7 is a bf16 value; the row below makes ties and near-overflow
+    a[5, :], b[2, :] = 0.0, 0.0
+    a[5, 0], a[5, 1], b[2, 0], b[2, 1] = 1.0, 2.0 ** -8, 1.0, 1.0   # 1 + 2^-8: a tie, rounds to even (1.0)
+    a[6, :], b[3, :] = 0.0, 0.0
+    a[6, 0], a[6, 1], b[3, 0], b[3, 1] = 2.0 ** 127, 2.0 ** 127, 1.0, 0.99609375  # 2^127 * 1.996: rounds up to inf
+    ab, bb = bf16_bits(a), bf16_bits(b)
+    with tile_env(PTOAMD_TILE=tile):
+        got32 = host(pa.gemm(dev(ab).view(torch.bfloat16), dev(bb).view(torch.bfloat16), pa.BF16, pa.F32, pa.B_DN))
+        got16 = host(pa.gemm(dev(ab).view(torch.bfloat16), dev(bb).view(torch.bfloat16), pa.BF16, pa.BF16, pa.B_DN))
+    want = oracle.store_f32(got32, ob.ST_BF16)
+    nan = np.isnan(got32)
+    assert nan[1].all() and np.isinf(got32[0]).any() and np.isinf(got32[2, 0])
+    assert np.array_equal(got16[~nan], want[~nan])
+    assert ((got16[nan] & 0x7FFF) > 0x7F80).all()  # NaN stays NaN (the payload is not part of the contract)
+    assert got16[5, 2] == 0x3F80 and got16[6, 3] == 0x7F80
+
+
 def test_gemm_golden_fixtures(pa, golden):
     g = golden
     a, bt, cin = g["mm_f16_a"], g["mm_f16_bt"], g["mm_f16_cin"]
