@@ -426,7 +426,12 @@ int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_t
     StreamTemp bt(stream);
     const uint8_t* b_kmajor = reinterpret_cast<const uint8_t*>(b);
     long ldb_kmajor = ldb_b;
-    if (b_layout == PTOAMD_B_ND) {  // TLOAD of an ND B panel: re-order once so the MFMA path reads K-contiguous rows
+    // A row-major B with few output row-tiles is transposed on its way into LDS by the register-staged tiles (no
+    // temporary, one launch).  With many row-tiles every element of B would be scattered into LDS that many times, and
+    // the DMA tiles cannot do it at all: then B is re-ordered once in global memory and read K-contiguous from there.
+    const bool b_in_kernel = b_layout == PTOAMD_B_ND && m <= 1024 && (ebytes == 1 || ebytes == 2) && (n % (16 / ebytes)) == 0 &&
+                             (ldb_b % 16) == 0 && getenv("PTOAMD_B_ND_TRANSPOSE") == nullptr;
+    if (b_layout == PTOAMD_B_ND && !b_in_kernel) {  // TLOAD of an ND B panel: re-order once so the MFMA path reads K-contiguous rows
         PTOAMD_HIP_CHECK(bt.alloc((size_t)n * k_bytes));
         const int rc = ebytes == 2 ? transpose_b<uint16_t>(bt.ptr, b, k, n, ldb, stream)
                                    : transpose_b<uint8_t>(bt.ptr, b, k, n, ldb, stream);
@@ -446,7 +451,8 @@ int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_t
                    : ab_type == PTOAMD_F16 ? TOP_F16
                    : ab_type == PTOAMD_I8 ? TOP_I8
                    : ab_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E5E5;
-    const int tile = pick_tile(m, n, k_bytes, false, false, dma_offsets_fit(m, n, lda_b, ldb_kmajor, k_bytes));
+    p.b_nd = b_in_kernel; p.b_esz = ebytes;
+    const int tile = pick_tile(m, n, k_bytes, false, false, !b_in_kernel && dma_offsets_fit(m, n, lda_b, ldb_kmajor, k_bytes));
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;
@@ -475,7 +481,9 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
     StreamTemp bt(stream);
     const uint8_t* b_kmajor = reinterpret_cast<const uint8_t*>(b);
     long ldb_kmajor = ldb;
-    if (b_layout == PTOAMD_B_ND) {
+    const bool b_in_kernel = b_layout == PTOAMD_B_ND && m <= 1024 && (n % 16) == 0 && (ldb % 16) == 0 &&
+                             getenv("PTOAMD_B_ND_TRANSPOSE") == nullptr;  // (same rule as ptoamd_gemm)
+    if (b_layout == PTOAMD_B_ND && !b_in_kernel) {
         PTOAMD_HIP_CHECK(bt.alloc((size_t)n * k));
         const int rc = transpose_b<uint8_t>(bt.ptr, b, k, n, ldb, stream);
         if (rc != PTOAMD_OK)
@@ -489,19 +497,19 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
     p.c = out_bf16; p.acc_out = acc_out; p.row_scale = scale_a; p.col_scale = scale_b;
     p.m = m; p.n = n; p.k_bytes = k; p.lda_bytes = lda; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
     p.out_kind = OUT_W8A8_BF16; p.group_m = 4;
-    const int tile = pick_tile(m, n, k, false, false, dma_offsets_fit(m, n, lda, ldb_kmajor, k));
+    p.b_nd = b_in_kernel; p.b_esz = 1;
+    const int tile = pick_tile(m, n, k, false, false, !b_in_kernel && dma_offsets_fit(m, n, lda, ldb_kmajor, k));
     PTOAMD_HIP_CHECK(launch_tiles(tile, TOP_I8, p, stream));
     set_last_kernel(tile_kernel_name(tile, TOP_I8));
     return PTOAMD_OK;
 }
 
-// Shared body of the TMATMUL_MX entry points.  The MFMA kernels stream scales as [M][K/32] and [N][K/32]; other GM layouts
-// are re-laid first, into `ws` (ws_bytes; the caller's workspace or the library's static array) when one is given, else
-// into a stream-ordered allocation.
+// Shared body of the TMATMUL_MX entry points.  The DMA tiles stream scales as [M][K/32] and [N][K/32] rows; other GM
+// layouts are re-laid into `ws` (ws_bytes; the caller's workspace or the library's static array) when one is given, and
+// addressed in place by the register-staged tiles when not.
 static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, const void* b, int a_type, int b_type,
                           const uint8_t* sa, const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n,
-                          int k, int lda, int ldb, int ldc, int b_layout, uint8_t* ws, size_t ws_bytes, bool may_allocate,
-                          void* stream_)
+                          int k, int lda, int ldb, int ldc, int b_layout, uint8_t* ws, size_t ws_bytes, void* stream_)
 {
     hipStream_t stream = as_stream(stream_);
     PTOAMD_REQUIRE(c && a && b && sa && sb, PTOAMD_E_INVALID, "%s: null operand", who);
@@ -527,7 +535,9 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
     const int bits = a8 ? 8 : 4;
     const long k_bytes = (long)k * bits / 8, lda_b = (long)lda * bits / 8, ldb_b = (long)ldb * bits / 8;
     const bool e1m2 = a_type == PTOAMD_E1M2 || b_type == PTOAMD_E1M2;  // the scaled MFMA has no E1M2 format
-    const bool tile_ok = !force_generic() && !e1m2 && b_layout == PTOAMD_B_DN && aligned16(a) && aligned16(b) &&
+    // a row-major B of one-byte codes is transposed on its way into LDS by the register-staged tiles; packed fp4 is not
+    const bool b_in_kernel = b_layout == PTOAMD_B_ND && a8 && (n % 16) == 0;
+    const bool tile_ok = !force_generic() && !e1m2 && (b_layout == PTOAMD_B_DN || b_in_kernel) && aligned16(a) && aligned16(b) &&
                          (lda_b % 16) == 0 && (ldb_b % 16) == 0 && (k_bytes % 128) == 0;
     if (!tile_ok) {
         GenericParams g{};
@@ -540,45 +550,48 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
         return launch_generic(g, stream);
     }
     const int kg = k / 32;
-    StreamTemp ta(stream), tb(stream);
-    const uint8_t* sa_nd = sa;
-    const uint8_t* sb_dn = sb;
+    // Scales that are not plain [M][K/32] / [N][K/32] rows: with a workspace they are re-laid into it and the DMA tiles run
+    // (the fastest form for a large product); without one the register-staged tiles address the pairs of the caller's
+    // layout directly.  Nothing is allocated either way.
+    const uint8_t* sa_use = sa;
+    const uint8_t* sb_use = sb;
+    int sa_mode = sa_layout == PTOAMD_MX_A_ND ? 0 : (sa_layout == PTOAMD_MX_A_ZZ ? 1 : 2);
+    int sb_mode = sb_layout == PTOAMD_MX_B_DN ? 0 : (sb_layout == PTOAMD_MX_B_NN ? 1 : 2);
     // workspace layout: [M][K/32] scales of A, rounded up to 256 bytes, then [N][K/32] scales of B
-    const size_t need_a = sa_layout != PTOAMD_MX_A_ND ? (((size_t)m * kg + 255) & ~(size_t)255) : 0;
-    const size_t need_b = sb_layout != PTOAMD_MX_B_DN ? (size_t)n * kg : 0;
-    if (ws != nullptr || !may_allocate)
-        PTOAMD_REQUIRE(need_a + need_b <= ws_bytes && (need_a + need_b == 0 || ws != nullptr), PTOAMD_E_INVALID,
+    const size_t need_a = sa_mode != 0 ? (((size_t)m * kg + 255) & ~(size_t)255) : 0;
+    const size_t need_b = sb_mode != 0 ? (size_t)n * kg : 0;
+    if (ws != nullptr && need_a + need_b > 0) {
+        PTOAMD_REQUIRE(need_a + need_b <= ws_bytes, PTOAMD_E_INVALID,
                        "%s: the scale layouts need %zu bytes of workspace, %zu available", who, need_a + need_b, ws_bytes);
-    if (sa_layout != PTOAMD_MX_A_ND) {  // the kernel streams scales as [M][K/32] and [N][K/32]
-        uint8_t* dst = ws;
-        if (dst == nullptr) {
-            PTOAMD_HIP_CHECK(ta.alloc((size_t)m * kg));
-            dst = reinterpret_cast<uint8_t*>(ta.ptr);
+        if (sa_mode != 0) {
+            const int rc = ptoamd_mx_scale_relayout(ws, PTOAMD_MX_A_ND, sa, sa_layout, m, kg, stream_);
+            if (rc != PTOAMD_OK)
+                return rc;
+            sa_use = ws;
+            sa_mode = 0;
         }
-        const int rc = ptoamd_mx_scale_relayout(dst, PTOAMD_MX_A_ND, sa, sa_layout, m, kg, stream_);
-        if (rc != PTOAMD_OK)
-            return rc;
-        sa_nd = dst;
-    }
-    if (sb_layout != PTOAMD_MX_B_DN) {
-        uint8_t* dst = ws != nullptr ? ws + need_a : nullptr;
-        if (dst == nullptr) {
-            PTOAMD_HIP_CHECK(tb.alloc((size_t)n * kg));
-            dst = reinterpret_cast<uint8_t*>(tb.ptr);
+        if (sb_mode != 0) {
+            const int rc = ptoamd_mx_scale_relayout(ws + need_a, PTOAMD_MX_B_DN, sb, sb_layout, kg, n, stream_);
+            if (rc != PTOAMD_OK)
+                return rc;
+            sb_use = ws + need_a;
+            sb_mode = 0;
         }
-        const int rc = ptoamd_mx_scale_relayout(dst, PTOAMD_MX_B_DN, sb, sb_layout, kg, n, stream_);
-        if (rc != PTOAMD_OK)
-            return rc;
-        sb_dn = dst;
     }
-    PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(sa_nd) & 3u) == 0 && (reinterpret_cast<uintptr_t>(sb_dn) & 3u) == 0,
-                   PTOAMD_E_ALIGNMENT, "%s: scale arrays must be 4-byte aligned", who);
+    const bool plain_scales = sa_mode == 0 && sb_mode == 0;
+    PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(sa_use) & (sa_mode == 0 ? 3u : 1u)) == 0 &&
+                       (reinterpret_cast<uintptr_t>(sb_use) & (sb_mode == 0 ? 3u : 1u)) == 0,
+                   PTOAMD_E_ALIGNMENT, "%s: scale arrays must be 4-byte aligned (2-byte in the boxed and pair-major layouts)", who);
+    const uint8_t* sa_nd = sa_use;
+    const uint8_t* sb_dn = sb_use;
     TileGemmParams p{};
     p.a = reinterpret_cast<const uint8_t*>(a);
     p.b = reinterpret_cast<const uint8_t*>(b);
     p.c = c; p.c_in = c_in; p.sa = sa_nd; p.sb = sb_dn;
     p.m = m; p.n = n; p.k_bytes = (int)k_bytes; p.lda_bytes = lda_b; p.ldb_bytes = ldb_b; p.ldc = ldc;
     p.scale_ld = kg; p.out_kind = out_kind; p.group_m = 4;
+    p.sa_mode = sa_mode; p.sb_mode = sb_mode;
+    p.b_nd = b_in_kernel; p.b_esz = 1;
     int op;
     if (a4)
         op = TOP_FP4;
@@ -588,7 +601,8 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
         op = b_type == PTOAMD_E5M2 ? TOP_FP8_E5E5 : TOP_FP8_E5E4;
     // the DMA tiles fetch scales as 16-byte chunks per row: 4 slabs of fp8, 2 of fp4
     const long k_slabs = k_bytes / 128;
-    const bool scale_dma_ok = (kg % 16) == 0 && aligned16(sa_nd) && aligned16(sb_dn) && (k_slabs % (a4 ? 2 : 4)) == 0;
+    const bool scale_dma_ok = plain_scales && !b_in_kernel && (kg % 16) == 0 && aligned16(sa_nd) && aligned16(sb_dn) &&
+                              (k_slabs % (a4 ? 2 : 4)) == 0;
     const int tile = pick_tile(m, n, k_bytes, true, a4, scale_dma_ok && dma_offsets_fit(m, n, lda_b, ldb_b, k_bytes));
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
@@ -600,7 +614,7 @@ int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type
                    int ldb, int ldc, int b_layout, void* stream_)
 {
     return gemm_mx_common("ptoamd_gemm_mx", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k, lda, ldb,
-                          ldc, b_layout, nullptr, 0, true, stream_);
+                          ldc, b_layout, nullptr, 0, stream_);
 }
 
 int ptoamd_gemm_mx_ws(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
@@ -610,7 +624,7 @@ int ptoamd_gemm_mx_ws(void* c, int c_type, const void* a, const void* b, int a_t
     PTOAMD_REQUIRE(workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, PTOAMD_E_ALIGNMENT,
                    "ptoamd_gemm_mx_ws: the workspace must be 256-byte aligned");
     return gemm_mx_common("ptoamd_gemm_mx_ws", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k, lda,
-                          ldb, ldc, b_layout, reinterpret_cast<uint8_t*>(workspace), workspace ? workspace_bytes : 0, false, stream_);
+                          ldb, ldc, b_layout, reinterpret_cast<uint8_t*>(workspace), workspace ? workspace_bytes : 0, stream_);
 }
 
 int ptoamd_gemm_mx_static(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
@@ -626,7 +640,7 @@ int ptoamd_gemm_mx_static(void* c, int c_type, const void* a, const void* b, int
     if (rc != PTOAMD_OK)
         return rc;
     return gemm_mx_common("ptoamd_gemm_mx_static", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k,
-                          lda, ldb, ldc, b_layout, ws, PTOAMD_STATIC_SCRATCH_BYTES, false, stream_);
+                          lda, ldb, ldc, b_layout, ws, PTOAMD_STATIC_SCRATCH_BYTES, stream_);
 }
 
 size_t ptoamd_gemm_mx_workspace_bytes(int m, int n, int k, int sa_layout, int sb_layout)

@@ -36,7 +36,21 @@ struct TileGemmParams {
     int relu;
     int out_kind;           // OutKind
     int group_m;            // tile-order grouping for L2 reuse
+    int b_nd;               // register-staged tiles only: b is [k][ldb_bytes] (rows of N), transposed on the way into LDS
+    int b_esz;              // element bytes of B (1 or 2) when b_nd is set
+    // register-staged tiles only: how the E8M0 bytes of a tile row are laid out.  Every MX layout keeps the two scales of
+    // a K-group pair adjacent: byte (x, g) of row / column x sits at base(x) + (g / 2) * pair_stride + g % 2.
+    //   0  [X][K/32] (MX_A_ND, MX_B_DN): base = x * scale_ld, pair_stride 2 (plain rows; the DMA tiles need this one)
+    //   1  16-row x 2-group boxes (MX_A_ZZ, MX_B_NN): base = (x / 16) * scale_ld * 16 + (x % 16) * 2, pair_stride 32
+    //   2  pair-major (MX_A_DN, MX_B_ND): base = x * 2, pair_stride = 2 * rows (m for A, n for B)
+    int sa_mode, sb_mode;
 };
+
+__device__ __forceinline__ long mx_scale_base(int mode, int x, int scale_ld)
+{
+    return mode == 0 ? (long)x * scale_ld : (mode == 1 ? (long)(x >> 4) * scale_ld * 16 + (x & 15) * 2 : (long)x * 2);
+}
+__device__ __forceinline__ long mx_pair_stride(int mode, int rows) { return mode == 0 ? 2 : (mode == 1 ? 32 : 2L * rows); }
 
 enum OutKind { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2, OUT_I32 = 3, OUT_W8A8_BF16 = 4 };
 
@@ -433,11 +447,33 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
         ga[i] = p.a + (long)min(m0 + r, p.m - 1) * p.lda_bytes + ld_chunk * 16;
         sa_off[i] = r * 128 + swizzle_chunk(r, ld_chunk) * 16;
     }
+    // B as [N][K] (Layout::DN): the same chunks as A.  B as [K][N] (Layout::ND, p.b_nd): a 16-byte chunk holds EPC
+    // consecutive columns of one k; the thread scatters its elements into the K-contiguous LDS rows of those columns,
+    // so the slab in LDS, the fragment reads and the MFMA loop are the same for both layouts and no transposed copy
+    // of B is made in global memory.  Chunk c of a slab: k = 8 * EPC * (c / BN) ... , see below.
+    int b_koff[LB];          // byte offset (along K) of the chunk's first element inside a slab; huge = never loaded
+    int sb_k[LB], sb_n[LB];  // b_nd: the chunk's k-chunk (0..7) and first column inside the tile
+    const long b_slab_stride = p.b_nd ? (long)(128 / p.b_esz) * p.ldb_bytes : 128;
 #pragma unroll
     for (int i = 0; i < LB; ++i) {
         const int r = ld_row + i * (NT / 8);
-        gb[i] = p.b + (long)min(n0 + r, p.n - 1) * p.ldb_bytes + ld_chunk * 16;
-        sb_off[i] = Cfg::A_BYTES + r * 128 + swizzle_chunk(r, ld_chunk) * 16;
+        if (!p.b_nd) {
+            gb[i] = p.b + (long)min(n0 + r, p.n - 1) * p.ldb_bytes + ld_chunk * 16;
+            sb_off[i] = Cfg::A_BYTES + r * 128 + swizzle_chunk(r, ld_chunk) * 16;
+            b_koff[i] = ld_chunk * 16;
+            sb_k[i] = sb_n[i] = 0;
+        } else {
+            const int epc = 16 / p.b_esz;  // elements per chunk = k rows per LDS chunk
+            const int c = tid + i * NT;
+            const int k_lo = c % epc, nc = (c / epc) % (BN / epc), k_hi = c / BN;
+            const int krow = k_hi * epc + k_lo;
+            const bool inside = n0 + nc * epc < p.n;  // (N is a multiple of EPC: a chunk is inside or outside as a whole)
+            gb[i] = p.b + (long)krow * p.ldb_bytes + (long)(inside ? n0 + nc * epc : 0) * p.b_esz;
+            sb_off[i] = Cfg::A_BYTES + nc * epc * 128 + k_lo * p.b_esz;
+            b_koff[i] = inside ? krow * p.b_esz : (1 << 30);
+            sb_k[i] = k_hi;
+            sb_n[i] = nc * epc;
+        }
     }
     const int k_slabs = (p.k_bytes + 127) / 128;
 
@@ -449,16 +485,36 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
             ra[i] = live ? *reinterpret_cast<const uint4*>(ga[i] + (long)kt * 128) : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < LB; ++i)
-            rb[i] = live ? *reinterpret_cast<const uint4*>(gb[i] + (long)kt * 128) : make_uint4(0, 0, 0, 0);
+            rb[i] = kt * 128 + b_koff[i] < p.k_bytes ? *reinterpret_cast<const uint4*>(gb[i] + kt * b_slab_stride)
+                                                     : make_uint4(0, 0, 0, 0);
     };
     auto stage = [&](int buf) {
         uint8_t* base = smem + buf * Cfg::STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < LA; ++i)
             *reinterpret_cast<uint4*>(base + sa_off[i]) = ra[i];
+        if (!p.b_nd) {
 #pragma unroll
-        for (int i = 0; i < LB; ++i)
-            *reinterpret_cast<uint4*>(base + sb_off[i]) = rb[i];
+            for (int i = 0; i < LB; ++i)
+                *reinterpret_cast<uint4*>(base + sb_off[i]) = rb[i];
+        } else if (p.b_esz == 2) {
+#pragma unroll
+            for (int i = 0; i < LB; ++i) {
+                const uint32_t w[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    *reinterpret_cast<uint16_t*>(base + sb_off[i] + e * 128 + swizzle_chunk(sb_n[i] + e, sb_k[i]) * 16) =
+                        (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < LB; ++i) {
+                const uint32_t w[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    *(base + sb_off[i] + e * 128 + swizzle_chunk(sb_n[i] + e, sb_k[i]) * 16) = (uint8_t)(w[e >> 2] >> (8 * (e & 3)));
+            }
+        }
     };
 
     // ---- MX block scales: one E8M0 byte per row per 32 elements, fetched per slab straight into registers
@@ -467,24 +523,35 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
     const uint8_t* gsa[MB];
     const uint8_t* gsb[NB];
     const bool has_scales = Op::SCALED && p.sa != nullptr;
+    const long spa = mx_pair_stride(p.sa_mode, p.m), spb = mx_pair_stride(p.sb_mode, p.n);
     if (has_scales) {
 #pragma unroll
         for (int i = 0; i < MB; ++i)
-            gsa[i] = p.sa + (long)min(m0 + wm * Cfg::WTM + i * 32 + l32, p.m - 1) * p.scale_ld;
+            gsa[i] = p.sa + mx_scale_base(p.sa_mode, min(m0 + wm * Cfg::WTM + i * 32 + l32, p.m - 1), p.scale_ld);
 #pragma unroll
         for (int j = 0; j < NB; ++j)
-            gsb[j] = p.sb + (long)min(n0 + wn * Cfg::WTN + j * 32 + l32, p.n - 1) * p.scale_ld;
+            gsb[j] = p.sb + mx_scale_base(p.sb_mode, min(n0 + wn * Cfg::WTN + j * 32 + l32, p.n - 1), p.scale_ld);
     }
+    // the SW dwords (4 SW scale bytes) of slab kt of one row: one dword load per dword in the plain layout, two 2-byte
+    // loads (one K-group pair each) in the others
+    auto load_row_scales = [&](const uint8_t* row, int mode, long pair_stride, int kt, int w) -> uint32_t {
+        if (mode == 0)
+            return *reinterpret_cast<const uint32_t*>(row + (long)kt * (SW * 4) + w * 4);
+        const long pair = (long)kt * (SW * 2) + w * 2;
+        const uint32_t lo = *reinterpret_cast<const uint16_t*>(row + pair * pair_stride);
+        const uint32_t hi = *reinterpret_cast<const uint16_t*>(row + (pair + 1) * pair_stride);
+        return lo | (hi << 16);
+    };
     auto load_scales = [&](int kt) {
         if (has_scales) {
 #pragma unroll
             for (int w = 0; w < SW; ++w) {
 #pragma unroll
                 for (int i = 0; i < MB; ++i)
-                    sca_n[i][w] = *reinterpret_cast<const uint32_t*>(gsa[i] + (long)kt * (SW * 4) + w * 4);
+                    sca_n[i][w] = load_row_scales(gsa[i], p.sa_mode, spa, kt, w);
 #pragma unroll
                 for (int j = 0; j < NB; ++j)
-                    scb_n[j][w] = *reinterpret_cast<const uint32_t*>(gsb[j] + (long)kt * (SW * 4) + w * 4);
+                    scb_n[j][w] = load_row_scales(gsb[j], p.sb_mode, spb, kt, w);
             }
         }
     };

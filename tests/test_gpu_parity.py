@@ -90,6 +90,52 @@ def test_config1_fp16_512_cubed(pa, oracle):
     assert np.array_equal(exact.view(np.uint32), ref.view(np.uint32))  # k-order-exact kernel: bit for bit
 
 
+@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("kind", ["f16", "bf16", "i8", "e4m3"])
+@pytest.mark.parametrize("m,n,k,ldb_pad", [(64, 64, 64, 0), (100, 136, 200, 8), (512, 512, 512, 0), (33, 48, 1040, 16), (1, 16, 16, 0)])
+def test_row_major_b_is_transposed_inside_the_kernel(pa, oracle, tile, kind, m, n, k, ldb_pad):
+    """B as [K][N] (Layout::ND): the register-staged tiles scatter it into the K-contiguous LDS slab themselves.  The
+    sums run in the same order as with a column-major copy of the same matrix, so the two results are identical, and
+    both match the oracle."""
+    if kind in ("i8", "e4m3"):  # 16-byte chunks: 16 one-byte elements
+        n, ldb_pad, k = (n + 15) // 16 * 16, (ldb_pad + 15) // 16 * 16, (k + 15) // 16 * 16
+    r = np.random.default_rng(m + 3 * n + 5 * k)
+    ldb = n + ldb_pad
+    if kind == "i8":
+        a, b = r.integers(-128, 128, (m, k)).astype(np.int8), r.integers(-128, 128, (k, ldb)).astype(np.int8)
+        ta, tc, ref = pa.I8, pa.I32, oracle.matmul_i8(a, np.ascontiguousarray(b[:, :n]))
+        da, db = dev(a), dev(b)
+    elif kind == "e4m3":
+        a, b = r.integers(0, 256, (m, k)).astype(np.uint8), r.integers(0, 256, (k, ldb)).astype(np.uint8)
+        a[(a & 0x7F) == 0x7F] = 0x38
+        b[(b & 0x7F) == 0x7F] = 0x38
+        ta, tc, ref = pa.E4M3, pa.F32, oracle.matmul_fp8(a, np.ascontiguousarray(b[:, :n]))
+        da, db = dev(a), dev(b)
+    else:
+        x, y = r.uniform(-1, 1, (m, k)).astype(np.float32), r.uniform(-1, 1, (k, ldb)).astype(np.float32)
+        if kind == "f16":
+            a, b = x.astype(np.float16).view(np.uint16), y.astype(np.float16).view(np.uint16)
+            ta, tc, ref = pa.F16, pa.F32, oracle.matmul_f16(a, np.ascontiguousarray(b[:, :n]))
+            da, db = dev(a).view(torch.float16), dev(b).view(torch.float16)
+        else:
+            a, b = bf16_bits(x), bf16_bits(y)
+            ta, tc, ref = pa.BF16, pa.F32, oracle.matmul_bf16(a, np.ascontiguousarray(b[:, :n]))
+            da, db = dev(a).view(torch.bfloat16), dev(b).view(torch.bfloat16)
+    bt = db[:, :n].t().contiguous()  # [n][k]
+    with tile_env(PTOAMD_TILE=tile):
+        got = host(pa.gemm(da, db, ta, tc, pa.B_ND, n=n))
+        assert pa.last_kernel().startswith(TILE_NAMES[tile])
+        same = host(pa.gemm(da, bt, ta, tc, pa.B_DN))
+        with tile_env(PTOAMD_B_ND_TRANSPOSE=1):
+            via_copy = host(pa.gemm(da, db, ta, tc, pa.B_ND, n=n))
+    assert np.array_equal(got.view(np.uint32), same.view(np.uint32))
+    assert np.array_equal(got.view(np.uint32), via_copy.view(np.uint32))
+    if kind == "i8":
+        assert np.array_equal(got, ref)
+    else:
+        assert relerr(got, ref) <= (2e-2 if kind == "e4m3" else 1e-2)
+
+
 TILE_NAMES = ("tile256x256_", "tile128x128_", "tile64x64_", "tile256x256w4_dtl", "tile256x256w8_dtl", "tile128x128_dtl",
               "tile256x128_dtl")
 ALL_TILES = [0, 1, 2, 3, 4, 5, 6]
@@ -250,6 +296,16 @@ def test_w8a8_fused_dequant(pa, oracle):
     ref_acc, ref_out = _w8a8_reference(oracle, a, b, sa, sb)
     assert np.array_equal(host(acc), ref_acc)
     assert np.array_equal(host(out), ref_out)  # same three roundings in the same order: bit-exact
+    # B as [K][N]: transposed inside the kernel (staged and element-wise drains), or through a copy
+    b_nd = dev(np.ascontiguousarray(b.T))
+    out_nd = pa.gemm_w8a8(dev(a), b_nd, dev(sa), dev(sb), b_layout=pa.B_ND)
+    assert pa.last_kernel() == "tile64x64_i8"  # (a register-staged tile: the DMA tiles cannot transpose)
+    assert np.array_equal(host(out_nd), ref_out)
+    out_nd, acc_nd = pa.gemm_w8a8(dev(a), b_nd, dev(sa), dev(sb), b_layout=pa.B_ND, want_acc=True)
+    assert np.array_equal(host(out_nd), ref_out) and np.array_equal(host(acc_nd), ref_acc)
+    with tile_env(PTOAMD_B_ND_TRANSPOSE=1):
+        out_nd = pa.gemm_w8a8(dev(a), b_nd, dev(sa), dev(sb), b_layout=pa.B_ND)
+    assert np.array_equal(host(out_nd), ref_out)
 
 
 def test_config3_w8a8_full_size(pa, oracle):
@@ -447,8 +503,9 @@ def test_mx_golden_and_scale_layouts(pa, golden):
 
 
 def test_gemm_mx_workspace_form(pa, oracle):
-    """ptoamd_gemm_mx_ws: scales in the boxed ZZ / NN layouts are re-laid into the caller's workspace; same kernels, same
-    bits as the allocating form, and no workspace is needed for the two natural layouts."""
+    """ptoamd_gemm_mx_ws: scales in the boxed ZZ / NN layouts are re-laid into the caller's workspace and the DMA tiles run;
+    without a workspace the register-staged tiles address the boxes in place.  Same bits either way, and no workspace is
+    needed for the two natural layouts."""
     r = np.random.default_rng(77)
     m, n, k = 256, 384, 1024
     a, b, sa, sb = _mx_inputs(r, ob.E4M3, m, n, k)
@@ -464,9 +521,10 @@ def test_gemm_mx_workspace_form(pa, oracle):
         got = host(pa.gemm_mx(da, db, sa_zz, sb_nn, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sa_layout=pa.MX_A_ZZ,
                               sb_layout=pa.MX_B_NN, workspace=ws))
         assert "_dtl_" in pa.last_kernel(), pa.last_kernel()
-        alloc = host(pa.gemm_mx(da, db, sa_zz, sb_nn, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sa_layout=pa.MX_A_ZZ,
-                                sb_layout=pa.MX_B_NN))
-    assert np.array_equal(got.view(np.uint32), alloc.view(np.uint32))
+        in_place = host(pa.gemm_mx(da, db, sa_zz, sb_nn, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sa_layout=pa.MX_A_ZZ,
+                                   sb_layout=pa.MX_B_NN))
+        assert pa.last_kernel().startswith("tile128x128_fp8"), pa.last_kernel()
+    assert np.array_equal(got.view(np.uint32), in_place.view(np.uint32))
     assert relerr(got, ref) <= 2e-2
     with tile_env(PTOAMD_TILE=5):
         nat = host(pa.gemm_mx(da, db, dev(sa), dev(sb), m, n, k, pa.E4M3, pa.E4M3, pa.F32, workspace=ws[:0]))
@@ -474,6 +532,44 @@ def test_gemm_mx_workspace_form(pa, oracle):
     with pytest.raises(pa.PtoAmdError, match="workspace"):
         pa.gemm_mx(da, db, sa_zz, sb_nn, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sa_layout=pa.MX_A_ZZ, sb_layout=pa.MX_B_NN,
                    workspace=ws[:need - 256])
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("typ", [ob.E4M3, ob.E2M1])
+@pytest.mark.parametrize("la,lb", [("MX_A_ZZ", "MX_B_NN"), ("MX_A_DN", "MX_B_ND"), ("MX_A_ND", "MX_B_NN"), ("MX_A_ZZ", "MX_B_DN")])
+def test_mx_scale_layouts_addressed_in_place(pa, oracle, typ, la, lb, tile):
+    """Every GM layout of the E8M0 scales keeps the two scales of a K-group pair adjacent; the register-staged tiles read
+    them where they lie (no re-laid copy, nothing allocated).  Identical to the product on the plain row layouts."""
+    r = np.random.default_rng(5)
+    m, n, k = 176, 208, 512  # m, n multiples of 16 (the boxed layouts), ragged against every tile size
+    a, b, sa, sb = _mx_inputs(r, typ, m, n, k)
+    t = PA_T[typ]
+    da, db, dsa, dsb = dev(a), dev(b), dev(sa), dev(sb)
+    sa_l = pa.mx_scale_relayout(dsa, pa.MX_A_ND, getattr(pa, la), m, k // 32) if la != "MX_A_ND" else dsa
+    sb_l = pa.mx_scale_relayout(dsb, pa.MX_B_DN, getattr(pa, lb), k // 32, n) if lb != "MX_B_DN" else dsb
+    with tile_env(PTOAMD_TILE=tile):
+        plain = host(pa.gemm_mx(da, db, dsa, dsb, m, n, k, t, t, pa.F32))
+        got = host(pa.gemm_mx(da, db, sa_l, sb_l, m, n, k, t, t, pa.F32, sa_layout=getattr(pa, la), sb_layout=getattr(pa, lb)))
+        assert pa.last_kernel().startswith(TILE_NAMES[tile]), pa.last_kernel()
+    assert np.array_equal(got.view(np.uint32), plain.view(np.uint32))
+    assert relerr(got, oracle.matmul_mx(a, b, sa, sb, m, k, n, typ, typ)) <= 2e-2
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_mx_fp8_row_major_b_in_kernel(pa, oracle, tile):
+    """TMATMUL_MX with B as [K][N] one-byte codes: transposed into the LDS slab by the kernel, scales in any layout."""
+    r = np.random.default_rng(6)
+    m, n, k = 96, 160, 384
+    a, b, sa, sb = _mx_inputs(r, ob.E4M3, m, n, k)  # b is [n][k]
+    b_nd = np.ascontiguousarray(b.T)                # [k][n]
+    sb_nd = pa.mx_scale_relayout(dev(sb), pa.MX_B_DN, pa.MX_B_ND, k // 32, n)
+    with tile_env(PTOAMD_TILE=tile):
+        want = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, pa.E4M3, pa.E4M3, pa.F32))
+        got = host(pa.gemm_mx(dev(a), dev(b_nd), dev(sa), sb_nd, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sb_layout=pa.MX_B_ND,
+                              b_layout=pa.B_ND))
+        assert pa.last_kernel().startswith(TILE_NAMES[tile]), pa.last_kernel()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert relerr(got, oracle.matmul_mx(a, b, sa, sb, m, k, n, ob.E4M3, ob.E4M3)) <= 2e-2
 
 
 def test_mx_scale_relayout_matches_reference_offsets(pa, golden):
