@@ -127,6 +127,25 @@ int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_t
                      int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream);
 
 /*
+ * The same pipeline drained through the fix-pipe quantiser: TSTORE of the accumulator tile with a scalar quantisation
+ * word (TSTORE(dst, src, preQuantScalar)) or one word per column (TSTORE_FP with a Scaling tile):
+ *   r = acc(i, j) * scale(word);  s8 / u8: clamp(rint(r + offset(word)), byte range chosen by the word's sign bit);
+ *   f16: clamp to +-65504 (finite values only for float accumulators);  then relu, then the store.
+ * Cin and bias are added to the accumulator before the quantisation.
+ * reference: include/pto/cpu/common.hpp:117-185 (extract_m1_from_quant, quantize_element), cpu/TStore.hpp:118-181,
+ *            common/pto_instr.hpp:439-490; test shapes tests/cpu/st/testcase/tstore_acc2gm, tstore_quant.
+ *   c_type      : PTOAMD_I8 | PTOAMD_U8 | PTOAMD_F16 (the byte's signedness comes from bit 46 of the word, as in the
+ *                 reference: it must agree with c_type)
+ *   quant_words : device memory, 8-byte aligned; one uint64 (per_column == 0) or N of them (per_column != 0).  Scalar
+ *                 words hold an fp32 scale in bits 0..31; per-column words a 19-bit (1, 8, 10) float in bits 13..31;
+ *                 both the offset in bits 37..45 and the sign bit 46
+ *   ab_type     : as ptoamd_gemm (float inputs accumulate in f32, int8 in i32: the DEQF16 / REQ8 forms)
+ */
+int ptoamd_gemm_requant(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
+                        const uint64_t* quant_words, int per_column, int m, int n, int k, int lda, int ldb, int ldc,
+                        int b_layout, int relu, void* stream);
+
+/*
  * W8A8: int8 x int8 -> int32 accumulate, then the dequantising drain fused in registers:
  *   out(i, j) = bf16( (float(acc(i, j)) * scale_a[i]) * scale_b[j] )
  * i.e. TMATMUL (cpu/TMatmul.hpp:106) -> TDEQUANT with offset 0 (cpu/TDeQuant.hpp:31-34) -> per-column multiply
@@ -151,11 +170,19 @@ int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type
                    int ldb, int ldc, int b_layout, void* stream);
 
 /*
+ * TMATMUL_MX with a bias row: C = A * B (+ Cin) + bias, bias [N] f32 added to every row after the K loop.
+ * reference: include/pto/cpu/TMatmul.hpp:273-292 (TMATMUL_MX_IMPL with a bias tile), common/pto_instr.hpp (TMATMUL_MX).
+ */
+int ptoamd_gemm_mx_bias(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
+                        const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, const float* bias, int m, int n,
+                        int k, int lda, int ldb, int ldc, int b_layout, void* stream);
+
+/*
  * ptoamd_gemm_mx with a caller-provided device workspace for what the kernels need beyond inputs and outputs: the MFMA
  * kernels stream scales as [M][K/32] (MX_A_ND) and [N][K/32] (MX_B_DN), and scales that arrive in another GM layout
  * (the TLOAD + TMOV of a scale tile, cpu/TLoad.hpp:287-321 with the MX_* maps of cpu/tile_offsets.hpp:233-268) are
- * re-laid into the workspace first.  ptoamd_gemm_mx takes that memory from a stream-ordered allocation per call; this
- * form allocates nothing.  workspace: 256-byte aligned, at least ptoamd_gemm_mx_workspace_bytes(...) bytes (0 for the
+ * re-laid into the workspace first, and the fastest (direct-to-LDS) kernels run.  ptoamd_gemm_mx reads such scales where
+ * they lie instead, with the register-staged kernels; neither form allocates.  workspace: 256-byte aligned, at least ptoamd_gemm_mx_workspace_bytes(...) bytes (0 for the
  * two natural layouts: workspace may then be NULL).
  */
 int ptoamd_gemm_mx_ws(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,

@@ -40,7 +40,8 @@ EXPORTS = [
     "ptoamd_malloc_host", "ptoamd_free_host", "ptoamd_memcpy", "ptoamd_memcpy_async", "ptoamd_memset",
     "ptoamd_stream_create", "ptoamd_stream_destroy", "ptoamd_stream_synchronize", "ptoamd_event_create",
     "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
-    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_ws",
+    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_requant", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
+    "ptoamd_gemm_mx_ws",
     "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
     "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_mx_scale_relayout", "ptoamd_last_kernel",
 ]
@@ -97,6 +98,20 @@ def gemm(a, b, ab_type, c_type=F32, b_layout=B_DN, c_in=None, relu=False, m=None
     return out
 
 
+def gemm_requant(a, b, ab_type, c_type, quant_words, per_column=False, b_layout=B_DN, c_in=None, bias=None, relu=False,
+                 n=None, stream=None, out=None):
+    """TLOAD -> TMATMUL -> TSTORE through the fix-pipe quantiser.  quant_words: int64 / uint64 device tensor holding one
+    word, or one word per column; c_type: I8, U8 or F16."""
+    m, k = a.shape
+    n = (b.shape[0] if b_layout == B_DN else b.shape[1]) if n is None else n
+    if out is None:
+        out = torch.empty((m, n), dtype={I8: torch.int8, U8: torch.uint8, F16: torch.float16}[c_type], device=a.device)
+    _check(_lib.ptoamd_gemm_requant(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), _ptr(bias), _ptr(quant_words),
+                                    int(per_column), m, n, k, a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu),
+                                    _stream(stream)), "ptoamd_gemm_requant")
+    return out
+
+
 def gemm_w8a8(a, b, scale_a, scale_b, b_layout=B_DN, want_acc=False, stream=None, out=None):
     """int8 x int8 -> int32 accumulate with the fused dequantising drain to bf16."""
     m, k = a.shape
@@ -130,7 +145,7 @@ def gemm_mx_workspace_bytes(m, n, k, sa_layout=MX_A_ND, sb_layout=MX_B_DN):
 
 
 def gemm_mx(a, b, sa, sb, m, n, k, a_type, b_type, c_type=F32, sa_layout=MX_A_ND, sb_layout=MX_B_DN, b_layout=B_DN,
-            c_in=None, stream=None, out=None, workspace=None):
+            c_in=None, stream=None, out=None, workspace=None, bias=None):
     """TMATMUL_MX.  a / b hold element codes (uint8; fp4 packed two per byte); sa / sb hold E8M0 bytes.  workspace: a
     uint8 device tensor of gemm_mx_workspace_bytes(...) bytes selects the form that allocates nothing."""
     if out is None:
@@ -142,6 +157,11 @@ def gemm_mx(a, b, sa, sb, m, n, k, a_type, b_type, c_type=F32, sa_layout=MX_A_ND
                                       sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _ptr(workspace),
                                       C.c_size_t(workspace.numel() * workspace.element_size()), _stream(stream)),
                "ptoamd_gemm_mx_ws")
+        return out
+    if bias is not None:
+        _check(_lib.ptoamd_gemm_mx_bias(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
+                                        sb_layout, _ptr(c_in), _ptr(bias), m, n, k, lda, ldb, out.stride(0), b_layout,
+                                        _stream(stream)), "ptoamd_gemm_mx_bias")
         return out
     _check(_lib.ptoamd_gemm_mx(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
                                sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),

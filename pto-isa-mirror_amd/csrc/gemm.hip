@@ -107,6 +107,8 @@ struct GenericParams {
     int ldc;
     int a_type, b_type, out_kind, relu;
     int sa_layout, sb_layout, mx;
+    const uint64_t* qwords;  // OUT_Q8 / OUT_QF16: fix-pipe quantisation words
+    int q_per_column;
 };
 
 __device__ __forceinline__ float load_elem_f32(const void* p, long idx, int type)
@@ -123,8 +125,31 @@ __device__ __forceinline__ float load_elem_f32(const void* p, long idx, int type
     }
 }
 
+// the quantising drains: word -> scale / offset / range, relu after the quantisation
+template <bool SRC_INT>
+__device__ __forceinline__ void store_quant(const GenericParams& p, long o, float acc, int gj)
+{
+    const uint64_t w = p.qwords[p.q_per_column ? gj : 0];
+    const bool byte = p.out_kind == OUT_Q8;
+    float r;
+    if (byte)
+        r = p.q_per_column ? fixpipe_quantize<true, true, SRC_INT>(acc, w) : fixpipe_quantize<false, true, SRC_INT>(acc, w);
+    else
+        r = p.q_per_column ? fixpipe_quantize<true, false, SRC_INT>(acc, w) : fixpipe_quantize<false, false, SRC_INT>(acc, w);
+    if (p.relu)
+        r = r > 0 ? r : 0;
+    if (byte)
+        reinterpret_cast<uint8_t*>(p.c)[o] = (uint8_t)(int32_t)r;
+    else
+        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits(r);
+}
+
 __device__ __forceinline__ void store_out(const GenericParams& p, long o, float v, int gi, int gj)
 {
+    if (p.out_kind == OUT_Q8 || p.out_kind == OUT_QF16) {
+        store_quant<false>(p, o, v, gj);
+        return;
+    }
     if (p.relu)
         v = v > 0 ? v : 0;
     switch (p.out_kind) {
@@ -152,6 +177,10 @@ __global__ void gemm_generic_kernel(const GenericParams p)
         if (p.bias)
             acc += (uint32_t) reinterpret_cast<const int32_t*>(p.bias)[gj];
         int32_t v = (int32_t)acc;
+        if (p.out_kind == OUT_Q8 || p.out_kind == OUT_QF16) {
+            store_quant<true>(p, o, (float)v, gj);
+            return;
+        }
         if (p.relu)
             v = v > 0 ? v : 0;
         if (p.out_kind == OUT_I32) {
@@ -264,7 +293,7 @@ static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStr
             if (e != hipSuccess)
                 return e;
             TileGemmParams tail = p;
-            const size_t esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : 2;
+            const size_t esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : (p.out_kind == OUT_Q8 ? 1 : 2);
             tail.n = p.n - n1;
             tail.b = p.b + (long)n1 * p.ldb_bytes;
             tail.c = static_cast<uint8_t*>(p.c) + (size_t)n1 * esz;
@@ -278,6 +307,8 @@ static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStr
                 tail.sb = p.sb + (long)n1 * p.scale_ld;
             if (p.col_scale)
                 tail.col_scale = p.col_scale + n1;
+            if (p.qwords && p.q_per_column)
+                tail.qwords = p.qwords + n1;
             return launch_gemm_tile(5, op, tail, stream);
         }
     }
@@ -386,8 +417,32 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
     return ptoamd_gemm_bias(c, c_type, a, b, ab_type, c_in, nullptr, m, n, k, lda, ldb, ldc, b_layout, relu, stream_);
 }
 
+static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
+                       const uint64_t* qwords, int q_per_column, int m, int n, int k, int lda, int ldb, int ldc, int b_layout,
+                       int relu, void* stream_);
+
 int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                      int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream_)
+{
+    return gemm_common(c, c_type, a, b, ab_type, c_in, bias, nullptr, 0, m, n, k, lda, ldb, ldc, b_layout, relu, stream_);
+}
+
+int ptoamd_gemm_requant(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
+                        const uint64_t* quant_words, int per_column, int m, int n, int k, int lda, int ldb, int ldc,
+                        int b_layout, int relu, void* stream_)
+{
+    PTOAMD_REQUIRE(quant_words != nullptr, PTOAMD_E_INVALID, "ptoamd_gemm_requant: null quantisation words");
+    PTOAMD_REQUIRE(c_type == PTOAMD_I8 || c_type == PTOAMD_U8 || c_type == PTOAMD_F16, PTOAMD_E_UNSUPPORTED,
+                   "ptoamd_gemm_requant: the fix-pipe quantiser stores s8, u8 or f16 (got type %d)", c_type);
+    PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(quant_words) & 7u) == 0, PTOAMD_E_ALIGNMENT,
+                   "ptoamd_gemm_requant: quantisation words must be 8-byte aligned");
+    return gemm_common(c, c_type, a, b, ab_type, c_in, bias, quant_words, per_column ? 1 : 0, m, n, k, lda, ldb, ldc, b_layout,
+                       relu, stream_);
+}
+
+static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
+                       const uint64_t* qwords, int q_per_column, int m, int n, int k, int lda, int ldb, int ldc, int b_layout,
+                       int relu, void* stream_)
 {
     hipStream_t stream = as_stream(stream_);
     PTOAMD_REQUIRE(c && a && b, PTOAMD_E_INVALID, "ptoamd_gemm: null operand");
@@ -401,7 +456,9 @@ int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_t
     PTOAMD_REQUIRE(is_int || is_float, PTOAMD_E_UNSUPPORTED,
                    "ptoamd_gemm: operand type %d is not a TMATMUL input type (s8, f16, bf16, f32, e4m3, e5m2)", ab_type);
     int out_kind;
-    if (is_int) {
+    if (qwords != nullptr) {
+        out_kind = c_type == PTOAMD_F16 ? OUT_QF16 : OUT_Q8;
+    } else if (is_int) {
         PTOAMD_REQUIRE(c_type == PTOAMD_I32, PTOAMD_E_UNSUPPORTED, "ptoamd_gemm: int8 operands accumulate to int32 only");
         out_kind = OUT_I32;
     } else {
@@ -421,6 +478,7 @@ int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_t
         g.sbk = b_layout == PTOAMD_B_DN ? 1 : ldb;
         g.sbn = b_layout == PTOAMD_B_DN ? ldb : 1;
         g.a_type = g.b_type = ab_type; g.out_kind = out_kind; g.relu = relu;
+        g.qwords = qwords; g.q_per_column = q_per_column;
         return launch_generic(g, stream);
     }
     StreamTemp bt(stream);
@@ -447,6 +505,7 @@ int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_t
     p.m = m; p.n = n; p.k_bytes = (int)k_bytes;
     p.lda_bytes = lda_b; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
     p.relu = relu; p.out_kind = out_kind; p.group_m = 4;
+    p.qwords = qwords; p.q_per_column = q_per_column;
     const int op = ab_type == PTOAMD_BF16 ? TOP_BF16
                    : ab_type == PTOAMD_F16 ? TOP_F16
                    : ab_type == PTOAMD_I8 ? TOP_I8
@@ -509,7 +568,8 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
 // addressed in place by the register-staged tiles when not.
 static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, const void* b, int a_type, int b_type,
                           const uint8_t* sa, const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n,
-                          int k, int lda, int ldb, int ldc, int b_layout, uint8_t* ws, size_t ws_bytes, void* stream_)
+                          int k, int lda, int ldb, int ldc, int b_layout, uint8_t* ws, size_t ws_bytes, void* stream_,
+                          const float* bias = nullptr)
 {
     hipStream_t stream = as_stream(stream_);
     PTOAMD_REQUIRE(c && a && b && sa && sb, PTOAMD_E_INVALID, "%s: null operand", who);
@@ -541,7 +601,7 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
                          (lda_b % 16) == 0 && (ldb_b % 16) == 0 && (k_bytes % 128) == 0;
     if (!tile_ok) {
         GenericParams g{};
-        g.a = a; g.b = b; g.c = c; g.c_in = c_in; g.sa = sa; g.sb = sb;
+        g.a = a; g.b = b; g.c = c; g.c_in = c_in; g.sa = sa; g.sb = sb; g.bias = bias;
         g.m = m; g.n = n; g.k = k; g.lda = lda; g.ldc = ldc;
         g.sbk = b_layout == PTOAMD_B_DN ? 1 : ldb;
         g.sbn = b_layout == PTOAMD_B_DN ? ldb : 1;
@@ -587,7 +647,7 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
     TileGemmParams p{};
     p.a = reinterpret_cast<const uint8_t*>(a);
     p.b = reinterpret_cast<const uint8_t*>(b);
-    p.c = c; p.c_in = c_in; p.sa = sa_nd; p.sb = sb_dn;
+    p.c = c; p.c_in = c_in; p.sa = sa_nd; p.sb = sb_dn; p.bias = bias;
     p.m = m; p.n = n; p.k_bytes = (int)k_bytes; p.lda_bytes = lda_b; p.ldb_bytes = ldb_b; p.ldc = ldc;
     p.scale_ld = kg; p.out_kind = out_kind; p.group_m = 4;
     p.sa_mode = sa_mode; p.sb_mode = sb_mode;
@@ -615,6 +675,14 @@ int ptoamd_gemm_mx(void* c, int c_type, const void* a, const void* b, int a_type
 {
     return gemm_mx_common("ptoamd_gemm_mx", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k, lda, ldb,
                           ldc, b_layout, nullptr, 0, stream_);
+}
+
+int ptoamd_gemm_mx_bias(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
+                        const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, const float* bias, int m, int n,
+                        int k, int lda, int ldb, int ldc, int b_layout, void* stream_)
+{
+    return gemm_mx_common("ptoamd_gemm_mx_bias", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k, lda,
+                          ldb, ldc, b_layout, nullptr, 0, stream_, bias);
 }
 
 int ptoamd_gemm_mx_ws(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,

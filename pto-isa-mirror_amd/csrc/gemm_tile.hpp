@@ -44,6 +44,9 @@ struct TileGemmParams {
     //   1  16-row x 2-group boxes (MX_A_ZZ, MX_B_NN): base = (x / 16) * scale_ld * 16 + (x % 16) * 2, pair_stride 32
     //   2  pair-major (MX_A_DN, MX_B_ND): base = x * 2, pair_stride = 2 * rows (m for A, n for B)
     int sa_mode, sb_mode;
+    // OUT_Q8 / OUT_QF16: the fix-pipe quantisation words of the drain, one for the whole matrix or one per column
+    const uint64_t* qwords;
+    int q_per_column;
 };
 
 __device__ __forceinline__ long mx_scale_base(int mode, int x, int scale_ld)
@@ -52,7 +55,8 @@ __device__ __forceinline__ long mx_scale_base(int mode, int x, int scale_ld)
 }
 __device__ __forceinline__ long mx_pair_stride(int mode, int rows) { return mode == 0 ? 2 : (mode == 1 ? 32 : 2L * rows); }
 
-enum OutKind { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2, OUT_I32 = 3, OUT_W8A8_BF16 = 4 };
+// OUT_Q8: one byte per element, signed or unsigned as the quantisation word says; OUT_QF16: half through the same words
+enum OutKind { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2, OUT_I32 = 3, OUT_W8A8_BF16 = 4, OUT_Q8 = 5, OUT_QF16 = 6 };
 
 // ---- MFMA operand traits ------------------------------------------------------------------------------------
 // Every mma() hands the matrix instruction B's fragment as its first operand and A's as its second, so a 32x32
@@ -213,7 +217,8 @@ __device__ __forceinline__ constexpr int acc_col(int r, int lhi) { return 8 * (r
 // wave-uniform branch per term and block; tested per element they turn the epilogue into thousands of basic blocks,
 // hundreds of KiB of code, and the instruction fetch -- not the stores -- sets its duration.
 // gi: the lane's row of C; col_b: first column of the block.
-template <bool FULL, class Cfg, class Acc>
+// RELU: apply p.relu here (the quantising kinds clamp at zero after the quantisation instead).
+template <bool FULL, bool RELU, class Cfg, class Acc>
 __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int gi, int col_b, int lhi)
 {
     using Elem = typename Cfg::Op::Elem;
@@ -234,7 +239,7 @@ __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int 
                 v[r] += reinterpret_cast<const Elem*>(p.bias)[gj];
         }
     }
-    if (p.relu) {
+    if (RELU && p.relu) {
 #pragma unroll
         for (int r = 0; r < 16; ++r)
             v[r] = v[r] > 0 ? v[r] : 0;
@@ -242,10 +247,10 @@ __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int 
     return v;
 }
 
-// bits of one output element (2-byte kinds in the low half); W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16, each
-// step rounded to f32
+// bits of one output element (1- and 2-byte kinds in the low part); W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16,
+// each step rounded to f32; the quantising kinds: fix-pipe word `qw`, then relu
 template <int KIND, class V>
-__device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs)
+__device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_t qw = 0, bool q_vector = false, bool relu = false)
 {
     if (KIND == OUT_F32)
         return __builtin_bit_cast(uint32_t, (float)v);
@@ -255,10 +260,20 @@ __device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs)
         return f32_to_f16_bits((float)v);
     if (KIND == OUT_BF16)
         return f32_to_bf16_bits((float)v);
+    if (KIND == OUT_Q8 || KIND == OUT_QF16) {
+        constexpr bool src_int = std::is_same<V, int32_t>::value || std::is_same<V, int>::value;
+        constexpr bool byte = KIND == OUT_Q8;
+        float r = q_vector ? fixpipe_quantize<true, byte, src_int>((float)v, qw) : fixpipe_quantize<false, byte, src_int>((float)v, qw);
+        if (relu)
+            r = r > 0 ? r : 0;
+        return byte ? ((uint32_t)(int32_t)r & 0xFFu) : (uint32_t)f32_to_f16_bits(r);
+    }
     return f32_to_bf16_bits(__fmul_rn(__fmul_rn((float)v, rs), cs));
 }
 template <int KIND>
-constexpr int out_bytes = (KIND == OUT_F32 || KIND == OUT_I32) ? 4 : 2;
+constexpr int out_bytes = (KIND == OUT_F32 || KIND == OUT_I32) ? 4 : (KIND == OUT_Q8 ? 1 : 2);
+template <int KIND>
+constexpr bool out_quant = KIND == OUT_Q8 || KIND == OUT_QF16;
 
 // Element-wise form: any alignment, any edge.  A lane's elements are 4-column runs of one row, so this form is slow
 // (short scattered stores); whole, aligned wave tiles take the staged form below.
@@ -267,7 +282,7 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
 {
     const int gi = row_b + l32;
     const float rs = (KIND == OUT_W8A8_BF16 && (FULL || gi < p.m)) ? p.row_scale[gi] : 1.0f;
-    const Acc v = tstore_terms<FULL, Cfg>(p, acc, gi, col_b, lhi);
+    const Acc v = tstore_terms<FULL, !out_quant<KIND>, Cfg>(p, acc, gi, col_b, lhi);
     const bool raw = KIND == OUT_W8A8_BF16 && p.acc_out != nullptr;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -275,11 +290,14 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
         if (FULL || (gi < p.m && gj < p.n)) {
             const long o = (long)gi * p.ldc + gj;
             const float cs = KIND == OUT_W8A8_BF16 ? p.col_scale[gj] : 1.0f;
-            const uint32_t bits = tstore_bits<KIND>(v[r], rs, cs);
+            const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? gj : 0] : 0;
+            const uint32_t bits = tstore_bits<KIND>(v[r], rs, cs, qw, p.q_per_column != 0, p.relu != 0);
             if (out_bytes<KIND> == 4)
                 reinterpret_cast<uint32_t*>(p.c)[o] = bits;
-            else
+            else if (out_bytes<KIND> == 2)
                 reinterpret_cast<uint16_t*>(p.c)[o] = (uint16_t)bits;
+            else
+                reinterpret_cast<uint8_t*>(p.c)[o] = (uint8_t)bits;
             if (raw)
                 p.acc_out[o] = (int32_t)v[r];
         }
@@ -291,7 +309,11 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
 template <bool FULL, class Cfg, class Acc>
 __device__ __forceinline__ void tstore_block_kind(const TileGemmParams& p, const Acc& acc, int row_b, int col_b, int l32, int lhi)
 {
-    if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
+    if (p.out_kind == OUT_Q8) {
+        tstore_block<OUT_Q8, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
+    } else if (p.out_kind == OUT_QF16) {
+        tstore_block<OUT_QF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
+    } else if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
         if (p.out_kind == OUT_I32)
             tstore_block<OUT_I32, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
         else
@@ -315,7 +337,7 @@ struct StagedStore {
     // sized for 4-byte outputs; the 16 pad bytes per row keep the 32 rows a band's lanes write off each other's banks
     static constexpr int WAVE_BYTES = 32 * (Cfg::WTN * 4 + 16);
     static_assert(Cfg::THREADS / 64 * WAVE_BYTES <= Cfg::LDS_BYTES, "staging regions fit in the operand ring");
-    static_assert((32 * Cfg::WTN * 2 / 16) % 64 == 0, "a band is a whole number of 64-lane reads");
+    static_assert((32 * Cfg::WTN / 16) % 64 == 0, "a band is a whole number of 64-lane reads, down to one-byte outputs");
 };
 
 // `stage` is the calling wave's private LDS region of StagedStore<Cfg>::WAVE_BYTES bytes; the wave's tile lies inside
@@ -335,7 +357,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
             constexpr int j = decltype(jc)::value;
             __builtin_amdgcn_sched_barrier(0);
             const int col_b = col0 + j * 32;
-            const Acc v = tstore_terms<true, Cfg>(p, acc[i][j], gi, col_b, lhi);
+            const Acc v = tstore_terms<true, !out_quant<KIND>, Cfg>(p, acc[i][j], gi, col_b, lhi);
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 uint8_t* dst = stage + l32 * ROW_BYTES + (j * 32 + 8 * g + 4 * lhi) * ESZ;
@@ -351,12 +373,16 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
                 } else {
                     uint32_t bits[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f);
+                    for (int e = 0; e < 4; ++e) {
+                        const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? col_b + 8 * g + 4 * lhi + e : 0] : 0;
+                        bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0);
+                    }
                     if (ESZ == 4)
                         *reinterpret_cast<uint4*>(dst) = make_uint4(bits[0], bits[1], bits[2], bits[3]);
-                    else
+                    else if (ESZ == 2)
                         *reinterpret_cast<uint2*>(dst) = make_uint2(bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16));
+                    else
+                        *reinterpret_cast<uint32_t*>(dst) = bits[0] | (bits[1] << 8) | (bits[2] << 16) | (bits[3] << 24);
                 }
             }
         });
@@ -380,10 +406,14 @@ __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::
                                        int lhi, uint8_t* stage = nullptr)
 {
     const bool full = row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n;
-    const int esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : 2;
+    const int esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : (p.out_kind == OUT_Q8 ? 1 : 2);
     const bool aligned = (((long)p.ldc * esz) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
     if (stage != nullptr && full && aligned && !(p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr)) {
-        if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
+        if (p.out_kind == OUT_QF16) {
+            tstore_staged<OUT_QF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
+        } else if (p.out_kind == OUT_Q8) {
+            tstore_staged<OUT_Q8, Cfg>(p, acc, row0, col0, l32, lhi, stage);
+        } else if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
             if (p.out_kind == OUT_I32)
                 tstore_staged<OUT_I32, Cfg>(p, acc, row0, col0, l32, lhi, stage);
             else

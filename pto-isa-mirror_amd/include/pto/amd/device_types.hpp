@@ -55,6 +55,40 @@ __device__ __forceinline__ float e8m0_to_f32(uint32_t e)
     return e == 0 ? u2f(0x00400000u) : u2f(e << 23);
 }
 
+// Fix-pipe quantisation words (reference: cpu/common.hpp:117-185).  A scalar word carries an fp32 scale in its low 32
+// bits; a vector (per-column) word a 19-bit (1, 8, 10) float at bits 13..31.  Bits 37..45 hold the offset added before
+// rounding to an 8-bit target and bit 46 that target's signedness.
+template <bool VECTOR>
+__device__ __forceinline__ float fixpipe_word_scale(uint64_t word)
+{
+    if (!VECTOR)
+        return u2f((uint32_t)(word & 0xFFFFFFFFu));
+    const uint32_t m1 = (uint32_t)((word >> 13) & 0x7FFFFu);
+    const uint32_t s = (m1 >> 18) & 1u, e = (m1 >> 10) & 0xFFu, mant = m1 & 0x3FFu;
+    if (e == 0 && mant == 0)
+        return 0.0f;
+    const float mv = 1.0f + (float)mant / 1024.0f;
+    return __fmul_rn(__fmul_rn(s ? -1.0f : 1.0f, mv), e8m0_to_f32(e));
+}
+// acc * scale, then: 8-bit targets add the offset, round to nearest even and clamp to the signed or unsigned byte range
+// (the result is the integer as a float); the half target clamps finite values to +-65504 (every value when the
+// accumulator was an integer)
+template <bool VECTOR, bool TO_BYTE, bool SRC_INT>
+__device__ __forceinline__ float fixpipe_quantize(float acc, uint64_t word)
+{
+    float r = __fmul_rn(acc, fixpipe_word_scale<VECTOR>(word));
+    if (TO_BYTE) {
+        const float offset = (float)(uint32_t)((word >> 37) & 0x1FFu);
+        const bool sign = (word >> 46) & 1u;
+        const float rounded = rintf(__fadd_rn(r, offset));
+        const float lo = sign ? -128.0f : 0.0f, hi = sign ? 127.0f : 255.0f;
+        r = rounded < lo ? lo : (rounded > hi ? hi : rounded);
+    } else if (SRC_INT || (r == r && fabsf(r) != __builtin_inff())) {
+        r = r < -65504.0f ? -65504.0f : (r > 65504.0f ? 65504.0f : r);
+    }
+    return r;
+}
+
 __device__ __forceinline__ float e4m3_to_f32(uint32_t c)
 {
     const uint32_t mag = c & 0x7Fu;

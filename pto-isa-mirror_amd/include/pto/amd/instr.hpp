@@ -408,16 +408,7 @@ PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
 template <bool VECTOR>
 PTO_INST float quant_word_scale(uint64_t word)
 {
-    if constexpr (!VECTOR) {
-        return ptoamd::u2f((uint32_t)(word & 0xFFFFFFFFu));
-    } else {
-        const uint32_t m1 = (uint32_t)((word >> 13) & 0x7FFFFu);
-        const uint32_t s = (m1 >> 18) & 1u, e = (m1 >> 10) & 0xFFu, mant = m1 & 0x3FFu;
-        if (e == 0 && mant == 0)
-            return 0.0f;
-        const float mv = 1.0f + (float)mant / 1024.0f;
-        return __fmul_rn(__fmul_rn(s ? -1.0f : 1.0f, mv), ptoamd::e8m0_to_f32(e));
-    }
+    return ptoamd::fixpipe_word_scale<VECTOR>(word);
 }
 template <bool VECTOR, typename G, typename Reg>
 PTO_INST float quantize_element(Reg acc, uint64_t word)
@@ -433,14 +424,9 @@ PTO_INST float quantize_element(Reg acc, uint64_t word)
         const int shift = (int)((word >> 32) & 0xFu) + 1;
         r = (float)(int16_t)((int32_t)acc >> shift);
     } else if constexpr (sizeof(G) == 1) {
-        const float offset = (float)(uint32_t)((word >> 37) & 0x1FFu);
-        const bool sign = (word >> 46) & 1u;
-        const float rounded = rintf(__fadd_rn(r, offset));
-        const float lo = sign ? -128.0f : 0.0f, hi = sign ? 127.0f : 255.0f;
-        r = rounded < lo ? lo : (rounded > hi ? hi : rounded);
+        r = ptoamd::fixpipe_quantize<VECTOR, true, src_is_int>((float)acc, word);
     } else if constexpr (std::is_same_v<G, _Float16>) {
-        if (src_is_int || (r == r && fabsf(r) != __builtin_inff()))
-            r = r < -65504.0f ? -65504.0f : (r > 65504.0f ? 65504.0f : r);
+        r = ptoamd::fixpipe_quantize<VECTOR, false, src_is_int>((float)acc, word);
     } else {
         if (r == r && fabsf(r) != __builtin_inff())
             r = r < -3.402823466e38f ? -3.402823466e38f : (r > 3.402823466e38f ? 3.402823466e38f : r);

@@ -330,6 +330,99 @@ def test_config3_w8a8_full_size(pa, oracle):
     assert torch.equal(acc[:64].to(torch.int64).sum(1), want)
 
 
+def _word_scalar(scale, offset=0, sign=1):
+    return int(np.float32(scale).view(np.uint32)) | (offset << 37) | (sign << 46)
+
+
+def _word_vector(scale, offset=0, sign=1):
+    bits = int(np.float32(scale).view(np.uint32))
+    m1 = ((bits >> 31) << 18) | (((bits >> 23) & 0xFF) << 10) | ((bits >> 13) & 0x3FF)
+    return (m1 << 13) | (offset << 37) | (sign << 46)
+
+
+# (m, n, k) of the reference's tstore_acc2gm / tstore_quant cases that quantise, plus shapes that fill whole MFMA tiles
+REQUANT_SHAPES = [(128, 128, 64), (31, 32, 96), (65, 96, 80), (256, 256, 128), (300, 200, 136)]
+
+
+@pytest.mark.parametrize("tile", [None, 2, 4, 5])
+@pytest.mark.parametrize("m,n,k", REQUANT_SHAPES)
+def test_requant_drain_float_accumulator(pa, oracle, tile, m, n, k):
+    """f16 x f16 -> f32 accumulator -> int8 / uint8 / f16 through scalar and per-column words (integer-valued inputs:
+    the accumulator is exact, so the drain must equal oracle.store_quant bit for bit)."""
+    r = np.random.default_rng(m + n + k)
+    a = r.integers(-4, 5, (m, k)).astype(np.float16)
+    b = r.integers(-4, 5, (n, k)).astype(np.float16)
+    bias = r.integers(-20, 20, n).astype(np.float32)
+    acc = oracle.matmul_f16(a.view(np.uint16), b.view(np.uint16), b_dn=True)
+    da, db = dev(a), dev(b)
+    scalar = np.array([_word_scalar(0.37, offset=3)], np.uint64)
+    scalar_u = np.array([_word_scalar(0.21, offset=100, sign=0)], np.uint64)
+    vector = np.array([_word_vector(s, offset=int(o)) for s, o in zip(r.uniform(0.01, 0.9, n), r.integers(0, 8, n))], np.uint64)
+    env = tile_env(PTOAMD_TILE=tile) if tile is not None else tile_env()
+    with env:
+        got = host(pa.gemm_requant(da, db, pa.F16, pa.I8, dev(scalar.view(np.int64))))
+        assert pa.last_kernel().startswith("tile")
+        assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I8, scalar, per_column=False))
+        got = host(pa.gemm_requant(da, db, pa.F16, pa.U8, dev(scalar_u.view(np.int64)), relu=True))
+        assert np.array_equal(got, oracle.store_quant(acc, ob.ST_U8, scalar_u, per_column=False, relu=True))
+        got = host(pa.gemm_requant(da, db, pa.F16, pa.I8, dev(vector.view(np.int64)), per_column=True, relu=True))
+        assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I8, vector, per_column=True, relu=True))
+        got = host(pa.gemm_requant(da, db, pa.F16, pa.F16, dev(vector.view(np.int64)), per_column=True))
+        assert np.array_equal(got.view(np.uint16), oracle.store_quant(acc, ob.ST_F16, vector, per_column=True))
+        got = host(pa.gemm_requant(da, db, pa.F16, pa.I8, dev(scalar.view(np.int64)), bias=dev(bias)))
+        assert np.array_equal(got, oracle.store_quant(acc + bias, ob.ST_I8, scalar, per_column=False))
+    with tile_env(PTOAMD_FORCE_GENERIC=1):
+        got = host(pa.gemm_requant(da, db, pa.F16, pa.I8, dev(vector.view(np.int64)), per_column=True, relu=True))
+        assert pa.last_kernel() == "generic"
+        assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I8, vector, per_column=True, relu=True))
+
+
+@pytest.mark.parametrize("tile", [None, 2, 4, 5])
+@pytest.mark.parametrize("m,n,k", REQUANT_SHAPES)
+def test_requant_drain_int32_accumulator(pa, oracle, tile, m, n, k):
+    """int8 x int8 -> int32 -> int8 (requant) and -> f16 (dequant), scalar and per-column words."""
+    k = (k + 15) // 16 * 16
+    r = np.random.default_rng(m * 3 + n + k)
+    a = r.integers(-128, 128, (m, k)).astype(np.int8)
+    b = r.integers(-128, 128, (n, k)).astype(np.int8)
+    acc = oracle.matmul_i8(a, b, b_dn=True)
+    da, db = dev(a), dev(b)
+    scalar = np.array([_word_scalar(2.0 ** -9, offset=5)], np.uint64)
+    vector = np.array([_word_vector(s) for s in r.uniform(1e-4, 3e-3, n)], np.uint64)
+    env = tile_env(PTOAMD_TILE=tile) if tile is not None else tile_env()
+    with env:
+        got = host(pa.gemm_requant(da, db, pa.I8, pa.I8, dev(scalar.view(np.int64))))
+        assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I8, scalar, per_column=False))
+        got = host(pa.gemm_requant(da, db, pa.I8, pa.F16, dev(vector.view(np.int64)), per_column=True))
+        assert np.array_equal(got.view(np.uint16), oracle.store_quant(acc, ob.ST_F16, vector, per_column=True))
+        got = host(pa.gemm_requant(da, db, pa.I8, pa.I8, dev(vector.view(np.int64)), per_column=True, relu=True))
+        assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I8, vector, per_column=True, relu=True))
+
+
+def test_requant_rejects_other_output_types(pa):
+    a = torch.zeros((16, 16), dtype=torch.float16, device=DEV)
+    w = torch.zeros(1, dtype=torch.int64, device=DEV)
+    with pytest.raises(pa.PtoAmdError, match="fix-pipe quantiser"):
+        pa.gemm_requant(a, a, pa.F16, pa.F32, w, out=torch.zeros((16, 16), dtype=torch.float32, device=DEV))
+
+
+def test_mx_gemm_with_bias(pa, oracle):
+    """TMATMUL_MX with a bias tile: added to every row after the K loop, on the MFMA tiles and the generic kernel."""
+    r = np.random.default_rng(9)
+    m, n, k = 200, 192, 256
+    a, b, sa, sb = _mx_inputs(r, ob.E4M3, m, n, k)
+    bias = r.uniform(-50, 50, n).astype(np.float32)
+    ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ob.E4M3, ob.E4M3, bias=bias)
+    plain = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, pa.E4M3, pa.E4M3, pa.F32))
+    got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, pa.E4M3, pa.E4M3, pa.F32, bias=dev(bias)))
+    assert pa.last_kernel().startswith("tile")
+    assert np.array_equal(got, plain + bias)  # one fp32 add after the sum
+    assert relerr(got, ref) <= 2e-2
+    with tile_env(PTOAMD_FORCE_GENERIC=1):
+        exact = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, pa.E4M3, pa.E4M3, pa.F32, bias=dev(bias)))
+    assert np.array_equal(exact.view(np.uint32), ref.view(np.uint32))
+
+
 @pytest.mark.parametrize("tile", [2, 4, 5])
 def test_tmatmul_bias(pa, oracle, tile):
     """TMATMUL_BIAS: the bias row is added to every row after the K loop, before relu and the TSTORE conversion
