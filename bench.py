@@ -140,6 +140,59 @@ def config5(pa, ev, gen, steps, warmup):
                 frac_of_peak=nbytes / ker / 1e6 / PEAK_HBM_GBPS)
 
 
+def _elementwise(name, kernel, nbytes, wall, ker):
+    return dict(config=name, kernel=kernel, ms=ker, wall_ms=wall, gbps=nbytes / ker / 1e6, bound="hbm",
+                frac_of_peak=nbytes / ker / 1e6 / PEAK_HBM_GBPS, algorithmic_bytes=nbytes)
+
+
+def _rotating(make, copies):
+    """`copies` instances of an input, used in turn, so that every launch reads from HBM and not from the 256 MB MALL."""
+    items = [make() for _ in range(copies)]
+    state = {"i": 0}
+
+    def nxt():
+        state["i"] += 1
+        return items[state["i"] % copies]
+    return nxt
+
+
+def quant_mxfp8(pa, ev, gen, steps, warmup):
+    rows, cols = 14336, 4096  # the weight matrix of configs[3]
+    src = _rotating(lambda: randn_bf16((rows, cols), gen), 4)
+    out = (torch.empty((rows, cols), dtype=torch.uint8, device=DEV), torch.empty((rows, cols // 32), dtype=torch.uint8, device=DEV))
+    wall, ker = time_launches(ev, lambda: pa.tquant_mx(src(), pa.OCP_MXFP8, want_aux=False, out=out), steps, warmup)
+    return _elementwise("TQUANT OCP-MXFP8, bf16 14336x4096 -> E4M3 codes + E8M0 exponents", "tquant_mx_rows",
+                        rows * cols * 2 + rows * cols + rows * cols // 32, wall, ker)
+
+
+def quant_mxfp4(pa, ev, gen, steps, warmup):
+    rows, cols = 28672, 8192  # the weight matrix of configs[4]; 470 MB of bf16, larger than the MALL
+    src = randn_bf16((rows, cols), gen)
+    out = (torch.empty((rows, cols // 2), dtype=torch.uint8, device=DEV), torch.empty((rows, cols // 32), dtype=torch.uint8, device=DEV))
+    wall, ker = time_launches(ev, lambda: pa.tquant_mx(src, pa.OCP_MXFP4, want_aux=False, out=out), steps, warmup)
+    return _elementwise("TQUANT OCP-MXFP4, bf16 28672x8192 -> E2M1 codes + E8M0 exponents", "tquant_mx_rows",
+                        rows * cols * 2 + rows * cols // 2 + rows * cols // 32, wall, ker)
+
+
+def quant_int8(pa, ev, gen, steps, warmup):
+    rows, cols = 2048, 8192  # the activation matrix of configs[2]
+    src = _rotating(lambda: torch.randn((rows, cols), generator=gen, device=DEV), 8)
+    scale = torch.rand(rows, generator=gen, device=DEV) * 20 + 1
+    out = torch.empty((rows, cols), dtype=torch.int8, device=DEV)
+    wall, ker = time_launches(ev, lambda: pa.tquant_int8(src(), scale, out=out), steps, warmup)
+    return _elementwise("TQUANT INT8_SYM, f32 2048x8192 -> int8", "tquant_int8", rows * cols * 5 + rows * 4, wall, ker)
+
+
+def dequant_int8(pa, ev, gen, steps, warmup):
+    rows, cols = 2048, 8192
+    src = _rotating(lambda: torch.randint(-128, 128, (rows, cols), generator=gen, device=DEV, dtype=torch.int8), 8)
+    scale = torch.rand(rows, generator=gen, device=DEV) + 0.5
+    offset = torch.rand(rows, generator=gen, device=DEV) * 10
+    out = torch.empty((rows, cols), dtype=torch.float32, device=DEV)
+    wall, ker = time_launches(ev, lambda: pa.tdequant(src(), scale, offset, out=out), steps, warmup)
+    return _elementwise("TDEQUANT int8 2048x8192 -> f32", "tdequant", rows * cols * 5 + rows * 8, wall, ker)
+
+
 def cpu_baseline():
     """The reference CPU simulator itself where its compiled form is present (oracle/_ref, built from the reference's
     headers: TLOAD / TMOV / TMATMUL_ACC / TSTORE on 256 x 256 output tiles, K walked by 512), else the plain-C port of
@@ -162,8 +215,9 @@ def cpu_baseline():
         dt = time.perf_counter() - t0
         flop = 2.0 * m * n * cols * k
         return {"value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "reference",
-                "sample": f"{cols} output tiles of 256 x 256 (rows 0-255, columns 0-{cols * n - 1}) x K=4096, fp16 inputs "
-                          f"({flop / 1e9:.1f} GFLOP) in {dt:.1f} s; full 4096^3 extrapolates to {dt * 256 / cols:.0f} s"}
+                "sample": f"{cols} independent 256 x 256 x 4096 output tiles of the workload (one A row panel against {cols} "
+                          f"B column panels), fp16 stand-in for bf16 ({flop / 1e9:.1f} GFLOP) in {dt:.1f} s; the full 4096^3 "
+                          f"is 256 such tiles and extrapolates to {dt * 256 / cols:.0f} s"}
     orc = Oracle()
     m, n = 256, 4096
     a = ((rng.standard_normal((m, k)) * 0.02).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
@@ -187,8 +241,9 @@ def main():
                     help="untimed run-in of the same launches before the warmup steps, for the GPU clock to settle")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-config measurements after the headline")
-    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4], default=None,
-                    help="measure just BASELINE.json configs[N] (a per_config entry) and print it: for profiling one kernel")
+    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4, 5, 6, 7, 8], default=None,
+                    help="measure just BASELINE.json configs[N] (a per_config entry) and print it: for profiling one kernel; "
+                         "5-8 are the elementwise kernels (TQUANT MXFP8, TQUANT MXFP4, TQUANT INT8, TDEQUANT)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -209,7 +264,8 @@ def main():
         del src, dst
     gen = torch.Generator(device=DEV).manual_seed(1)
     if args.only is not None:
-        fn = {0: config1, 2: config3, 3: config4, 4: config5}[args.only]
+        fn = {0: config1, 2: config3, 3: config4, 4: config5, 5: quant_mxfp8, 6: quant_mxfp4, 7: quant_int8,
+              8: dequant_int8}[args.only]
         print(json.dumps(fn(pa, ev, gen, args.steps, args.warmup)))
         return
 
@@ -235,7 +291,7 @@ def main():
     }
     if not args.no_extra:
         per = []
-        for fn in (config1, config3, config4, config5):
+        for fn in (config1, config3, config4, config5, quant_mxfp8, quant_mxfp4, quant_int8, dequant_int8):
             per.append(fn(pa, ev, gen, 50, 5))
             torch.cuda.empty_cache()
         line["per_config"] = per

@@ -179,9 +179,10 @@ def gemv_mxfp4(a_bf16, w, sw, n, k, c_type=F32, stream=None, out=None):
     return out
 
 
-def tquant_int8(src, scale, offset=None, stream=None):
+def tquant_int8(src, scale, offset=None, stream=None, out=None):
     rows, cols = src.shape
-    out = torch.empty((rows, cols), dtype=torch.int8 if offset is None else torch.uint8, device=src.device)
+    if out is None:
+        out = torch.empty((rows, cols), dtype=torch.int8 if offset is None else torch.uint8, device=src.device)
     _check(_lib.ptoamd_tquant_int8(_ptr(out), _ptr(src), _ptr(scale), _ptr(offset), rows, cols, _stream(stream)),
            "ptoamd_tquant_int8")
     return out
@@ -190,13 +191,16 @@ def tquant_int8(src, scale, offset=None, stream=None):
 _SRC_TYPE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 
-def tquant_mx(src, alg, axis=1, want_aux=True, stream=None):
-    """TQUANT<MXFP8 | MXFP4_E2M1>: returns (codes, exp[, max, scaling])."""
+def tquant_mx(src, alg, axis=1, want_aux=True, stream=None, out=None):
+    """TQUANT<MXFP8 | MXFP4_E2M1>: returns (codes, exp[, max, scaling]).  out: (codes, exp) tensors to write into."""
     rows, cols = src.shape
     fp4 = alg in (OCP_MXFP4, NV_MXFP4)
-    codes = torch.empty((rows, cols // 2 if fp4 else cols), dtype=torch.uint8, device=src.device)
     gshape = (rows, cols // 32) if axis == 1 else (rows // 32, cols)
-    exp = torch.empty(gshape, dtype=torch.uint8, device=src.device)
+    if out is not None:
+        codes, exp = out
+    else:
+        codes = torch.empty((rows, cols // 2 if fp4 else cols), dtype=torch.uint8, device=src.device)
+        exp = torch.empty(gshape, dtype=torch.uint8, device=src.device)
     mx = torch.empty(gshape, dtype=torch.float32, device=src.device) if want_aux else None
     sc = torch.empty(gshape, dtype=torch.float32, device=src.device) if want_aux else None
     _check(_lib.ptoamd_tquant_mx(_ptr(codes), _ptr(exp), _ptr(mx), _ptr(sc), _ptr(src), _SRC_TYPE[src.dtype], rows, cols,
@@ -207,9 +211,10 @@ def tquant_mx(src, alg, axis=1, want_aux=True, stream=None):
 _INT_TYPE = {torch.int8: I8, torch.int16: I16, torch.int32: I32}
 
 
-def tdequant(src, scale, offset, stream=None):
+def tdequant(src, scale, offset, stream=None, out=None):
     rows, cols = src.shape
-    out = torch.empty((rows, cols), dtype=torch.float32, device=src.device)
+    if out is None:
+        out = torch.empty((rows, cols), dtype=torch.float32, device=src.device)
     _check(_lib.ptoamd_tdequant(_ptr(out), _ptr(src), _INT_TYPE[src.dtype], _ptr(scale), _ptr(offset), rows, cols,
                                 _stream(stream)), "ptoamd_tdequant")
     return out

@@ -3,6 +3,7 @@
 // codes, shared exponents, group maxima and scalings are bit-identical; citations are given per function.
 #include "common_host.hpp"
 #include "device_types.hpp"
+#include "lds_dma.hpp"
 #include "../include/pto/amd/quant_math.hpp"
 
 namespace ptoamd {
@@ -11,48 +12,91 @@ static_assert(PTOAMD_OCP_MXFP8 == MX_OCP_FP8 && PTOAMD_NV_MXFP8 == MX_NV_FP8 && 
                   PTOAMD_NV_MXFP4 == MX_NV_FP4,
               "the C ABI's algorithm ids are the kernels' template arguments");
 
-// ---- axis 1: 32-element groups along a row.  8 lanes own one group, 4 consecutive elements each. --------------
+// ---- axis 1: 32-element groups along a row.  A lane owns one 16-byte piece of the source (4 f32 or 8 half / bf16
+// elements), so a group is 8 or 4 neighbouring lanes and a wave reads 1 KiB per load instruction; every thread handles
+// UNITS such pieces, one block-wide span apart, with all its loads in flight before the first is used.
+// FP4 codes come from the packed hardware conversion (v_cvt_scalef32_pk_fp4_f32, round to nearest even, saturating): on
+// finite input it is EncodeE2M1Magic (TQuant.hpp:155-176) -- the magic-number add there is a round-to-nearest-even onto
+// the same grid with the same clamp -- and the two cases where that function does not depend on the value alone (an
+// infinite or NaN scaling) are resolved per group before the conversion is consulted.  The bf16 source's re-rounding of
+// the scaled value (TQuant.hpp:68-76) is the identity here: the scaling is a power of two, so the product of a bf16
+// value is a bf16 value again unless it is subnormal, and then it is far below the smallest code either way.
 template <int ALG, typename T, bool SRC_BF16>
-__global__ void tquant_mx_rows_kernel(uint8_t* dst, uint8_t* exp, float* mx, float* scaling, const T* src, long groups)
+__global__ void __launch_bounds__(256) tquant_mx_rows_kernel(uint8_t* dst, uint8_t* exp, float* mx, float* scaling, const T* src, long units)
 {
     constexpr bool FP4 = ALG == PTOAMD_OCP_MXFP4 || ALG == PTOAMD_NV_MXFP4;
-    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    const long g = t >> 3;  // all 8 lanes of a group are in or out together (blockDim is a multiple of 8)
-    const bool live = g < groups;
-    float v[4] = {0, 0, 0, 0};
-    if (live) {
-        const T* p = src + g * 32 + (t & 7) * 4;
+    constexpr int EPL = 16 / (int)sizeof(T), LPG = 32 / EPL, UNITS = 4;
+    const long first = (long)blockIdx.x * (UNITS * 256) + threadIdx.x;
+    uint4 raw[UNITS];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            v[i] = widen<T>(p[i]);
+    for (int u = 0; u < UNITS; ++u) {
+        const long unit = first + u * 256;
+        raw[u] = unit < units ? reinterpret_cast<const uint4*>(src)[unit] : make_uint4(0, 0, 0, 0);
     }
-    uint32_t run = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        run = max_step<ALG>(run, v[i]);
+    for (int u = 0; u < UNITS; ++u) {
+        const long unit = first + u * 256;
+        const bool live = unit < units;  // (a block's span starts on a group boundary: all lanes of a group agree)
+        float v[EPL];
+        const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
 #pragma unroll
-    for (int off = 1; off < 8; off <<= 1)
-        run = max_merge<ALG>(run, (uint32_t)__shfl_xor((int)run, off, 8));
-    if (!live)
-        return;
-    const float maxabs = max_value<ALG>(run, u2f(0x7FC00000u));
-    const uint32_t e = shared_exponent<ALG>(maxabs);
-    const float sc = group_scaling<ALG>(maxabs, e);
-    if ((t & 7) == 0) {
-        exp[g] = (uint8_t)e;
-        if (mx)
-            mx[g] = maxabs;
-        if (scaling)
-            scaling[g] = sc;
-    }
-    uint32_t c[4];
+        for (int i = 0; i < EPL; ++i) {
+            if constexpr (sizeof(T) == 4) {
+                v[i] = u2f(w[i]);
+            } else {
+                T t;
+                t.b = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
+                v[i] = widen<T>(t);
+            }
+        }
+        uint32_t run = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        c[i] = encode_mx<ALG, SRC_BF16>(v[i], sc);
-    if (FP4) {
-        reinterpret_cast<uint16_t*>(dst)[g * 8 + (t & 7)] = (uint16_t)(c[0] | (c[1] << 4) | (c[2] << 8) | (c[3] << 12));
-    } else {
-        reinterpret_cast<uint32_t*>(dst)[g * 8 + (t & 7)] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+        for (int i = 0; i < EPL; ++i)
+            run = max_step<ALG>(run, v[i]);
+#pragma unroll
+        for (int off = 1; off < LPG; off <<= 1)
+            run = max_merge<ALG>(run, (uint32_t)__shfl_xor((int)run, off, LPG));
+        const float maxabs = max_value<ALG>(run, u2f(0x7FC00000u));
+        const uint32_t e = shared_exponent<ALG>(maxabs);
+        const float sc = group_scaling<ALG>(maxabs, e);
+        const long g = unit / LPG;
+        if (live && (threadIdx.x & (LPG - 1)) == 0) {
+            exp[g] = (uint8_t)e;
+            if (mx)
+                mx[g] = maxabs;
+            if (scaling)
+                scaling[g] = sc;
+        }
+        if (FP4) {
+            uint32_t packed = 0;
+            static_for<EPL / 2>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, __fmul_rn(v[2 * i], sc), __fmul_rn(v[2 * i + 1], sc), 1.0f, i);
+            });
+            const uint32_t sb = f2u(sc);  // StoreMxEncodedValue's two special scalings (TQuant.hpp:349-372)
+            if ((sb & 0x7FFFFFFFu) == 0x7F800000u)
+                packed = (sb >> 31) ? 0xFFFFFFFFu : 0x77777777u;
+            else if ((sb & 0x7FFFFFFFu) > 0x7F800000u)
+                packed = 0x77777777u;
+            if (live) {
+                if (EPL == 8)
+                    reinterpret_cast<uint32_t*>(dst)[unit] = packed;
+                else
+                    reinterpret_cast<uint16_t*>(dst)[unit] = (uint16_t)packed;
+            }
+        } else {
+            uint32_t c[EPL];
+#pragma unroll
+            for (int i = 0; i < EPL; ++i)
+                c[i] = encode_mx<ALG, SRC_BF16>(v[i], sc);
+            if (live) {
+                const uint32_t lo = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+                if constexpr (EPL == 8)
+                    reinterpret_cast<uint2*>(dst)[unit] = make_uint2(lo, c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24));
+                else
+                    reinterpret_cast<uint32_t*>(dst)[unit] = lo;
+            }
+        }
     }
 }
 
@@ -129,6 +173,62 @@ __global__ void tquant_int8_kernel(uint8_t* dst, const float* src, const float* 
     }
 }
 
+// Row-parallel forms for matrices whose rows are whole 4-element pieces: blockIdx.y is the row (no division to find the
+// per-row scale), a lane moves four elements per piece -- 16 bytes of f32 in, one dword out -- and UNITS pieces per thread.
+template <bool ASYM>
+__global__ void __launch_bounds__(256) tquant_int8_rows_kernel(uint8_t* dst, const float* src, const float* scale, const float* offset, int cols)
+{
+    constexpr int UNITS = 2;
+    const int r = blockIdx.y;
+    const float s = scale[r], o = ASYM ? offset[r] : 0.0f;
+    const float4* in = reinterpret_cast<const float4*>(src + (long)r * cols);
+    uint32_t* out = reinterpret_cast<uint32_t*>(dst + (long)r * cols);
+    const int pieces = cols >> 2, first = blockIdx.x * (UNITS * 256) + threadIdx.x;
+    float4 v[UNITS];
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u)
+        v[u] = first + u * 256 < pieces ? in[first + u * 256] : make_float4(0, 0, 0, 0);
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+        const float x[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+        uint32_t packed = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float q = __fmul_rn(x[i], s);
+            if (ASYM)
+                q = __fadd_rn(q, o);
+            q = rintf(q);
+            const float lo = ASYM ? 0.0f : -128.0f, hi = ASYM ? 255.0f : 127.0f;
+            q = q < lo ? lo : (q > hi ? hi : q);
+            packed |= ((uint32_t)(int)q & 0xFFu) << (8 * i);
+        }
+        if (first + u * 256 < pieces)
+            out[first + u * 256] = packed;
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) tdequant_rows_kernel(float* dst, const T* src, const float* scale, const float* offset, int cols)
+{
+    constexpr int UNITS = 2;
+    const int r = blockIdx.y;
+    const float s = scale[r], o = offset[r];
+    struct alignas(4 * sizeof(T)) Piece { T e[4]; };
+    const Piece* in = reinterpret_cast<const Piece*>(src + (long)r * cols);
+    float4* out = reinterpret_cast<float4*>(dst + (long)r * cols);
+    const int pieces = cols >> 2, first = blockIdx.x * (UNITS * 256) + threadIdx.x;
+    Piece v[UNITS];
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u)
+        if (first + u * 256 < pieces)
+            v[u] = in[first + u * 256];
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u)
+        if (first + u * 256 < pieces)
+            out[first + u * 256] = make_float4(__fmul_rn(__fsub_rn((float)v[u].e[0], o), s), __fmul_rn(__fsub_rn((float)v[u].e[1], o), s),
+                                               __fmul_rn(__fsub_rn((float)v[u].e[2], o), s), __fmul_rn(__fsub_rn((float)v[u].e[3], o), s));
+}
+
 // ---- TDEQUANT (TDeQuant.hpp:18-37) ---------------------------------------------------------------------------
 template <typename T>
 __global__ void tdequant_kernel(float* dst, const T* src, const float* scale, const float* offset, int rows, int cols)
@@ -146,10 +246,9 @@ static int launch_tquant_mx(uint8_t* dst, uint8_t* exp, float* mx, float* scalin
 {
     const T* s = reinterpret_cast<const T*>(src);
     if (axis == 1) {
-        const long groups = (long)rows * (cols / 32);
-        const long threads = groups * 8;
-        hipLaunchKernelGGL((tquant_mx_rows_kernel<ALG, T, SRC_BF16>), dim3((unsigned)((threads + 255) / 256)), dim3(256),
-                           0, stream, dst, exp, mx, scaling, s, groups);
+        const long units = (long)rows * cols * (long)sizeof(T) / 16;  // 16-byte pieces; a row is a whole number of them
+        hipLaunchKernelGGL((tquant_mx_rows_kernel<ALG, T, SRC_BF16>), dim3((unsigned)((units + 1023) / 1024)), dim3(256),
+                           0, stream, dst, exp, mx, scaling, s, units);
     } else {
         dim3 block(128), grid((cols / 2 + 127) / 128, rows / 32);
         hipLaunchKernelGGL((tquant_mx_cols_kernel<ALG, T, SRC_BF16>), grid, block, 0, stream, dst, exp, mx, scaling, s,
@@ -182,6 +281,17 @@ int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const fl
     PTOAMD_REQUIRE(dst && src && scale, PTOAMD_E_INVALID, "ptoamd_tquant_int8: null operand");
     PTOAMD_REQUIRE(rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_tquant_int8: rows and cols must be positive");
     const long total = (long)rows * cols;
+    if ((cols & 3) == 0 && rows <= 65535 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0 && (reinterpret_cast<uintptr_t>(dst) & 3u) == 0) {
+        const dim3 grid((unsigned)((cols / 4 + 511) / 512), (unsigned)rows);
+        if (offset)
+            hipLaunchKernelGGL(tquant_int8_rows_kernel<true>, grid, dim3(256), 0, as_stream(stream),
+                               reinterpret_cast<uint8_t*>(dst), src, scale, offset, cols);
+        else
+            hipLaunchKernelGGL(tquant_int8_rows_kernel<false>, grid, dim3(256), 0, as_stream(stream),
+                               reinterpret_cast<uint8_t*>(dst), src, scale, offset, cols);
+        PTOAMD_HIP_CHECK(hipGetLastError());
+        return PTOAMD_OK;
+    }
     const unsigned blocks = (unsigned)((total / 4 + 256) / 256);
     if (offset)
         hipLaunchKernelGGL(tquant_int8_kernel<true>, dim3(blocks), dim3(256), 0, as_stream(stream),
@@ -204,8 +314,8 @@ int ptoamd_tquant_mx(uint8_t* dst, uint8_t* exp, float* max, float* scaling, con
     PTOAMD_REQUIRE(axis == 1 ? cols % 32 == 0 : rows % 32 == 0, PTOAMD_E_INVALID,
                    "ptoamd_tquant_mx: the grouped axis must be a multiple of 32 (rows %d, cols %d, axis %d)", rows, cols, axis);
     PTOAMD_REQUIRE(cols % 2 == 0, PTOAMD_E_INVALID, "ptoamd_tquant_mx: cols must be even");
-    PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(dst) & 3u) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0,
-                   PTOAMD_E_ALIGNMENT, "ptoamd_tquant_mx: dst must be 4-byte and src 16-byte aligned");
+    PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(dst) & 7u) == 0 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0,
+                   PTOAMD_E_ALIGNMENT, "ptoamd_tquant_mx: dst must be 8-byte and src 16-byte aligned");
     hipStream_t s = as_stream(stream);
     switch (alg) {
         case PTOAMD_OCP_MXFP8: return dispatch_src<PTOAMD_OCP_MXFP8>(dst, exp, max, scaling, src, src_type, rows, cols, axis, s);
@@ -224,6 +334,23 @@ int ptoamd_tdequant(float* dst, const void* src, int src_type, const float* scal
     const long total = (long)rows * cols;
     const dim3 grid((unsigned)((total + 255) / 256)), block(256);
     hipStream_t s = as_stream(stream);
+    if ((cols & 3) == 0 && rows <= 65535 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+        const dim3 rgrid((unsigned)((cols / 4 + 511) / 512), (unsigned)rows);
+        switch (src_type) {
+            case PTOAMD_I8:
+                hipLaunchKernelGGL(tdequant_rows_kernel<int8_t>, rgrid, block, 0, s, dst, reinterpret_cast<const int8_t*>(src), scale, offset, cols);
+                break;
+            case PTOAMD_I16:
+                hipLaunchKernelGGL(tdequant_rows_kernel<int16_t>, rgrid, block, 0, s, dst, reinterpret_cast<const int16_t*>(src), scale, offset, cols);
+                break;
+            case PTOAMD_I32:
+                hipLaunchKernelGGL(tdequant_rows_kernel<int32_t>, rgrid, block, 0, s, dst, reinterpret_cast<const int32_t*>(src), scale, offset, cols);
+                break;
+            default: set_error("ptoamd_tdequant: source type %d is not int8, int16 or int32", src_type); return PTOAMD_E_UNSUPPORTED;
+        }
+        PTOAMD_HIP_CHECK(hipGetLastError());
+        return PTOAMD_OK;
+    }
     switch (src_type) {
         case PTOAMD_I8:
             hipLaunchKernelGGL(tdequant_kernel<int8_t>, grid, block, 0, s, dst, reinterpret_cast<const int8_t*>(src), scale, offset, rows, cols);
