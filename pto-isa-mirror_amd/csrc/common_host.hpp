@@ -15,6 +15,30 @@ hipError_t ensure_dynamic_lds(const void* kernel, int bytes);
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// One record per C-ABI launch, written as a JSON line to $PTOAMD_TRACE_DIR/ptoamd_trace_<pid>.jsonl when that variable
+// names a directory (no-op otherwise).  Field names follow the reference simulator's InstructionTraceRecord
+// (include/pto/cpu/trace.hpp:67-87: sequence_id, opcode, input_tiles / output_tiles with address, shape, layout, dtype),
+// plus what identifies the launch here: the pipeline (cube / vector), m / n / k and the kernel that ran.  An entry point
+// declares a scope on entry; the record is written when the scope ends, if a kernel was launched inside it.
+class TraceScope {
+public:
+    TraceScope(const char* opcode, const char* pipeline, long m, long n, long k);
+    ~TraceScope();
+    TraceScope& in(const void* address, long rows, long cols, const char* layout, int dtype);
+    TraceScope& out(const void* address, long rows, long cols, const char* layout, int dtype);
+    TraceScope(const TraceScope&) = delete;
+    TraceScope& operator=(const TraceScope&) = delete;
+
+private:
+    struct Tile { const void* address; long rows, cols; const char* layout; int dtype; };
+    bool on_;
+    const char *opcode_, *pipeline_;
+    long m_, n_, k_;
+    unsigned long launches_before_;
+    Tile in_[6], out_[4];
+    int nin_ = 0, nout_ = 0;
+};
+
 #define PTOAMD_HIP_CHECK(expr)                                                                   \
     do {                                                                                         \
         hipError_t e_ = (expr);                                                                  \

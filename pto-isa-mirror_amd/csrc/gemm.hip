@@ -391,6 +391,10 @@ extern "C" {
 int ptoamd_mx_scale_relayout(uint8_t* dst, int dst_layout, const uint8_t* src, int src_layout, int rows, int cols,
                              void* stream)
 {
+    static const char* const names[] = {"MX_A_ZZ", "MX_A_ND", "MX_A_DN", "MX_B_NN", "MX_B_ND", "MX_B_DN"};
+    TraceScope trace("TMOV", "vector", rows, cols, 0);
+    trace.in(src, rows, cols, src_layout >= 0 && src_layout <= 5 ? names[src_layout] : "?", 100)
+        .out(dst, rows, cols, dst_layout >= 0 && dst_layout <= 5 ? names[dst_layout] : "?", 100);
     PTOAMD_REQUIRE(dst && src && rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_mx_scale_relayout: bad argument");
     PTOAMD_REQUIRE(dst_layout >= 0 && dst_layout <= 5 && src_layout >= 0 && src_layout <= 5, PTOAMD_E_INVALID,
                    "ptoamd_mx_scale_relayout: unknown layout");
@@ -408,6 +412,7 @@ int ptoamd_mx_scale_relayout(uint8_t* dst, int dst_layout, const uint8_t* src, i
     hipLaunchKernelGGL(mx_scale_relayout_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream),
                        dst, dst_layout, src, src_layout, rows, cols);
     PTOAMD_HIP_CHECK(hipGetLastError());
+    set_last_kernel("mx_scale_relayout");
     return PTOAMD_OK;
 }
 
@@ -445,6 +450,10 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
                        int relu, void* stream_)
 {
     hipStream_t stream = as_stream(stream_);
+    TraceScope trace(qwords ? "TMATMUL+TSTORE_FP" : (bias ? "TMATMUL_BIAS" : (c_in ? "TMATMUL_ACC" : "TMATMUL")), "cube", m, n, k);
+    trace.in(a, m, k, "ND", ab_type).in(b, k, n, b_layout == PTOAMD_B_DN ? "DN" : "ND", ab_type)
+        .in(c_in, m, n, "ND", ab_type == PTOAMD_I8 ? PTOAMD_I32 : PTOAMD_F32).in(bias, 1, n, "ND", ab_type == PTOAMD_I8 ? PTOAMD_I32 : PTOAMD_F32)
+        .in(qwords, 1, q_per_column ? n : 1, "ND", 101).out(c, m, n, "ND", c_type);
     PTOAMD_REQUIRE(c && a && b, PTOAMD_E_INVALID, "ptoamd_gemm: null operand");
     PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemm: m, n, k must be positive (%d, %d, %d)", m, n, k);
     PTOAMD_REQUIRE(b_layout == PTOAMD_B_ND || b_layout == PTOAMD_B_DN, PTOAMD_E_INVALID, "ptoamd_gemm: unknown b_layout");
@@ -521,6 +530,9 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
                      const float* scale_b, int m, int n, int k, int lda, int ldb, int ldc, int b_layout, void* stream_)
 {
     hipStream_t stream = as_stream(stream_);
+    TraceScope trace("TMATMUL+TDEQUANT", "cube", m, n, k);
+    trace.in(a, m, k, "ND", PTOAMD_I8).in(b, k, n, b_layout == PTOAMD_B_DN ? "DN" : "ND", PTOAMD_I8).in(scale_a, m, 1, "ND", PTOAMD_F32)
+        .in(scale_b, 1, n, "ND", PTOAMD_F32).out(out_bf16, m, n, "ND", PTOAMD_BF16).out(acc_out, m, n, "ND", PTOAMD_I32);
     PTOAMD_REQUIRE(out_bf16 && a && b && scale_a && scale_b, PTOAMD_E_INVALID, "ptoamd_gemm_w8a8: null operand");
     PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemm_w8a8: m, n, k must be positive");
     PTOAMD_REQUIRE(b_layout == PTOAMD_B_ND || b_layout == PTOAMD_B_DN, PTOAMD_E_INVALID, "ptoamd_gemm_w8a8: unknown b_layout");
@@ -572,6 +584,12 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
                           const float* bias = nullptr)
 {
     hipStream_t stream = as_stream(stream_);
+    static const char* const mx_layouts[] = {"MX_A_ZZ", "MX_A_ND", "MX_A_DN", "MX_B_NN", "MX_B_ND", "MX_B_DN"};
+    TraceScope trace(bias ? "TMATMUL_MX_BIAS" : (c_in ? "TMATMUL_MX_ACC" : "TMATMUL_MX"), "cube", m, n, k);
+    trace.in(a, m, k, "ND", a_type).in(b, k, n, b_layout == PTOAMD_B_DN ? "DN" : "ND", b_type)
+        .in(sa, m, k / 32, sa_layout >= 0 && sa_layout < 6 ? mx_layouts[sa_layout] : "?", 100)
+        .in(sb, k / 32, n, sb_layout >= 0 && sb_layout < 6 ? mx_layouts[sb_layout] : "?", 100).in(c_in, m, n, "ND", PTOAMD_F32)
+        .in(bias, 1, n, "ND", PTOAMD_F32).out(c, m, n, "ND", c_type);
     PTOAMD_REQUIRE(c && a && b && sa && sb, PTOAMD_E_INVALID, "%s: null operand", who);
     PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "%s: m, n, k must be positive", who);
     PTOAMD_REQUIRE(k % 64 == 0, PTOAMD_E_INVALID, "%s: k = %d must be a multiple of 64", who, k);

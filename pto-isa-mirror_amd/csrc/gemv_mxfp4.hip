@@ -607,6 +607,8 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
                                  int n, int k, int lda, int ldw, int ldc, void* stream_)
 {
     hipStream_t stream = as_stream(stream_);
+    TraceScope trace("TGEMV_MX", "cube", m, n, k);
+    trace.in(a_bf16, m, k, "ND", PTOAMD_BF16).in(w, k, n, "DN", PTOAMD_E2M1).in(sw, k / 32, n, "MX_B_DN", 100).out(out, m, n, "ND", c_type);
     PTOAMD_REQUIRE(out && a_bf16 && w && sw, PTOAMD_E_INVALID, "ptoamd_gemv_mxfp4: null operand");
     PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemv_mxfp4: m, n, k must be positive");
     PTOAMD_REQUIRE(m <= 16, PTOAMD_E_UNSUPPORTED, "ptoamd_gemv_mxfp4: m = %d exceeds the decode batch of 16 (use ptoamd_gemm_mx)", m);

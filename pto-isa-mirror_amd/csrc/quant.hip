@@ -255,6 +255,7 @@ static int launch_tquant_mx(uint8_t* dst, uint8_t* exp, float* mx, float* scalin
                            rows, cols);
     }
     PTOAMD_HIP_CHECK(hipGetLastError());
+    set_last_kernel(axis == 1 ? "tquant_mx_rows" : "tquant_mx_cols");
     return PTOAMD_OK;
 }
 
@@ -278,6 +279,9 @@ extern "C" {
 int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const float* offset, int rows, int cols,
                        void* stream)
 {
+    TraceScope trace(offset ? "TQUANT_INT8_ASYM" : "TQUANT_INT8_SYM", "vector", rows, cols, 0);
+    trace.in(src, rows, cols, "ND", PTOAMD_F32).in(scale, rows, 1, "ND", PTOAMD_F32).in(offset, rows, 1, "ND", PTOAMD_F32)
+        .out(dst, rows, cols, "ND", offset ? PTOAMD_U8 : PTOAMD_I8);
     PTOAMD_REQUIRE(dst && src && scale, PTOAMD_E_INVALID, "ptoamd_tquant_int8: null operand");
     PTOAMD_REQUIRE(rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_tquant_int8: rows and cols must be positive");
     const long total = (long)rows * cols;
@@ -290,6 +294,7 @@ int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const fl
             hipLaunchKernelGGL(tquant_int8_rows_kernel<false>, grid, dim3(256), 0, as_stream(stream),
                                reinterpret_cast<uint8_t*>(dst), src, scale, offset, cols);
         PTOAMD_HIP_CHECK(hipGetLastError());
+        set_last_kernel("tquant_int8_rows");
         return PTOAMD_OK;
     }
     const unsigned blocks = (unsigned)((total / 4 + 256) / 256);
@@ -300,12 +305,19 @@ int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const fl
         hipLaunchKernelGGL(tquant_int8_kernel<false>, dim3(blocks), dim3(256), 0, as_stream(stream),
                            reinterpret_cast<uint8_t*>(dst), src, scale, offset, rows, cols);
     PTOAMD_HIP_CHECK(hipGetLastError());
+    set_last_kernel("tquant_int8");
     return PTOAMD_OK;
 }
 
 int ptoamd_tquant_mx(uint8_t* dst, uint8_t* exp, float* max, float* scaling, const void* src, int src_type, int rows,
                      int cols, int alg, int axis, void* stream)
 {
+    const bool fp4 = alg == PTOAMD_OCP_MXFP4 || alg == PTOAMD_NV_MXFP4;
+    TraceScope trace(fp4 ? "TQUANT_MXFP4" : "TQUANT_MXFP8", "vector", rows, cols, 0);
+    trace.in(src, rows, cols, "ND", src_type).out(dst, rows, cols, "ND", fp4 ? PTOAMD_E2M1 : PTOAMD_E4M3)
+        .out(exp, axis == 1 ? rows : rows / 32, axis == 1 ? cols / 32 : cols, "ND", 100)
+        .out(max, axis == 1 ? rows : rows / 32, axis == 1 ? cols / 32 : cols, "ND", PTOAMD_F32)
+        .out(scaling, axis == 1 ? rows : rows / 32, axis == 1 ? cols / 32 : cols, "ND", PTOAMD_F32);
     PTOAMD_REQUIRE(dst && exp && src, PTOAMD_E_INVALID, "ptoamd_tquant_mx: null operand");
     PTOAMD_REQUIRE(rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_tquant_mx: rows and cols must be positive");
     PTOAMD_REQUIRE(axis == 0 || axis == 1, PTOAMD_E_INVALID, "ptoamd_tquant_mx: axis must be 0 or 1");
@@ -329,6 +341,9 @@ int ptoamd_tquant_mx(uint8_t* dst, uint8_t* exp, float* max, float* scaling, con
 int ptoamd_tdequant(float* dst, const void* src, int src_type, const float* scale, const float* offset, int rows,
                     int cols, void* stream)
 {
+    TraceScope trace("TDEQUANT", "vector", rows, cols, 0);
+    trace.in(src, rows, cols, "ND", src_type).in(scale, rows, 1, "ND", PTOAMD_F32).in(offset, rows, 1, "ND", PTOAMD_F32)
+        .out(dst, rows, cols, "ND", PTOAMD_F32);
     PTOAMD_REQUIRE(dst && src && scale && offset, PTOAMD_E_INVALID, "ptoamd_tdequant: null operand");
     PTOAMD_REQUIRE(rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_tdequant: rows and cols must be positive");
     const long total = (long)rows * cols;
@@ -349,6 +364,7 @@ int ptoamd_tdequant(float* dst, const void* src, int src_type, const float* scal
             default: set_error("ptoamd_tdequant: source type %d is not int8, int16 or int32", src_type); return PTOAMD_E_UNSUPPORTED;
         }
         PTOAMD_HIP_CHECK(hipGetLastError());
+        set_last_kernel("tdequant_rows");
         return PTOAMD_OK;
     }
     switch (src_type) {
@@ -364,6 +380,7 @@ int ptoamd_tdequant(float* dst, const void* src, int src_type, const float* scal
         default: set_error("ptoamd_tdequant: source type %d is not int8, int16 or int32", src_type); return PTOAMD_E_UNSUPPORTED;
     }
     PTOAMD_HIP_CHECK(hipGetLastError());
+    set_last_kernel("tdequant");
     return PTOAMD_OK;
 }
 

@@ -1,6 +1,9 @@
 // Host runtime of the gfx950 backend: the counterpart of the fake aclrt* runtime the reference's tests and demos use
 // (include/pto/common/cpu_stub.hpp:73-120, 524-555), on the HIP runtime.
+#include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
+#include <unistd.h>
 
 #include <mutex>
 #include <set>
@@ -19,10 +22,84 @@ void set_error(const char* fmt, ...)
     vsnprintf(g_error, sizeof g_error, fmt, ap);
     va_end(ap);
 }
+static thread_local unsigned long g_launches = 0;
 void set_last_kernel(const char* name)
 {
     strncpy(g_kernel, name, sizeof g_kernel - 1);
     g_kernel[sizeof g_kernel - 1] = 0;
+    ++g_launches;
+}
+
+// ---- launch trace -----------------------------------------------------------------------------------------------------
+namespace {
+struct TraceSink {
+    std::mutex mu;
+    FILE* file = nullptr;
+    unsigned long sequence = 0;
+    bool enabled = false;
+    TraceSink()
+    {
+        const char* dir = getenv("PTOAMD_TRACE_DIR");
+        if (dir == nullptr || *dir == 0)
+            return;
+        char path[1024];
+        snprintf(path, sizeof path, "%s/ptoamd_trace_%ld.jsonl", dir, (long)getpid());
+        file = fopen(path, "a");
+        enabled = file != nullptr;
+    }
+    ~TraceSink()
+    {
+        if (file)
+            fclose(file);
+    }
+};
+TraceSink& trace_sink()
+{
+    static TraceSink sink;
+    return sink;
+}
+const char* dtype_name(int t)
+{
+    static const char* names[] = {"f32", "f16", "bf16", "i32", "i8", "u8", "e4m3", "e5m2", "e2m1x2", "e1m2x2", "i16"};
+    return t >= 0 && t < 11 ? names[t] : (t == 100 ? "e8m0" : (t == 101 ? "u64" : "?"));
+}
+}  // namespace
+
+TraceScope::TraceScope(const char* opcode, const char* pipeline, long m, long n, long k)
+    : on_(trace_sink().enabled), opcode_(opcode), pipeline_(pipeline), m_(m), n_(n), k_(k), launches_before_(g_launches)
+{
+}
+TraceScope& TraceScope::in(const void* address, long rows, long cols, const char* layout, int dtype)
+{
+    if (on_ && address != nullptr && nin_ < 6)
+        in_[nin_++] = Tile{address, rows, cols, layout, dtype};
+    return *this;
+}
+TraceScope& TraceScope::out(const void* address, long rows, long cols, const char* layout, int dtype)
+{
+    if (on_ && address != nullptr && nout_ < 4)
+        out_[nout_++] = Tile{address, rows, cols, layout, dtype};
+    return *this;
+}
+TraceScope::~TraceScope()
+{
+    if (!on_ || g_launches == launches_before_)
+        return;  // tracing off, or the call was rejected before anything ran
+    TraceSink& sink = trace_sink();
+    std::lock_guard<std::mutex> lock(sink.mu);
+    fprintf(sink.file, "{\"sequence_id\": %lu, \"opcode\": \"%s\", \"pipeline\": \"%s\", \"kernel\": \"%s\", \"m\": %ld, \"n\": %ld, \"k\": %ld",
+            sink.sequence++, opcode_, pipeline_, g_kernel, m_, n_, k_);
+    for (int side = 0; side < 2; ++side) {
+        const Tile* t = side == 0 ? in_ : out_;
+        const int cnt = side == 0 ? nin_ : nout_;
+        fprintf(sink.file, ", \"%s\": [", side == 0 ? "input_tiles" : "output_tiles");
+        for (int i = 0; i < cnt; ++i)
+            fprintf(sink.file, "%s{\"address\": %llu, \"shape\": [%ld, %ld], \"layout\": \"%s\", \"dtype\": \"%s\"}", i ? ", " : "",
+                    (unsigned long long)(uintptr_t)t[i].address, t[i].rows, t[i].cols, t[i].layout, dtype_name(t[i].dtype));
+        fprintf(sink.file, "]");
+    }
+    fprintf(sink.file, "}\n");
+    fflush(sink.file);
 }
 
 // hipFuncAttributeMaxDynamicSharedMemorySize is a property of (kernel, device): it is set once per pair, under a lock,

@@ -374,3 +374,44 @@ def test_tstore_fix_pipe_quantisation(kernels, oracle, case):
     got = out.cpu().numpy().view(out_dt).reshape(m, n)
     assert np.array_equal(got, ref.view(out_dt))
     assert len(np.unique(got)) > 8  # the case exercises the quantiser, not a saturated constant
+
+
+# ------------------------------------------------------------------------------- framework-free runner + launch trace
+RUNNER = os.path.join(HERE, "pto_kernels", "build", "case_runner")
+
+
+def test_case_runner_and_launch_trace(tmp_path):
+    """The C++ test main (aclrt* calls, Launch, host golden, ResultCmp) passes its cases, exits non-zero otherwise, and
+    with PTOAMD_TRACE_DIR set every C-ABI launch leaves one JSON record."""
+    import json
+
+    if not os.path.exists(RUNNER):
+        raise RuntimeError(f"{RUNNER} is missing: run __graft_entry__.build()")
+    env = dict(os.environ, PTOAMD_TRACE_DIR=str(tmp_path))
+    for case in ("tmatmul", "tmatmul_i8", "tmatmul_mx", "gemm", "gemm_mx", "quant_gemm"):
+        res = subprocess.run([RUNNER, case], capture_output=True, text=True, timeout=120, env=env)
+        assert res.returncode == 0, case + "\n" + res.stdout + res.stderr
+        assert f"{case}: PASS" in res.stdout and "err count: 0," in res.stdout, res.stdout
+    assert subprocess.run([RUNNER, "no_such_case"], capture_output=True, timeout=60, env=env).returncode == 2
+    records = []
+    for name in sorted(os.listdir(tmp_path)):
+        assert name.startswith("ptoamd_trace_") and name.endswith(".jsonl")
+        with open(tmp_path / name) as f:
+            records.append([json.loads(line) for line in f])
+    by_len = sorted(records, key=len)
+    # the three C-ABI cases: one, one and three launches (PTO-kernel cases launch no C-ABI kernel and write no file)
+    assert [len(r) for r in by_len] == [1, 1, 3]
+    ops = sorted(r[0]["opcode"] for r in by_len[:2])
+    assert ops == ["TMATMUL", "TMATMUL_MX"]
+    for recs in by_len:
+        for i, rec in enumerate(recs):
+            assert rec["sequence_id"] == i and rec["kernel"] and rec["pipeline"] in ("cube", "vector")
+            assert all({"address", "shape", "layout", "dtype"} <= set(t) for t in rec["input_tiles"] + rec["output_tiles"])
+    gemm = next(r[0] for r in by_len[:2] if r[0]["opcode"] == "TMATMUL")
+    assert (gemm["m"], gemm["n"], gemm["k"]) == (256, 384, 512) and gemm["kernel"].startswith("tile")
+    assert [t["dtype"] for t in gemm["input_tiles"]] == ["bf16", "bf16"] and gemm["input_tiles"][1]["layout"] == "DN"
+    assert gemm["output_tiles"][0]["dtype"] == "f32" and gemm["output_tiles"][0]["shape"] == [256, 384]
+    quant = by_len[2]
+    assert [r["opcode"] for r in quant] == ["TQUANT_MXFP8", "TQUANT_MXFP8", "TMATMUL_MX"]
+    assert quant[0]["pipeline"] == "vector" and quant[0]["kernel"] == "tquant_mx_rows"
+    assert [t["layout"] for t in quant[2]["input_tiles"][2:4]] == ["MX_A_ND", "MX_B_DN"]
