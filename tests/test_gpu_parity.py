@@ -54,6 +54,21 @@ def relerr(got, ref):
     return float(np.abs(got.astype(np.float64) - ref.astype(np.float64)).max() / max(np.abs(ref).max(), 1e-30))
 
 
+def check_f32_drain(got, ref, absdot, k, label, max_rel=1e-4, eps=None):
+    """The two bars of an fp32 drain against the oracle's sequential fp32 sum, with the achieved errors printed:
+    max|got - ref| <= max_rel * max|ref|, and element by element |got - ref| <= 1e-2 |ref| + eps * sum|a||b| with
+    eps = 8 k 2^-24 (what k fp32 roundings of partial sums bounded by sum|a||b| can add up to, eight-fold)."""
+    got, ref = got.astype(np.float64), ref.astype(np.float64)
+    err = np.abs(got - ref)
+    eps = 8 * k * 2.0 ** -24 if eps is None else eps
+    bound = 1e-2 * np.abs(ref) + eps * absdot
+    print(f"{label}: {err.size} outputs, max|got-ref| = {err.max():.3e}, max|ref| = {np.abs(ref).max():.3e} "
+          f"(ratio {err.max() / np.abs(ref).max():.2e}, bar {max_rel:.0e}), worst error / element bound = {(err / bound).max():.3e}, "
+          f"max error / sum|a||b| = {(err / np.maximum(absdot, 1e-300)).max():.2e}")
+    assert err.max() <= max_rel * np.abs(ref).max()
+    assert (err <= bound).all()
+
+
 class tile_env:
     def __init__(self, **kw):
         self.kw = kw
@@ -161,7 +176,8 @@ def test_bf16_gemm_every_tile_shape(pa, oracle, tile, m, n, k):
         got32 = host(pa.gemm(dev(a).view(torch.bfloat16), dev(b).view(torch.bfloat16), pa.BF16, pa.F32, pa.B_DN))
         expect_tile(pa, tile, 2 * k)
         got16 = host(pa.gemm(dev(a).view(torch.bfloat16), dev(b).view(torch.bfloat16), pa.BF16, pa.BF16, pa.B_DN))
-    assert relerr(got32, ref) <= 1e-2
+    absdot = np.abs(bf16_to_f32(a).astype(np.float64)) @ np.abs(bf16_to_f32(b).astype(np.float64)).T
+    check_f32_drain(got32, ref, absdot, k, f"bf16 {m}x{n}x{k} tile {tile}")
     # TSTORE f32 -> bf16 is round-to-nearest-even of the same accumulator
     assert np.array_equal(got16, oracle.store_f32(got32, ob.ST_BF16))
 
@@ -222,32 +238,37 @@ def test_gemm_golden_fixtures(pa, golden):
 
 
 def test_config2_bf16_4096_cubed(pa, oracle):
-    """configs[1]: bf16 4096^3, A row-major, B column-major, N(0,1)*0.02, fp32 accumulate, bf16 output."""
+    """configs[1]: bf16 4096^3, A row-major, B column-major, N(0,1)*0.02, fp32 accumulate, bf16 output.  4096 sampled
+    outputs and two whole 256 x 256 output tiles against the oracle, on the fp32 drain (both error bars) and on the bf16
+    drain (which must be the rounding of the fp32 drain, bit for bit, everywhere)."""
     m = n = k = 4096
     gen = torch.Generator(device=DEV).manual_seed(2)
     a = (torch.randn((m, k), generator=gen, device=DEV) * 0.02).to(torch.bfloat16)
     b = (torch.randn((n, k), generator=gen, device=DEV) * 0.02).to(torch.bfloat16)
     out = pa.gemm(a, b, pa.BF16, pa.BF16, pa.B_DN)
     assert pa.last_kernel() == "tile256x256w8_dtl_bf16"
-    rows = np.array([0, 1, 255, 256, 1000, 2047, 2048, 3333, 4095])
-    cols = np.arange(0, 4096, 37)
-    ref = oracle.matmul_bf16(host(sel(a, rows)), host(sel(b, cols)), b_dn=True)
-    got = bf16_to_f32(host(out)[np.ix_(rows, cols)])
-    assert relerr(got, ref) <= 1e-2
-    # two whole output tiles, one at each end of the grid
-    for r0, c0 in ((0, 0), (3840, 3840)):
-        ref = oracle.matmul_bf16(host(a[r0:r0 + 64]), host(b[c0:c0 + 256]), b_dn=True)
-        assert relerr(bf16_to_f32(host(out)[r0:r0 + 64, c0:c0 + 256]), ref) <= 1e-2
-    # size-independent properties on the fp32 drain: exact power-of-two scaling and K-split additivity
     f = pa.gemm(a, b, pa.BF16, pa.F32, pa.B_DN)
+    assert pa.last_kernel() == "tile256x256w8_dtl_bf16"
+    out_h, f_h = host(out), host(f)
+    assert np.array_equal(out_h, oracle.store_f32(f_h, ob.ST_BF16))
+    rows = np.unique(np.concatenate([[0, 1, 255, 256, 2047, 2048, 4095], np.arange(5, 4096, 72)]))[:64]
+    cols = np.arange(0, 4096, 64) + np.arange(64) % 64
+    blocks = [("samples", rows, cols), ("tile (0, 0)", np.arange(256), np.arange(256)),
+              ("tile (15, 15)", np.arange(3840, 4096), np.arange(3840, 4096))]
+    for label, rr, cc in blocks:
+        ar, bc = host(sel(a, rr)), host(sel(b, cc))
+        ref = oracle.matmul_bf16(ar, bc, b_dn=True)
+        absdot = np.abs(bf16_to_f32(ar).astype(np.float64)) @ np.abs(bf16_to_f32(bc).astype(np.float64)).T
+        check_f32_drain(f_h[np.ix_(rr, cc)], ref, absdot, k, f"configs[1] bf16 4096^3, {label}")
+        assert relerr(bf16_to_f32(out_h[np.ix_(rr, cc)]), ref) <= 1e-2
+    # size-independent properties on the fp32 drain: exact power-of-two scaling and K-split additivity
     f2 = pa.gemm((a.float() * 4).to(torch.bfloat16), b, pa.BF16, pa.F32, pa.B_DN)
     assert torch.equal(f2, f * 4)
     lo = pa.gemm(a[:, :2048].contiguous(), b[:, :2048].contiguous(), pa.BF16, pa.F32, pa.B_DN)
     hi = pa.gemm(a[:, 2048:].contiguous(), b[:, 2048:].contiguous(), pa.BF16, pa.F32, pa.B_DN, c_in=lo)
-    assert relerr(host(hi), host(f)) <= 1e-5  # TMATMUL then TMATMUL_ACC over the two K halves
+    assert relerr(host(hi), f_h) <= 1e-5  # TMATMUL then TMATMUL_ACC over the two K halves
 
 
-# ------------------------------------------------------------------------------------------- int8 / W8A8
 @pytest.mark.parametrize("tile", ALL_TILES)
 def test_int8_accumulators_bit_exact(pa, oracle, tile):
     r = np.random.default_rng(tile)
@@ -318,12 +339,17 @@ def test_config3_w8a8_full_size(pa, oracle):
     sb = torch.rand(n, generator=gen, device=DEV) * 0.01 + 0.001
     out, acc = pa.gemm_w8a8(a, b, sa, sb, want_acc=True)
     assert pa.last_kernel() == "tile256x256w8_dtl_i8"
-    rows = np.array([0, 255, 256, 1023, 2047])
-    cols = np.arange(0, n, 257)
-    ra, rb = host(sel(a, rows)), host(sel(b, cols))
-    ref_acc, ref_out = _w8a8_reference(oracle, ra, rb, host(sa)[rows], host(sb)[cols])
-    assert np.array_equal(host(acc)[np.ix_(rows, cols)], ref_acc)
-    assert np.array_equal(host(out)[np.ix_(rows, cols)], ref_out)
+    acc_h, out_h, sa_h, sb_h = host(acc), host(out), host(sa), host(sb)
+    rows = np.unique(np.concatenate([[0, 255, 256, 1023, 2047], np.arange(3, m, 33)]))[:64]
+    cols = np.arange(0, n, 128) + np.arange(64) % 128
+    # 4096 sampled outputs and two whole 256 x 256 output tiles: raw accumulators and dequantised bf16, bit for bit
+    for label, rr, cc in (("samples", rows, cols), ("tile (0, 0)", np.arange(256), np.arange(256)),
+                          ("tile (7, 31)", np.arange(m - 256, m), np.arange(n - 256, n))):
+        ref_acc, ref_out = _w8a8_reference(oracle, host(sel(a, rr)), host(sel(b, cc)), sa_h[rr], sb_h[cc])
+        bad_acc = int((acc_h[np.ix_(rr, cc)] != ref_acc).sum())
+        bad_out = int((out_h[np.ix_(rr, cc)] != ref_out).sum())
+        print(f"configs[2] W8A8 2048x8192x8192, {label}: {ref_acc.size} outputs, {bad_acc} accumulators and {bad_out} bf16 values differ")
+        assert bad_acc == 0 and bad_out == 0
     # checksum identity over the whole result: sum_j C[i, j] = A[i, :] . (sum_j B[j, :]) in exact integers
     colsum = b.to(torch.int64).sum(0)
     want = (a[:64].to(torch.int64) * colsum[None, :]).sum(1)
@@ -514,6 +540,16 @@ def _mx_inputs(r, typ, m, n, k, spread=8):
 PA_T = {ob.E4M3: 6, ob.E5M2: 7, ob.E2M1: 8, ob.E1M2: 9}
 
 
+def _mx_unpack(oracle, codes, typ):
+    """Decoded float64 values of a code matrix (fp4: two codes per byte, even element in the low nibble)."""
+    table = oracle.mx_decode_table(typ)
+    if typ in (ob.E2M1, ob.E1M2):
+        out = np.empty((codes.shape[0], codes.shape[1] * 2), np.float64)
+        out[:, 0::2], out[:, 1::2] = table[codes & 0xF], table[codes >> 4]
+        return out
+    return table[codes]
+
+
 @pytest.mark.parametrize("ta,tb", [(ob.E4M3, ob.E4M3), (ob.E5M2, ob.E5M2), (ob.E4M3, ob.E5M2), (ob.E5M2, ob.E4M3),
                                    (ob.E2M1, ob.E2M1)])
 @pytest.mark.parametrize("tile", ALL_TILES)
@@ -526,7 +562,14 @@ def test_mx_gemm(pa, oracle, ta, tb, tile):
         with tile_env(PTOAMD_TILE=tile):
             got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[ta], PA_T[tb], pa.F32))
             assert pa.last_kernel().startswith("tile"), pa.last_kernel()
-        assert relerr(got, ref) <= 2e-2
+        # codes from the whole range (a 2^17 spread inside one 64-product instruction): FP4 products add up like fp32
+        # sums; the FP8 form aligns the products of one instruction to their largest exponent and keeps about 13 bits
+        # below it (measured up to 2.4e-4 sum|a||b| and 1e-4 max|ref|), hence 2^-11 sum|a||b| and 1e-3 max|ref| there
+        fp4 = ta in (ob.E2M1, ob.E1M2)
+        ua = _mx_unpack(oracle, a, ta) * np.repeat(2.0 ** (sa.astype(np.float64) - 127), 32, 1)
+        ub = _mx_unpack(oracle, b, tb) * np.repeat(2.0 ** (sb.astype(np.float64) - 127), 32, 1)
+        check_f32_drain(got, ref, np.abs(ua) @ np.abs(ub).T, k, f"MX {ta}x{tb} {m}x{n}x{k} tile {tile}",
+                        max_rel=1e-4 if fp4 else 1e-3, eps=None if fp4 else 2.0 ** -11)
         with tile_env(PTOAMD_FORCE_GENERIC=1):
             exact = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[ta], PA_T[tb], pa.F32))
         assert np.array_equal(exact.view(np.uint32), ref.view(np.uint32))  # double-add-then-round order, bit for bit
@@ -687,18 +730,32 @@ def test_config4_mxfp8_full_size(pa, oracle):
     b, sb = pa.tquant_mx(xb, pa.OCP_MXFP8, want_aux=False)
     out = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E4M3, pa.E4M3, pa.BF16)
     assert pa.last_kernel() == "tile256x256w8_dtl_fp8_e4m3_e4m3"
-    rows = np.array([0, 255, 256, 2049, 4095])
-    cols = np.arange(0, n, 449)
+    f = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E4M3, pa.E4M3, pa.F32)
+    out_h, f_h = host(out), host(f)
+    assert np.array_equal(out_h, oracle.store_f32(f_h, ob.ST_BF16))  # the bf16 drain is the rounding of the fp32 drain
+    table = oracle.mx_decode_table(ob.E4M3)
+    rows = np.unique(np.concatenate([[0, 255, 256, 2049, 4095], np.arange(7, m, 66)]))[:64]
+    cols = np.arange(0, n, 224) + np.arange(64) % 224
+    for label, rr, cc in (("samples", rows, cols), ("tile (0, 0)", np.arange(256), np.arange(256)),
+                          ("tile (15, 55)", np.arange(m - 256, m), np.arange(n - 256, n))):
+        ar, bc, sar, sbc = host(sel(a, rr)), host(sel(b, cc)), host(sel(sa, rr)), host(sel(sb, cc))
+        ref = oracle.matmul_mx(ar, bc, sar, sbc, len(rr), k, len(cc), ob.E4M3, ob.E4M3)
+        wa = np.abs(table[ar]) * np.repeat(2.0 ** (sar.astype(np.float64) - 127), 32, 1)
+        wb = np.abs(table[bc]) * np.repeat(2.0 ** (sbc.astype(np.float64) - 127), 32, 1)
+        # (The FP8 form of the scaled MFMA aligns the 64 products of one instruction to their largest exponent and keeps a
+        # limited number of bits below it; on operands of one magnitude, as here, that costs nothing measurable -- 2e-6
+        # sum|a||b| -- and the plain fp32 bars hold.  test_mx_gemm draws from the whole code range, where it shows.)
+        check_f32_drain(f_h[np.ix_(rr, cc)], ref, wa @ wb.T, k, f"configs[3] MXFP8 4096x14336x4096, {label}")
+        assert relerr(bf16_to_f32(out_h[np.ix_(rr, cc)]), ref) <= 2e-2
+    # the quantised operands are close to the source: the GEMM of the dequantised data approximates xa . xb^T
     ref = oracle.matmul_mx(host(sel(a, rows)), host(sel(b, cols)), host(sel(sa, rows)), host(sel(sb, cols)), len(rows), k, len(cols),
                            ob.E4M3, ob.E4M3)
-    assert relerr(bf16_to_f32(host(out)[np.ix_(rows, cols)]), ref) <= 2e-2
-    # the quantised operands are close to the source: the GEMM of the dequantised data approximates xa . xb^T
     approx = (xa[rows.tolist()] @ xb[cols.tolist()].T).cpu().numpy()
     assert relerr(ref, approx) <= 0.1
     # raising every A scale by one doubles the fp32 result exactly
-    f = pa.gemm_mx(a[:512], b[:512], sa[:512], sb[:512], 512, 512, k, pa.E4M3, pa.E4M3, pa.F32)
-    f2 = pa.gemm_mx(a[:512], b[:512], sa[:512] + 1, sb[:512], 512, 512, k, pa.E4M3, pa.E4M3, pa.F32)
-    assert torch.equal(f2, f * 2)
+    g1 = pa.gemm_mx(a[:512], b[:512], sa[:512], sb[:512], 512, 512, k, pa.E4M3, pa.E4M3, pa.F32)
+    g2 = pa.gemm_mx(a[:512], b[:512], sa[:512] + 1, sb[:512], 512, 512, k, pa.E4M3, pa.E4M3, pa.F32)
+    assert torch.equal(g2, g1 * 2)
 
 
 def test_mxfp4_gemm_large_takes_the_256_tile(pa, oracle):
