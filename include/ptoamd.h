@@ -146,6 +146,16 @@ int ptoamd_gemm_requant(void* c, int c_type, const void* a, const void* b, int a
                         int b_layout, int relu, void* stream);
 
 /*
+ * The same pipeline drained with TSTORE<AtomicAdd>: C(i, j) += (A * B)(i, j), one atomic add per element, so that
+ * several launches (K split over calls or streams) may accumulate into one C.  c_type: PTOAMD_F32 (float inputs) or
+ * PTOAMD_I32 (int8 inputs).  The order of the additions between concurrent launches is not defined; float sums may
+ * therefore differ in the last bits from run to run, integer sums do not.
+ * reference: include/pto/cpu/TStore.hpp:64-78 (AtomicType::AtomicAdd), common/pto_instr.hpp (TSTORE<..., AtomicAdd>).
+ */
+int ptoamd_gemm_atomic_add(void* c, int c_type, const void* a, const void* b, int ab_type, int m, int n, int k, int lda, int ldb,
+                           int ldc, int b_layout, void* stream);
+
+/*
  * W8A8: int8 x int8 -> int32 accumulate, then the dequantising drain fused in registers:
  *   out(i, j) = bf16( (float(acc(i, j)) * scale_a[i]) * scale_b[j] )
  * i.e. TMATMUL (cpu/TMatmul.hpp:106) -> TDEQUANT with offset 0 (cpu/TDeQuant.hpp:31-34) -> per-column multiply

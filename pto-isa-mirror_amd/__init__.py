@@ -40,7 +40,7 @@ EXPORTS = [
     "ptoamd_malloc_host", "ptoamd_free_host", "ptoamd_memcpy", "ptoamd_memcpy_async", "ptoamd_memset",
     "ptoamd_stream_create", "ptoamd_stream_destroy", "ptoamd_stream_synchronize", "ptoamd_event_create",
     "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
-    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_requant", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
+    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_requant", "ptoamd_gemm_atomic_add", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
     "ptoamd_gemm_mx_ws",
     "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
     "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_mx_scale_relayout", "ptoamd_last_kernel",
@@ -95,6 +95,16 @@ def gemm(a, b, ab_type, c_type=F32, b_layout=B_DN, c_in=None, relu=False, m=None
         return out
     _check(_lib.ptoamd_gemm(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), m, n, k, a.stride(0), b.stride(0),
                             out.stride(0), b_layout, int(relu), _stream(stream)), "ptoamd_gemm")
+    return out
+
+
+def gemm_atomic_add(out, a, b, ab_type, b_layout=B_DN, stream=None):
+    """out += A . B through TSTORE<AtomicAdd> (out: f32 for float inputs, int32 for int8)."""
+    m, k = a.shape
+    n = out.shape[1]
+    c_type = F32 if out.dtype == torch.float32 else I32
+    _check(_lib.ptoamd_gemm_atomic_add(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, m, n, k, a.stride(0), b.stride(0),
+                                       out.stride(0), b_layout, _stream(stream)), "ptoamd_gemm_atomic_add")
     return out
 
 

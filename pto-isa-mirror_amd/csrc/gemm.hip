@@ -109,6 +109,7 @@ struct GenericParams {
     int sa_layout, sb_layout, mx;
     const uint64_t* qwords;  // OUT_Q8 / OUT_QF16: fix-pipe quantisation words
     int q_per_column;
+    int atomic_add;          // OUT_F32 / OUT_I32: C += result (TSTORE<AtomicAdd>)
 };
 
 __device__ __forceinline__ float load_elem_f32(const void* p, long idx, int type)
@@ -153,7 +154,12 @@ __device__ __forceinline__ void store_out(const GenericParams& p, long o, float 
     if (p.relu)
         v = v > 0 ? v : 0;
     switch (p.out_kind) {
-        case OUT_F32: reinterpret_cast<float*>(p.c)[o] = v; break;
+        case OUT_F32:
+            if (p.atomic_add)
+                atomicAdd(reinterpret_cast<float*>(p.c) + o, v);
+            else
+                reinterpret_cast<float*>(p.c)[o] = v;
+            break;
         case OUT_F16: reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_f16_bits(v); break;
         default: reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(v); break;
     }
@@ -184,7 +190,10 @@ __global__ void gemm_generic_kernel(const GenericParams p)
         if (p.relu)
             v = v > 0 ? v : 0;
         if (p.out_kind == OUT_I32) {
-            reinterpret_cast<int32_t*>(p.c)[o] = v;
+            if (p.atomic_add)
+                atomicAdd(reinterpret_cast<int*>(p.c) + o, v);
+            else
+                reinterpret_cast<int32_t*>(p.c)[o] = v;
         } else {
             if (p.acc_out)
                 p.acc_out[o] = v;
@@ -424,7 +433,7 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
 
 static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                        const uint64_t* qwords, int q_per_column, int m, int n, int k, int lda, int ldb, int ldc, int b_layout,
-                       int relu, void* stream_);
+                       int relu, void* stream_, int atomic_add = 0);
 
 int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                      int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream_)
@@ -445,12 +454,22 @@ int ptoamd_gemm_requant(void* c, int c_type, const void* a, const void* b, int a
                        relu, stream_);
 }
 
+int ptoamd_gemm_atomic_add(void* c, int c_type, const void* a, const void* b, int ab_type, int m, int n, int k, int lda, int ldb,
+                           int ldc, int b_layout, void* stream_)
+{
+    PTOAMD_REQUIRE(c_type == PTOAMD_F32 || c_type == PTOAMD_I32, PTOAMD_E_UNSUPPORTED,
+                   "ptoamd_gemm_atomic_add: atomic adds target f32 or i32 (got type %d)", c_type);
+    return gemm_common(c, c_type, a, b, ab_type, nullptr, nullptr, nullptr, 0, m, n, k, lda, ldb, ldc, b_layout, 0, stream_, 1);
+}
+
 static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                        const uint64_t* qwords, int q_per_column, int m, int n, int k, int lda, int ldb, int ldc, int b_layout,
-                       int relu, void* stream_)
+                       int relu, void* stream_, int atomic_add)
 {
     hipStream_t stream = as_stream(stream_);
-    TraceScope trace(qwords ? "TMATMUL+TSTORE_FP" : (bias ? "TMATMUL_BIAS" : (c_in ? "TMATMUL_ACC" : "TMATMUL")), "cube", m, n, k);
+    TraceScope trace(atomic_add ? "TMATMUL+TSTORE_ATOMIC_ADD"
+                                : (qwords ? "TMATMUL+TSTORE_FP" : (bias ? "TMATMUL_BIAS" : (c_in ? "TMATMUL_ACC" : "TMATMUL"))),
+                     "cube", m, n, k);
     trace.in(a, m, k, "ND", ab_type).in(b, k, n, b_layout == PTOAMD_B_DN ? "DN" : "ND", ab_type)
         .in(c_in, m, n, "ND", ab_type == PTOAMD_I8 ? PTOAMD_I32 : PTOAMD_F32).in(bias, 1, n, "ND", ab_type == PTOAMD_I8 ? PTOAMD_I32 : PTOAMD_F32)
         .in(qwords, 1, q_per_column ? n : 1, "ND", 101).out(c, m, n, "ND", c_type);
@@ -487,7 +506,7 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
         g.sbk = b_layout == PTOAMD_B_DN ? 1 : ldb;
         g.sbn = b_layout == PTOAMD_B_DN ? ldb : 1;
         g.a_type = g.b_type = ab_type; g.out_kind = out_kind; g.relu = relu;
-        g.qwords = qwords; g.q_per_column = q_per_column;
+        g.qwords = qwords; g.q_per_column = q_per_column; g.atomic_add = atomic_add;
         return launch_generic(g, stream);
     }
     StreamTemp bt(stream);
@@ -514,7 +533,7 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
     p.m = m; p.n = n; p.k_bytes = (int)k_bytes;
     p.lda_bytes = lda_b; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
     p.relu = relu; p.out_kind = out_kind; p.group_m = 4;
-    p.qwords = qwords; p.q_per_column = q_per_column;
+    p.qwords = qwords; p.q_per_column = q_per_column; p.atomic_add = atomic_add;
     const int op = ab_type == PTOAMD_BF16 ? TOP_BF16
                    : ab_type == PTOAMD_F16 ? TOP_F16
                    : ab_type == PTOAMD_I8 ? TOP_I8

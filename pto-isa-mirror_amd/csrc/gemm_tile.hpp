@@ -47,6 +47,7 @@ struct TileGemmParams {
     // OUT_Q8 / OUT_QF16: the fix-pipe quantisation words of the drain, one for the whole matrix or one per column
     const uint64_t* qwords;
     int q_per_column;
+    int atomic_add;         // OUT_F32 / OUT_I32 only: C += result with atomic adds (TSTORE<AtomicAdd>)
 };
 
 __device__ __forceinline__ long mx_scale_base(int mode, int x, int scale_ld)
@@ -292,7 +293,11 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
             const float cs = KIND == OUT_W8A8_BF16 ? p.col_scale[gj] : 1.0f;
             const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? gj : 0] : 0;
             const uint32_t bits = tstore_bits<KIND>(v[r], rs, cs, qw, p.q_per_column != 0, p.relu != 0);
-            if (out_bytes<KIND> == 4)
+            if (KIND == OUT_F32 && p.atomic_add)
+                atomicAdd(reinterpret_cast<float*>(p.c) + o, __builtin_bit_cast(float, bits));
+            else if (KIND == OUT_I32 && p.atomic_add)
+                atomicAdd(reinterpret_cast<int*>(p.c) + o, (int)bits);
+            else if (out_bytes<KIND> == 4)
                 reinterpret_cast<uint32_t*>(p.c)[o] = bits;
             else if (out_bytes<KIND> == 2)
                 reinterpret_cast<uint16_t*>(p.c)[o] = (uint16_t)bits;
@@ -408,7 +413,7 @@ __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::
     const bool full = row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n;
     const int esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : (p.out_kind == OUT_Q8 ? 1 : 2);
     const bool aligned = (((long)p.ldc * esz) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
-    if (stage != nullptr && full && aligned && !(p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr)) {
+    if (stage != nullptr && full && aligned && !p.atomic_add && !(p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr)) {
         if (p.out_kind == OUT_QF16) {
             tstore_staged<OUT_QF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
         } else if (p.out_kind == OUT_Q8) {

@@ -425,6 +425,36 @@ def test_requant_drain_int32_accumulator(pa, oracle, tile, m, n, k):
         assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I8, vector, per_column=True, relu=True))
 
 
+@pytest.mark.parametrize("tile", [None, 2, 5])
+def test_atomic_add_drain_accumulates_k_halves(pa, oracle, tile):
+    """TSTORE<AtomicAdd> in the fused launcher: two launches over the two K halves add up in C (exact on integers)."""
+    r = np.random.default_rng(31)
+    m, n, k = 200, 264, 256
+    a = r.integers(-4, 5, (m, k)).astype(np.float16)
+    b = r.integers(-4, 5, (n, k)).astype(np.float16)
+    init = r.integers(-50, 50, (m, n)).astype(np.float32)
+    want = init + oracle.matmul_f16(a.view(np.uint16), b.view(np.uint16), b_dn=True)
+    env = tile_env(PTOAMD_TILE=tile) if tile is not None else tile_env()
+    with env:
+        out = dev(init.copy())
+        pa.gemm_atomic_add(out, dev(np.ascontiguousarray(a[:, :128])), dev(np.ascontiguousarray(b[:, :128])), pa.F16)
+        assert pa.last_kernel().startswith("tile")
+        pa.gemm_atomic_add(out, dev(np.ascontiguousarray(a[:, 128:])), dev(np.ascontiguousarray(b[:, 128:])), pa.F16)
+    assert np.array_equal(host(out), want)
+    ai, bi = r.integers(-128, 128, (m, k)).astype(np.int8), r.integers(-128, 128, (n, k)).astype(np.int8)
+    initi = r.integers(-2 ** 20, 2 ** 20, (m, n)).astype(np.int32)
+    outi = dev(initi.copy())
+    pa.gemm_atomic_add(outi, dev(ai), dev(bi), pa.I8)
+    assert np.array_equal(host(outi), initi + oracle.matmul_i8(ai, bi, b_dn=True))
+    with tile_env(PTOAMD_FORCE_GENERIC=1):
+        outi = dev(initi.copy())
+        pa.gemm_atomic_add(outi, dev(ai), dev(bi), pa.I8)
+    assert np.array_equal(host(outi), initi + oracle.matmul_i8(ai, bi, b_dn=True))
+    with pytest.raises(pa.PtoAmdError, match="atomic adds target"):
+        _lib = pa.lib()
+        pa._check(_lib.ptoamd_gemm_atomic_add(None, pa.BF16, None, None, pa.BF16, 1, 1, 16, 16, 16, 1, pa.B_DN, None), "x")
+
+
 def test_requant_rejects_other_output_types(pa):
     a = torch.zeros((16, 16), dtype=torch.float16, device=DEV)
     w = torch.zeros(1, dtype=torch.int64, device=DEV)
