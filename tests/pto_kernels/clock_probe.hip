@@ -1,0 +1,120 @@
+// Per-workgroup timestamps of the direct-to-LDS 256 x 256 tile GEMM kernel on one problem (default 4096^3 bf16).
+//
+// Compiled with -DPTOAMD_CLOCK_PROBE the kernel writes, per workgroup, eight 64-bit words through p.acc_out:
+// [0] core clocks spent in the K loop, [1] wall clock (100 MHz) at entry, [2] at the start of the K loop, [3] at its end,
+// [4] at exit.  This program runs the launch back to back until the clocks have settled, then prints the phases of the
+// last launch (mean / max over the workgroups) and the K loop per XCD (workgroup id mod 8).  Timing tool only: it checks
+// no results.  Build: make -C tests/pto_kernels build/clock_probe   (not part of the default target; ~2 minutes)
+//        run:   tests/pto_kernels/build/clock_probe [m n k]
+#define PTOAMD_CLOCK_PROBE 1
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "../../pto-isa-mirror_amd/csrc/gemm_tile_dtl.hpp"
+
+using namespace ptoamd;
+using Cfg = TileCfg<256, 256, 2, 4, OpBF16>;
+
+#define CK(x)                                                                          \
+    do {                                                                               \
+        hipError_t e_ = (x);                                                           \
+        if (e_ != hipSuccess) {                                                        \
+            printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__);      \
+            return 1;                                                                  \
+        }                                                                              \
+    } while (0)
+
+int main(int argc, char** argv)
+{
+    const int m = argc > 1 ? atoi(argv[1]) : 4096, n = argc > 2 ? atoi(argv[2]) : 4096, k = argc > 3 ? atoi(argv[3]) : 4096;
+    if (m <= 0 || n <= 0 || k <= 0 || m % 256 || n % 256 || k % 64) {
+        printf("m and n must be multiples of 256, k a multiple of 64\n");
+        return 2;
+    }
+    const size_t kb = (size_t)k * 2;
+    if ((size_t)(std::max(m, n) - 1) * kb + kb > 0xffffffffull) {
+        printf("operands must stay below 4 GiB (32-bit DMA offsets)\n");
+        return 2;
+    }
+    std::vector<uint16_t> ha((size_t)m * k), hb((size_t)n * k);
+    srand(1);
+    for (auto& v : ha) v = (uint16_t)(0x3c00 + (rand() & 0x3ff) - ((rand() & 1) << 15));
+    for (auto& v : hb) v = (uint16_t)(0x3c00 + (rand() & 0x3ff) - ((rand() & 1) << 15));
+    uint8_t *a, *b;
+    void* c;
+    long* stamps;
+    const int tiles = (m / 256) * (n / 256);
+    CK(hipMalloc(&a, ha.size() * 2));
+    CK(hipMalloc(&b, hb.size() * 2));
+    CK(hipMalloc(&c, (size_t)m * n * 2));
+    CK(hipMalloc(&stamps, (size_t)tiles * 64));
+    CK(hipMemcpy(a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
+    CK(hipMemcpy(b, hb.data(), hb.size() * 2, hipMemcpyHostToDevice));
+    CK(hipMemset(stamps, 0, (size_t)tiles * 64));
+
+    TileGemmParams p{};
+    p.a = a;
+    p.b = b;
+    p.c = c;
+    p.m = m;
+    p.n = n;
+    p.k_bytes = (int)kb;
+    p.lda_bytes = (long)kb;
+    p.ldb_bytes = (long)kb;
+    p.ldc = n;
+    p.out_kind = OUT_BF16;
+    p.group_m = 4;
+    p.acc_out = (int32_t*)stamps;
+    auto kernel = gemm_tile_dtl_kernel<Cfg>;
+    CK(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    for (int i = 0; i < 300; ++i) hipLaunchKernelGGL(kernel, dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, 0, p);
+    CK(hipEventRecord(e0));
+    for (int i = 0; i < 100; ++i) hipLaunchKernelGGL(kernel, dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, 0, p);
+    CK(hipEventRecord(e1));
+    CK(hipEventSynchronize(e1));
+    float ms;
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    printf("%d x %d x %d bf16, %d workgroups: %.2f us per launch with the stamps compiled in\n", m, n, k, tiles, ms * 10.f);
+
+    std::vector<long> h((size_t)tiles * 8);
+    CK(hipMemcpy(h.data(), stamps, (size_t)tiles * 64, hipMemcpyDeviceToHost));
+    long first = h[1], last = 0;
+    for (int t = 0; t < tiles; ++t) {
+        first = std::min(first, h[8 * t + 1]);
+        last = std::max(last, h[8 * t + 4]);
+    }
+    double sum[4] = {0, 0, 0, 0}, mx[4] = {0, 0, 0, 0}, clocks = 0;
+    double xcd_loop[8] = {0}, xcd_clk[8] = {0}, xcd_max[8] = {0};
+    int xcd_cnt[8] = {0};
+    for (int t = 0; t < tiles; ++t) {
+        const long* o = &h[8 * t];
+        const double ph[4] = {double(o[1] - first), double(o[2] - o[1]), double(o[3] - o[2]), double(o[4] - o[3])};
+        for (int i = 0; i < 4; ++i) {
+            sum[i] += ph[i];
+            mx[i] = std::max(mx[i], ph[i]);
+        }
+        clocks += o[0];
+        xcd_loop[t % 8] += ph[2];
+        xcd_clk[t % 8] += o[0];
+        xcd_max[t % 8] = std::max(xcd_max[t % 8], ph[2]);
+        ++xcd_cnt[t % 8];
+    }
+    const char* names[4] = {"entry after the first workgroup's", "prologue", "K loop", "TSTORE"};
+    for (int i = 0; i < 4; ++i) printf("%-34s mean %7.2f us  max %7.2f us\n", names[i], sum[i] / tiles / 100, mx[i] / 100);
+    printf("K loop: %.0f core clocks per workgroup = %.0f per 128-byte slab, %.3f GHz\n", clocks / tiles,
+           clocks / tiles / (kb / 128.0), clocks / sum[2] / 10.0);
+    printf("first entry -> last exit %.2f us\n", (last - first) / 100.0);
+    for (int x = 0; x < 8; ++x)
+        if (xcd_cnt[x])
+            printf("  XCD %d: K loop mean %.2f us, max %.2f us, %.3f GHz\n", x, xcd_loop[x] / xcd_cnt[x] / 100, xcd_max[x] / 100,
+                   xcd_clk[x] / xcd_loop[x] / 10.0);
+    return 0;
+}
