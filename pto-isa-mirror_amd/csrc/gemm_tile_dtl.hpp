@@ -133,7 +133,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // per lane from global memory they are 64 separate small requests per load instruction and keep the CU's address
     // unit busier than the operand DMAs do.  Instead the 16 scale bytes of every row of the tile -- SPG slabs' worth --
     // are DMAed into one of two LDS scale buffers, one instruction per 64 rows, and each wave reads the dwords of its
-    // rows from there.  Chunk g + 1 is requested in the last k-step of slab g * SPG and read from the last k-step of
+    // rows from there.  Chunk g + 1 is requested when slab g * SPG starts and read from the last k-step of
     // slab (g + 1) * SPG - 1 on, i.e. at least one slab barrier (with its vmcnt(0)) later.
     constexpr int GPS = Op::SCALED ? Op::GROUPS_PER_SLAB : 4;  // scale bytes per row per slab
     constexpr int SW = GPS / 4, SPG = 16 / GPS;
@@ -206,10 +206,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     static_assert(Cfg::WTM % 32 == 0 && Cfg::WTN % 32 == 0, "wave tiles start on 32-row boundaries");
     const uint32_t fa_lane = (wm * Cfg::WTM + l32) * 128 + ((lhi ^ swizzle_chunk(l32, 0)) << 4);
     const uint32_t fb_lane = Cfg::A_BYTES + (wn * Cfg::WTN + l32) * 128 + ((lhi ^ swizzle_chunk(l32, 0)) << 4);
-    // Two fragment register sets (next k-step's reads overlap this k-step's MFMAs) unless 32-byte fragments of a
-    // large wave tile would not fit the register file next to the accumulators; then one set is refilled piecewise,
-    // each block right after the last MFMA that reads it, and the second wave of the SIMD covers the LDS latency.
-    constexpr int SETS = ((FR == 2 && MB * NB >= 8) || NT > 512) ? 1 : 2;  // 16 waves: 128 registers per lane
+    // Two fragment register sets (next k-step's reads overlap this k-step's MFMAs).  Where 32-byte fragments of a large
+    // wave tile would not fit the register file twice next to the accumulators (HYBRID), only the fragments that stay
+    // live until the end of a k-step get a second copy -- all of B and A's last row block; the other A row blocks are
+    // refilled in place right after their last MFMA, several MFMAs before the next k-step reads them.  16 waves
+    // (128 registers per lane) keep one set, refilled piecewise, and the SIMD's other waves cover the LDS latency.
+    // (The hybrid read schedule needs one first-column MFMA per double-buffered fragment, NB + 1 <= MB; the square wave
+    // tile of the 4-wave form has accumulators for 16 blocks and keeps the single set.)
+    constexpr bool BIG_FRAGS = FR == 2 && MB * NB >= 8;
+    constexpr bool HYBRID = BIG_FRAGS && NT <= 512 && NB + 1 <= MB;
+    constexpr int SETS = (NT > 512 || (BIG_FRAGS && !HYBRID)) ? 1 : 2;
     uint4 fa[SETS][MB][FR], fb[SETS][NB][FR];
     constexpr int NREAD = (MB + NB) * FR, NMMA = MB * NB, NDMA = LA + LB;
     // fragment read number q of k-step s of ring buffer buf into register set `set`; B fragments come first because the
@@ -233,15 +239,28 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         static_for<NMMA>([&](auto xc) {
             constexpr int x = decltype(xc)::value;
             constexpr int i = x / NB, j = x % NB;
+            const int aset = (HYBRID && i != MB - 1) ? 0 : set;  // register set of A's row block i
             // MX group 2 s + lhi of the slab lives in dword s >> 1 (either lane half) at byte 2 (s & 1) + lhi; the
             // dwords were shifted right by 8 lhi when the slab started, so both halves select byte 2 (s & 1) and the
             // instruction's own byte select does the extraction.  Without scale arrays every byte is E8M0 127.
             if (s & 1)
-                Op::template mma_sel<2>(acc[i][j], fa[set][i], fb[set][j], sca[i][s >> 1], scb[j][s >> 1]);
+                Op::template mma_sel<2>(acc[i][j], fa[aset][i], fb[set][j], sca[i][s >> 1], scb[j][s >> 1]);
             else
-                Op::template mma_sel<0>(acc[i][j], fa[set][i], fb[set][j], sca[i][s >> 1], scb[j][s >> 1]);
+                Op::template mma_sel<0>(acc[i][j], fa[aset][i], fb[set][j], sca[i][s >> 1], scb[j][s >> 1]);
             if (reads) {
-                if constexpr (SETS == 2) {
+                if constexpr (HYBRID) {
+                    // pinned behind the MFMA that frees the registers (hoisted above it the refill would need a second
+                    // copy after all).  First-column MFMAs 0 .. NB - 1 are followed by the next step's B blocks and
+                    // MFMA NB by A's last row block, into the other set; a row's last MFMA by that row's refill.
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (j == 0 && i < NB)
+                        static_for<FR>([&](auto fc) { textract_piece(nset, rbuf, rs, i * FR + decltype(fc)::value); });
+                    if constexpr (j == 0 && i == NB)
+                        static_for<FR>([&](auto fc) { textract_piece(nset, rbuf, rs, NB * FR + (MB - 1) * FR + decltype(fc)::value); });
+                    if constexpr (j == NB - 1 && i < MB - 1)
+                        static_for<FR>([&](auto fc) { textract_piece(0, rbuf, rs, NB * FR + i * FR + decltype(fc)::value); });
+                    __builtin_amdgcn_sched_barrier(0);
+                } else if constexpr (SETS == 2) {
                     constexpr int q0 = x * NREAD / NMMA, q1 = (x + 1) * NREAD / NMMA;
                     static_for<q1 - q0>([&](auto qc) { textract_piece(nset, rbuf, rs, q0 + decltype(qc)::value); });
                 } else {
@@ -259,7 +278,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
                 static_for<q1 - q0>([&](auto qc) { tload_piece(dkt, dbuf, q0 + decltype(qc)::value); });
             }
         });
-        if constexpr (SETS == 2)
+        if constexpr (SETS == 2 && !HYBRID)
             sched_kstep<NMMA, NREAD, 0>();
     };
 
@@ -283,6 +302,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     auto slab = [&](int kt, bool more, bool dma) {
         const int cur = kt & 1;
         if (Op::SCALED) {
+            // The request for the next scale chunk sits here, at the top of the slab, and not between two k-steps: a
+            // branch between them splits the slab into basic blocks, and the compiler then sinks the first k-step's
+            // MFMAs (pure register operations) below the barrier into the block that uses their results, where they
+            // no longer overlap the fragment reads.  The buffer it overwrites was last read a whole slab ago (every
+            // wave has passed the previous slab's barrier, and consumed those scale dwords before it).
+            if (kt % SPG == 0 && (kt / SPG + 1) * SPG < k_slabs)
+                tload_scales(kt / SPG + 1);
             if constexpr (!SC_AHEAD)
                 read_scales(kt);
 #pragma unroll
@@ -304,8 +330,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         __syncthreads();
         if (SC_AHEAD && more)
             read_scales(kt + 1);
-        if (kt % SPG == 0 && (kt / SPG + 1) * SPG < k_slabs)
-            tload_scales(kt / SPG + 1);
         kstep(std::integral_constant<int, 0>{}, KS - 1, more, cur ^ 1, 0, dma, kt + 2, cur);
     };
     int kt = 0;

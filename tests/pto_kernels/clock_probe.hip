@@ -1,11 +1,14 @@
-// Per-workgroup timestamps of the direct-to-LDS 256 x 256 tile GEMM kernel on one problem (default 4096^3 bf16).
+// Per-workgroup timestamps of the direct-to-LDS 256 x 256 tile GEMM kernel on one problem (default 4096^3).
+// -DPROBE_KIND=0 bf16 (default), 1 int8 -> i32, 2 MXFP8 (E4M3 x E4M3, unit block scales) -> bf16.
 //
 // Compiled with -DPTOAMD_CLOCK_PROBE the kernel writes, per workgroup, eight 64-bit words through p.acc_out:
 // [0] core clocks spent in the K loop, [1] wall clock (100 MHz) at entry, [2] at the start of the K loop, [3] at its end,
 // [4] at exit.  This program runs the launch back to back until the clocks have settled, then prints the phases of the
 // last launch (mean / max over the workgroups) and the K loop per XCD (workgroup id mod 8).  Timing tool only: it checks
-// no results.  Build: make -C tests/pto_kernels build/clock_probe   (not part of the default target; ~2 minutes)
-//        run:   tests/pto_kernels/build/clock_probe [m n k]
+// no results.  Build: make -C tests/pto_kernels build/clock_probe   (not part of the default target; under a minute;
+//                     build/clock_probe_i8 and build/clock_probe_fp8 are the other two kinds)
+//        run:   tests/pto_kernels/build/clock_probe [m n k [zeros]]   (a fourth argument fills the operands with zeros:
+//               the same instruction stream at the lowest switching power)
 #define PTOAMD_CLOCK_PROBE 1
 #include <hip/hip_runtime.h>
 
@@ -17,7 +20,23 @@
 #include "../../pto-isa-mirror_amd/csrc/gemm_tile_dtl.hpp"
 
 using namespace ptoamd;
-using Cfg = TileCfg<256, 256, 2, 4, OpBF16>;
+#ifndef PROBE_KIND
+#define PROBE_KIND 0
+#endif
+#if PROBE_KIND == 0
+using ProbeOp = OpBF16;
+constexpr int ESZ = 2, CSZ = 2, OUT = OUT_BF16;
+constexpr const char* KIND = "bf16";
+#elif PROBE_KIND == 1
+using ProbeOp = OpI8;
+constexpr int ESZ = 1, CSZ = 4, OUT = OUT_I32;
+constexpr const char* KIND = "int8";
+#else
+using ProbeOp = OpFP8<0, 0>;
+constexpr int ESZ = 1, CSZ = 2, OUT = OUT_BF16;
+constexpr const char* KIND = "MXFP8";
+#endif
+using Cfg = TileCfg<256, 256, 2, 4, ProbeOp>;
 
 #define CK(x)                                                                          \
     do {                                                                               \
@@ -31,30 +50,46 @@ using Cfg = TileCfg<256, 256, 2, 4, OpBF16>;
 int main(int argc, char** argv)
 {
     const int m = argc > 1 ? atoi(argv[1]) : 4096, n = argc > 2 ? atoi(argv[2]) : 4096, k = argc > 3 ? atoi(argv[3]) : 4096;
-    if (m <= 0 || n <= 0 || k <= 0 || m % 256 || n % 256 || k % 64) {
-        printf("m and n must be multiples of 256, k a multiple of 64\n");
+    if (m <= 0 || n <= 0 || k <= 0 || m % 256 || n % 256 || k % 512) {
+        printf("m and n must be multiples of 256, k a multiple of 512\n");
         return 2;
     }
-    const size_t kb = (size_t)k * 2;
+    const size_t kb = (size_t)k * ESZ;
     if ((size_t)(std::max(m, n) - 1) * kb + kb > 0xffffffffull) {
         printf("operands must stay below 4 GiB (32-bit DMA offsets)\n");
         return 2;
     }
-    std::vector<uint16_t> ha((size_t)m * k), hb((size_t)n * k);
+    // operand bytes: 16-bit patterns 0x3c00 + 10 random bits with a random sign are bf16 values of magnitude 1 - 2; as
+    // byte pairs they are ordinary int8 values and, with bit 3 of each byte cleared, finite E4M3 codes
+    std::vector<uint16_t> ha((size_t)m * kb / 2), hb((size_t)n * kb / 2);
     srand(1);
     for (auto& v : ha) v = (uint16_t)(0x3c00 + (rand() & 0x3ff) - ((rand() & 1) << 15));
     for (auto& v : hb) v = (uint16_t)(0x3c00 + (rand() & 0x3ff) - ((rand() & 1) << 15));
-    uint8_t *a, *b;
+    if (argc > 4) {
+        std::fill(ha.begin(), ha.end(), 0);
+        std::fill(hb.begin(), hb.end(), 0);
+    }
+    if (ProbeOp::SCALED) {
+        for (auto& v : ha) v &= 0xf7f7;
+        for (auto& v : hb) v &= 0xf7f7;
+    }
+    uint8_t *a, *b, *sa = nullptr, *sb = nullptr;
     void* c;
     long* stamps;
     const int tiles = (m / 256) * (n / 256);
     CK(hipMalloc(&a, ha.size() * 2));
     CK(hipMalloc(&b, hb.size() * 2));
-    CK(hipMalloc(&c, (size_t)m * n * 2));
+    CK(hipMalloc(&c, (size_t)m * n * CSZ));
     CK(hipMalloc(&stamps, (size_t)tiles * 64));
     CK(hipMemcpy(a, ha.data(), ha.size() * 2, hipMemcpyHostToDevice));
     CK(hipMemcpy(b, hb.data(), hb.size() * 2, hipMemcpyHostToDevice));
     CK(hipMemset(stamps, 0, (size_t)tiles * 64));
+    if (ProbeOp::SCALED) {
+        CK(hipMalloc(&sa, (size_t)m * (k / 32)));
+        CK(hipMalloc(&sb, (size_t)n * (k / 32)));
+        CK(hipMemset(sa, 127, (size_t)m * (k / 32)));
+        CK(hipMemset(sb, 127, (size_t)n * (k / 32)));
+    }
 
     TileGemmParams p{};
     p.a = a;
@@ -66,8 +101,11 @@ int main(int argc, char** argv)
     p.lda_bytes = (long)kb;
     p.ldb_bytes = (long)kb;
     p.ldc = n;
-    p.out_kind = OUT_BF16;
+    p.out_kind = OUT;
     p.group_m = 4;
+    p.sa = sa;
+    p.sb = sb;
+    p.scale_ld = k / 32;
     p.acc_out = (int32_t*)stamps;
     auto kernel = gemm_tile_dtl_kernel<Cfg>;
     CK(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
@@ -82,7 +120,7 @@ int main(int argc, char** argv)
     CK(hipEventSynchronize(e1));
     float ms;
     CK(hipEventElapsedTime(&ms, e0, e1));
-    printf("%d x %d x %d bf16, %d workgroups: %.2f us per launch with the stamps compiled in\n", m, n, k, tiles, ms * 10.f);
+    printf("%d x %d x %d %s%s, %d workgroups: %.2f us per launch with the stamps compiled in\n", m, n, k, KIND, argc > 4 ? " (zero operands)" : "", tiles, ms * 10.f);
 
     std::vector<long> h((size_t)tiles * 8);
     CK(hipMemcpy(h.data(), stamps, (size_t)tiles * 64, hipMemcpyDeviceToHost));
@@ -112,6 +150,20 @@ int main(int argc, char** argv)
     printf("K loop: %.0f core clocks per workgroup = %.0f per 128-byte slab, %.3f GHz\n", clocks / tiles,
            clocks / tiles / (kb / 128.0), clocks / sum[2] / 10.0);
     printf("first entry -> last exit %.2f us\n", (last - first) / 100.0);
+    if (tiles > 256) {  // more workgroups than CUs: when each round of the chip starts and ends
+        std::vector<long> entry(tiles), exit_(tiles);
+        for (int t = 0; t < tiles; ++t) {
+            entry[t] = h[8 * t + 1] - first;
+            exit_[t] = h[8 * t + 4] - first;
+        }
+        std::sort(entry.begin(), entry.end());
+        std::sort(exit_.begin(), exit_.end());
+        for (int r = 0; r * 256 < tiles; ++r) {
+            const int lo = r * 256, hi = std::min(tiles, lo + 256) - 1;
+            printf("  workgroups %4d-%4d by start: entries %.2f .. %.2f us; by end: exits %.2f .. %.2f us\n", lo, hi,
+                   entry[lo] / 100.0, entry[hi] / 100.0, exit_[lo] / 100.0, exit_[hi] / 100.0);
+        }
+    }
     for (int x = 0; x < 8; ++x)
         if (xcd_cnt[x])
             printf("  XCD %d: K loop mean %.2f us, max %.2f us, %.3f GHz\n", x, xcd_loop[x] / xcd_cnt[x] / 100, xcd_max[x] / 100,
