@@ -130,11 +130,13 @@ int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_t
  * The same pipeline drained through the fix-pipe quantiser: TSTORE of the accumulator tile with a scalar quantisation
  * word (TSTORE(dst, src, preQuantScalar)) or one word per column (TSTORE_FP with a Scaling tile):
  *   r = acc(i, j) * scale(word);  s8 / u8: clamp(rint(r + offset(word)), byte range chosen by the word's sign bit);
- *   f16: clamp to +-65504 (finite values only for float accumulators);  then relu, then the store.
+ *   f16: clamp to +-65504 (finite values only for float accumulators);  bf16: the product rounded to bfloat16;
+ *   s16 (int32 accumulators only, the SHIFTS322S16 mode): (int16)(acc >> (bits 32..35 of the word + 1)), wrapping as
+ *   the reference does;  then relu, then the store.
  * Cin and bias are added to the accumulator before the quantisation.
  * reference: include/pto/cpu/common.hpp:117-185 (extract_m1_from_quant, quantize_element), cpu/TStore.hpp:118-181,
  *            common/pto_instr.hpp:439-490; test shapes tests/cpu/st/testcase/tstore_acc2gm, tstore_quant.
- *   c_type      : PTOAMD_I8 | PTOAMD_U8 | PTOAMD_F16 (the byte's signedness comes from bit 46 of the word, as in the
+ *   c_type      : PTOAMD_I8 | PTOAMD_U8 | PTOAMD_F16 | PTOAMD_BF16 | PTOAMD_I16 (the byte's signedness comes from bit 46 of the word, as in the
  *                 reference: it must agree with c_type)
  *   quant_words : device memory, 8-byte aligned; one uint64 (per_column == 0) or N of them (per_column != 0).  Scalar
  *                 words hold an fp32 scale in bits 0..31; per-column words a 19-bit (1, 8, 10) float in bits 13..31;
@@ -229,6 +231,11 @@ int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, const uint8_t* 
  * offset == NULL selects the symmetric form (int8 output); otherwise the output is uint8.  src is [rows][cols] f32. */
 int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const float* offset, int rows, int cols,
                        void* stream);
+/* The same with the parameter tiles described as the reference's GetParamValue reads them (cpu/TQuant.hpp:78-84):
+ * scale / offset are [para_rows][para_ld] f32, column 0 is used and the row index is clamped to para_rows - 1 (a
+ * parameter tile with fewer valid rows than src repeats its last row). */
+int ptoamd_tquant_int8_para(void* dst, const float* src, const float* scale, const float* offset, int rows, int cols,
+                            int para_rows, int para_ld, void* stream);
 
 /* TQUANT<MXFP8 | MXFP4_E2M1> (cpu/TQuant.hpp:461-493, 524-547).  src [rows][cols] of src_type (F32 | F16 | BF16);
  * axis 1 groups 32 elements along a row (exp / max / scaling are [rows][cols/32]), axis 0 along a column
@@ -240,6 +247,10 @@ int ptoamd_tquant_mx(uint8_t* dst, uint8_t* exp, float* max, float* scaling, con
  * src_type PTOAMD_I8 | PTOAMD_I16 | PTOAMD_I32. */
 int ptoamd_tdequant(float* dst, const void* src, int src_type, const float* scale, const float* offset, int rows,
                     int cols, void* stream);
+/* The same with parameter tiles wider than one column (cpu/TDeQuant.hpp:24-30): scale / offset are [rows][para_ld] f32
+ * with para_cols valid columns, and element (r, c) uses parameter column min(c, para_cols - 1). */
+int ptoamd_tdequant_para(float* dst, const void* src, int src_type, const float* scale, const float* offset, int rows,
+                         int cols, int para_cols, int para_ld, void* stream);
 
 /* Copies an E8M0 scale matrix between GM layouts (the TLOAD + TMOV of a scale tile, cpu/tile_offsets.hpp:233-268):
  * rows x cols is the logical extent ([M][K/32] for the A side, [K/32][N] for the B side). */

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 
 E4M3, E5M2, E2M1, E1M2, E8M0 = 0, 1, 2, 3, 4
 ND, DN, NZ, MX_A_ZZ, MX_A_ND, MX_A_DN, MX_B_NN, MX_B_ND, MX_B_DN = range(9)
-ST_F32, ST_F16, ST_BF16, ST_I32, ST_I8, ST_U8 = range(6)
+ST_F32, ST_F16, ST_BF16, ST_I32, ST_I8, ST_U8, ST_I16 = range(7)
 OCP_FP8, NV_FP8, OCP_FP4, NV_FP4 = range(4)
 SRC_F32, SRC_F16, SRC_BF16 = range(3)
 
@@ -167,7 +167,7 @@ class Oracle:
 
     # -- store -------------------------------------------------------------------------------
     _ST_DT = {ST_F32: np.float32, ST_F16: np.uint16, ST_BF16: np.uint16, ST_I32: np.int32, ST_I8: np.int8,
-              ST_U8: np.uint8}
+              ST_U8: np.uint8, ST_I16: np.int16}
 
     def store_f32(self, acc, dst_kind, relu=False):
         acc = _c(acc, np.float32)
@@ -222,6 +222,26 @@ class Oracle:
         out = np.empty((r, c), np.float32)
         self.lib.pto_tdequant(_p(out), _p(src), kind, _p(_c(scale, np.float32)), _p(_c(offset, np.float32)), r, c)
         return out
+
+    def tdequant_para(self, src, scale, offset):
+        """scale / offset: [rows][para_cols]; element (r, c) uses parameter column min(c, para_cols - 1)."""
+        kind = {np.dtype(np.int8): 0, np.dtype(np.int16): 1, np.dtype(np.int32): 2}[src.dtype]
+        src = np.ascontiguousarray(src)
+        scale, offset = _c(scale, np.float32), _c(offset, np.float32)
+        r, c = src.shape
+        out = np.empty((r, c), np.float32)
+        self.lib.pto_tdequant_para(_p(out), _p(src), kind, _p(scale), _p(offset), r, c, scale.shape[1], scale.shape[1])
+        return out
+
+    def tquant_int8_para(self, src, scale, offset=None, para_ld=1):
+        """scale / offset: [para_rows * para_ld] flat; row r uses element min(r, para_rows - 1) * para_ld."""
+        src = _c(src, np.float32)
+        scale = _c(scale, np.float32)
+        r, c = src.shape
+        out = np.empty((r, c), np.uint8)
+        off = None if offset is None else _p(_c(offset, np.float32))
+        self.lib.pto_tquant_int8_para(_p(out), _p(src), _p(scale), off, r, c, scale.size // para_ld, para_ld)
+        return out if offset is not None else out.view(np.int8)
 
     # -- CPU-simulator-shaped baseline --------------------------------------------------------
     def sim_gemm_tiled(self, a, b, dtype, out_kind, b_dn, max_threads=0):
@@ -314,7 +334,7 @@ class RefLib:
         words = _c(words, np.uint64)
         m, n = acc.shape
         key = ("i32" if acc.dtype == np.int32 else "f32") + "_" + dst
-        out_dt = {"i8": np.int8, "u8": np.uint8, "f16": np.uint16}[dst]
+        out_dt = {"i8": np.int8, "u8": np.uint8, "f16": np.uint16, "i16": np.int16}[dst]
         out = np.empty((m, n), out_dt)
         acc = np.ascontiguousarray(acc)
         rc = getattr(self.lib, "ref_store_" + key)(_p(out), _p(acc), m, n, _p(words), int(per_column), int(relu))
@@ -364,6 +384,23 @@ class RefLib:
                                     _p(_c(src, np.float32)))
         assert rc == 0, rc
         return (dst.reshape(r, c // 2) if fp4 else dst.reshape(r, c)), exp, mx, sc
+
+    def tdequant_para(self, src, scale, offset):
+        """16 x 64 int8 source, scale / offset [16][para_cols] with para_cols 1, 3 or 8."""
+        out = np.empty((16, 64), np.float32)
+        scale, offset = _c(scale, np.float32), _c(offset, np.float32)
+        rc = self.lib.ref_tdequant_para(scale.shape[1], _p(out), _p(_c(src, np.int8)), _p(scale), _p(offset))
+        assert rc == 0, rc
+        return out
+
+    def tquant_int8_para(self, src, scale, offset=None):
+        """16 x 64 f32 source, scale / offset [para_rows] with para_rows 1, 5 or 16."""
+        out = np.empty((16, 64), np.uint8)
+        scale = _c(scale, np.float32)
+        off = _c(np.zeros_like(scale) if offset is None else offset, np.float32)
+        rc = self.lib.ref_tquant_int8_para(scale.size, int(offset is not None), _p(out), _p(_c(src, np.float32)), _p(scale), _p(off))
+        assert rc == 0, rc
+        return out if offset is not None else out.view(np.int8)
 
     def tdequant(self, shape_id, src, scale, offset):
         r, c = self.shape(shape_id)

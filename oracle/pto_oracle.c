@@ -538,6 +538,7 @@ static void put_converted(void* out, int dst_kind, size_t idx, float v)
         case PTO_ST_BF16: ((uint16_t*)out)[idx] = pto_f32_to_bf16(v); break;
         case PTO_ST_I32: ((int32_t*)out)[idx] = (int32_t)v; break;
         case PTO_ST_I8: ((int8_t*)out)[idx] = (int8_t)v; break;
+        case PTO_ST_I16: ((int16_t*)out)[idx] = (int16_t)v; break;
         default: ((uint8_t*)out)[idx] = (uint8_t)v; break;
     }
 }
@@ -569,8 +570,10 @@ float pto_quant_word_scale(uint64_t word, int vector_mode)
     return sv * mv * ev;
 }
 
-/* common.hpp:139-185 (quantize_element) for the 8-bit, f16 and bf16 targets */
-static float quant_core(float src, uint64_t word, int vector_mode, int dst_kind, int src_is_int, int saturate_inf)
+/* common.hpp:139-185 (quantize_element) for the 8-bit, f16, bf16 and (int32 source only) int16 targets; isrc is the
+ * integer accumulator when src_is_int */
+static float quant_core(float src, int32_t isrc, uint64_t word, int vector_mode, int dst_kind, int src_is_int,
+                        int saturate_inf)
 {
     const float f_scale = pto_quant_word_scale(word, vector_mode);
     const uint32_t offset = (uint32_t)((word >> 37) & 0x1FFu);
@@ -593,6 +596,11 @@ static float quant_core(float src, uint64_t word, int vector_mode, int dst_kind,
             r = 0.0f;
         else if (isfinite(r) || saturate_inf)
             r = r < -3.402823466e38f ? -3.402823466e38f : (r > 3.402823466e38f ? 3.402823466e38f : r);
+    } else if (dst_kind == PTO_ST_I16 && src_is_int) {
+        /* SHIFTS322S16 / VSHIFTS322S16 (common.hpp:174-180): arithmetic shift by bits 32..35 of the word plus one; the
+         * value is narrowed to int16 BEFORE the clamp, so it wraps and the clamp never acts */
+        const int shift = (int)((word >> 32) & 0xFu) + 1;
+        r = (float)(int16_t)(isrc >> shift);
     }
     return r;
 }
@@ -602,7 +610,7 @@ void pto_store_quant_f32(void* out, int dst_kind, const float* acc, int m, int n
 {
     for (int i = 0; i < m; ++i)
         for (int j = 0; j < n; ++j) {
-            float r = quant_core(acc[(size_t)i * n + j], words[per_column ? j : 0], per_column, dst_kind, 0,
+            float r = quant_core(acc[(size_t)i * n + j], 0, words[per_column ? j : 0], per_column, dst_kind, 0,
                                  saturate_inf);
             if (relu)
                 r = r > 0 ? r : 0;
@@ -615,7 +623,8 @@ void pto_store_quant_i32(void* out, int dst_kind, const int32_t* acc, int m, int
 {
     for (int i = 0; i < m; ++i)
         for (int j = 0; j < n; ++j) {
-            float r = quant_core((float)acc[(size_t)i * n + j], words[per_column ? j : 0], per_column, dst_kind, 1, 0);
+            const int32_t a = acc[(size_t)i * n + j];
+            float r = quant_core((float)a, a, words[per_column ? j : 0], per_column, dst_kind, 1, 0);
             if (relu)
                 r = r > 0 ? r : 0;
             put_converted(out, dst_kind, (size_t)i * n + j, r);
@@ -627,21 +636,33 @@ void pto_store_quant_i32(void* out, int dst_kind, const int32_t* acc, int m, int
 static inline float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 /* TQuant.hpp:86-96, 496-522.  The "scale" operand is multiplied (it is the inverse scale). */
+/* GetParamValue (TQuant.hpp:78-84) as TQUANT INT8 calls it: column 0 of a [para_rows][para_ld] parameter tile, the
+ * row clamped to para_rows - 1.  offset == NULL: symmetric (int8 codes in dst), else asymmetric (uint8 codes). */
+void pto_tquant_int8_para(uint8_t* dst, const float* src, const float* scale, const float* offset, int rows, int cols,
+                          int para_rows, int para_ld)
+{
+    for (int r = 0; r < rows; ++r) {
+        const size_t pr = (size_t)(r < para_rows - 1 ? r : para_rows - 1) * para_ld;
+        for (int c = 0; c < cols; ++c) {
+            const float prod = src[(size_t)r * cols + c] * scale[pr];
+            if (offset) {
+                const float v = prod + offset[pr]; /* two roundings: multiply, then add */
+                dst[(size_t)r * cols + c] = (uint8_t)clampf(nearbyintf(v), 0.0f, 255.0f);
+            } else {
+                dst[(size_t)r * cols + c] = (uint8_t)(int8_t)clampf(nearbyintf(prod), -128.0f, 127.0f);
+            }
+        }
+    }
+}
+
 void pto_tquant_int8_sym(int8_t* dst, const float* src, const float* scale, int rows, int cols)
 {
-    for (int r = 0; r < rows; ++r)
-        for (int c = 0; c < cols; ++c)
-            dst[(size_t)r * cols + c] = (int8_t)clampf(nearbyintf(src[(size_t)r * cols + c] * scale[r]), -128.0f, 127.0f);
+    pto_tquant_int8_para((uint8_t*)dst, src, scale, NULL, rows, cols, rows, 1);
 }
 
 void pto_tquant_int8_asym(uint8_t* dst, const float* src, const float* scale, const float* offset, int rows, int cols)
 {
-    for (int r = 0; r < rows; ++r)
-        for (int c = 0; c < cols; ++c) {
-            const float prod = src[(size_t)r * cols + c] * scale[r];
-            const float v = prod + offset[r]; /* two roundings: multiply, then add */
-            dst[(size_t)r * cols + c] = (uint8_t)clampf(nearbyintf(v), 0.0f, 255.0f);
-        }
+    pto_tquant_int8_para(dst, src, scale, offset, rows, cols, rows, 1);
 }
 
 static float e4m3_pos_value(unsigned code) /* TQuant.hpp:98-116 for codes 0..0x7E */
@@ -821,18 +842,27 @@ void pto_reorder_exp_zz(uint8_t* dst, const uint8_t* exp, int rows, int group_co
 }
 
 /* cpu/TDeQuant.hpp:18-37 with a single scale/offset column */
-void pto_tdequant(float* dst, const void* src, int src_kind, const float* scale, const float* offset, int rows,
-                  int cols)
+/* TDeQuant.hpp:18-37.  scale / offset are [rows][para_ld] with para_cols valid columns; element (r, c) reads
+ * parameter column min(c, para_cols - 1) (TDeQuant.hpp:24-30). */
+void pto_tdequant_para(float* dst, const void* src, int src_kind, const float* scale, const float* offset, int rows,
+                       int cols, int para_cols, int para_ld)
 {
     for (int r = 0; r < rows; ++r)
         for (int c = 0; c < cols; ++c) {
             const size_t i = (size_t)r * cols + c;
+            const size_t pi = (size_t)r * para_ld + (c < para_cols - 1 ? c : para_cols - 1);
             const float s = src_kind == 0 ? (float)((const int8_t*)src)[i]
                                           : (src_kind == 1 ? (float)((const int16_t*)src)[i]
                                                            : (float)((const int32_t*)src)[i]);
-            const float d = s - offset[r];
-            dst[i] = d * scale[r];
+            const float d = s - offset[pi];
+            dst[i] = d * scale[pi];
         }
+}
+
+void pto_tdequant(float* dst, const void* src, int src_kind, const float* scale, const float* offset, int rows,
+                  int cols)
+{
+    pto_tdequant_para(dst, src, src_kind, scale, offset, rows, cols, 1, 1);
 }
 
 /* ============================== CPU-simulator-shaped tiled GEMM ============================ */

@@ -81,7 +81,7 @@ void pto_matmul_mx(float* out, const uint8_t* a, const uint8_t* b, const uint8_t
                    int a_type, int b_type, int sa_layout, int sb_layout);
 
 /* ---- TSTORE value conversion (Acc -> GM), incl. fix-pipe requantisation ------------------- */
-enum pto_store_dst { PTO_ST_F32 = 0, PTO_ST_F16 = 1, PTO_ST_BF16 = 2, PTO_ST_I32 = 3, PTO_ST_I8 = 4, PTO_ST_U8 = 5 };
+enum pto_store_dst { PTO_ST_F32 = 0, PTO_ST_F16 = 1, PTO_ST_BF16 = 2, PTO_ST_I32 = 3, PTO_ST_I8 = 4, PTO_ST_U8 = 5, PTO_ST_I16 = 6 };
 /* no-quant path: optional relu then static_cast */
 void pto_store_f32(void* out, int dst_kind, const float* acc, int m, int n, int ldacc, int ldout, int relu);
 /* quant path: words[j] per column when per_column, else words[0] */
@@ -94,6 +94,8 @@ void pto_store_quant_i32(void* out, int dst_kind, const int32_t* acc, int m, int
 /* ---- TQUANT / TDEQUANT -------------------------------------------------------------------- */
 void pto_tquant_int8_sym(int8_t* dst, const float* src, const float* scale, int rows, int cols);
 void pto_tquant_int8_asym(uint8_t* dst, const float* src, const float* scale, const float* offset, int rows, int cols);
+void pto_tquant_int8_para(uint8_t* dst, const float* src, const float* scale, const float* offset, int rows, int cols,
+                          int para_rows, int para_ld);
 
 enum pto_mx_alg { PTO_OCP_FP8 = 0, PTO_NV_FP8 = 1, PTO_OCP_FP4 = 2, PTO_NV_FP4 = 3 };
 enum pto_src_kind { PTO_SRC_F32 = 0, PTO_SRC_F16 = 1, PTO_SRC_BF16 = 2 };
@@ -111,6 +113,8 @@ void pto_reorder_exp_zz(uint8_t* dst, const uint8_t* exp, int rows, int group_co
 /* dst(r, c) = (float(src(r, c)) - offset[r]) * scale[r];  src_kind: 0 int8, 1 int16, 2 int32 */
 void pto_tdequant(float* dst, const void* src, int src_kind, const float* scale, const float* offset, int rows,
                   int cols);
+void pto_tdequant_para(float* dst, const void* src, int src_kind, const float* scale, const float* offset, int rows,
+                       int cols, int para_cols, int para_ld);
 
 /* ---- CPU-simulator-shaped tiled GEMM (the "port" CPU baseline) ---------------------------- */
 /* Walks 128x128 output tiles with a K step of 64 the way the reference demo does: TLOAD copies into a private

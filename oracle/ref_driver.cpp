@@ -309,6 +309,61 @@ int RunDequant(float* dst, const SrcT* src, const float* scale, const float* off
     return 0;
 }
 
+// Parameter tiles as the reference reads them: TDEQUANT clamps the parameter column to the tile's valid columns
+// (TDeQuant.hpp:24-30); TQUANT INT8 reads column 0 and clamps the row to the valid rows (GetParamValue, TQuant.hpp:78-84).
+template <int PC>
+int RunDequantPara(float* dst, const int8_t* src, const float* scale, const float* offset)
+{
+    constexpr int R = 16, C = 64;
+    using SrcTile = Tile<TileType::Vec, int8_t, R, C>;
+    using DstTile = Tile<TileType::Vec, float, R, C>;
+    using ParaTile = Tile<TileType::Vec, float, R, 8, BLayout::RowMajor, R, PC>;
+    SrcTile s;
+    DstTile d;
+    ParaTile sc, off;
+    for (int r = 0; r < R; ++r) {
+        for (int c = 0; c < PC; ++c) {
+            sc.SetElement(r, c, scale[r * PC + c]);
+            off.SetElement(r, c, offset[r * PC + c]);
+        }
+        for (int c = 0; c < C; ++c)
+            s.SetElement(r, c, src[r * C + c]);
+    }
+    TDEQUANT(d, s, sc, off);
+    for (int r = 0; r < R; ++r)
+        for (int c = 0; c < C; ++c)
+            dst[r * C + c] = d.GetElement(r, c);
+    return 0;
+}
+
+template <int PR, bool asym>
+int RunQuantInt8Para(uint8_t* dst, const float* src, const float* scale, const float* offset)
+{
+    constexpr int R = 16, C = 64;
+    using SrcTile = Tile<TileType::Vec, float, R, C>;
+    using DstTile = Tile<TileType::Vec, std::conditional_t<asym, uint8_t, int8_t>, R, C>;
+    using ParaTile = Tile<TileType::Vec, float, R, 8, BLayout::RowMajor, PR, 3>;
+    SrcTile s;
+    DstTile d;
+    ParaTile sc, off;
+    for (int r = 0; r < PR; ++r)
+        for (int c = 0; c < 3; ++c) {  // columns 1 and 2 hold other values: only column 0 may be read
+            sc.SetElement(r, c, c == 0 ? scale[r] : -1000.0f);
+            off.SetElement(r, c, c == 0 ? offset[r] : 999.0f);
+        }
+    for (int r = 0; r < R; ++r)
+        for (int c = 0; c < C; ++c)
+            s.SetElement(r, c, src[r * C + c]);
+    if constexpr (asym)
+        TQUANT<QuantType::INT8_ASYM>(d, s, sc, &off);
+    else
+        TQUANT<QuantType::INT8_SYM>(d, s, sc);
+    for (int r = 0; r < R; ++r)
+        for (int c = 0; c < C; ++c)
+            dst[r * C + c] = (uint8_t)d.GetElement(r, c);
+    return 0;
+}
+
 template <typename TileT>
 int64_t TileOffset(int r, int c)
 {
@@ -418,6 +473,12 @@ int ref_store_i32_f16(uint16_t* out, const int32_t* acc, int m, int n, const uin
                   RunStoreQuant<half, int32_t, false>((half*)out, acc, m, n, q, per_col);
 }
 
+int ref_store_i32_i16(int16_t* out, const int32_t* acc, int m, int n, const uint64_t* q, int per_col, int relu)
+{
+    return relu ? RunStoreQuant<int16_t, int32_t, true>(out, acc, m, n, q, per_col) :
+                  RunStoreQuant<int16_t, int32_t, false>(out, acc, m, n, q, per_col);
+}
+
 // ---- TQUANT / TDEQUANT; shape_id selects one of the compiled static shapes -------------------
 // shape ids: 0 = 4x32, 1 = 2x128, 2 = 2x256, 3 = 16x64, 4 = 8x512, 5 = 64x64, 6 = 32x96
 #define PTO_REF_SHAPES(X) X(0, 4, 32) X(1, 2, 128) X(2, 2, 256) X(3, 16, 64) X(4, 8, 512) X(5, 64, 64) X(6, 32, 96)
@@ -496,6 +557,29 @@ int ref_tdequant(int shape_id, int src_kind, float* dst, const void* src, const 
     }
     PTO_REF_SHAPES(X)
 #undef X
+    return -1;
+}
+
+// 16 x 64 int8 source; scale / offset [16][para_cols], para_cols 1, 3 or 8
+int ref_tdequant_para(int para_cols, float* dst, const int8_t* src, const float* scale, const float* offset)
+{
+    switch (para_cols) {
+        case 1: return RunDequantPara<1>(dst, src, scale, offset);
+        case 3: return RunDequantPara<3>(dst, src, scale, offset);
+        case 8: return RunDequantPara<8>(dst, src, scale, offset);
+        default: return -1;
+    }
+}
+
+// 16 x 64 f32 source; scale / offset [para_rows], para_rows 1, 5 or 16
+int ref_tquant_int8_para(int para_rows, int asym, uint8_t* dst, const float* src, const float* scale, const float* offset)
+{
+#define P(n)                                                                         \
+    if (para_rows == n)                                                              \
+        return asym ? RunQuantInt8Para<n, true>(dst, src, scale, offset) :           \
+                      RunQuantInt8Para<n, false>(dst, src, scale, offset);
+    P(1) P(5) P(16)
+#undef P
     return -1;
 }
 

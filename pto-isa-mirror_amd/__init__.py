@@ -43,7 +43,8 @@ EXPORTS = [
     "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_requant", "ptoamd_gemm_atomic_add", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
     "ptoamd_gemm_mx_ws",
     "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
-    "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_mx_scale_relayout", "ptoamd_last_kernel",
+    "ptoamd_tquant_int8_para", "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_tdequant_para", "ptoamd_mx_scale_relayout",
+    "ptoamd_last_kernel",
 ]
 
 
@@ -111,11 +112,11 @@ def gemm_atomic_add(out, a, b, ab_type, b_layout=B_DN, stream=None):
 def gemm_requant(a, b, ab_type, c_type, quant_words, per_column=False, b_layout=B_DN, c_in=None, bias=None, relu=False,
                  n=None, stream=None, out=None):
     """TLOAD -> TMATMUL -> TSTORE through the fix-pipe quantiser.  quant_words: int64 / uint64 device tensor holding one
-    word, or one word per column; c_type: I8, U8 or F16."""
+    word, or one word per column; c_type: I8, U8, F16, BF16 or (int8 operands) I16."""
     m, k = a.shape
     n = (b.shape[0] if b_layout == B_DN else b.shape[1]) if n is None else n
     if out is None:
-        out = torch.empty((m, n), dtype={I8: torch.int8, U8: torch.uint8, F16: torch.float16}[c_type], device=a.device)
+        out = torch.empty((m, n), dtype={I8: torch.int8, U8: torch.uint8, F16: torch.float16, BF16: torch.bfloat16, I16: torch.int16}[c_type], device=a.device)
     _check(_lib.ptoamd_gemm_requant(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), _ptr(bias), _ptr(quant_words),
                                     int(per_column), m, n, k, a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu),
                                     _stream(stream)), "ptoamd_gemm_requant")
@@ -190,9 +191,15 @@ def gemv_mxfp4(a_bf16, w, sw, n, k, c_type=F32, stream=None, out=None):
 
 
 def tquant_int8(src, scale, offset=None, stream=None, out=None):
+    """scale / offset: one value per row (1-D), or a 2-D parameter tile [para_rows][para_ld]: column 0 is read and rows
+    past the tile's last repeat it (the reference's GetParamValue)."""
     rows, cols = src.shape
     if out is None:
         out = torch.empty((rows, cols), dtype=torch.int8 if offset is None else torch.uint8, device=src.device)
+    if scale.dim() == 2:
+        _check(_lib.ptoamd_tquant_int8_para(_ptr(out), _ptr(src), _ptr(scale), _ptr(offset), rows, cols, scale.shape[0],
+                                            scale.stride(0), _stream(stream)), "ptoamd_tquant_int8_para")
+        return out
     _check(_lib.ptoamd_tquant_int8(_ptr(out), _ptr(src), _ptr(scale), _ptr(offset), rows, cols, _stream(stream)),
            "ptoamd_tquant_int8")
     return out
@@ -222,9 +229,15 @@ _INT_TYPE = {torch.int8: I8, torch.int16: I16, torch.int32: I32}
 
 
 def tdequant(src, scale, offset, stream=None, out=None):
+    """scale / offset: one value per row (1-D), or a 2-D parameter tile [rows][para_cols]: element (r, c) reads parameter
+    column min(c, para_cols - 1)."""
     rows, cols = src.shape
     if out is None:
         out = torch.empty((rows, cols), dtype=torch.float32, device=src.device)
+    if scale.dim() == 2:
+        _check(_lib.ptoamd_tdequant_para(_ptr(out), _ptr(src), _INT_TYPE[src.dtype], _ptr(scale), _ptr(offset), rows, cols,
+                                         scale.shape[1], scale.stride(0), _stream(stream)), "ptoamd_tdequant_para")
+        return out
     _check(_lib.ptoamd_tdequant(_ptr(out), _ptr(src), _INT_TYPE[src.dtype], _ptr(scale), _ptr(offset), rows, cols,
                                 _stream(stream)), "ptoamd_tdequant")
     return out

@@ -131,6 +131,13 @@ template <bool SRC_INT>
 __device__ __forceinline__ void store_quant(const GenericParams& p, long o, float acc, int gj)
 {
     const uint64_t w = p.qwords[p.q_per_column ? gj : 0];
+    if (p.out_kind == OUT_QBF16) {
+        float r = __fmul_rn(acc, p.q_per_column ? fixpipe_word_scale<true>(w) : fixpipe_word_scale<false>(w));
+        if (p.relu)
+            r = r > 0 ? r : 0;
+        reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(r);
+        return;
+    }
     const bool byte = p.out_kind == OUT_Q8;
     float r;
     if (byte)
@@ -147,7 +154,7 @@ __device__ __forceinline__ void store_quant(const GenericParams& p, long o, floa
 
 __device__ __forceinline__ void store_out(const GenericParams& p, long o, float v, int gi, int gj)
 {
-    if (p.out_kind == OUT_Q8 || p.out_kind == OUT_QF16) {
+    if (p.out_kind == OUT_Q8 || p.out_kind == OUT_QF16 || p.out_kind == OUT_QBF16) {
         store_quant<false>(p, o, v, gj);
         return;
     }
@@ -183,7 +190,14 @@ __global__ void gemm_generic_kernel(const GenericParams p)
         if (p.bias)
             acc += (uint32_t) reinterpret_cast<const int32_t*>(p.bias)[gj];
         int32_t v = (int32_t)acc;
-        if (p.out_kind == OUT_Q8 || p.out_kind == OUT_QF16) {
+        if (p.out_kind == OUT_QS16) {
+            int32_t r = fixpipe_shift_s16(v, p.qwords[p.q_per_column ? gj : 0]);
+            if (p.relu)
+                r = r > 0 ? r : 0;
+            reinterpret_cast<int16_t*>(p.c)[o] = (int16_t)r;
+            return;
+        }
+        if (p.out_kind == OUT_Q8 || p.out_kind == OUT_QF16 || p.out_kind == OUT_QBF16) {
             store_quant<true>(p, o, (float)v, gj);
             return;
         }
@@ -294,7 +308,7 @@ static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStr
         while (whole > 0 && ((long)tiles_m * whole) % 256 != 0)
             --whole;
         const long tail_tiles = (long)tiles_m * (tiles_n - whole);
-        if (whole > 0 && whole < tiles_n && tail_tiles <= 160) {
+        if (whole > 0 && whole < tiles_n && tail_tiles <= 100) {
             const int n1 = whole * 256;
             TileGemmParams head = p;
             head.n = n1;
@@ -446,8 +460,8 @@ int ptoamd_gemm_requant(void* c, int c_type, const void* a, const void* b, int a
                         int b_layout, int relu, void* stream_)
 {
     PTOAMD_REQUIRE(quant_words != nullptr, PTOAMD_E_INVALID, "ptoamd_gemm_requant: null quantisation words");
-    PTOAMD_REQUIRE(c_type == PTOAMD_I8 || c_type == PTOAMD_U8 || c_type == PTOAMD_F16, PTOAMD_E_UNSUPPORTED,
-                   "ptoamd_gemm_requant: the fix-pipe quantiser stores s8, u8 or f16 (got type %d)", c_type);
+    PTOAMD_REQUIRE(c_type == PTOAMD_I8 || c_type == PTOAMD_U8 || c_type == PTOAMD_F16 || c_type == PTOAMD_BF16 || c_type == PTOAMD_I16,
+                   PTOAMD_E_UNSUPPORTED, "ptoamd_gemm_requant: the fix-pipe quantiser stores s8, u8, f16, bf16 or s16 (got type %d)", c_type);
     PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(quant_words) & 7u) == 0, PTOAMD_E_ALIGNMENT,
                    "ptoamd_gemm_requant: quantisation words must be 8-byte aligned");
     return gemm_common(c, c_type, a, b, ab_type, c_in, bias, quant_words, per_column ? 1 : 0, m, n, k, lda, ldb, ldc, b_layout,
@@ -485,7 +499,9 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
                    "ptoamd_gemm: operand type %d is not a TMATMUL input type (s8, f16, bf16, f32, e4m3, e5m2)", ab_type);
     int out_kind;
     if (qwords != nullptr) {
-        out_kind = c_type == PTOAMD_F16 ? OUT_QF16 : OUT_Q8;
+        PTOAMD_REQUIRE(c_type != PTOAMD_I16 || is_int, PTOAMD_E_UNSUPPORTED,
+                       "ptoamd_gemm_requant: the int16 shift mode takes int32 accumulators (int8 operands)");
+        out_kind = c_type == PTOAMD_F16 ? OUT_QF16 : (c_type == PTOAMD_BF16 ? OUT_QBF16 : (c_type == PTOAMD_I16 ? OUT_QS16 : OUT_Q8));
     } else if (is_int) {
         PTOAMD_REQUIRE(c_type == PTOAMD_I32, PTOAMD_E_UNSUPPORTED, "ptoamd_gemm: int8 operands accumulate to int32 only");
         out_kind = OUT_I32;

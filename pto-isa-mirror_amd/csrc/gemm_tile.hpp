@@ -56,8 +56,10 @@ __device__ __forceinline__ long mx_scale_base(int mode, int x, int scale_ld)
 }
 __device__ __forceinline__ long mx_pair_stride(int mode, int rows) { return mode == 0 ? 2 : (mode == 1 ? 32 : 2L * rows); }
 
-// OUT_Q8: one byte per element, signed or unsigned as the quantisation word says; OUT_QF16: half through the same words
-enum OutKind { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2, OUT_I32 = 3, OUT_W8A8_BF16 = 4, OUT_Q8 = 5, OUT_QF16 = 6 };
+// OUT_Q8: one byte per element, signed or unsigned as the quantisation word says; OUT_QF16 / OUT_QBF16: half / bfloat16
+// through the same words; OUT_QS16: int32 accumulators shifted right into int16 (the word's shift field)
+enum OutKind { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2, OUT_I32 = 3, OUT_W8A8_BF16 = 4, OUT_Q8 = 5, OUT_QF16 = 6, OUT_QBF16 = 7,
+               OUT_QS16 = 8 };
 
 // ---- MFMA operand traits ------------------------------------------------------------------------------------
 // Every mma() hands the matrix instruction B's fragment as its first operand and A's as its second, so a 32x32
@@ -269,12 +271,24 @@ __device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_
             r = r > 0 ? r : 0;
         return byte ? ((uint32_t)(int32_t)r & 0xFFu) : (uint32_t)f32_to_f16_bits(r);
     }
+    if (KIND == OUT_QBF16) {
+        float r = __fmul_rn((float)v, q_vector ? fixpipe_word_scale<true>(qw) : fixpipe_word_scale<false>(qw));
+        if (relu)
+            r = r > 0 ? r : 0;
+        return f32_to_bf16_bits(r);
+    }
+    if (KIND == OUT_QS16) {
+        int32_t r = fixpipe_shift_s16((int32_t)v, qw);
+        if (relu)
+            r = r > 0 ? r : 0;
+        return (uint32_t)r & 0xFFFFu;
+    }
     return f32_to_bf16_bits(__fmul_rn(__fmul_rn((float)v, rs), cs));
 }
 template <int KIND>
 constexpr int out_bytes = (KIND == OUT_F32 || KIND == OUT_I32) ? 4 : (KIND == OUT_Q8 ? 1 : 2);
 template <int KIND>
-constexpr bool out_quant = KIND == OUT_Q8 || KIND == OUT_QF16;
+constexpr bool out_quant = KIND == OUT_Q8 || KIND == OUT_QF16 || KIND == OUT_QBF16 || KIND == OUT_QS16;
 
 // Element-wise form: any alignment, any edge.  A lane's elements are 4-column runs of one row, so this form is slow
 // (short scattered stores); whole, aligned wave tiles take the staged form below.
@@ -318,8 +332,12 @@ __device__ __forceinline__ void tstore_block_kind(const TileGemmParams& p, const
         tstore_block<OUT_Q8, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
     } else if (p.out_kind == OUT_QF16) {
         tstore_block<OUT_QF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
+    } else if (p.out_kind == OUT_QBF16) {
+        tstore_block<OUT_QBF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
     } else if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
-        if (p.out_kind == OUT_I32)
+        if (p.out_kind == OUT_QS16)
+            tstore_block<OUT_QS16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
+        else if (p.out_kind == OUT_I32)
             tstore_block<OUT_I32, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
         else
             tstore_block<OUT_W8A8_BF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
@@ -418,8 +436,12 @@ __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::
             tstore_staged<OUT_QF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
         } else if (p.out_kind == OUT_Q8) {
             tstore_staged<OUT_Q8, Cfg>(p, acc, row0, col0, l32, lhi, stage);
+        } else if (p.out_kind == OUT_QBF16) {
+            tstore_staged<OUT_QBF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
         } else if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
-            if (p.out_kind == OUT_I32)
+            if (p.out_kind == OUT_QS16)
+                tstore_staged<OUT_QS16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
+            else if (p.out_kind == OUT_I32)
                 tstore_staged<OUT_I32, Cfg>(p, acc, row0, col0, l32, lhi, stage);
             else
                 tstore_staged<OUT_W8A8_BF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);

@@ -143,7 +143,7 @@ __global__ void tquant_mx_cols_kernel(uint8_t* dst, uint8_t* exp, float* mx, flo
 // ---- TQUANT INT8 (TQuant.hpp:86-96, 496-522): the "scale" operand multiplies -----------------------------------
 template <bool ASYM>
 __global__ void tquant_int8_kernel(uint8_t* dst, const float* src, const float* scale, const float* offset, int rows,
-                                   int cols)
+                                   int cols, int para_rows, int para_ld)
 {
     const long idx4 = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     const long total = (long)rows * cols;
@@ -155,10 +155,11 @@ __global__ void tquant_int8_kernel(uint8_t* dst, const float* src, const float* 
         const long idx = idx4 + i;
         if (idx >= total)
             break;
-        const int r = (int)(idx / cols);
-        float v = __fmul_rn(src[idx], scale[r]);
+        // GetParamValue (TQuant.hpp:78-84): column 0 of the parameter tile, the row clamped to its last valid one
+        const long pr = (long)min((int)(idx / cols), para_rows - 1) * para_ld;
+        float v = __fmul_rn(src[idx], scale[pr]);
         if (ASYM)
-            v = __fadd_rn(v, offset[r]);
+            v = __fadd_rn(v, offset[pr]);
         v = rintf(v);
         const float lo = ASYM ? 0.0f : -128.0f, hi = ASYM ? 255.0f : 127.0f;
         v = v < lo ? lo : (v > hi ? hi : v);
@@ -231,13 +232,15 @@ __global__ void __launch_bounds__(256) tdequant_rows_kernel(float* dst, const T*
 
 // ---- TDEQUANT (TDeQuant.hpp:18-37) ---------------------------------------------------------------------------
 template <typename T>
-__global__ void tdequant_kernel(float* dst, const T* src, const float* scale, const float* offset, int rows, int cols)
+__global__ void tdequant_kernel(float* dst, const T* src, const float* scale, const float* offset, int rows, int cols,
+                                int para_cols, int para_ld)
 {
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (long)rows * cols)
         return;
-    const int r = (int)(idx / cols);
-    dst[idx] = __fmul_rn(__fsub_rn((float)src[idx], offset[r]), scale[r]);
+    const int r = (int)(idx / cols), c = (int)(idx - (long)r * cols);
+    const long pi = (long)r * para_ld + min(c, para_cols - 1);  // TDeQuant.hpp:24-30: the parameter column is clamped
+    dst[idx] = __fmul_rn(__fsub_rn((float)src[idx], offset[pi]), scale[pi]);
 }
 
 template <int ALG, typename T, bool SRC_BF16>
@@ -279,13 +282,21 @@ extern "C" {
 int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const float* offset, int rows, int cols,
                        void* stream)
 {
+    return ptoamd_tquant_int8_para(dst, src, scale, offset, rows, cols, rows, 1, stream);
+}
+
+int ptoamd_tquant_int8_para(void* dst, const float* src, const float* scale, const float* offset, int rows, int cols,
+                            int para_rows, int para_ld, void* stream)
+{
     TraceScope trace(offset ? "TQUANT_INT8_ASYM" : "TQUANT_INT8_SYM", "vector", rows, cols, 0);
-    trace.in(src, rows, cols, "ND", PTOAMD_F32).in(scale, rows, 1, "ND", PTOAMD_F32).in(offset, rows, 1, "ND", PTOAMD_F32)
+    trace.in(src, rows, cols, "ND", PTOAMD_F32).in(scale, para_rows, 1, "ND", PTOAMD_F32).in(offset, para_rows, 1, "ND", PTOAMD_F32)
         .out(dst, rows, cols, "ND", offset ? PTOAMD_U8 : PTOAMD_I8);
     PTOAMD_REQUIRE(dst && src && scale, PTOAMD_E_INVALID, "ptoamd_tquant_int8: null operand");
     PTOAMD_REQUIRE(rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_tquant_int8: rows and cols must be positive");
+    PTOAMD_REQUIRE(para_rows > 0 && para_ld > 0, PTOAMD_E_INVALID,
+                   "ptoamd_tquant_int8: the parameter tile needs at least one row and a positive row pitch");
     const long total = (long)rows * cols;
-    if ((cols & 3) == 0 && rows <= 65535 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0 && (reinterpret_cast<uintptr_t>(dst) & 3u) == 0) {
+    if (para_rows >= rows && para_ld == 1 && (cols & 3) == 0 && rows <= 65535 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0 && (reinterpret_cast<uintptr_t>(dst) & 3u) == 0) {
         const dim3 grid((unsigned)((cols / 4 + 511) / 512), (unsigned)rows);
         if (offset)
             hipLaunchKernelGGL(tquant_int8_rows_kernel<true>, grid, dim3(256), 0, as_stream(stream),
@@ -300,10 +311,10 @@ int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const fl
     const unsigned blocks = (unsigned)((total / 4 + 256) / 256);
     if (offset)
         hipLaunchKernelGGL(tquant_int8_kernel<true>, dim3(blocks), dim3(256), 0, as_stream(stream),
-                           reinterpret_cast<uint8_t*>(dst), src, scale, offset, rows, cols);
+                           reinterpret_cast<uint8_t*>(dst), src, scale, offset, rows, cols, para_rows, para_ld);
     else
         hipLaunchKernelGGL(tquant_int8_kernel<false>, dim3(blocks), dim3(256), 0, as_stream(stream),
-                           reinterpret_cast<uint8_t*>(dst), src, scale, offset, rows, cols);
+                           reinterpret_cast<uint8_t*>(dst), src, scale, offset, rows, cols, para_rows, para_ld);
     PTOAMD_HIP_CHECK(hipGetLastError());
     set_last_kernel("tquant_int8");
     return PTOAMD_OK;
@@ -341,15 +352,23 @@ int ptoamd_tquant_mx(uint8_t* dst, uint8_t* exp, float* max, float* scaling, con
 int ptoamd_tdequant(float* dst, const void* src, int src_type, const float* scale, const float* offset, int rows,
                     int cols, void* stream)
 {
+    return ptoamd_tdequant_para(dst, src, src_type, scale, offset, rows, cols, 1, 1, stream);
+}
+
+int ptoamd_tdequant_para(float* dst, const void* src, int src_type, const float* scale, const float* offset, int rows,
+                         int cols, int para_cols, int para_ld, void* stream)
+{
     TraceScope trace("TDEQUANT", "vector", rows, cols, 0);
-    trace.in(src, rows, cols, "ND", src_type).in(scale, rows, 1, "ND", PTOAMD_F32).in(offset, rows, 1, "ND", PTOAMD_F32)
+    trace.in(src, rows, cols, "ND", src_type).in(scale, rows, para_cols, "ND", PTOAMD_F32).in(offset, rows, para_cols, "ND", PTOAMD_F32)
         .out(dst, rows, cols, "ND", PTOAMD_F32);
     PTOAMD_REQUIRE(dst && src && scale && offset, PTOAMD_E_INVALID, "ptoamd_tdequant: null operand");
     PTOAMD_REQUIRE(rows > 0 && cols > 0, PTOAMD_E_INVALID, "ptoamd_tdequant: rows and cols must be positive");
+    PTOAMD_REQUIRE(para_cols > 0 && para_ld >= para_cols, PTOAMD_E_INVALID,
+                   "ptoamd_tdequant: the parameter tile needs at least one column and a row pitch that holds its columns");
     const long total = (long)rows * cols;
     const dim3 grid((unsigned)((total + 255) / 256)), block(256);
     hipStream_t s = as_stream(stream);
-    if ((cols & 3) == 0 && rows <= 65535 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+    if (para_cols == 1 && para_ld == 1 && (cols & 3) == 0 && rows <= 65535 && (reinterpret_cast<uintptr_t>(src) & 15u) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
         const dim3 rgrid((unsigned)((cols / 4 + 511) / 512), (unsigned)rows);
         switch (src_type) {
             case PTOAMD_I8:
@@ -369,13 +388,13 @@ int ptoamd_tdequant(float* dst, const void* src, int src_type, const float* scal
     }
     switch (src_type) {
         case PTOAMD_I8:
-            hipLaunchKernelGGL(tdequant_kernel<int8_t>, grid, block, 0, s, dst, reinterpret_cast<const int8_t*>(src), scale, offset, rows, cols);
+            hipLaunchKernelGGL(tdequant_kernel<int8_t>, grid, block, 0, s, dst, reinterpret_cast<const int8_t*>(src), scale, offset, rows, cols, para_cols, para_ld);
             break;
         case PTOAMD_I16:
-            hipLaunchKernelGGL(tdequant_kernel<int16_t>, grid, block, 0, s, dst, reinterpret_cast<const int16_t*>(src), scale, offset, rows, cols);
+            hipLaunchKernelGGL(tdequant_kernel<int16_t>, grid, block, 0, s, dst, reinterpret_cast<const int16_t*>(src), scale, offset, rows, cols, para_cols, para_ld);
             break;
         case PTOAMD_I32:
-            hipLaunchKernelGGL(tdequant_kernel<int32_t>, grid, block, 0, s, dst, reinterpret_cast<const int32_t*>(src), scale, offset, rows, cols);
+            hipLaunchKernelGGL(tdequant_kernel<int32_t>, grid, block, 0, s, dst, reinterpret_cast<const int32_t*>(src), scale, offset, rows, cols, para_cols, para_ld);
             break;
         default: set_error("ptoamd_tdequant: source type %d is not int8, int16 or int32", src_type); return PTOAMD_E_UNSUPPORTED;
     }

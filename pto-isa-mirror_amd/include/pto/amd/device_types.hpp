@@ -89,6 +89,13 @@ __device__ __forceinline__ float fixpipe_quantize(float acc, uint64_t word)
     return r;
 }
 
+// the int16 shift mode of the fix-pipe (cpu/common.hpp:174-180): arithmetic shift right by bits 32..35 of the word plus
+// one; the reference narrows to int16 before it clamps, so the value wraps
+__device__ __forceinline__ int32_t fixpipe_shift_s16(int32_t acc, uint64_t word)
+{
+    return (int32_t)(int16_t)(acc >> ((int)((word >> 32) & 0xFu) + 1));
+}
+
 __device__ __forceinline__ float e4m3_to_f32(uint32_t c)
 {
     const uint32_t mag = c & 0x7Fu;

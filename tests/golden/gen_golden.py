@@ -178,6 +178,30 @@ def main():
     e = r.integers(0, 256, (48, 6)).astype(np.uint8)
     g["zz_exp"], g["zz_reordered"] = e, ref.reorder_exp_zz(e)
 
+    # --- parameter tiles wider / shorter than the data tile; the int16 shift mode of the requantising store ---
+    src8 = r.integers(-128, 128, (16, 64)).astype(np.int8)
+    g["dqp_src"] = src8
+    for pc in (1, 3, 8):
+        sc = r.uniform(0.25, 2.0, (16, pc)).astype(np.float32)
+        of = r.uniform(-20, 20, (16, pc)).astype(np.float32)
+        g[f"dqp_scale_{pc}"], g[f"dqp_off_{pc}"] = sc, of
+        g[f"dqp_out_{pc}"] = ref.tdequant_para(src8, sc, of)
+    srcf = (r.standard_normal((16, 64)) * 40).astype(np.float32)
+    g["q8p_src"] = srcf
+    for pr in (1, 5, 16):
+        sc = r.uniform(0.5, 4.0, pr).astype(np.float32)
+        of = r.uniform(0, 200, pr).astype(np.float32)
+        g[f"q8p_scale_{pr}"], g[f"q8p_off_{pr}"] = sc, of
+        g[f"q8p_sym_{pr}"] = ref.tquant_int8_para(srcf, sc)
+        g[f"q8p_asym_{pr}"] = ref.tquant_int8_para(srcf, sc, of)
+    acc = r.integers(-2 ** 31, 2 ** 31, (24, 40)).astype(np.int32)
+    acc[0, :8] = [0, 1, -1, 65535, 65536, -65536, 2 ** 31 - 1, -2 ** 31]
+    wsh = (r.integers(0, 16, 40).astype(np.uint64) << np.uint64(32)) | r.integers(0, 2 ** 32, 40).astype(np.uint64)
+    g["s16_acc"], g["s16_words"] = acc, wsh
+    for per_col in (0, 1):
+        for relu in (0, 1):
+            g[f"s16_out_{per_col}_{relu}"] = ref.store_quant(acc, "i16", wsh, per_col, relu=bool(relu))
+
     out = os.path.join(ROOT, "tests", "golden", "pto_golden.npz")
     np.savez_compressed(out, **g)
     print(f"wrote {out}: {len(g)} arrays, {os.path.getsize(out)} bytes")

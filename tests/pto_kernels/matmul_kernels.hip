@@ -535,6 +535,8 @@ extern "C" int pto_kernels_launch_quant(int id, void* dst, void* exp, void* max,
 
 // store-quant cases: 1: f16 -> f32 acc -> int8, scalar word     2: f16 -> f32 acc -> uint8, per-column words, relu
 //                    3: int8 -> i32 acc -> f16 (dequant), per-column words     4: int8 -> i32 acc -> int8 (requant), scalar
+//                    5: f16 -> f32 acc -> bf16, scalar word     6: int8 -> i32 acc -> bf16, per-column words, relu
+//                    7: int8 -> i32 acc -> int16 (shift mode), scalar word     8: the same, per-column words, relu
 extern "C" int pto_kernels_launch_store_quant(int id, void* out, void* a, void* b, void* words, void* stream)
 {
     switch (id) {
@@ -542,6 +544,10 @@ extern "C" int pto_kernels_launch_store_quant(int id, void* out, void* a, void* 
     case 2: return run<&RunTMATMUL_QUANT<uint8_t, float, half, 33, 64, 70, true, true>>(stream, 1, (uint8_t*)out, (half*)a, (half*)b, (uint64_t*)words);
     case 3: return run<&RunTMATMUL_QUANT<half, int32_t, int8_t, 24, 96, 40, true, false>>(stream, 1, (half*)out, (int8_t*)a, (int8_t*)b, (uint64_t*)words);
     case 4: return run<&RunTMATMUL_QUANT<int8_t, int32_t, int8_t, 24, 96, 40, false, false>>(stream, 1, (int8_t*)out, (int8_t*)a, (int8_t*)b, (uint64_t*)words);
+    case 5: return run<&RunTMATMUL_QUANT<bfloat16_t, float, half, 40, 50, 60, false, false>>(stream, 1, (bfloat16_t*)out, (half*)a, (half*)b, (uint64_t*)words);
+    case 6: return run<&RunTMATMUL_QUANT<bfloat16_t, int32_t, int8_t, 24, 96, 40, true, true>>(stream, 1, (bfloat16_t*)out, (int8_t*)a, (int8_t*)b, (uint64_t*)words);
+    case 7: return run<&RunTMATMUL_QUANT<int16_t, int32_t, int8_t, 24, 96, 40, false, false>>(stream, 1, (int16_t*)out, (int8_t*)a, (int8_t*)b, (uint64_t*)words);
+    case 8: return run<&RunTMATMUL_QUANT<int16_t, int32_t, int8_t, 24, 96, 40, true, true>>(stream, 1, (int16_t*)out, (int8_t*)a, (int8_t*)b, (uint64_t*)words);
     default: return -1;
     }
 }

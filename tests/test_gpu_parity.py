@@ -397,10 +397,18 @@ def test_requant_drain_float_accumulator(pa, oracle, tile, m, n, k):
         assert np.array_equal(got.view(np.uint16), oracle.store_quant(acc, ob.ST_F16, vector, per_column=True))
         got = host(pa.gemm_requant(da, db, pa.F16, pa.I8, dev(scalar.view(np.int64)), bias=dev(bias)))
         assert np.array_equal(got, oracle.store_quant(acc + bias, ob.ST_I8, scalar, per_column=False))
+        # bfloat16 target (QF322BF16_PRE / VQF322BF16_PRE)
+        got = pa.gemm_requant(da, db, pa.F16, pa.BF16, dev(vector.view(np.int64)), per_column=True, relu=True)
+        assert np.array_equal(host(got.view(torch.int16)).view(np.uint16),
+                              oracle.store_quant(acc, ob.ST_BF16, vector, per_column=True, relu=True))
+        got = pa.gemm_requant(da, db, pa.F16, pa.BF16, dev(scalar.view(np.int64)))
+        assert np.array_equal(host(got.view(torch.int16)).view(np.uint16), oracle.store_quant(acc, ob.ST_BF16, scalar, per_column=False))
     with tile_env(PTOAMD_FORCE_GENERIC=1):
         got = host(pa.gemm_requant(da, db, pa.F16, pa.I8, dev(vector.view(np.int64)), per_column=True, relu=True))
         assert pa.last_kernel() == "generic"
         assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I8, vector, per_column=True, relu=True))
+        got = pa.gemm_requant(da, db, pa.F16, pa.BF16, dev(vector.view(np.int64)), per_column=True)
+        assert np.array_equal(host(got.view(torch.int16)).view(np.uint16), oracle.store_quant(acc, ob.ST_BF16, vector, per_column=True))
 
 
 @pytest.mark.parametrize("tile", [None, 2, 4, 5])
@@ -423,6 +431,20 @@ def test_requant_drain_int32_accumulator(pa, oracle, tile, m, n, k):
         assert np.array_equal(got.view(np.uint16), oracle.store_quant(acc, ob.ST_F16, vector, per_column=True))
         got = host(pa.gemm_requant(da, db, pa.I8, pa.I8, dev(vector.view(np.int64)), per_column=True, relu=True))
         assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I8, vector, per_column=True, relu=True))
+        # bfloat16 target (QS322BF16_PRE) and the int16 shift mode (SHIFTS322S16 / VSHIFTS322S16: the shift count sits in
+        # bits 32..35 of the word; the other bits are noise here and must not matter)
+        got = pa.gemm_requant(da, db, pa.I8, pa.BF16, dev(vector.view(np.int64)), per_column=True)
+        assert np.array_equal(host(got.view(torch.int16)).view(np.uint16), oracle.store_quant(acc, ob.ST_BF16, vector, per_column=True))
+        shifts = (r.integers(0, 16, n).astype(np.uint64) << np.uint64(32)) | r.integers(0, 2 ** 32, n).astype(np.uint64)
+        got = host(pa.gemm_requant(da, db, pa.I8, pa.I16, dev(shifts.view(np.int64)), per_column=True))
+        want = oracle.store_quant(acc, ob.ST_I16, shifts, per_column=True)
+        assert np.array_equal(got, want) and len(np.unique(want)) > 16
+        got = host(pa.gemm_requant(da, db, pa.I8, pa.I16, dev(shifts[3:4].view(np.int64).copy()), relu=True))
+        assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I16, shifts[3:4], per_column=False, relu=True))
+    with tile_env(PTOAMD_FORCE_GENERIC=1):
+        got = host(pa.gemm_requant(da, db, pa.I8, pa.I16, dev(shifts.view(np.int64)), per_column=True, relu=True))
+        assert pa.last_kernel() == "generic"
+        assert np.array_equal(got, oracle.store_quant(acc, ob.ST_I16, shifts, per_column=True, relu=True))
 
 
 @pytest.mark.parametrize("tile", [None, 2, 5])
@@ -460,6 +482,37 @@ def test_requant_rejects_other_output_types(pa):
     w = torch.zeros(1, dtype=torch.int64, device=DEV)
     with pytest.raises(pa.PtoAmdError, match="fix-pipe quantiser"):
         pa.gemm_requant(a, a, pa.F16, pa.F32, w, out=torch.zeros((16, 16), dtype=torch.float32, device=DEV))
+    with pytest.raises(pa.PtoAmdError, match="int16 shift mode"):
+        pa.gemm_requant(a, a, pa.F16, pa.I16, w)
+
+
+def test_parameter_tiles_wider_and_shorter_than_the_data(pa, oracle, golden):
+    """TDEQUANT clamps the parameter column to the parameter tile's valid columns, TQUANT INT8 reads column 0 and
+    clamps the row (vectors frozen from the compiled reference), then larger shapes against the oracle."""
+    src8 = golden["dqp_src"]
+    for pc in (1, 3, 8):
+        sc, of = golden[f"dqp_scale_{pc}"], golden[f"dqp_off_{pc}"]
+        got = host(pa.tdequant(dev(src8), dev(sc), dev(of)))
+        assert np.array_equal(got.view(np.uint32), golden[f"dqp_out_{pc}"].view(np.uint32)), pc
+    srcf = golden["q8p_src"]
+    for pr in (1, 5, 16):
+        sc, of = golden[f"q8p_scale_{pr}"], golden[f"q8p_off_{pr}"]
+        # parameter tiles three columns wide: only column 0 may be read
+        sc3 = np.full((pr, 3), -1000.0, np.float32)
+        of3 = np.full((pr, 3), 999.0, np.float32)
+        sc3[:, 0], of3[:, 0] = sc, of
+        assert np.array_equal(host(pa.tquant_int8(dev(srcf), dev(sc3))), golden[f"q8p_sym_{pr}"]), pr
+        assert np.array_equal(host(pa.tquant_int8(dev(srcf), dev(sc3), dev(of3))), golden[f"q8p_asym_{pr}"]), pr
+    r = np.random.default_rng(5)
+    src = r.integers(-2 ** 15, 2 ** 15, (70, 333)).astype(np.int16)
+    sc = r.uniform(0.1, 2, (70, 5)).astype(np.float32)
+    of = r.uniform(-9, 9, (70, 5)).astype(np.float32)
+    got = host(pa.tdequant(dev(src), dev(sc), dev(of)))
+    assert np.array_equal(got.view(np.uint32), oracle.tdequant_para(src, sc, of).view(np.uint32))
+    srcf = (r.standard_normal((70, 333)) * 30).astype(np.float32)
+    scq = r.uniform(0.5, 3, (9, 2)).astype(np.float32)
+    got = host(pa.tquant_int8(dev(srcf), dev(scq)))
+    assert np.array_equal(got, oracle.tquant_int8_para(srcf, scq.ravel(), para_ld=2))
 
 
 def test_mx_gemm_with_bias(pa, oracle):

@@ -419,6 +419,58 @@ def test_tdequant_closed_form(oracle):
     assert np.array_equal(bits(want), bits(oracle.tdequant(q, scale, off)))
 
 
+def test_parameter_tile_fixtures(oracle, golden):
+    """Parameter tiles as the reference reads them: TDEQUANT clamps the column, TQUANT INT8 reads column 0 and clamps
+    the row (vectors from the compiled reference); plus the numpy closed form, which a swapped clamp would fail."""
+    g = golden
+    for pc in (1, 3, 8):
+        got = oracle.tdequant_para(g["dqp_src"], g[f"dqp_scale_{pc}"], g[f"dqp_off_{pc}"])
+        assert np.array_equal(bits(got), bits(g[f"dqp_out_{pc}"])), pc
+        col = np.minimum(np.arange(64), pc - 1)
+        want = (g["dqp_src"].astype(np.float32) - g[f"dqp_off_{pc}"][:, col]) * g[f"dqp_scale_{pc}"][:, col]
+        assert np.array_equal(bits(got), bits(want))
+    for pr in (1, 5, 16):
+        sc, of = g[f"q8p_scale_{pr}"], g[f"q8p_off_{pr}"]
+        assert np.array_equal(oracle.tquant_int8_para(g["q8p_src"], sc), g[f"q8p_sym_{pr}"]), pr
+        assert np.array_equal(oracle.tquant_int8_para(g["q8p_src"], sc, of), g[f"q8p_asym_{pr}"]), pr
+        row = np.minimum(np.arange(16), pr - 1)
+        want = np.clip(np.rint(g["q8p_src"] * sc[row][:, None]), -128, 127).astype(np.int8)
+        assert np.array_equal(g[f"q8p_sym_{pr}"], want)
+
+
+def test_store_int16_shift_mode(oracle, golden):
+    """SHIFTS322S16: (int16)(acc >> (bits 32..35 + 1)), narrowed before the clamp (so it wraps), then relu: the
+    compiled reference's outputs and the closed form."""
+    g = golden
+    acc, words = g["s16_acc"], g["s16_words"]
+    for per_col in (0, 1):
+        w = words if per_col else words[:1]
+        shift = ((w >> np.uint64(32)) & np.uint64(15)).astype(np.int64) + 1
+        want = (acc.astype(np.int64) >> (shift[None, :] if per_col else shift[0])).astype(np.int16)
+        for relu in (0, 1):
+            got = oracle.store_quant(acc, ob.ST_I16, w, per_col, relu)
+            assert np.array_equal(got, g[f"s16_out_{per_col}_{relu}"]), (per_col, relu)
+            assert np.array_equal(got, np.maximum(want, 0) if relu else want)
+    assert (g["s16_out_0_0"] < 0).any() and len(np.unique(g["s16_out_1_0"])) > 100
+
+
+def test_store_quant_bf16_target_against_torch(oracle):
+    """QF322BF16_PRE / QS322BF16_PRE: the product acc * scale rounded to bfloat16 (the compiled reference cannot pin
+    this target: its bfloat16_t is a half in this build), checked against float32 multiply + torch's bf16 rounding."""
+    import torch
+    r = np.random.default_rng(12)
+    accf = (r.standard_normal((24, 40)) * 300).astype(np.float32)
+    acci = r.integers(-2 ** 24, 2 ** 24, (24, 40)).astype(np.int32)
+    scales = r.uniform(0.001, 3.0, 40).astype(np.float32)
+    words = np.array([int(s.view(np.uint32)) for s in scales], np.uint64)
+    for acc in (accf, acci):
+        for relu in (False, True):
+            prod = acc.astype(np.float32) * scales[0]
+            prod = np.maximum(prod, 0) if relu else prod
+            want = torch.from_numpy(prod).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+            assert np.array_equal(oracle.store_quant(acc, ob.ST_BF16, words[:1], False, relu), want)
+
+
 # ---------------------------------------------------------------- the CPU-simulator-shaped baseline walk
 def test_sim_tiled_equals_one_shot(oracle):
     r = np.random.default_rng(9)

@@ -210,6 +210,31 @@ def test_store_quant(oracle, reflib, per_col, relu):
                           oracle.store_quant(acci, ob.ST_F16, words, per_col, relu))
 
 
+def test_store_int16_shift_mode(oracle, reflib):
+    r = _rng(23)
+    acc = r.integers(-2 ** 31, 2 ** 31, (24, 40)).astype(np.int32)
+    words = (r.integers(0, 16, 40).astype(np.uint64) << np.uint64(32)) | r.integers(0, 2 ** 32, 40).astype(np.uint64)
+    for per_col in (0, 1):
+        for relu in (False, True):
+            assert np.array_equal(reflib.store_quant(acc, "i16", words, per_col, relu),
+                                  oracle.store_quant(acc, ob.ST_I16, words, per_col, relu))
+
+
+def test_parameter_tiles(oracle, reflib):
+    r = _rng(29)
+    src8 = r.integers(-128, 128, (16, 64)).astype(np.int8)
+    for pc in (1, 3, 8):
+        sc = r.uniform(0.25, 2.0, (16, pc)).astype(np.float32)
+        of = r.uniform(-20, 20, (16, pc)).astype(np.float32)
+        assert np.array_equal(reflib.tdequant_para(src8, sc, of).view(np.uint32), oracle.tdequant_para(src8, sc, of).view(np.uint32))
+    srcf = (r.standard_normal((16, 64)) * 40).astype(np.float32)
+    for pr in (1, 5, 16):
+        sc = r.uniform(0.5, 4.0, pr).astype(np.float32)
+        of = r.uniform(0, 200, pr).astype(np.float32)
+        assert np.array_equal(reflib.tquant_int8_para(srcf, sc), oracle.tquant_int8_para(srcf, sc))
+        assert np.array_equal(reflib.tquant_int8_para(srcf, sc, of), oracle.tquant_int8_para(srcf, sc, of))
+
+
 def test_store_f32_to_f16(oracle, reflib):
     r = _rng(23)
     a = _f16(r.uniform(-4, 4, (40, 64)))
