@@ -647,11 +647,18 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
     const int out_kind = c_type == PTOAMD_F32 ? OUT_F32 : (c_type == PTOAMD_F16 ? OUT_F16 : OUT_BF16);
     const int bits = a8 ? 8 : 4;
     const long k_bytes = (long)k * bits / 8, lda_b = (long)lda * bits / 8, ldb_b = (long)ldb * bits / 8;
-    const bool e1m2 = a_type == PTOAMD_E1M2 || b_type == PTOAMD_E1M2;  // the scaled MFMA has no E1M2 format
+    // The scaled MFMA has no E1M2 operand format, but every E1M2 (and E2M1) value is an E4M3 value: a product with an
+    // E1M2 operand runs on the E4M3 x E4M3 instruction, the register-staged loader expanding both operands' packed
+    // nibbles to E4M3 bytes on their way into LDS (the block scales are per 32 elements in either form).
+    const bool e1m2 = a_type == PTOAMD_E1M2 || b_type == PTOAMD_E1M2;
+    const bool expand_ok = e1m2 && b_layout == PTOAMD_B_DN && (k % 128) == 0 && (reinterpret_cast<uintptr_t>(a) & 7u) == 0 &&
+                           (reinterpret_cast<uintptr_t>(b) & 7u) == 0 && (lda_b % 8) == 0 && (ldb_b % 8) == 0;
     // a row-major B of one-byte codes is transposed on its way into LDS by the register-staged tiles; packed fp4 is not
     const bool b_in_kernel = b_layout == PTOAMD_B_ND && a8 && (n % 16) == 0;
-    const bool tile_ok = !force_generic() && !e1m2 && (b_layout == PTOAMD_B_DN || b_in_kernel) && aligned16(a) && aligned16(b) &&
-                         (lda_b % 16) == 0 && (ldb_b % 16) == 0 && (k_bytes % 128) == 0;
+    const bool tile_ok = !force_generic() &&
+                         (e1m2 ? expand_ok
+                               : ((b_layout == PTOAMD_B_DN || b_in_kernel) && aligned16(a) && aligned16(b) && (lda_b % 16) == 0 &&
+                                  (ldb_b % 16) == 0 && (k_bytes % 128) == 0));
     if (!tile_ok) {
         GenericParams g{};
         g.a = a; g.b = b; g.c = c; g.c_in = c_in; g.sa = sa; g.sb = sb; g.bias = bias;
@@ -706,7 +713,12 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
     p.sa_mode = sa_mode; p.sb_mode = sb_mode;
     p.b_nd = b_in_kernel; p.b_esz = 1;
     int op;
-    if (a4)
+    if (e1m2) {
+        op = TOP_FP8_E4E4;
+        p.k_bytes = k;  // one E4M3 byte per element once expanded; the row pitches stay those of the packed operands
+        p.a_expand = a_type == PTOAMD_E2M1 ? 1 : 2;
+        p.b_expand = b_type == PTOAMD_E2M1 ? 1 : 2;
+    } else if (a4)
         op = TOP_FP4;
     else if (a_type == PTOAMD_E4M3)
         op = b_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E4E5;
@@ -716,7 +728,8 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
     const long k_slabs = k_bytes / 128;
     const bool scale_dma_ok = plain_scales && !b_in_kernel && (kg % 16) == 0 && aligned16(sa_nd) && aligned16(sb_dn) &&
                               (k_slabs % (a4 ? 2 : 4)) == 0;
-    const int tile = pick_tile(m, n, k_bytes, true, a4, scale_dma_ok && dma_offsets_fit(m, n, lda_b, ldb_b, k_bytes));
+    const int tile = e1m2 ? pick_tile(m, n, k, true, false, false)
+                          : pick_tile(m, n, k_bytes, true, a4, scale_dma_ok && dma_offsets_fit(m, n, lda_b, ldb_b, k_bytes));
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;

@@ -48,6 +48,11 @@ struct TileGemmParams {
     const uint64_t* qwords;
     int q_per_column;
     int atomic_add;         // OUT_F32 / OUT_I32 only: C += result with atomic adds (TSTORE<AtomicAdd>)
+    // register-staged E4M3 x E4M3 tiles only: the operand arrives as packed fp4 codes (two per byte, even k in the low
+    // nibble; lda_bytes / ldb_bytes are the packed row pitches, k_bytes counts elements) and the loader expands every
+    // code to the E4M3 byte of the same value: 0 = no, 1 = E2M1, 2 = E1M2.  Every value of either fp4 format is an E4M3
+    // value, and the scaled MFMA has no E1M2 operand format.
+    int a_expand, b_expand;
 };
 
 __device__ __forceinline__ long mx_scale_base(int mode, int x, int scale_ld)
@@ -149,6 +154,27 @@ struct OpFP8 {
         c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, BFMT, AFMT, SEL, (int)sb, SEL, (int)sa);
     }
 };
+// 16 packed fp4 codes (8 bytes, even k in the low nibble) -> the 16 E4M3 bytes of the same values.  mode 1: E2M1
+// (0, 0.5, 1, 1.5, 2, 3, 4, 6), mode 2: E1M2 (0, 0.25, ... 1.75); bit 3 of a code is the sign.
+__device__ __forceinline__ uint4 expand_fp4_to_e4m3(uint2 x, int mode)
+{
+    const uint32_t lut_lo = mode == 1 ? 0x3C383000u : 0x34302800u;  // codes 0..3
+    const uint32_t lut_hi = mode == 1 ? 0x4C484440u : 0x3E3C3A38u;  // codes 4..7
+    uint32_t out[4];
+    const uint32_t w[2] = {x.x, x.y};
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+        const uint32_t lo_n = w[d] & 0x0F0F0F0Fu, hi_n = (w[d] >> 4) & 0x0F0F0F0Fu;  // elements 0, 2, 4, 6 / 1, 3, 5, 7
+        const uint32_t lo_e = __builtin_amdgcn_perm(lut_hi, lut_lo, lo_n & 0x07070707u) | ((lo_n & 0x08080808u) << 4);
+        const uint32_t hi_e = __builtin_amdgcn_perm(lut_hi, lut_lo, hi_n & 0x07070707u) | ((hi_n & 0x08080808u) << 4);
+        out[2 * d] = __builtin_amdgcn_perm(hi_e, lo_e, 0x05010400u);
+        out[2 * d + 1] = __builtin_amdgcn_perm(hi_e, lo_e, 0x07030602u);
+    }
+    return make_uint4(out[0], out[1], out[2], out[3]);
+}
+template <class Op>
+constexpr bool expands_fp4 = std::is_same<Op, OpFP8<0, 0>>::value;
+
 // fp4 E2M1 (format 4): 32 elements = 16 bytes per lane = one MX group
 struct OpFP4 {
     using Acc = f32x16;
@@ -498,10 +524,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
     const uint8_t* ga[LA];
     const uint8_t* gb[LB];
     int sa_off[LA], sb_off[LB];
+    const int a_exp = expands_fp4<Op> ? p.a_expand : 0, b_exp = expands_fp4<Op> ? p.b_expand : 0;
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
         const int r = ld_row + i * (NT / 8);
-        ga[i] = p.a + (long)min(m0 + r, p.m - 1) * p.lda_bytes + ld_chunk * 16;
+        ga[i] = p.a + (long)min(m0 + r, p.m - 1) * p.lda_bytes + (a_exp ? ld_chunk * 8 : ld_chunk * 16);
         sa_off[i] = r * 128 + swizzle_chunk(r, ld_chunk) * 16;
     }
     // B as [N][K] (Layout::DN): the same chunks as A.  B as [K][N] (Layout::ND, p.b_nd): a 16-byte chunk holds EPC
@@ -515,7 +542,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
     for (int i = 0; i < LB; ++i) {
         const int r = ld_row + i * (NT / 8);
         if (!p.b_nd) {
-            gb[i] = p.b + (long)min(n0 + r, p.n - 1) * p.ldb_bytes + ld_chunk * 16;
+            gb[i] = p.b + (long)min(n0 + r, p.n - 1) * p.ldb_bytes + (b_exp ? ld_chunk * 8 : ld_chunk * 16);
             sb_off[i] = Cfg::A_BYTES + r * 128 + swizzle_chunk(r, ld_chunk) * 16;
             b_koff[i] = ld_chunk * 16;
             sb_k[i] = sb_n[i] = 0;
@@ -538,12 +565,20 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
     auto tload = [&](int kt) {
         const bool live = kt * 128 + ld_chunk * 16 < p.k_bytes;  // partial last slab: missing chunks are zero
 #pragma unroll
-        for (int i = 0; i < LA; ++i)
-            ra[i] = live ? *reinterpret_cast<const uint4*>(ga[i] + (long)kt * 128) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < LA; ++i) {
+            if (expands_fp4<Op> && a_exp)
+                ra[i] = live ? expand_fp4_to_e4m3(*reinterpret_cast<const uint2*>(ga[i] + (long)kt * 64), a_exp) : make_uint4(0, 0, 0, 0);
+            else
+                ra[i] = live ? *reinterpret_cast<const uint4*>(ga[i] + (long)kt * 128) : make_uint4(0, 0, 0, 0);
+        }
 #pragma unroll
-        for (int i = 0; i < LB; ++i)
-            rb[i] = kt * 128 + b_koff[i] < p.k_bytes ? *reinterpret_cast<const uint4*>(gb[i] + kt * b_slab_stride)
-                                                     : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < LB; ++i) {
+            if (expands_fp4<Op> && b_exp)  // (B is [N][K] here: the host sends row-major packed B elsewhere)
+                rb[i] = live ? expand_fp4_to_e4m3(*reinterpret_cast<const uint2*>(gb[i] + (long)kt * 64), b_exp) : make_uint4(0, 0, 0, 0);
+            else
+                rb[i] = kt * 128 + b_koff[i] < p.k_bytes ? *reinterpret_cast<const uint4*>(gb[i] + kt * b_slab_stride)
+                                                         : make_uint4(0, 0, 0, 0);
+        }
     };
     auto stage = [&](int buf) {
         uint8_t* base = smem + buf * Cfg::STAGE_BYTES;

@@ -658,6 +658,51 @@ def test_mx_gemm(pa, oracle, ta, tb, tile):
         assert np.array_equal(exact.view(np.uint32), ref.view(np.uint32))  # double-add-then-round order, bit for bit
 
 
+@pytest.mark.parametrize("ta,tb", [(ob.E1M2, ob.E1M2), (ob.E1M2, ob.E2M1), (ob.E2M1, ob.E1M2)])
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_mx_e1m2_operands_run_on_the_fp8_mfma(pa, oracle, ta, tb, tile):
+    """The scaled MFMA has no E1M2 format; every E1M2 and E2M1 value is an E4M3 value, so the register-staged loader
+    expands the nibbles and the E4M3 x E4M3 instruction runs the product.  All 16 x 16 code pairs occur; block scales
+    in the plain and in the boxed layouts; ragged M and N.  The bound is the fp8 instruction's (it keeps about 13 bits
+    below the largest of its 64 products); with one scale per row the sums are exact and must match bit for bit."""
+    r = np.random.default_rng(ta * 16 + tb + tile)
+    for m, n, k in ((128, 128, 256), (200, 72, 512)):
+        a, _, sa, sb = _mx_inputs(r, ta, m, n, k)
+        _, b, _, _ = _mx_inputs(r, tb, m, n, k)
+        ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ta, tb)
+        with tile_env(PTOAMD_TILE=tile):
+            got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[ta], PA_T[tb], pa.F32))
+            assert pa.last_kernel().endswith("fp8_e4m3_e4m3") and "_dtl_" not in pa.last_kernel(), pa.last_kernel()
+        ua = _mx_unpack(oracle, a, ta) * np.repeat(2.0 ** (sa.astype(np.float64) - 127), 32, 1)
+        ub = _mx_unpack(oracle, b, tb) * np.repeat(2.0 ** (sb.astype(np.float64) - 127), 32, 1)
+        check_f32_drain(got, ref, np.abs(ua) @ np.abs(ub).T, k, f"MX {ta}x{tb} {m}x{n}x{k} tile {tile} (expanded to E4M3)",
+                        max_rel=1e-3, eps=2.0 ** -11)
+        # one scale per row / column: all products of a row share a binade range of 2^6, the sums are exact in fp32
+        sa1 = np.repeat(r.integers(120, 134, (m, 1)).astype(np.uint8), k // 32, 1)
+        sb1 = np.repeat(r.integers(120, 134, (n, 1)).astype(np.uint8), k // 32, 1)
+        ref1 = oracle.matmul_mx(a, b, sa1, sb1, m, k, n, ta, tb)
+        with tile_env(PTOAMD_TILE=tile):
+            got1 = host(pa.gemm_mx(dev(a), dev(b), dev(sa1), dev(sb1), m, n, k, PA_T[ta], PA_T[tb], pa.F32))
+        assert np.array_equal(got1.view(np.uint32), ref1.view(np.uint32))
+    # boxed scale layouts in place, bf16 drain, bias
+    m, n, k = 64, 96, 256
+    a, _, sa, sb = _mx_inputs(r, ta, m, n, k)
+    _, b, _, _ = _mx_inputs(r, tb, m, n, k)
+    ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ta, tb)
+    sa_zz = pa.mx_scale_relayout(dev(sa), pa.MX_A_ND, pa.MX_A_ZZ, m, k // 32)
+    sb_nn = pa.mx_scale_relayout(dev(sb), pa.MX_B_DN, pa.MX_B_NN, k // 32, n)
+    with tile_env(PTOAMD_TILE=tile):
+        got = host(pa.gemm_mx(dev(a), dev(b), sa_zz, sb_nn, m, n, k, PA_T[ta], PA_T[tb], pa.F32,
+                              sa_layout=pa.MX_A_ZZ, sb_layout=pa.MX_B_NN))
+    assert relerr(got, ref) <= 1e-3
+    # shapes the expansion path does not take (k not a multiple of 128) still run, on the order-exact kernel
+    a, _, sa, sb = _mx_inputs(r, ta, 40, 24, 192)
+    _, b, _, _ = _mx_inputs(r, tb, 40, 24, 192)
+    got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), 40, 24, 192, PA_T[ta], PA_T[tb], pa.F32))
+    assert pa.last_kernel() == "generic"
+    assert np.array_equal(got.view(np.uint32), oracle.matmul_mx(a, b, sa, sb, 40, 192, 24, ta, tb).view(np.uint32))
+
+
 def test_mx_block_scales_select_the_right_group(pa, oracle):
     """One scale group at a time carries a large exponent: a wrong byte/lane selection shows up as a gross error."""
     r = np.random.default_rng(8)
