@@ -117,6 +117,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     const uint32_t lds_wave_base = __builtin_amdgcn_readfirstlane(lds_address(smem) + wave * 1024);
     // DMA number q (0 .. LA + LB - 1) of slab kt into ring buffer buf
     auto tload_piece = [&](int kt, int buf, int q) {
+#if defined(PTOAMD_CLOCK_PROBE) && defined(PTOAMD_PROBE_DMA_EVERY)
+        // timing experiment (results are wrong): after the first two slabs issue no DMA (0) or every n-th piece only
+        if (kt > 1 && (PTOAMD_PROBE_DMA_EVERY == 0 || q % (PTOAMD_PROBE_DMA_EVERY ? PTOAMD_PROBE_DMA_EVERY : 1) != 0))
+            return;
+#endif
         const uint32_t dst = lds_wave_base + buf * Cfg::STAGE_BYTES;
         if (q < LA)
             lds_dma16_off(p.a + (long)kt * 128, goff_a[q], dst + q * (NT * 16));
@@ -139,10 +144,14 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     constexpr int SW = GPS / 4, SPG = 16 / GPS;
     constexpr int SROWS = BM + BN, NSI = SROWS / 64, NW = NT / 64, NSW = (NSI + NW - 1) / NW;
     static_assert(SROWS % 64 == 0 && BM % 64 == 0, "one scale DMA covers 64 rows of one operand");
-    // The scale dwords of slab kt + 1 are read one k-step ahead, except where 32-byte fragments of a large wave tile
-    // leave no registers for the second copy: there they are read when the slab starts and the SIMD's other wave
-    // covers the LDS latency.
+    // The scale dwords of slab kt + 1 are read one k-step ahead (after slab kt's barrier), so that the slab's first
+    // MFMA does not wait for an LDS round trip.  PTOAMD_SCALES_AT_SLAB_START reads them when the slab starts instead
+    // (one register set fewer) for the 32-byte fragments of a large wave tile.
+#ifdef PTOAMD_SCALES_AT_SLAB_START
     constexpr bool SC_AHEAD = !(Op::FRAG_BYTES == 32 && MB * NB >= 8);
+#else
+    constexpr bool SC_AHEAD = true;
+#endif
     uint32_t sca[MB][SW], scb[NB][SW], sca_n[MB][SW], scb_n[NB][SW];
     const bool has_scales = Op::SCALED && p.sa != nullptr;
 #pragma unroll
@@ -175,8 +184,11 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         }
     };
     // slab kt's scales of this lane's rows, LDS -> sca_n / scb_n
+    // (No test of has_scales here: a branch between two k-steps lets the compiler sink the earlier k-step's MFMAs
+    // below it, away from the fragment reads they should overlap.  Without scale arrays the LDS scale area is filled
+    // with E8M0 127 once, in the prologue.)
     auto read_scales = [&](int kt) {
-        if (has_scales) {
+        if (Op::SCALED) {
             const uint8_t* base = smem + 2 * Cfg::STAGE_BYTES + ((kt / SPG) & 1) * (SROWS * 16) + (kt % SPG) * GPS;
 #pragma unroll
             for (int w = 0; w < SW; ++w) {
@@ -285,6 +297,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // ---- prologue: slabs 0 and 1 in flight, first fragments in registers
     tload(0, 0);
     tload_scales(0);
+    if (Op::SCALED && !has_scales) {
+        for (int o = tid * 16; o < 2 * SROWS * 16; o += NT * 16)
+            *reinterpret_cast<uint4*>(smem + 2 * Cfg::STAGE_BYTES + o) = make_uint4(0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu);
+    }
     if (k_slabs > 1)
         static_for<dma_phase_begin<NDMA, KS>(1)>([&](auto qc) { tload_piece(1, 1, decltype(qc)::value); });
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMAs have landed

@@ -6,7 +6,8 @@
 // [4] at exit.  This program runs the launch back to back until the clocks have settled, then prints the phases of the
 // last launch (mean / max over the workgroups) and the K loop per XCD (workgroup id mod 8).  Timing tool only: it checks
 // no results.  Build: make -C tests/pto_kernels build/clock_probe   (not part of the default target; under a minute;
-//                     build/clock_probe_i8 and build/clock_probe_fp8 are the other two kinds)
+//                     build/clock_probe_i8 and build/clock_probe_fp8 are the other two kinds; build/clock_probe_nodma and
+//                     build/clock_probe_halfdma leave out all / half of the slab DMAs to show what the copy-in costs)
 //        run:   tests/pto_kernels/build/clock_probe [m n k [zeros]]   (a fourth argument fills the operands with zeros:
 //               the same instruction stream at the lowest switching power)
 #define PTOAMD_CLOCK_PROBE 1
