@@ -390,6 +390,89 @@ static int run(void* stream, int blocks, Args... args)
 //   2: e4m3 x e4m3 127x72x64      3: e4m3 x e5m2 128x110x63     5: e1m2 x e2m1 117x64x60     6: e2m1 x e1m2 128x118x64
 //   15: e2m1 x e1m2 35x128x56 + bias     11: gemv e1m2 x e1m2 1x128x62, B scales MX_B_ND     12: gemv e4m3 x e5m2 1x256x20, MX_B_ND
 //   21: gemv e2m1 x e2m1 1x192x40, B scales MX_B_DN
+// ---- quantise, then multiply: the step between TQUANT and TMATMUL_MX inside one kernel --------------------------------
+// A arrives as f32.  TQUANT<MXFP8> turns it into E4M3 codes plus one E8M0 exponent per 32 elements in Vec (unified
+// buffer) tiles; TMOV carries the codes from the row-major Vec tile into the fractal (NZ) Mat tile and the exponents,
+// viewed as an [M][K/32] scale tile at the same unified-buffer address, into the scale Mat tile; from there on the
+// kernel is the ordinary TMATMUL_MX pipeline.  B and its scales come quantised from global memory.
+template <int M, int K, int N>
+__global__ AICORE void RunQUANT_TMATMUL_MX(__gm__ float* out, __gm__ float* src0, __gm__ float8_e4m3_t* src1, __gm__ float8_e8m0_t* src3)
+{
+    using ScaleType = float8_e8m0_t;
+    using E4 = float8_e4m3_t;
+    constexpr int kMX = K / 32, G = M * kMX;
+    static_assert(M % 16 == 0 && K % 64 == 0 && N % 32 == 0, "whole fractals");
+
+    using SrcTile = Tile<TileType::Vec, float, M, K, BLayout::RowMajor, M, K>;
+    using CodeTile = Tile<TileType::Vec, E4, M, K, BLayout::RowMajor, M, K>;
+    using ExpTile = Tile<TileType::Vec, uint8_t, 1, G, BLayout::RowMajor, 1, G>;
+    using ExpView = Tile<TileType::Vec, ScaleType, M, kMX, BLayout::RowMajor, M, kMX>;
+    using FlatTile = Tile<TileType::Vec, float, 1, G, BLayout::RowMajor, 1, G>;
+    SrcTile srcTile;
+    CodeTile codeTile;
+    ExpTile expTile;
+    ExpView expView;
+    FlatTile maxTile, scalingTile;
+    constexpr int u1 = CeilAlign<int>(SrcTile::Bytes, 32), u2 = u1 + CeilAlign<int>(CodeTile::Bytes, 32),
+                  u3 = u2 + CeilAlign<int>(ExpTile::Bytes, 32), u4 = u3 + CeilAlign<int>(FlatTile::Bytes, 32);
+    TASSIGN(srcTile, 0x0);
+    TASSIGN(codeTile, u1);
+    TASSIGN(expTile, u2);
+    TASSIGN(expView, u2);  // the same bytes, seen as M rows of K / 32 scales
+    TASSIGN(maxTile, u3);
+    TASSIGN(scalingTile, u4);
+
+    using MatA = Tile<TileType::Mat, E4, M, K, BLayout::ColMajor, M, K, SLayout::RowMajor, 512>;
+    using MatB = Tile<TileType::Mat, E4, K, N, BLayout::ColMajor, K, N, SLayout::RowMajor, 512>;
+    using MatSA = Tile<TileType::Mat, ScaleType, M, kMX, BLayout::RowMajor, M, kMX, SLayout::RowMajor, 32>;
+    using MatSB = Tile<TileType::Mat, ScaleType, kMX, N, BLayout::ColMajor, kMX, N, SLayout::ColMajor, 32>;
+    MatA aMat;
+    MatB bMat;
+    MatSA saMat;
+    MatSB sbMat;
+    TASSIGN(aMat, 0x0);
+    TASSIGN(bMat, M * K);
+    TASSIGN(saMat, M * K + K * N);
+    TASSIGN(sbMat, M * K + K * N + M * kMX);
+    TileLeft<E4, M, K, M, K> aTile;
+    TileRight<E4, K, N, K, N> bTile;
+    TileLeftScale<ScaleType, M, kMX, M, kMX> saTile;
+    TileRightScale<ScaleType, kMX, N, kMX, N> sbTile;
+    TileAcc<float, M, N, M, N> cTile;
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(cTile, 0x0);
+    TASSIGN(saTile, GetScaleAddr(aTile.data()));
+    TASSIGN(sbTile, GetScaleAddr(bTile.data()));
+
+    GlobalTensor<float, TileShape2D<float, M, K>, BaseShape2D<float, M, K>> aGlobal(src0);
+    GlobalTensor<E4, TileShape2D<E4, K, N>, BaseShape2D<E4, K, N>> bGlobal(src1);
+    using GlobalSB = GlobalTensor<ScaleType, TileShape2D<ScaleType, kMX, N, Layout::MX_B_NN>, BaseShape2D<ScaleType, kMX, N, Layout::MX_B_NN>, Layout::MX_B_NN>;
+    GlobalSB sbGlobal(src3);
+    GlobalTensor<float, TileShape2D<float, M, N>, BaseShape2D<float, M, N>> outGlobal(out);
+
+    TLOAD(srcTile, aGlobal);
+    TLOAD(bMat, bGlobal);
+    TLOAD<MatSB, GlobalSB>(sbMat, sbGlobal);
+    set_flag(PIPE_MTE2, PIPE_V, EVENT_ID0);
+    wait_flag(PIPE_MTE2, PIPE_V, EVENT_ID0);
+    TQUANT<QuantType::MXFP8>(codeTile, srcTile, &expTile, &maxTile, &scalingTile);
+    set_flag(PIPE_V, PIPE_MTE1, EVENT_ID0);
+    wait_flag(PIPE_V, PIPE_MTE1, EVENT_ID0);
+    TMOV(aMat, codeTile);   // codes: ND (row-major Vec tile) -> NZ (fractal Mat tile)
+    TMOV(saMat, expView);   // exponents: [M][K / 32] rows -> the scale Mat tile
+    TMOV(aTile, aMat);
+    TMOV(bTile, bMat);
+    TMOV(saTile, saMat);
+    TMOV(sbTile, sbMat);
+    set_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
+    wait_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
+    TMATMUL_MX(cTile, aTile, saTile, bTile, sbTile);
+    set_flag(PIPE_M, PIPE_FIX, EVENT_ID0);
+    wait_flag(PIPE_M, PIPE_FIX, EVENT_ID0);
+    TSTORE(outGlobal, cTile);
+}
+
 extern "C" int pto_boundary_launch_mx(int id, void* out, void* a, void* b, void* sa, void* sb, void* bias, void* stream)
 {
     using S = float8_e8m0_t;
@@ -443,7 +526,7 @@ extern "C" int pto_boundary_launch_cvt(int id, void* dst, void* src, int mode, i
 //   30 / 31: 5-D global tensor half ND / DN (out = packed, src1 = scattered)     32: float ND
 //   40..44: fix-pipe TMOV / TEXTRACT modes 0..4 on a half 48x64x96 product (src2 = quant words)
 //   45: mode 1 on an int8 48x64x96 product (int32 accumulator -> int8)
-//   50: TRESHAPE     60: TASSIGN at the address in `arg`
+//   50: TRESHAPE     60: TASSIGN at the address in `arg`     70: TQUANT<MXFP8> of an f32 A, TMOV ND -> NZ, TMATMUL_MX
 extern "C" int pto_boundary_launch(int id, void* out, void* src0, void* src1, void* src2, unsigned arg, void* stream)
 {
     using E4 = float8_e4m3_t;
@@ -468,6 +551,7 @@ extern "C" int pto_boundary_launch(int id, void* out, void* src0, void* src1, vo
     case 45: return run<&RunTMOV_FIXPIPE<int8_t, int32_t, int8_t, 48, 64, 96, 1>>(stream, 1, (int8_t*)out, (int8_t*)src0, (int8_t*)src1, (uint64_t*)src2);
     case 50: return run<&RunTRESHAPE>(stream, 1, (float*)out, (float*)src0);
     case 60: return run<&RunTASSIGN_OUT_OF_RANGE>(stream, 1, (float*)out, (float*)src0, (uint32_t)arg);
+    case 70: return run<&RunQUANT_TMATMUL_MX<32, 128, 64>>(stream, 1, (float*)out, (float*)src0, (E4*)src1, (float8_e8m0_t*)src2);
     default: return -1;
     }
 }

@@ -167,6 +167,42 @@ def test_tmatmul_mx_unaligned_k_with_tfillpad(lib, oracle, case, dist):
         assert_sum_close(got, exact, absdot, k, f"mx case {case} vs float64", **_mx_bound(ta))
 
 
+@pytest.mark.parametrize("dist", ["powers", "normal"])
+def test_quantise_then_matmul_mx_in_one_kernel(lib, oracle, dist):
+    """f32 A -> TQUANT<MXFP8> in Vec tiles -> TMOV codes ND -> NZ Mat tile, exponents -> scale Mat tile -> TMATMUL_MX.
+    The kernel's result is compared with the oracle's TMATMUL_MX of the oracle's own quantisation of A: a wrong code
+    layout, exponent row or scale pairing after the TMOVs shows as a gross error.  'powers': A holds signed powers of
+    two and B small integers, so codes, scales and sums are all exact and the match must be bit for bit."""
+    m, k, n = 32, 128, 64
+    kg = k // 32
+    r = np.random.default_rng(70 + len(dist))
+    if dist == "powers":
+        # a different binade per 64 elements (one MFMA's worth, so that nothing is shifted out inside the instruction),
+        # narrow enough that every partial sum fits 24 bits and the order of the additions cannot matter
+        e = np.repeat(r.integers(-2, 3, (m, k // 64)), 64, 1) + r.integers(-3, 1, (m, k))
+        a = (np.ldexp(1.0, e) * r.choice([-1.0, 1.0], (m, k))).astype(np.float32)
+        b, bv = _mx_operand(oracle, r, ob.E4M3, (k, n), "ints")
+        sb = r.integers(125, 130, (kg, n)).astype(np.uint8)
+    else:
+        a = (r.standard_normal((m, k)) * np.exp(r.uniform(-3, 3, (m, 1)))).astype(np.float32)
+        b, bv = _mx_operand(oracle, r, ob.E4M3, (k, n), "codes")
+        sb = r.integers(118, 136, (kg, n)).astype(np.uint8)
+    codes, exp, _, _ = oracle.tquant_mx(a, ob.OCP_FP8, 1)
+    ref = oracle.matmul_mx(codes, b, exp, np.ascontiguousarray(sb.T), m, k, n, ob.E4M3, ob.E4M3,
+                           sa_layout=ob.MX_A_ND, sb_layout=ob.MX_B_DN, b_dn=False)
+    sb_gm = np.zeros(kg * n, np.uint8)
+    sb_gm[oracle.mx_scale_offsets(ob.MX_B_NN, kg, n)] = sb
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
+    launch(lib, 70, out, dev(a), dev(b), dev(sb_gm))
+    got = out.cpu().numpy()
+    wa = oracle.mx_decode_table(ob.E4M3)[codes] * np.repeat(2.0 ** (exp.astype(np.float64) - 127), 32, 1)
+    wb = bv * np.repeat(2.0 ** (sb.astype(np.float64) - 127), 32, 0)
+    assert np.abs(ref).max() > 0 and len(np.unique(exp)) > 3
+    assert_sum_close(got, ref, np.abs(wa) @ np.abs(wb), k, "quantise-then-matmul " + dist, **_mx_bound(ob.E4M3))
+    if dist == "powers":
+        assert np.array_equal(got, ref)
+
+
 @pytest.mark.parametrize("dist", ["ints", "codes"])
 @pytest.mark.parametrize("case", sorted(MX_GEMV))
 def test_tgemv_mx(lib, oracle, case, dist):
