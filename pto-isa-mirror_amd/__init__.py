@@ -68,7 +68,9 @@ def init(device=0):
 def _ptr(t):
     if t is None:
         return C.c_void_p(0)
-    assert t.is_cuda and t.is_contiguous(), "operands must be contiguous device tensors"
+    # contiguous, or a 2-D view with unit column stride (its row pitch goes to the library as the leading dimension)
+    assert t.is_cuda and (t.is_contiguous() or (t.dim() == 2 and t.stride(1) == 1)), \
+        "operands must be device tensors, contiguous or row-strided"
     return C.c_void_p(t.data_ptr())
 
 

@@ -151,6 +151,34 @@ def test_row_major_b_is_transposed_inside_the_kernel(pa, oracle, tile, kind, m, 
         assert relerr(got, ref) <= (2e-2 if kind == "e4m3" else 1e-2)
 
 
+def test_operands_past_4_gib_leave_the_dma_tiles(pa, oracle):
+    """The direct-to-LDS tiles keep lane addresses as 32-bit offsets from a scalar base.  An A whose last row starts more
+    than 4 GiB after its first (a large row pitch here: only K elements of each row are used) must be routed to the
+    register-staged tiles, which carry 64-bit pointers, and give the right result."""
+    r = np.random.default_rng(64)
+    m, n, k = 512, 512, 256
+    lda = (1 << 32) // 2 // (m - 1) + 64            # elements: (m - 1) * lda * 2 bytes is just past 2^32
+    base = torch.zeros(m * lda, dtype=torch.bfloat16, device=DEV)
+    a_h = bf16_bits(r.standard_normal((m, k)))
+    b_h = bf16_bits(r.standard_normal((n, k)))
+    a = base.view(m, lda)[:, :k]
+    a.copy_(dev(a_h).view(torch.bfloat16))
+    assert a.stride(0) * 2 * (m - 1) + k * 2 > 2 ** 32
+    rows = np.array([0, 1, 255, 256, 510, 511])
+    ref = oracle.matmul_bf16(a_h[rows], b_h, b_dn=True)
+    for tile, name in ((None, "tile64x64_bf16"), (4, "tile256x256_bf16"), (5, "tile128x128_bf16")):
+        env = tile_env(PTOAMD_TILE=tile) if tile is not None else tile_env()
+        with env:
+            got = host(pa.gemm(a, dev(b_h).view(torch.bfloat16), pa.BF16, pa.F32, pa.B_DN))
+            assert pa.last_kernel() == name, pa.last_kernel()
+        assert relerr(got[rows], ref) <= 1e-4
+    # the same product with an ordinary pitch does take the DMA tile
+    with tile_env(PTOAMD_TILE=4):
+        pa.gemm(dev(a_h).view(torch.bfloat16), dev(b_h).view(torch.bfloat16), pa.BF16, pa.F32, pa.B_DN)
+        assert pa.last_kernel() == "tile256x256w8_dtl_bf16"
+    del base, a
+
+
 TILE_NAMES = ("tile256x256_", "tile128x128_", "tile64x64_", "tile256x256w4_dtl", "tile256x256w8_dtl", "tile128x128_dtl",
               "tile256x128_dtl")
 ALL_TILES = [0, 1, 2, 3, 4, 5, 6]
