@@ -8,6 +8,8 @@
 
 namespace ptoamd {
 
+typedef short short2v __attribute__((ext_vector_type(2)));
+
 static_assert(PTOAMD_OCP_MXFP8 == MX_OCP_FP8 && PTOAMD_NV_MXFP8 == MX_NV_FP8 && PTOAMD_OCP_MXFP4 == MX_OCP_FP4 &&
                   PTOAMD_NV_MXFP4 == MX_NV_FP4,
               "the C ABI's algorithm ids are the kernels' template arguments");
@@ -85,16 +87,46 @@ __global__ void __launch_bounds__(256) tquant_mx_rows_kernel(uint8_t* dst, uint8
                     reinterpret_cast<uint16_t*>(dst)[unit] = (uint16_t)packed;
             }
         } else {
-            uint32_t c[EPL];
+            uint32_t words[EPL / 4];
+            // The hardware conversion rounds every finite value inside +-448 exactly as EncodeE4M3Fn does (all 2^32
+            // float patterns compared); it differs beyond 448 (NaN code instead of saturation), on NaN (0xFF instead
+            // of 0x7F) and on negative values that round to zero (0x80 instead of 0x00).  So a lane whose own elements
+            // hold no NaN (the group maximum ignores NaNs, so it cannot tell) clamps, converts in pairs and clears
+            // the sign of zero codes; a lane with a NaN takes the software encoder.  Both give the same codes wherever
+            // both apply, so the lanes of a group need not agree.
+            uint32_t largest = 0;
 #pragma unroll
             for (int i = 0; i < EPL; ++i)
-                c[i] = encode_mx<ALG, SRC_BF16>(v[i], sc);
+                largest = max(largest, f2u(v[i]) & 0x7FFFFFFFu);
+            const bool fast = ALG == PTOAMD_OCP_MXFP8 && largest <= 0x7F800000u && (f2u(sc) & 0x7F800000u) != 0x7F800000u;
+            if (fast) {
+                static_for<EPL / 4>([&](auto wc) {
+                    constexpr int w = decltype(wc)::value;
+                    float t[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        t[i] = __builtin_amdgcn_fmed3f(__fmul_rn(v[4 * w + i], sc), -448.0f, 448.0f);
+                    short2v pk = {0, 0};
+                    pk = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(pk, t[0], t[1], 1.0f, false);
+                    pk = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(pk, t[2], t[3], 1.0f, true);
+                    const uint32_t x = __builtin_bit_cast(uint32_t, pk);
+                    const uint32_t nonzero = ((x & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) & 0x80808080u;  // bit 7 of bytes whose magnitude is not 0
+                    words[w] = x & (nonzero | 0x7F7F7F7Fu);
+                });
+            } else {
+                uint32_t c[EPL];
+#pragma unroll
+                for (int i = 0; i < EPL; ++i)
+                    c[i] = encode_mx<ALG, SRC_BF16>(v[i], sc);
+#pragma unroll
+                for (int w = 0; w < EPL / 4; ++w)
+                    words[w] = c[4 * w] | (c[4 * w + 1] << 8) | (c[4 * w + 2] << 16) | (c[4 * w + 3] << 24);
+            }
             if (live) {
-                const uint32_t lo = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
                 if constexpr (EPL == 8)
-                    reinterpret_cast<uint2*>(dst)[unit] = make_uint2(lo, c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24));
+                    reinterpret_cast<uint2*>(dst)[unit] = make_uint2(words[0], words[1]);
                 else
-                    reinterpret_cast<uint32_t*>(dst)[unit] = lo;
+                    reinterpret_cast<uint32_t*>(dst)[unit] = words[0];
             }
         }
     }

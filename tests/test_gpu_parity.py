@@ -1059,6 +1059,51 @@ def test_tquant_mx_half_sources(pa, oracle, dtype, kind, alg):
     assert np.array_equal(exp, re) and np.array_equal(codes, rc) and _eq_f32(mx, rm) and _eq_f32(sc, rs)
 
 
+@pytest.mark.parametrize("alg", [0, 1])
+def test_tquant_mxfp8_every_bf16_pattern_and_edge_groups(pa, oracle, alg):
+    """The MXFP8 quantiser's packed hardware conversion against the oracle's nearest-code search, bit for bit: every
+    bf16 bit pattern (NaNs and infinities included) as a bf16 and as an f32 source, sorted (groups of one magnitude) and
+    shuffled (groups spanning the whole range), plus f32 groups built to hit what the hardware conversion does
+    differently: scaled values between 448 and 512, negative values that round to zero, ties between codes, groups
+    holding a NaN or an infinity, all-zero groups."""
+    r = np.random.default_rng(90 + alg)
+    pats = np.arange(65536, dtype=np.uint16)
+    for order in ("sorted", "shuffled"):
+        bits = pats.copy() if order == "sorted" else r.permutation(pats)
+        f32 = (bits.astype(np.uint32) << 16).view(np.float32).reshape(64, 1024)
+        src16 = torch.from_numpy(bits.view(np.int16).reshape(64, 1024)).view(torch.bfloat16)
+        for src, kind in ((torch.from_numpy(f32.copy()), ob.SRC_F32), (src16, ob.SRC_BF16)):
+            codes, exp, mx, sc = (host(t) for t in pa.tquant_mx(src.to(DEV), alg, 1))
+            rc, re, rm, rs = oracle.tquant_mx(f32, alg, 1, kind)
+            assert np.array_equal(exp, re), (order, kind)
+            assert np.array_equal(codes, rc), (order, kind, int((codes != rc).sum()))
+            assert _eq_f32(mx, rm) and _eq_f32(sc, rs)
+    g = np.zeros((16, 32), np.float32)
+    g[0] = np.linspace(440, 511.9, 32)                      # shared exponent 2^0: values above 448 saturate to 0x7E
+    g[1] = -g[0]
+    g[2] = 300.0; g[2, 1:] = -(2.0 ** (-np.arange(1, 32) / 2.0 - 6))            # negatives down to below half the smallest code
+    g[3] = 1.0; g[3, 1:] = (np.arange(31) + 0.5) * 2.0 ** -9 * 2.0 ** -8 * 256   # exact ties between subnormal codes
+    g[4] = 1.0; g[4, 1:] = 1.0 + (2 * np.arange(31) + 1) / 16.0                 # exact ties between normal codes
+    g[5] = r.standard_normal(32); g[5, 7] = np.nan
+    g[6] = r.standard_normal(32); g[6, 3] = np.inf
+    g[7] = r.standard_normal(32); g[7, 9] = -np.inf
+    g[8] = 0.0
+    g[9] = -0.0
+    g[10] = np.float32(1e-42)                                # denormal f32 input
+    g[11] = r.standard_normal(32) * 1e38
+    g[12] = r.standard_normal(32) * 1e-38
+    g[13] = 447.9; g[13, ::2] = -448.1
+    g[14] = r.standard_normal(32); g[14, 0] = np.nan; g[14, 1] = np.inf
+    g[15] = 2.0 ** -127
+    src = np.ascontiguousarray(np.tile(g, (1, 4)))         # 16 rows x 128: four copies of each group per row
+    codes, exp, mx, sc = (host(t) for t in pa.tquant_mx(dev(src), alg, 1))
+    rc, re, rm, rs = oracle.tquant_mx(src, alg, 1)
+    assert np.array_equal(exp, re)
+    bad = np.argwhere(codes != rc)
+    assert bad.size == 0, (bad[:5], codes[codes != rc][:5], rc[codes != rc][:5])
+    assert _eq_f32(mx, rm) and _eq_f32(sc, rs)
+
+
 def test_tquant_int8_and_tdequant_bit_exact(pa, oracle, golden):
     g = golden
     src, scale, off = g["q8_src"], g["q8_scale"], g["q8_off"]
