@@ -279,7 +279,8 @@ __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int 
 // bits of one output element (1- and 2-byte kinds in the low part); W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16,
 // each step rounded to f32; the quantising kinds: fix-pipe word `qw`, then relu
 template <int KIND, class V>
-__device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_t qw = 0, bool q_vector = false, bool relu = false)
+__device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_t qw = 0, bool q_vector = false, bool relu = false,
+                                                int q16_kind = OUT_QF16)
 {
     if (KIND == OUT_F32)
         return __builtin_bit_cast(uint32_t, (float)v);
@@ -289,32 +290,38 @@ __device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_
         return f32_to_f16_bits((float)v);
     if (KIND == OUT_BF16)
         return f32_to_bf16_bits((float)v);
-    if (KIND == OUT_Q8 || KIND == OUT_QF16) {
-        constexpr bool src_int = std::is_same<V, int32_t>::value || std::is_same<V, int>::value;
-        constexpr bool byte = KIND == OUT_Q8;
-        float r = q_vector ? fixpipe_quantize<true, byte, src_int>((float)v, qw) : fixpipe_quantize<false, byte, src_int>((float)v, qw);
+    constexpr bool src_int = std::is_same<V, int32_t>::value || std::is_same<V, int>::value;
+    if (KIND == OUT_Q8) {
+        float r = q_vector ? fixpipe_quantize<true, true, src_int>((float)v, qw) : fixpipe_quantize<false, true, src_int>((float)v, qw);
         if (relu)
             r = r > 0 ? r : 0;
-        return byte ? ((uint32_t)(int32_t)r & 0xFFu) : (uint32_t)f32_to_f16_bits(r);
+        return (uint32_t)(int32_t)r & 0xFFu;
     }
-    if (KIND == OUT_QBF16) {
-        float r = __fmul_rn((float)v, q_vector ? fixpipe_word_scale<true>(qw) : fixpipe_word_scale<false>(qw));
+    if (KIND == OUT_QF16) {
+        // the three 16-bit targets of the quantiser share one instance; which one is a (uniform) run-time choice
+        if (src_int && q16_kind == OUT_QS16) {
+            int32_t r = fixpipe_shift_s16((int32_t)v, qw);
+            if (relu)
+                r = r > 0 ? r : 0;
+            return (uint32_t)r & 0xFFFFu;
+        }
+        if (q16_kind == OUT_QBF16) {
+            float r = __fmul_rn((float)v, q_vector ? fixpipe_word_scale<true>(qw) : fixpipe_word_scale<false>(qw));
+            if (relu)
+                r = r > 0 ? r : 0;
+            return f32_to_bf16_bits(r);
+        }
+        float r = q_vector ? fixpipe_quantize<true, false, src_int>((float)v, qw) : fixpipe_quantize<false, false, src_int>((float)v, qw);
         if (relu)
             r = r > 0 ? r : 0;
-        return f32_to_bf16_bits(r);
-    }
-    if (KIND == OUT_QS16) {
-        int32_t r = fixpipe_shift_s16((int32_t)v, qw);
-        if (relu)
-            r = r > 0 ? r : 0;
-        return (uint32_t)r & 0xFFFFu;
+        return (uint32_t)f32_to_f16_bits(r);
     }
     return f32_to_bf16_bits(__fmul_rn(__fmul_rn((float)v, rs), cs));
 }
 template <int KIND>
 constexpr int out_bytes = (KIND == OUT_F32 || KIND == OUT_I32) ? 4 : (KIND == OUT_Q8 ? 1 : 2);
 template <int KIND>
-constexpr bool out_quant = KIND == OUT_Q8 || KIND == OUT_QF16 || KIND == OUT_QBF16 || KIND == OUT_QS16;
+constexpr bool out_quant = KIND == OUT_Q8 || KIND == OUT_QF16;  // (OUT_QF16 instances also serve OUT_QBF16 and OUT_QS16)
 
 // Element-wise form: any alignment, any edge.  A lane's elements are 4-column runs of one row, so this form is slow
 // (short scattered stores); whole, aligned wave tiles take the staged form below.
@@ -332,7 +339,7 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
             const long o = (long)gi * p.ldc + gj;
             const float cs = KIND == OUT_W8A8_BF16 ? p.col_scale[gj] : 1.0f;
             const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? gj : 0] : 0;
-            const uint32_t bits = tstore_bits<KIND>(v[r], rs, cs, qw, p.q_per_column != 0, p.relu != 0);
+            const uint32_t bits = tstore_bits<KIND>(v[r], rs, cs, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
             if (KIND == OUT_F32 && p.atomic_add)
                 atomicAdd(reinterpret_cast<float*>(p.c) + o, __builtin_bit_cast(float, bits));
             else if (KIND == OUT_I32 && p.atomic_add)
@@ -356,14 +363,10 @@ __device__ __forceinline__ void tstore_block_kind(const TileGemmParams& p, const
 {
     if (p.out_kind == OUT_Q8) {
         tstore_block<OUT_Q8, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
-    } else if (p.out_kind == OUT_QF16) {
+    } else if (p.out_kind >= OUT_QF16) {
         tstore_block<OUT_QF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
-    } else if (p.out_kind == OUT_QBF16) {
-        tstore_block<OUT_QBF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
     } else if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
-        if (p.out_kind == OUT_QS16)
-            tstore_block<OUT_QS16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
-        else if (p.out_kind == OUT_I32)
+        if (p.out_kind == OUT_I32)
             tstore_block<OUT_I32, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
         else
             tstore_block<OUT_W8A8_BF16, FULL, Cfg>(p, acc, row_b, col_b, l32, lhi);
@@ -424,7 +427,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? col_b + 8 * g + 4 * lhi + e : 0] : 0;
-                        bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0);
+                        bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
                     }
                     if (ESZ == 4)
                         *reinterpret_cast<uint4*>(dst) = make_uint4(bits[0], bits[1], bits[2], bits[3]);
@@ -458,16 +461,12 @@ __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::
     const int esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : (p.out_kind == OUT_Q8 ? 1 : 2);
     const bool aligned = (((long)p.ldc * esz) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
     if (stage != nullptr && full && aligned && !p.atomic_add && !(p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr)) {
-        if (p.out_kind == OUT_QF16) {
+        if (p.out_kind >= OUT_QF16) {
             tstore_staged<OUT_QF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
         } else if (p.out_kind == OUT_Q8) {
             tstore_staged<OUT_Q8, Cfg>(p, acc, row0, col0, l32, lhi, stage);
-        } else if (p.out_kind == OUT_QBF16) {
-            tstore_staged<OUT_QBF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
         } else if constexpr (std::is_same<typename Cfg::Op::Elem, int32_t>::value) {
-            if (p.out_kind == OUT_QS16)
-                tstore_staged<OUT_QS16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
-            else if (p.out_kind == OUT_I32)
+            if (p.out_kind == OUT_I32)
                 tstore_staged<OUT_I32, Cfg>(p, acc, row0, col0, l32, lhi, stage);
             else
                 tstore_staged<OUT_W8A8_BF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
@@ -485,10 +484,9 @@ __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::
         // keep the address arithmetic of one 32x32 block from being hoisted over the others (register pressure)
         __builtin_amdgcn_sched_barrier(0);
         const Acc block = acc[i][j];
-        if (full)
-            tstore_block_kind<true, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi);
-        else
-            tstore_block_kind<false, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi);
+        // (bounds-checked also where the wave's tile lies inside the matrix: this form is store-bound either way, and a
+        // second, unchecked copy of every output kind costs more compile time than it saves run time)
+        tstore_block_kind<false, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi);
     });
 }
 
