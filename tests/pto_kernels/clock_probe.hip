@@ -37,7 +37,10 @@ using ProbeOp = OpFP8<0, 0>;
 constexpr int ESZ = 1, CSZ = 2, OUT = OUT_BF16;
 constexpr const char* KIND = "MXFP8";
 #endif
-using Cfg = TileCfg<256, 256, 2, 4, ProbeOp>;
+#ifndef PROBE_WAVES_N
+#define PROBE_WAVES_N 4  // 4: eight waves with 128 x 64 wave tiles (the default tile); 2: four waves with 128 x 128 wave tiles
+#endif
+using Cfg = TileCfg<256, 256, 2, PROBE_WAVES_N, ProbeOp>;
 
 #define CK(x)                                                                          \
     do {                                                                               \
