@@ -126,6 +126,11 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
 int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                      int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream);
 
+/* TMATMUL / _ACC / _BIAS on a mixed fp8 pair (cpu/TMatmul.hpp:31-49 admits all four E4M3 / E5M2 pairings of Left and Right):
+ * as ptoamd_gemm_bias with separate operand types; bias may be NULL. */
+int ptoamd_gemm_fp8(void* c, int c_type, const void* a, int a_type, const void* b, int b_type, const void* c_in, const void* bias,
+                    int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream);
+
 /*
  * The same pipeline drained through the fix-pipe quantiser: TSTORE of the accumulator tile with a scalar quantisation
  * word (TSTORE(dst, src, preQuantScalar)) or one word per column (TSTORE_FP with a Scaling tile):

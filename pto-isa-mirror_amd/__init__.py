@@ -40,7 +40,7 @@ EXPORTS = [
     "ptoamd_malloc_host", "ptoamd_free_host", "ptoamd_memcpy", "ptoamd_memcpy_async", "ptoamd_memset",
     "ptoamd_stream_create", "ptoamd_stream_destroy", "ptoamd_stream_synchronize", "ptoamd_event_create",
     "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
-    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_requant", "ptoamd_gemm_atomic_add", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
+    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_fp8", "ptoamd_gemm_requant", "ptoamd_gemm_atomic_add", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
     "ptoamd_gemm_mx_ws",
     "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
     "ptoamd_tquant_int8_para", "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_tdequant_para", "ptoamd_mx_scale_relayout",
@@ -98,6 +98,17 @@ def gemm(a, b, ab_type, c_type=F32, b_layout=B_DN, c_in=None, relu=False, m=None
         return out
     _check(_lib.ptoamd_gemm(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), m, n, k, a.stride(0), b.stride(0),
                             out.stride(0), b_layout, int(relu), _stream(stream)), "ptoamd_gemm")
+    return out
+
+
+def gemm_fp8(a, b, a_type, b_type, c_type=F32, b_layout=B_DN, c_in=None, bias=None, relu=False, stream=None, out=None):
+    """TMATMUL on an fp8 pair whose two types may differ (E4M3 / E5M2)."""
+    m, k = a.shape
+    n = b.shape[0] if b_layout == B_DN else b.shape[1]
+    if out is None:
+        out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
+    _check(_lib.ptoamd_gemm_fp8(_ptr(out), c_type, _ptr(a), a_type, _ptr(b), b_type, _ptr(c_in), _ptr(bias), m, n, k,
+                                a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu), _stream(stream)), "ptoamd_gemm_fp8")
     return out
 
 

@@ -447,12 +447,20 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
 
 static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                        const uint64_t* qwords, int q_per_column, int m, int n, int k, int lda, int ldb, int ldc, int b_layout,
-                       int relu, void* stream_, int atomic_add = 0);
+                       int relu, void* stream_, int atomic_add = 0, int b_type = -1);
 
 int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                      int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream_)
 {
     return gemm_common(c, c_type, a, b, ab_type, c_in, bias, nullptr, 0, m, n, k, lda, ldb, ldc, b_layout, relu, stream_);
+}
+
+int ptoamd_gemm_fp8(void* c, int c_type, const void* a, int a_type, const void* b, int b_type, const void* c_in, const void* bias,
+                    int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream_)
+{
+    const bool a8 = a_type == PTOAMD_E4M3 || a_type == PTOAMD_E5M2, b8 = b_type == PTOAMD_E4M3 || b_type == PTOAMD_E5M2;
+    PTOAMD_REQUIRE(a8 && b8, PTOAMD_E_UNSUPPORTED, "ptoamd_gemm_fp8: both operand types must be e4m3 or e5m2 (got %d, %d)", a_type, b_type);
+    return gemm_common(c, c_type, a, b, a_type, c_in, bias, nullptr, 0, m, n, k, lda, ldb, ldc, b_layout, relu, stream_, 0, b_type);
 }
 
 int ptoamd_gemm_requant(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
@@ -478,13 +486,16 @@ int ptoamd_gemm_atomic_add(void* c, int c_type, const void* a, const void* b, in
 
 static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                        const uint64_t* qwords, int q_per_column, int m, int n, int k, int lda, int ldb, int ldc, int b_layout,
-                       int relu, void* stream_, int atomic_add)
+                       int relu, void* stream_, int atomic_add, int b_type)
 {
+    // b_type: -1 = as ab_type; otherwise the second type of a mixed fp8 pair (ab_type is then A's)
+    if (b_type < 0)
+        b_type = ab_type;
     hipStream_t stream = as_stream(stream_);
     TraceScope trace(atomic_add ? "TMATMUL+TSTORE_ATOMIC_ADD"
                                 : (qwords ? "TMATMUL+TSTORE_FP" : (bias ? "TMATMUL_BIAS" : (c_in ? "TMATMUL_ACC" : "TMATMUL"))),
                      "cube", m, n, k);
-    trace.in(a, m, k, "ND", ab_type).in(b, k, n, b_layout == PTOAMD_B_DN ? "DN" : "ND", ab_type)
+    trace.in(a, m, k, "ND", ab_type).in(b, k, n, b_layout == PTOAMD_B_DN ? "DN" : "ND", b_type)
         .in(c_in, m, n, "ND", ab_type == PTOAMD_I8 ? PTOAMD_I32 : PTOAMD_F32).in(bias, 1, n, "ND", ab_type == PTOAMD_I8 ? PTOAMD_I32 : PTOAMD_F32)
         .in(qwords, 1, q_per_column ? n : 1, "ND", 101).out(c, m, n, "ND", c_type);
     PTOAMD_REQUIRE(c && a && b, PTOAMD_E_INVALID, "ptoamd_gemm: null operand");
@@ -521,7 +532,7 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
         g.m = m; g.n = n; g.k = k; g.lda = lda; g.ldc = ldc;
         g.sbk = b_layout == PTOAMD_B_DN ? 1 : ldb;
         g.sbn = b_layout == PTOAMD_B_DN ? ldb : 1;
-        g.a_type = g.b_type = ab_type; g.out_kind = out_kind; g.relu = relu;
+        g.a_type = ab_type; g.b_type = b_type; g.out_kind = out_kind; g.relu = relu;
         g.qwords = qwords; g.q_per_column = q_per_column; g.atomic_add = atomic_add;
         return launch_generic(g, stream);
     }
@@ -553,7 +564,8 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
     const int op = ab_type == PTOAMD_BF16 ? TOP_BF16
                    : ab_type == PTOAMD_F16 ? TOP_F16
                    : ab_type == PTOAMD_I8 ? TOP_I8
-                   : ab_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E5E5;
+                   : ab_type == PTOAMD_E4M3 ? (b_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E4E5)
+                                            : (b_type == PTOAMD_E5M2 ? TOP_FP8_E5E5 : TOP_FP8_E5E4);
     p.b_nd = b_in_kernel; p.b_esz = ebytes;
     const int tile = pick_tile(m, n, k_bytes, false, false, !b_in_kernel && dma_offsets_fit(m, n, lda_b, ldb_kmajor, k_bytes));
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));

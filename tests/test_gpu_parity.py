@@ -298,6 +298,26 @@ def test_config2_bf16_4096_cubed(pa, oracle):
 
 
 @pytest.mark.parametrize("tile", ALL_TILES)
+def test_plain_fp8_tmatmul_every_tile_shape(pa, oracle, tile):
+    """TMATMUL on fp8 operands without block scales runs on the scaled instruction with every scale 2^0: the DMA tiles
+    read their scale bytes from LDS, which holds E8M0 127 throughout when no scale arrays are given."""
+    r = np.random.default_rng(300 + tile)
+    for (ta, tb), (m, n, k) in zip(((ob.E4M3, ob.E4M3), (ob.E5M2, ob.E4M3), (ob.E4M3, ob.E5M2), (ob.E5M2, ob.E5M2)),
+                                   ((256, 256, 512), (200, 136, 1024), (64, 72, 128), (130, 256, 256))):
+        a, _, _, _ = _mx_inputs(r, ta, m, n, k)
+        _, b, _, _ = _mx_inputs(r, tb, m, n, k)
+        ref = oracle.matmul_fp8(a, b, b_dn=True, a_type=ta, b_type=tb)
+        with tile_env(PTOAMD_TILE=tile):
+            if ta == tb:
+                got = host(pa.gemm(dev(a), dev(b), PA_T[ta], pa.F32, pa.B_DN))
+            else:  # a mixed pair: the two types are passed separately
+                got = host(pa.gemm_fp8(dev(a), dev(b), PA_T[ta], PA_T[tb]))
+            expect_tile(pa, tile, k)
+        ua, ub = _mx_unpack(oracle, a, ta), _mx_unpack(oracle, b, tb)
+        check_f32_drain(got, ref, np.abs(ua) @ np.abs(ub).T, k, f"fp8 {m}x{n}x{k} tile {tile}", max_rel=1e-3, eps=2.0 ** -11)
+
+
+@pytest.mark.parametrize("tile", ALL_TILES)
 def test_int8_accumulators_bit_exact(pa, oracle, tile):
     r = np.random.default_rng(tile)
     for m, n, k in ((256, 256, 512), (130, 70, 208), (33, 500, 4096)):
