@@ -74,6 +74,7 @@ enum OutKind { OUT_F32 = 0, OUT_F16 = 1, OUT_BF16 = 2, OUT_I32 = 3, OUT_W8A8_BF1
 // FRAG_BYTES: operand bytes one lane feeds one MFMA; a k-step spans 2 * FRAG_BYTES of a slab row (lanes 0-31 take
 // the first half, lanes 32-63 the second), so a 128-byte slab is 128 / (2 * FRAG_BYTES) k-steps.
 struct OpBF16 {
+    static constexpr int BLK = 32, ACC_REGS = 16;
     using Acc = f32x16;
     using Elem = float;
     static constexpr int FRAG_BYTES = 16;
@@ -91,6 +92,7 @@ struct OpBF16 {
     }
 };
 struct OpF16 {
+    static constexpr int BLK = 32, ACC_REGS = 16;
     using Acc = f32x16;
     using Elem = float;
     static constexpr int FRAG_BYTES = 16;
@@ -108,6 +110,7 @@ struct OpF16 {
     }
 };
 struct OpI8 {
+    static constexpr int BLK = 32, ACC_REGS = 16;
     using Acc = i32x16;
     using Elem = int32_t;
     static constexpr int FRAG_BYTES = 16;
@@ -124,10 +127,70 @@ struct OpI8 {
         mma(c, a, b, sa, sb);
     }
 };
+// The same three operand types on the 16x16 matrix instructions (k = 32 elements of 16 bits, 64 of 8 bits): a block is
+// 16 x 16, the four lane groups of 16 take consecutive 16-byte chunks, so a k-step spans 64 bytes of a slab row.  Lane
+// (l % 16, l / 16) holds row l % 16 of the (transposed) block and its columns 4 (l / 16) .. + 3.  Per FLOP these
+// instructions draw less power than the 32x32 forms: a loop of nothing but MFMAs on random operands sustains 1.97 GHz
+// (bf16) and 2.18 GHz (int8) against 1.74 and 1.85 GHz, which is what bounds the large tiles.
+struct OpBF16x16 {
+    static constexpr int BLK = 16, ACC_REGS = 4;
+    using Acc = f32x4;
+    using Elem = float;
+    static constexpr int FRAG_BYTES = 16;
+    static constexpr bool SCALED = false;
+    static constexpr int GROUPS_PER_SLAB = 0;
+    __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t, uint32_t)
+    {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, b[0]), __builtin_bit_cast(bf16x8, a[0]),
+                                                    c, 0, 0, 0);
+    }
+    template <int SEL>
+    __device__ static __forceinline__ void mma_sel(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        mma(c, a, b, sa, sb);
+    }
+};
+struct OpF16x16 {
+    static constexpr int BLK = 16, ACC_REGS = 4;
+    using Acc = f32x4;
+    using Elem = float;
+    static constexpr int FRAG_BYTES = 16;
+    static constexpr bool SCALED = false;
+    static constexpr int GROUPS_PER_SLAB = 0;
+    __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t, uint32_t)
+    {
+        c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, b[0]), __builtin_bit_cast(f16x8, a[0]), c,
+                                                   0, 0, 0);
+    }
+    template <int SEL>
+    __device__ static __forceinline__ void mma_sel(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        mma(c, a, b, sa, sb);
+    }
+};
+struct OpI8x16 {
+    static constexpr int BLK = 16, ACC_REGS = 4;
+    using Acc = i32x4;
+    using Elem = int32_t;
+    static constexpr int FRAG_BYTES = 16;
+    static constexpr bool SCALED = false;
+    static constexpr int GROUPS_PER_SLAB = 0;
+    __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t, uint32_t)
+    {
+        c = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, b[0]), __builtin_bit_cast(i32x4, a[0]), c,
+                                                  0, 0, 0);
+    }
+    template <int SEL>
+    __device__ static __forceinline__ void mma_sel(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        mma(c, a, b, sa, sb);
+    }
+};
 // fp8 (E4M3 = format 0, E5M2 = format 1) through the block-scaled MFMA; each lane's 32 bytes are one MX group.
 // Without scale pointers both scales are 2^0 (E8M0 127) and the instruction is a plain fp8 TMATMUL.
 template <int AFMT, int BFMT>
 struct OpFP8 {
+    static constexpr int BLK = 32, ACC_REGS = 16;
     using Acc = f32x16;
     using Elem = float;
     static constexpr int FRAG_BYTES = 32;
@@ -177,6 +240,7 @@ constexpr bool expands_fp4 = std::is_same<Op, OpFP8<0, 0>>::value;
 
 // fp4 E2M1 (format 4): 32 elements = 16 bytes per lane = one MX group
 struct OpFP4 {
+    static constexpr int BLK = 32, ACC_REGS = 16;
     using Acc = f32x16;
     using Elem = float;
     static constexpr int FRAG_BYTES = 16;
@@ -206,11 +270,12 @@ __device__ __forceinline__ int swizzle_chunk(int row, int chunk) { return chunk 
 // 16-byte fragments: the two lane halves take consecutive chunks.  32-byte fp8 fragments of the 32x32x64 scaled MFMA:
 // registers 0-3 of a lane belong to the k-step's first MX block (32 elements) and registers 4-7 to its second, each
 // block being split 16 + 16 bytes over the two lane halves, while lane half h supplies the E8M0 scale of block h.
-template <int FR>
+// (LG lane groups per wave: 2 for the 32x32 instructions, 4 for the 16x16 ones, which have 16-byte fragments only.)
+template <int FR, int LG = 2>
 __device__ __forceinline__ int frag_chunk(int s, int lhi, int f)
 {
     if (FR == 1)
-        return 2 * s + lhi;
+        return LG * s + lhi;
     return 4 * s + 2 * f + lhi;
 }
 
@@ -220,9 +285,10 @@ struct TileCfg {
     using Op = Op_;
     static constexpr int THREADS = WAVES_M * WAVES_N * 64;
     static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;  // per-wave output tile
-    static constexpr int MB = WTM / 32, NB = WTN / 32;            // 32x32 MFMA blocks per wave
+    static constexpr int BLK = Op::BLK, LG = 64 / BLK;            // MFMA block edge; lane groups of BLK lanes per wave
+    static constexpr int MB = WTM / BLK, NB = WTN / BLK;          // MFMA blocks per wave
     static constexpr int SLAB = 128;                              // bytes of K per slab row
-    static constexpr int KSTEPS = SLAB / (2 * Op::FRAG_BYTES);
+    static constexpr int KSTEPS = SLAB / (LG * Op::FRAG_BYTES);
     static constexpr int A_BYTES = BM * SLAB, B_BYTES = BN * SLAB, STAGE_BYTES = A_BYTES + B_BYTES;
     // the direct-to-LDS kernel of a block-scaled operand type keeps two buffers of 16 scale bytes per tile row behind
     // the operand ring
@@ -230,6 +296,7 @@ struct TileCfg {
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES + SCALE_BYTES;
     static constexpr int LA = BM * 8 / THREADS, LB = BN * 8 / THREADS;  // 16-byte chunks per thread per slab
     static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "wave tiles are made of 32x32 blocks");
+    static_assert(BLK == 32 || Op::FRAG_BYTES == 16, "the 16x16 instructions take 16-byte fragments");
     static_assert((BM * 8) % THREADS == 0 && (BN * 8) % THREADS == 0, "slab chunks must divide over the workgroup");
 };
 
@@ -240,7 +307,9 @@ struct TileCfg {
 // or 256 accumulator registers per lane pushes them through scratch memory.  The TMATMUL_ACC input is folded in here:
 // C = Cin + A.B.
 // column (inside its 32x32 block) of accumulator register r of a lane in half lhi
-__device__ __forceinline__ constexpr int acc_col(int r, int lhi) { return 8 * (r >> 2) + 4 * lhi + (r & 3); }
+// (a 16x16 block has one quad per lane: column 4 (lane / 16) + r)
+template <int BLK = 32>
+__device__ __forceinline__ constexpr int acc_col(int r, int lhi) { return BLK == 32 ? 8 * (r >> 2) + 4 * lhi + (r & 3) : 4 * lhi + r; }
 
 // The optional terms (accumulator input, bias row, relu) are applied in passes over the block's 16 registers, one
 // wave-uniform branch per term and block; tested per element they turn the epilogue into thousands of basic blocks,
@@ -254,23 +323,23 @@ __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int 
     const Elem* cin = reinterpret_cast<const Elem*>(p.c_in);
     if (cin != nullptr) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int gj = col_b + acc_col(r, lhi);
+        for (int r = 0; r < Cfg::Op::ACC_REGS; ++r) {
+            const int gj = col_b + acc_col<Cfg::BLK>(r, lhi);
             if (FULL || (gi < p.m && gj < p.n))
                 v[r] += cin[(long)gi * p.ldc + gj];
         }
     }
     if (p.bias != nullptr) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int gj = col_b + acc_col(r, lhi);
+        for (int r = 0; r < Cfg::Op::ACC_REGS; ++r) {
+            const int gj = col_b + acc_col<Cfg::BLK>(r, lhi);
             if (FULL || gj < p.n)
                 v[r] += reinterpret_cast<const Elem*>(p.bias)[gj];
         }
     }
     if (RELU && p.relu) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
+        for (int r = 0; r < Cfg::Op::ACC_REGS; ++r)
             v[r] = v[r] > 0 ? v[r] : 0;
     }
     return v;
@@ -333,8 +402,8 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
     const Acc v = tstore_terms<FULL, !out_quant<KIND>, Cfg>(p, acc, gi, col_b, lhi);
     const bool raw = KIND == OUT_W8A8_BF16 && p.acc_out != nullptr;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int gj = col_b + acc_col(r, lhi);
+    for (int r = 0; r < Cfg::Op::ACC_REGS; ++r) {
+        const int gj = col_b + acc_col<Cfg::BLK>(r, lhi);
         if (FULL || (gi < p.m && gj < p.n)) {
             const long o = (long)gi * p.ldc + gj;
             const float cs = KIND == OUT_W8A8_BF16 ? p.col_scale[gj] : 1.0f;
@@ -380,7 +449,7 @@ __device__ __forceinline__ void tstore_block_kind(const TileGemmParams& p, const
 }
 
 // ---- TSTORE through LDS ------------------------------------------------------------------------------------------------
-// A wave converts one 32-row band of its tile into a private, padded LDS region -- a lane writes its four consecutive
+// A wave converts one band (32 or 16 rows, the MFMA block's height) of its tile into a private, padded LDS region -- a lane writes its four consecutive
 // columns of a register quad as one 8-byte (16-bit outputs) or 16-byte (32-bit outputs) piece -- reads the band back as
 // 16-byte row chunks and stores whole row pieces of the wave tile's width.  LDS operations of one wave execute in
 // order, so the region is reused for the next band without a barrier.
@@ -389,7 +458,7 @@ struct StagedStore {
     // sized for 4-byte outputs; the 16 pad bytes per row keep the 32 rows a band's lanes write off each other's banks
     static constexpr int WAVE_BYTES = 32 * (Cfg::WTN * 4 + 16);
     static_assert(Cfg::THREADS / 64 * WAVE_BYTES <= Cfg::LDS_BYTES, "staging regions fit in the operand ring");
-    static_assert((32 * Cfg::WTN / 16) % 64 == 0, "a band is a whole number of 64-lane reads, down to one-byte outputs");
+    static_assert((Cfg::BLK * Cfg::WTN / 16) % 64 == 0, "a band is a whole number of 64-lane reads, down to one-byte outputs");
 };
 
 // `stage` is the calling wave's private LDS region of StagedStore<Cfg>::WAVE_BYTES bytes; the wave's tile lies inside
@@ -399,34 +468,36 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
                                               int l32, int lhi, uint8_t* stage)
 {
     constexpr int ESZ = out_bytes<KIND>;
-    constexpr int ROW_BYTES = Cfg::WTN * ESZ + 16, CHUNKS = Cfg::WTN * ESZ / 16, ITERS = 32 * CHUNKS / 64;
-    const int lane = lhi * 32 + l32;
+    constexpr int ROW_BYTES = Cfg::WTN * ESZ + 16, CHUNKS = Cfg::WTN * ESZ / 16, ITERS = Cfg::BLK * CHUNKS / 64;
+    constexpr int BLK = Cfg::BLK;
+    const int lane = lhi * BLK + l32;
     static_for<Cfg::MB>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        const int gi = row0 + i * 32 + l32;
+        const int gi = row0 + i * BLK + l32;
         const float rs = KIND == OUT_W8A8_BF16 ? p.row_scale[gi] : 1.0f;
         static_for<Cfg::NB>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             __builtin_amdgcn_sched_barrier(0);
-            const int col_b = col0 + j * 32;
+            const int col_b = col0 + j * BLK;
             const Acc v = tstore_terms<true, !out_quant<KIND>, Cfg>(p, acc[i][j], gi, col_b, lhi);
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                uint8_t* dst = stage + l32 * ROW_BYTES + (j * 32 + 8 * g + 4 * lhi) * ESZ;
+            for (int g = 0; g < Cfg::Op::ACC_REGS / 4; ++g) {
+                const int qc = acc_col<BLK>(4 * g, lhi);  // first of the quad's four columns
+                uint8_t* dst = stage + l32 * ROW_BYTES + (j * BLK + qc) * ESZ;
                 if constexpr (KIND == OUT_BF16 || KIND == OUT_W8A8_BF16) {  // packed conversion: one instruction per pair
                     float f[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         f[e] = (float)v[4 * g + e];
                         if (KIND == OUT_W8A8_BF16)
-                            f[e] = __fmul_rn(__fmul_rn(f[e], rs), p.col_scale[col_b + 8 * g + 4 * lhi + e]);
+                            f[e] = __fmul_rn(__fmul_rn(f[e], rs), p.col_scale[col_b + qc + e]);
                     }
                     *reinterpret_cast<uint2*>(dst) = make_uint2(f32x2_to_bf16x2_bits(f[0], f[1]), f32x2_to_bf16x2_bits(f[2], f[3]));
                 } else {
                     uint32_t bits[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? col_b + 8 * g + 4 * lhi + e : 0] : 0;
+                        const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? col_b + qc + e : 0] : 0;
                         bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
                     }
                     if (ESZ == 4)
@@ -445,7 +516,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
             const uint4 v = *reinterpret_cast<const uint4*>(stage + row * ROW_BYTES + ch * 16);
             typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
             nt_u32x4* dst = reinterpret_cast<nt_u32x4*>(reinterpret_cast<uint8_t*>(p.c) +
-                                                        ((long)(row0 + i * 32 + row) * p.ldc + col0) * ESZ + ch * 16);
+                                                        ((long)(row0 + i * BLK + row) * p.ldc + col0) * ESZ + ch * 16);
             const nt_u32x4 vv = {v.x, v.y, v.z, v.w};
             __builtin_nontemporal_store(vv, dst);  // C is not read again by this kernel: keep it out of the L2's way
         }
@@ -486,7 +557,7 @@ __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::
         const Acc block = acc[i][j];
         // (bounds-checked also where the wave's tile lies inside the matrix: this form is store-bound either way, and a
         // second, unchecked copy of every output kind costs more compile time than it saves run time)
-        tstore_block_kind<false, Cfg>(p, block, row0 + i * 32, col0 + j * 32, l32, lhi);
+        tstore_block_kind<false, Cfg>(p, block, row0 + i * Cfg::BLK, col0 + j * Cfg::BLK, l32, lhi);
     });
 }
 
@@ -497,6 +568,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
     using Acc = typename Op::Acc;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, LA = Cfg::LA, LB = Cfg::LB;
     constexpr int NT = Cfg::THREADS, FR = Op::FRAG_BYTES / 16;
+    static_assert(Op::BLK == 32, "the register-staged tiles use the 32x32 instructions");
     extern __shared__ __align__(16) uint8_t smem[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

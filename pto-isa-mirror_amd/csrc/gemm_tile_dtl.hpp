@@ -87,7 +87,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps the tile bookkeeping in scalar registers
     const int wm = wave % Cfg::WAVES_M, wn = wave / Cfg::WAVES_M;
-    const int l32 = lane & 31, lhi = lane >> 5;
+    // l32: the lane's row inside an MFMA block (32 or 16 rows), lhi: its lane group (0-1 or 0-3)
+    constexpr int BLK = Cfg::BLK, LG = Cfg::LG;
+    const int l32 = lane % BLK, lhi = lane / BLK;
 
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
     const int grid = tiles_m * tiles_n;
@@ -194,10 +196,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
             for (int w = 0; w < SW; ++w) {
 #pragma unroll
                 for (int i = 0; i < MB; ++i)
-                    sca_n[i][w] = *reinterpret_cast<const uint32_t*>(base + (wm * Cfg::WTM + i * 32 + l32) * 16 + w * 4);
+                    sca_n[i][w] = *reinterpret_cast<const uint32_t*>(base + (wm * Cfg::WTM + i * BLK + l32) * 16 + w * 4);
 #pragma unroll
                 for (int j = 0; j < NB; ++j)
-                    scb_n[j][w] = *reinterpret_cast<const uint32_t*>(base + (BM + wn * Cfg::WTN + j * 32 + l32) * 16 + w * 4);
+                    scb_n[j][w] = *reinterpret_cast<const uint32_t*>(base + (BM + wn * Cfg::WTN + j * BLK + l32) * 16 + w * 4);
             }
         }
     };
@@ -209,12 +211,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
+            for (int r = 0; r < Op::ACC_REGS; ++r)
                 acc[i][j][r] = 0;
-    // ---- fragment addressing.  A lane reads row l32 of every 32-row block of its wave tile; blocks are 32 * 128 bytes
+    // ---- fragment addressing.  A lane reads row l32 of every block of its wave tile; blocks are BLK * 128 bytes
     // apart and the swizzle depends on row % 16 only, so one lane-constant per operand serves all blocks: the byte
-    // offset of (row, chunk lhi ^ swizzle).  Chunk c = c0 + lhi with c0 even, and (c0 + lhi) ^ swz = c0 ^ (lhi ^ swz),
-    // so the address of chunk c is that constant XOR (c0 << 4): one VALU op per k-step piece, shared by the blocks.
+    // offset of (row, chunk lhi ^ swizzle).  Chunk c = c0 + lhi with c0 a multiple of the lane-group count, and
+    // (c0 + lhi) ^ swz = c0 ^ (lhi ^ swz), so the address of chunk c is that constant XOR (c0 << 4): one VALU op per
+    // k-step piece, shared by the blocks.
     static_assert(Cfg::WTM % 32 == 0 && Cfg::WTN % 32 == 0, "wave tiles start on 32-row boundaries");
     const uint32_t fa_lane = (wm * Cfg::WTM + l32) * 128 + ((lhi ^ swizzle_chunk(l32, 0)) << 4);
     const uint32_t fb_lane = Cfg::A_BYTES + (wn * Cfg::WTN + l32) * 128 + ((lhi ^ swizzle_chunk(l32, 0)) << 4);
@@ -225,7 +228,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // (128 registers per lane) keep one set, refilled piecewise, and the SIMD's other waves cover the LDS latency.
     // (The hybrid read schedule needs one first-column MFMA per double-buffered fragment, NB + 1 <= MB; the square wave
     // tile of the 4-wave form has accumulators for 16 blocks and keeps the single set.)
-    constexpr bool BIG_FRAGS = FR == 2 && MB * NB >= 8;
+    constexpr bool BIG_FRAGS = (MB + NB) * FR >= 12;  // 48 or more registers per fragment set
     constexpr bool HYBRID = BIG_FRAGS && NT <= 512 && NB + 1 <= MB;
     constexpr int SETS = (NT > 512 || (BIG_FRAGS && !HYBRID)) ? 1 : 2;
     uint4 fa[SETS][MB][FR], fb[SETS][NB][FR];
@@ -236,10 +239,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         const uint8_t* base = smem + buf * Cfg::STAGE_BYTES;
         if (q < NB * FR) {
             const int j = q / FR, f = q % FR;
-            fb[set][j][f] = *reinterpret_cast<const uint4*>(base + (fb_lane ^ (frag_chunk<FR>(s, 0, f) << 4)) + j * (32 * 128));
+            fb[set][j][f] = *reinterpret_cast<const uint4*>(base + (fb_lane ^ (frag_chunk<FR, LG>(s, 0, f) << 4)) + j * (BLK * 128));
         } else {
             const int i = (q - NB * FR) / FR, f = (q - NB * FR) % FR;
-            fa[set][i][f] = *reinterpret_cast<const uint4*>(base + (fa_lane ^ (frag_chunk<FR>(s, 0, f) << 4)) + i * (32 * 128));
+            fa[set][i][f] = *reinterpret_cast<const uint4*>(base + (fa_lane ^ (frag_chunk<FR, LG>(s, 0, f) << 4)) + i * (BLK * 128));
         }
     };
     // One k-step: the MFMAs of step s (register set s & 1), with the fragment reads of the next step (register set

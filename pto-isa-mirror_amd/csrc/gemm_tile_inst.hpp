@@ -32,7 +32,11 @@ hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 {
     switch (tile) {
         case 3: return launch_dtl<TileCfg<256, 256, 2, 2, PTOAMD_TILE_OP>>(p, stream);
+#ifdef PTOAMD_TILE_OP16  // the large eight-wave tile runs on the 16x16 instructions where the operand type has them
+        case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP16>>(p, stream);
+#else
         case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>>(p, stream);
+#endif
         case 5: return launch_dtl<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>>(p, stream);
         case 6: return launch_dtl<TileCfg<256, 128, 4, 2, PTOAMD_TILE_OP>>(p, stream);
         case 0: return launch_cfg<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>>(p, stream);

@@ -24,7 +24,18 @@ using namespace ptoamd;
 #ifndef PROBE_KIND
 #define PROBE_KIND 0
 #endif
-#if PROBE_KIND == 0
+#ifndef PROBE_BLK
+#define PROBE_BLK 16  // MFMA block edge of the bf16 / int8 kinds: 16 (the shipped tile) or 32
+#endif
+#if PROBE_KIND == 0 && PROBE_BLK == 16
+using ProbeOp = OpBF16x16;
+constexpr int ESZ = 2, CSZ = 2, OUT = OUT_BF16;
+constexpr const char* KIND = "bf16 (16x16x32)";
+#elif PROBE_KIND == 1 && PROBE_BLK == 16
+using ProbeOp = OpI8x16;
+constexpr int ESZ = 1, CSZ = 4, OUT = OUT_I32;
+constexpr const char* KIND = "int8 (16x16x64)";
+#elif PROBE_KIND == 0
 using ProbeOp = OpBF16;
 constexpr int ESZ = 2, CSZ = 2, OUT = OUT_BF16;
 constexpr const char* KIND = "bf16";
