@@ -449,7 +449,7 @@ __device__ __forceinline__ void tstore_block_kind(const TileGemmParams& p, const
 }
 
 // ---- TSTORE through LDS ------------------------------------------------------------------------------------------------
-// A wave converts one band (32 or 16 rows, the MFMA block's height) of its tile into a private, padded LDS region -- a lane writes its four consecutive
+// A wave converts one 32-row band (one or two block rows) of its tile into a private, padded LDS region -- a lane writes its four consecutive
 // columns of a register quad as one 8-byte (16-bit outputs) or 16-byte (32-bit outputs) piece -- reads the band back as
 // 16-byte row chunks and stores whole row pieces of the wave tile's width.  LDS operations of one wave execute in
 // order, so the region is reused for the next band without a barrier.
@@ -458,7 +458,7 @@ struct StagedStore {
     // sized for 4-byte outputs; the 16 pad bytes per row keep the 32 rows a band's lanes write off each other's banks
     static constexpr int WAVE_BYTES = 32 * (Cfg::WTN * 4 + 16);
     static_assert(Cfg::THREADS / 64 * WAVE_BYTES <= Cfg::LDS_BYTES, "staging regions fit in the operand ring");
-    static_assert((Cfg::BLK * Cfg::WTN / 16) % 64 == 0, "a band is a whole number of 64-lane reads, down to one-byte outputs");
+    static_assert((32 * Cfg::WTN / 16) % 64 == 0, "a band is a whole number of 64-lane reads, down to one-byte outputs");
 };
 
 // `stage` is the calling wave's private LDS region of StagedStore<Cfg>::WAVE_BYTES bytes; the wave's tile lies inside
@@ -467,47 +467,51 @@ template <int KIND, class Cfg, class Acc>
 __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0,
                                               int l32, int lhi, uint8_t* stage)
 {
-    constexpr int ESZ = out_bytes<KIND>;
-    constexpr int ROW_BYTES = Cfg::WTN * ESZ + 16, CHUNKS = Cfg::WTN * ESZ / 16, ITERS = Cfg::BLK * CHUNKS / 64;
-    constexpr int BLK = Cfg::BLK;
+    constexpr int ESZ = out_bytes<KIND>, BLK = Cfg::BLK;
+    constexpr int BPB = 32 / BLK;  // block rows per 32-row band (two for the 16x16 instructions)
+    constexpr int ROW_BYTES = Cfg::WTN * ESZ + 16, CHUNKS = Cfg::WTN * ESZ / 16, ITERS = 32 * CHUNKS / 64;
     const int lane = lhi * BLK + l32;
-    static_for<Cfg::MB>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        const int gi = row0 + i * BLK + l32;
-        const float rs = KIND == OUT_W8A8_BF16 ? p.row_scale[gi] : 1.0f;
-        static_for<Cfg::NB>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            __builtin_amdgcn_sched_barrier(0);
-            const int col_b = col0 + j * BLK;
-            const Acc v = tstore_terms<true, !out_quant<KIND>, Cfg>(p, acc[i][j], gi, col_b, lhi);
+    static_for<Cfg::MB / BPB>([&](auto bc) {
+        constexpr int band = decltype(bc)::value;
+        static_for<BPB>([&](auto hc) {
+            constexpr int i = band * BPB + decltype(hc)::value;
+            const int srow = decltype(hc)::value * BLK + l32;  // row inside the band
+            const int gi = row0 + i * BLK + l32;
+            const float rs = KIND == OUT_W8A8_BF16 ? p.row_scale[gi] : 1.0f;
+            static_for<Cfg::NB>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                __builtin_amdgcn_sched_barrier(0);
+                const int col_b = col0 + j * BLK;
+                const Acc v = tstore_terms<true, !out_quant<KIND>, Cfg>(p, acc[i][j], gi, col_b, lhi);
 #pragma unroll
-            for (int g = 0; g < Cfg::Op::ACC_REGS / 4; ++g) {
-                const int qc = acc_col<BLK>(4 * g, lhi);  // first of the quad's four columns
-                uint8_t* dst = stage + l32 * ROW_BYTES + (j * BLK + qc) * ESZ;
-                if constexpr (KIND == OUT_BF16 || KIND == OUT_W8A8_BF16) {  // packed conversion: one instruction per pair
-                    float f[4];
+                for (int g = 0; g < Cfg::Op::ACC_REGS / 4; ++g) {
+                    const int qc = acc_col<BLK>(4 * g, lhi);  // first of the quad's four columns
+                    uint8_t* dst = stage + srow * ROW_BYTES + (j * BLK + qc) * ESZ;
+                    if constexpr (KIND == OUT_BF16 || KIND == OUT_W8A8_BF16) {  // packed conversion: one instruction per pair
+                        float f[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        f[e] = (float)v[4 * g + e];
-                        if (KIND == OUT_W8A8_BF16)
-                            f[e] = __fmul_rn(__fmul_rn(f[e], rs), p.col_scale[col_b + qc + e]);
+                        for (int e = 0; e < 4; ++e) {
+                            f[e] = (float)v[4 * g + e];
+                            if (KIND == OUT_W8A8_BF16)
+                                f[e] = __fmul_rn(__fmul_rn(f[e], rs), p.col_scale[col_b + qc + e]);
+                        }
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(f32x2_to_bf16x2_bits(f[0], f[1]), f32x2_to_bf16x2_bits(f[2], f[3]));
+                    } else {
+                        uint32_t bits[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? col_b + qc + e : 0] : 0;
+                            bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
+                        }
+                        if (ESZ == 4)
+                            *reinterpret_cast<uint4*>(dst) = make_uint4(bits[0], bits[1], bits[2], bits[3]);
+                        else if (ESZ == 2)
+                            *reinterpret_cast<uint2*>(dst) = make_uint2(bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16));
+                        else
+                            *reinterpret_cast<uint32_t*>(dst) = bits[0] | (bits[1] << 8) | (bits[2] << 16) | (bits[3] << 24);
                     }
-                    *reinterpret_cast<uint2*>(dst) = make_uint2(f32x2_to_bf16x2_bits(f[0], f[1]), f32x2_to_bf16x2_bits(f[2], f[3]));
-                } else {
-                    uint32_t bits[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? col_b + qc + e : 0] : 0;
-                        bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
-                    }
-                    if (ESZ == 4)
-                        *reinterpret_cast<uint4*>(dst) = make_uint4(bits[0], bits[1], bits[2], bits[3]);
-                    else if (ESZ == 2)
-                        *reinterpret_cast<uint2*>(dst) = make_uint2(bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16));
-                    else
-                        *reinterpret_cast<uint32_t*>(dst) = bits[0] | (bits[1] << 8) | (bits[2] << 16) | (bits[3] << 24);
                 }
-            }
+            });
         });
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -516,7 +520,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
             const uint4 v = *reinterpret_cast<const uint4*>(stage + row * ROW_BYTES + ch * 16);
             typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
             nt_u32x4* dst = reinterpret_cast<nt_u32x4*>(reinterpret_cast<uint8_t*>(p.c) +
-                                                        ((long)(row0 + i * BLK + row) * p.ldc + col0) * ESZ + ch * 16);
+                                                        ((long)(row0 + band * 32 + row) * p.ldc + col0) * ESZ + ch * 16);
             const nt_u32x4 vv = {v.x, v.y, v.z, v.w};
             __builtin_nontemporal_store(vv, dst);  // C is not read again by this kernel: keep it out of the L2's way
         }

@@ -57,15 +57,22 @@ __device__ __forceinline__ void sched_kstep()
 #ifndef PTOAMD_DMA_PHASES
 #define PTOAMD_DMA_PHASES 4, 4
 #endif
-template <int NDMA, int KS>
+// The 16x16 instructions' slab has two long k-steps (32 MFMAs of a 128 x 64 wave tile each); their phase 1 is the FIRST
+// HALF of the next slab's first k-step, half a k-step ahead of the barrier that needs the data.
+#ifndef PTOAMD_DMA_PHASES_16
+#define PTOAMD_DMA_PHASES_16 8
+#endif
+template <int NDMA, int KS, int BLK = 32>
 __host__ __device__ constexpr int dma_phase_begin(int phase)
 {
-    constexpr int share[] = {PTOAMD_DMA_PHASES};
-    constexpr int n = sizeof(share) / sizeof(share[0]);
+    constexpr int share32[] = {PTOAMD_DMA_PHASES};
+    constexpr int share16[] = {PTOAMD_DMA_PHASES_16};
+    constexpr int n = BLK == 16 ? sizeof(share16) / sizeof(share16[0]) : sizeof(share32) / sizeof(share32[0]);
     int eighths = 0;
     for (int f = 0; f < phase && f < n; ++f)
-        eighths += share[f];
-    if (phase >= n || phase >= KS || (KS < 4 && phase >= 1))  // two k-steps per slab: phase 1 would be the k-step before the barrier
+        eighths += BLK == 16 ? share16[f] : share32[f];
+    // two k-steps per slab of the 32x32 instructions (fp8): phase 1 would be the k-step before the barrier
+    if (phase >= n || phase >= KS || (KS < 4 && BLK == 32 && phase >= 1))
         eighths = 8;
     return eighths * NDMA / 8;
 }
@@ -118,7 +125,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
 
     const uint32_t lds_wave_base = __builtin_amdgcn_readfirstlane(lds_address(smem) + wave * 1024);
     // DMA number q (0 .. LA + LB - 1) of slab kt into ring buffer buf
-    auto tload_piece = [&](int kt, int buf, int q) {
+    auto tload_piece = [&](int kt, int buf, int q) __attribute__((always_inline)) {
 #if defined(PTOAMD_CLOCK_PROBE) && defined(PTOAMD_PROBE_DMA_EVERY)
         // timing experiment (results are wrong): after the first two slabs issue no DMA (0) or every n-th piece only
         if (kt > 1 && (PTOAMD_PROBE_DMA_EVERY == 0 || q % (PTOAMD_PROBE_DMA_EVERY ? PTOAMD_PROBE_DMA_EVERY : 1) != 0))
@@ -130,7 +137,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         else
             lds_dma16_off(p.b + (long)kt * 128, goff_b[q - LA], dst + Cfg::A_BYTES + (q - LA) * (NT * 16));
     };
-    auto tload = [&](int kt, int buf) {
+    auto tload = [&](int kt, int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int q = 0; q < LA + LB; ++q)
             tload_piece(kt, buf, q);
@@ -175,7 +182,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
                                : p.sb + (long)min(n0 + max(r - BM, 0), p.n - 1) * p.scale_ld;
         }
     }
-    auto tload_scales = [&](int g) {
+    auto tload_scales = [&](int g) __attribute__((always_inline)) {
         if (has_scales) {
 #pragma unroll
             for (int w = 0; w < NSW; ++w) {
@@ -189,7 +196,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // (No test of has_scales here: a branch between two k-steps lets the compiler sink the earlier k-step's MFMAs
     // below it, away from the fragment reads they should overlap.  Without scale arrays the LDS scale area is filled
     // with E8M0 127 once, in the prologue.)
-    auto read_scales = [&](int kt) {
+    auto read_scales = [&](int kt) __attribute__((always_inline)) {
         if (Op::SCALED) {
             const uint8_t* base = smem + 2 * Cfg::STAGE_BYTES + ((kt / SPG) & 1) * (SROWS * 16) + (kt % SPG) * GPS;
 #pragma unroll
@@ -235,7 +242,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     constexpr int NREAD = (MB + NB) * FR, NMMA = MB * NB, NDMA = LA + LB;
     // fragment read number q of k-step s of ring buffer buf into register set `set`; B fragments come first because the
     // first MFMAs of a k-step need all of B's first block but only A's first
-    auto textract_piece = [&](int set, int buf, int s, int q) {
+    auto textract_piece = [&](int set, int buf, int s, int q) __attribute__((always_inline)) {
         const uint8_t* base = smem + buf * Cfg::STAGE_BYTES;
         if (q < NB * FR) {
             const int j = q / FR, f = q % FR;
@@ -247,8 +254,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     };
     // One k-step: the MFMAs of step s (register set s & 1), with the fragment reads of the next step (register set
     // (s + 1) & 1, from buffer rbuf step rs) and, in a slab's last step, the DMAs of slab dkt spread between them.
-    auto kstep = [&](auto phase, int s, bool reads, int rbuf, int rs, bool dmas, int dkt, int dbuf) {
-        constexpr int DQ0 = dma_phase_begin<NDMA, KS>(decltype(phase)::value), DN = dma_phase_begin<NDMA, KS>(decltype(phase)::value + 1) - DQ0;
+    auto kstep = [&](auto phase, int s, bool reads, int rbuf, int rs, bool dmas, int dkt, int dbuf) __attribute__((always_inline)) {
+        constexpr int PH = decltype(phase)::value;
+        constexpr int DQ0 = dma_phase_begin<NDMA, KS, BLK>(PH), DN = dma_phase_begin<NDMA, KS, BLK>(PH + 1) - DQ0;
+        constexpr int DSPAN = (BLK == 16 && PH > 0) ? NMMA / 2 : NMMA;  // MFMAs the phase's DMAs are spread over
         const int set = SETS == 2 ? (s & 1) : 0;
         const int nset = SETS == 2 ? (set ^ 1) : 0;
         static_for<NMMA>([&](auto xc) {
@@ -289,7 +298,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
                 }
             }
             if (dmas) {
-                constexpr int q0 = DQ0 + x * DN / NMMA, q1 = DQ0 + (x + 1) * DN / NMMA;
+                constexpr int xa = x < DSPAN ? x : DSPAN, xb = x + 1 < DSPAN ? x + 1 : DSPAN;
+                constexpr int q0 = DQ0 + xa * DN / DSPAN, q1 = DQ0 + xb * DN / DSPAN;
                 static_for<q1 - q0>([&](auto qc) { tload_piece(dkt, dbuf, q0 + decltype(qc)::value); });
             }
         });
@@ -305,7 +315,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
             *reinterpret_cast<uint4*>(smem + 2 * Cfg::STAGE_BYTES + o) = make_uint4(0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu);
     }
     if (k_slabs > 1)
-        static_for<dma_phase_begin<NDMA, KS>(1)>([&](auto qc) { tload_piece(1, 1, decltype(qc)::value); });
+        static_for<dma_phase_begin<NDMA, KS, BLK>(1)>([&](auto qc) { tload_piece(1, 1, decltype(qc)::value); });
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMAs have landed
     __syncthreads();
 #pragma unroll
@@ -318,7 +328,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
 
     // One slab.  `more` = slab kt+1 exists (read its first fragments in the last k-step), `dma` = slab kt+2 exists
     // (start its DMA into the buffer this slab frees); both are literal at the call sites so the branches fold.
-    auto slab = [&](int kt, bool more, bool dma) {
+    // (always_inline: out of line, a lambda takes the accumulators by reference and they live in scratch memory)
+    auto slab = [&](int kt, bool more, bool dma) __attribute__((always_inline)) {
         const int cur = kt & 1;
         if (Op::SCALED) {
             // The request for the next scale chunk sits here, at the top of the slab, and not between two k-steps: a
