@@ -2,7 +2,7 @@
 //
 //   TLOAD (GM -> L1 Mat tile)        128-bit coalesced global loads of a [rows][128 B] K-slab, staged into LDS
 //   TMOV/TEXTRACT (L1 -> L0A/L0B)    ds_read_b128 of MFMA operand fragments from the swizzled LDS slab
-//   TMATMUL / TMATMUL_ACC (Cube)     v_mfma_* on 32x32 blocks, accumulators (the L0C Acc tile) live in registers
+//   TMATMUL / TMATMUL_ACC (Cube)     v_mfma_* on 32x32 (or 16x16) blocks, accumulators (the L0C Acc tile) live in registers
 //   TSTORE (L0C -> GM, fix-pipe)     register epilogue: relu / dequant scales / f32->bf16|f16 RNE, then global stores
 //
 // Both operands are read K-contiguous: A is [M][K] row-major and B is [N][K] (Layout::DN).  A K-slab is 128 bytes per

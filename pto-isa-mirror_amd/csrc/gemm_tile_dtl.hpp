@@ -356,9 +356,17 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
             kstep(std::integral_constant<int, s + 1>{}, s, true, cur, s + 1, more, kt + 1, cur ^ 1);
         });
         // every wave is done reading slab kt, and its DMAs of slab kt+1 (issued one slab ago) have landed
+#if defined(PTOAMD_CLOCK_PROBE) && defined(PTOAMD_PROBE_NO_BARRIER)  // timing experiment (results are wrong)
+        __builtin_amdgcn_sched_barrier(0);
+#else
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
+#endif
+#if defined(PTOAMD_CLOCK_PROBE) && defined(PTOAMD_PROBE_NO_SCALE_READS)
+        if (false)
+#else
         if (SC_AHEAD && more)
+#endif
             read_scales(kt + 1);
         kstep(std::integral_constant<int, 0>{}, KS - 1, more, cur ^ 1, 0, dma, kt + 2, cur);
     };
