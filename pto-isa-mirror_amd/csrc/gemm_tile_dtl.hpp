@@ -314,9 +314,16 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         for (int o = tid * 16; o < 2 * SROWS * 16; o += NT * 16)
             *reinterpret_cast<uint4*>(smem + 2 * Cfg::STAGE_BYTES + o) = make_uint4(0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu);
     }
-    if (k_slabs > 1)
-        static_for<dma_phase_begin<NDMA, KS, BLK>(1)>([&](auto qc) { tload_piece(1, 1, decltype(qc)::value); });
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMAs have landed
+    // slab 1's first DMAs go out now but only slab 0 (and the scales) are waited for: the counter retires loads in
+    // order, so "at most N1 outstanding" means everything issued before slab 1's pieces has landed; slab 1 is covered
+    // by the first slab's barrier
+    constexpr int N1 = dma_phase_begin<NDMA, KS, BLK>(1);
+    if (k_slabs > 1) {
+        static_for<N1>([&](auto qc) { tload_piece(1, 1, decltype(qc)::value); });
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (N1 & 15) | ((N1 >> 4) << 14));  // vmcnt(N1)
+    } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMAs have landed
+    }
     __syncthreads();
 #pragma unroll
     for (int q = 0; q < NREAD; ++q)
