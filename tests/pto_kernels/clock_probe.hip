@@ -51,7 +51,13 @@ constexpr const char* KIND = "MXFP8";
 #ifndef PROBE_WAVES_N
 #define PROBE_WAVES_N 4  // 4: eight waves with 128 x 64 wave tiles (the default tile); 2: four waves with 128 x 128 wave tiles
 #endif
-using Cfg = TileCfg<256, 256, 2, PROBE_WAVES_N, ProbeOp>;
+#ifndef PROBE_BN
+#define PROBE_BN 256  // tile width: 256, or 128 (with PROBE_WAVES_N=2: the four-wave 256 x 128 tile)
+#endif
+#ifndef PROBE_WAVES_M
+#define PROBE_WAVES_M 2
+#endif
+using Cfg = TileCfg<256, PROBE_BN, PROBE_WAVES_M, PROBE_WAVES_N, ProbeOp>;
 
 #define CK(x)                                                                          \
     do {                                                                               \
@@ -70,13 +76,15 @@ int main(int argc, char** argv)
         return 2;
     }
     const size_t kb = (size_t)k * ESZ;
-    if ((size_t)(std::max(m, n) - 1) * kb + kb > 0xffffffffull) {
+    // row pitch of A and B: the K extent plus PTOAMD_PROBE_PITCH_PAD bytes (a multiple of 16; default 0 = contiguous rows)
+    const size_t pitch = kb + (getenv("PTOAMD_PROBE_PITCH_PAD") ? atoi(getenv("PTOAMD_PROBE_PITCH_PAD")) : 0);
+    if ((size_t)(std::max(m, n) - 1) * pitch + kb > 0xffffffffull || pitch % 16) {
         printf("operands must stay below 4 GiB (32-bit DMA offsets)\n");
         return 2;
     }
     // operand bytes: 16-bit patterns 0x3c00 + 10 random bits with a random sign are bf16 values of magnitude 1 - 2; as
     // byte pairs they are ordinary int8 values and, with bit 3 of each byte cleared, finite E4M3 codes
-    std::vector<uint16_t> ha((size_t)m * kb / 2), hb((size_t)n * kb / 2);
+    std::vector<uint16_t> ha((size_t)m * pitch / 2), hb((size_t)n * pitch / 2);
     srand(1);
     for (auto& v : ha) v = (uint16_t)(0x3c00 + (rand() & 0x3ff) - ((rand() & 1) << 15));
     for (auto& v : hb) v = (uint16_t)(0x3c00 + (rand() & 0x3ff) - ((rand() & 1) << 15));
@@ -91,7 +99,7 @@ int main(int argc, char** argv)
     uint8_t *a, *b, *sa = nullptr, *sb = nullptr;
     void* c;
     long* stamps;
-    const int tiles = (m / 256) * (n / 256);
+    const int tiles = (m / Cfg::BM) * (n / Cfg::BN);
     CK(hipMalloc(&a, ha.size() * 2));
     CK(hipMalloc(&b, hb.size() * 2));
     CK(hipMalloc(&c, (size_t)m * n * CSZ));
@@ -113,8 +121,8 @@ int main(int argc, char** argv)
     p.m = m;
     p.n = n;
     p.k_bytes = (int)kb;
-    p.lda_bytes = (long)kb;
-    p.ldb_bytes = (long)kb;
+    p.lda_bytes = (long)pitch;
+    p.ldb_bytes = (long)pitch;
     p.ldc = n;
     p.out_kind = OUT;
     p.group_m = 4;
