@@ -27,7 +27,7 @@ DEV = "cuda:0"
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of
 # known size: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000), see profiles/gemm_tile_dtl_256x256_bf16_4096cubed.md.
-HEADLINE_TRAFFIC_BYTES = 235_105_280
+HEADLINE_TRAFFIC_BYTES = 235_224_064
 
 
 class Events:
