@@ -391,6 +391,12 @@ __device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_
     }
     return f32_to_bf16_bits(__fmul_rn(__fmul_rn((float)v, rs), cs));
 }
+// (the timing build of the DMA kernel borrows acc_out for its time stamps: no raw accumulators are written then)
+#ifdef PTOAMD_CLOCK_PROBE
+constexpr bool acc_out_is_probe = true;
+#else
+constexpr bool acc_out_is_probe = false;
+#endif
 template <int KIND>
 constexpr int out_bytes = (KIND == OUT_F32 || KIND == OUT_I32) ? 4 : (KIND == OUT_Q8 ? 1 : 2);
 template <int KIND>
@@ -404,7 +410,7 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
     const int gi = row_b + l32;
     const float rs = (KIND == OUT_W8A8_BF16 && (FULL || gi < p.m)) ? p.row_scale[gi] : 1.0f;
     const Acc v = tstore_terms<FULL, !out_quant<KIND>, Cfg>(p, acc, gi, col_b, lhi);
-    const bool raw = KIND == OUT_W8A8_BF16 && p.acc_out != nullptr;
+    const bool raw = KIND == OUT_W8A8_BF16 && p.acc_out != nullptr && !acc_out_is_probe;
 #pragma unroll
     for (int r = 0; r < Cfg::Op::ACC_REGS; ++r) {
         const int gj = col_b + acc_col<Cfg::BLK>(r, lhi);
@@ -475,13 +481,27 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
     constexpr int BPB = 32 / BLK;  // block rows per 32-row band (two for the 16x16 instructions)
     constexpr int ROW_BYTES = Cfg::WTN * ESZ + 16, CHUNKS = Cfg::WTN * ESZ / 16, ITERS = 32 * CHUNKS / 64;
     const int lane = lhi * BLK + l32;
+    // W8A8: a lane's column scales are the same for every block row of the wave tile; fetched once here (fetched where
+    // they are used they are 128 separate loads per lane, and the store phase takes twice as long)
+    float cs_pre[Cfg::NB][Cfg::Op::ACC_REGS], rs_pre[Cfg::MB];
+    if constexpr (KIND == OUT_W8A8_BF16) {
+#pragma unroll
+        for (int i = 0; i < Cfg::MB; ++i)  // the row scales likewise: one load latency instead of one per block row
+            rs_pre[i] = p.row_scale[row0 + i * BLK + l32];
+        static_for<Cfg::NB>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+#pragma unroll
+            for (int r = 0; r < Cfg::Op::ACC_REGS; ++r)
+                cs_pre[j][r] = p.col_scale[col0 + j * BLK + acc_col<BLK>(r, lhi)];
+        });
+    }
     static_for<Cfg::MB / BPB>([&](auto bc) {
         constexpr int band = decltype(bc)::value;
         static_for<BPB>([&](auto hc) {
             constexpr int i = band * BPB + decltype(hc)::value;
             const int srow = decltype(hc)::value * BLK + l32;  // row inside the band
             const int gi = row0 + i * BLK + l32;
-            const float rs = KIND == OUT_W8A8_BF16 ? p.row_scale[gi] : 1.0f;
+            const float rs = KIND == OUT_W8A8_BF16 ? rs_pre[i] : 1.0f;
             static_for<Cfg::NB>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 __builtin_amdgcn_sched_barrier(0);
@@ -497,7 +517,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
                         for (int e = 0; e < 4; ++e) {
                             f[e] = (float)v[4 * g + e];
                             if (KIND == OUT_W8A8_BF16)
-                                f[e] = __fmul_rn(__fmul_rn(f[e], rs), p.col_scale[col_b + qc + e]);
+                                f[e] = __fmul_rn(__fmul_rn(f[e], rs), cs_pre[j][4 * g + e]);
                         }
                         *reinterpret_cast<uint2*>(dst) = make_uint2(f32x2_to_bf16x2_bits(f[0], f[1]), f32x2_to_bf16x2_bits(f[2], f[3]));
                     } else {
@@ -540,7 +560,8 @@ __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::
     const bool full = row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n;
     const int esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : (p.out_kind == OUT_Q8 ? 1 : 2);
     const bool aligned = (((long)p.ldc * esz) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
-    if (stage != nullptr && full && aligned && !p.atomic_add && !(p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr)) {
+    const bool raw_acc = p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr && !acc_out_is_probe;
+    if (stage != nullptr && full && aligned && !p.atomic_add && !raw_acc) {
         if (p.out_kind >= OUT_QF16) {
             tstore_staged<OUT_QF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
         } else if (p.out_kind == OUT_Q8) {

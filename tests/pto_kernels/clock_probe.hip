@@ -1,5 +1,6 @@
 // Per-workgroup timestamps of the direct-to-LDS 256 x 256 tile GEMM kernel on one problem (default 4096^3).
-// -DPROBE_KIND=0 bf16 (default), 1 int8 -> i32, 2 MXFP8 (E4M3 x E4M3, unit block scales) -> bf16.
+// -DPROBE_KIND=0 bf16 (default), 1 int8 -> i32, 2 MXFP8 (E4M3 x E4M3, unit block scales) -> bf16, 3 W8A8 (int8 -> bf16
+// through per-row and per-column float scales).
 //
 // Compiled with -DPTOAMD_CLOCK_PROBE the kernel writes, per workgroup, eight 64-bit words through p.acc_out:
 // [0] core clocks spent in the K loop, [1] wall clock (100 MHz) at entry, [2] at the start of the K loop, [3] at its end,
@@ -35,6 +36,10 @@ constexpr const char* KIND = "bf16 (16x16x32)";
 using ProbeOp = OpI8x16;
 constexpr int ESZ = 1, CSZ = 4, OUT = OUT_I32;
 constexpr const char* KIND = "int8 (16x16x64)";
+#elif PROBE_KIND == 3
+using ProbeOp = OpI8x16;
+constexpr int ESZ = 1, CSZ = 2, OUT = OUT_W8A8_BF16;
+constexpr const char* KIND = "W8A8 int8 (16x16x64) -> bf16 with row and column scales";
 #elif PROBE_KIND == 0
 using ProbeOp = OpBF16;
 constexpr int ESZ = 2, CSZ = 2, OUT = OUT_BF16;
@@ -115,6 +120,16 @@ int main(int argc, char** argv)
     }
 
     TileGemmParams p{};
+    if (OUT == OUT_W8A8_BF16) {
+        float *rs, *cs;
+        std::vector<float> hs(std::max(m, n), 0.001f);
+        CK(hipMalloc(&rs, (size_t)m * 4));
+        CK(hipMalloc(&cs, (size_t)n * 4));
+        CK(hipMemcpy(rs, hs.data(), (size_t)m * 4, hipMemcpyHostToDevice));
+        CK(hipMemcpy(cs, hs.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+        p.row_scale = rs;
+        p.col_scale = cs;
+    }
     p.a = a;
     p.b = b;
     p.c = c;
