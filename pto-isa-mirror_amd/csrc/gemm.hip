@@ -278,7 +278,9 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
     const bool dtl_ok = (k_bytes % 128) == 0 && scale_dma_ok;
     const char* env = getenv("PTOAMD_TILE");
     if (env && env[0] >= '0' && env[0] <= '6') {
-        const int t = env[0] - '0';
+        int t = env[0] - '0';
+        if (t == 3)  // the four-wave form of the 256 x 256 DMA tile is no longer built
+            t = 4;
         if (t < 3 || dtl_ok)
             return t;
         return t == 5 ? 1 : 0;

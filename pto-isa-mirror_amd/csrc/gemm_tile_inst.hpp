@@ -31,10 +31,13 @@ static hipError_t launch_dtl(const TileGemmParams& p, hipStream_t stream)
 hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 {
     switch (tile) {
-        case 3: return launch_dtl<TileCfg<256, 256, 2, 2, PTOAMD_TILE_OP>>(p, stream);
+        // (tile id 3 was a four-wave form of the 256 x 256 tile, 128 x 128 per wave: never faster than the eight-wave form
+        // and a third of this translation unit's compile time; the id now selects tile 4)
 #ifdef PTOAMD_TILE_OP16  // the large eight-wave tile runs on the 16x16 instructions where the operand type has them
+        case 3:
         case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP16>>(p, stream);
 #else
+        case 3:
         case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>>(p, stream);
 #endif
         case 5: return launch_dtl<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>>(p, stream);

@@ -181,7 +181,7 @@ def test_operands_past_4_gib_leave_the_dma_tiles(pa, oracle):
 
 TILE_NAMES = ("tile256x256_", "tile128x128_", "tile64x64_", "tile256x256w4_dtl", "tile256x256w8_dtl", "tile128x128_dtl",
               "tile256x128_dtl")
-ALL_TILES = [0, 1, 2, 3, 4, 5, 6]
+ALL_TILES = [0, 1, 2, 4, 5, 6]  # (id 3, a four-wave form of tile 4, is no longer built and selects tile 4)
 
 
 def expect_tile(pa, tile, k_bytes):
@@ -766,7 +766,7 @@ def test_mx_block_scales_select_the_right_group(pa, oracle):
         assert relerr(got, ref) <= 2e-2, g
 
 
-@pytest.mark.parametrize("tile", [3, 4, 5, 6])
+@pytest.mark.parametrize("tile", [4, 5, 6])
 @pytest.mark.parametrize("typ", [ob.E4M3, ob.E2M1])
 def test_mx_scale_chunks_across_slabs(pa, oracle, typ, tile):
     """The DMA tiles fetch scales as 16-byte chunks per row (4 fp8 slabs / 2 fp4 slabs) into two alternating LDS
