@@ -288,7 +288,7 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
     const long t256 = (long)((m + 255) / 256) * ((n + 255) / 256);
     const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128);
     if (scaled && dtl_ok && t256 >= 128)
-        return 4;  // half the copy-in bytes per MFMA of the 128x128 tile: fp8 2.03 vs 1.84, fp4 2.5 vs 2.3 PFLOP/s
+        return 4;  // half the copy-in bytes per MFMA of the 128x128 tile
     if (scaled)
         return t128 >= 96 ? (dtl_ok ? 5 : 1) : 2;
     if (t256 >= 128)
