@@ -1,6 +1,6 @@
 // Per-workgroup timestamps of the direct-to-LDS 256 x 256 tile GEMM kernel on one problem (default 4096^3).
 // -DPROBE_KIND=0 bf16 (default), 1 int8 -> i32, 2 MXFP8 (E4M3 x E4M3, unit block scales) -> bf16, 3 W8A8 (int8 -> bf16
-// through per-row and per-column float scales).
+// through per-row and per-column float scales), 4 MXFP4 (E2M1 x E2M1, unit block scales, k given in operand bytes) -> bf16.
 //
 // Compiled with -DPTOAMD_CLOCK_PROBE the kernel writes, per workgroup, eight 64-bit words through p.acc_out:
 // [0] core clocks spent in the K loop, [1] wall clock (100 MHz) at entry, [2] at the start of the K loop, [3] at its end,
@@ -36,6 +36,10 @@ constexpr const char* KIND = "bf16 (16x16x32)";
 using ProbeOp = OpI8x16;
 constexpr int ESZ = 1, CSZ = 4, OUT = OUT_I32;
 constexpr const char* KIND = "int8 (16x16x64)";
+#elif PROBE_KIND == 4
+using ProbeOp = OpFP4;   // k counts operand BYTES here (two E2M1 codes each)
+constexpr int ESZ = 1, CSZ = 2, OUT = OUT_BF16;
+constexpr const char* KIND = "MXFP4 (k in bytes)";
 #elif PROBE_KIND == 3
 using ProbeOp = OpI8x16;
 constexpr int ESZ = 1, CSZ = 2, OUT = OUT_W8A8_BF16;
@@ -72,6 +76,8 @@ using Cfg = TileCfg<256, PROBE_BN, PROBE_WAVES_M, PROBE_WAVES_N, ProbeOp>;
             return 1;                                                                  \
         }                                                                              \
     } while (0)
+
+constexpr int GROUP_BYTES = ProbeOp::SCALED ? 128 / ProbeOp::GROUPS_PER_SLAB : 32;  // operand bytes per MX group
 
 int main(int argc, char** argv)
 {
@@ -113,10 +119,10 @@ int main(int argc, char** argv)
     CK(hipMemcpy(b, hb.data(), hb.size() * 2, hipMemcpyHostToDevice));
     CK(hipMemset(stamps, 0, (size_t)tiles * 64));
     if (ProbeOp::SCALED) {
-        CK(hipMalloc(&sa, (size_t)m * (k / 32)));
-        CK(hipMalloc(&sb, (size_t)n * (k / 32)));
-        CK(hipMemset(sa, 127, (size_t)m * (k / 32)));
-        CK(hipMemset(sb, 127, (size_t)n * (k / 32)));
+        CK(hipMalloc(&sa, (size_t)m * (kb / GROUP_BYTES)));
+        CK(hipMalloc(&sb, (size_t)n * (kb / GROUP_BYTES)));
+        CK(hipMemset(sa, 127, (size_t)m * (kb / GROUP_BYTES)));
+        CK(hipMemset(sb, 127, (size_t)n * (kb / GROUP_BYTES)));
     }
 
     TileGemmParams p{};
@@ -143,7 +149,7 @@ int main(int argc, char** argv)
     p.group_m = 4;
     p.sa = sa;
     p.sb = sb;
-    p.scale_ld = k / 32;
+    p.scale_ld = (int)(kb / GROUP_BYTES);
     p.acc_out = (int32_t*)stamps;
     auto kernel = gemm_tile_dtl_kernel<Cfg>;
     CK(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
