@@ -317,7 +317,8 @@ __device__ __forceinline__ constexpr int acc_col(int r, int lhi) { return BLK ==
 // gi: the lane's row of C; col_b: first column of the block.
 // RELU: apply p.relu here (the quantising kinds clamp at zero after the quantisation instead).
 template <bool FULL, bool RELU, class Cfg, class Acc>
-__device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int gi, int col_b, int lhi)
+__device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int gi, int col_b, int lhi,
+                                             const typename Cfg::Op::Elem* bias_blk = nullptr)
 {
     using Elem = typename Cfg::Op::Elem;
     const Elem* cin = reinterpret_cast<const Elem*>(p.c_in);
@@ -337,7 +338,9 @@ __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int 
 #pragma unroll
         for (int r = 0; r < Cfg::Op::ACC_REGS; ++r) {
             const int gj = col_b + acc_col<Cfg::BLK>(r, lhi);
-            if (FULL || gj < p.n)
+            if (bias_blk != nullptr)  // (a literal at every call site) the block's bias values, fetched by the caller
+                v[r] += bias_blk[r];
+            else if (FULL || gj < p.n)
                 v[r] += reinterpret_cast<const Elem*>(p.bias)[gj];
         }
     }
@@ -483,6 +486,32 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
     const int lane = lhi * BLK + l32;
     // W8A8: a lane's column scales are the same for every block row of the wave tile; fetched once here (fetched where
     // they are used they are 128 separate loads per lane, and the store phase takes twice as long)
+    // What depends on the column only is the same for every block row of the wave tile and is fetched once, up front:
+    // fetched per block (with the blocks kept apart for register pressure) every block pays a load latency of its own.
+    using Elem = typename Cfg::Op::Elem;
+    Elem bias_pre[Cfg::NB][Cfg::Op::ACC_REGS];
+    const bool has_bias = p.bias != nullptr;
+    if (has_bias) {
+        static_for<Cfg::NB>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+#pragma unroll
+            for (int r = 0; r < Cfg::Op::ACC_REGS; ++r)
+                bias_pre[j][r] = reinterpret_cast<const Elem*>(p.bias)[col0 + j * BLK + acc_col<BLK>(r, lhi)];
+        });
+    }
+    uint64_t qw_pre[Cfg::NB][Cfg::Op::ACC_REGS];
+    uint64_t qw0 = 0;
+    if constexpr (out_quant<KIND>) {
+        qw0 = p.qwords[0];
+        if (p.q_per_column) {
+            static_for<Cfg::NB>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+#pragma unroll
+                for (int r = 0; r < Cfg::Op::ACC_REGS; ++r)
+                    qw_pre[j][r] = p.qwords[col0 + j * BLK + acc_col<BLK>(r, lhi)];
+            });
+        }
+    }
     float cs_pre[Cfg::NB][Cfg::Op::ACC_REGS], rs_pre[Cfg::MB];
     if constexpr (KIND == OUT_W8A8_BF16) {
 #pragma unroll
@@ -506,7 +535,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
                 constexpr int j = decltype(jc)::value;
                 __builtin_amdgcn_sched_barrier(0);
                 const int col_b = col0 + j * BLK;
-                const Acc v = tstore_terms<true, !out_quant<KIND>, Cfg>(p, acc[i][j], gi, col_b, lhi);
+                const Acc v = tstore_terms<true, !out_quant<KIND>, Cfg>(p, acc[i][j], gi, col_b, lhi, bias_pre[j]);  // (read only where p.bias is set)
 #pragma unroll
                 for (int g = 0; g < Cfg::Op::ACC_REGS / 4; ++g) {
                     const int qc = acc_col<BLK>(4 * g, lhi);  // first of the quad's four columns
@@ -524,7 +553,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
                         uint32_t bits[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? col_b + qc + e : 0] : 0;
+                            const uint64_t qw = out_quant<KIND> ? (p.q_per_column ? qw_pre[j][4 * g + e] : qw0) : 0;
                             bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
                         }
                         if (ESZ == 4)
