@@ -486,11 +486,17 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
     const int lane = lhi * BLK + l32;
     // W8A8: a lane's column scales are the same for every block row of the wave tile; fetched once here (fetched where
     // they are used they are 128 separate loads per lane, and the store phase takes twice as long)
+    // (nothing below may be scheduled up into the K loop's last slab, where every register is taken)
+    __builtin_amdgcn_sched_barrier(0);
     // What depends on the column only is the same for every block row of the wave tile and is fetched once, up front:
     // fetched per block (with the blocks kept apart for register pressure) every block pays a load latency of its own.
+    // (Only where a lane has at most 16 columns -- the 16x16 blocks of the large tile -- and one kind of item at a time:
+    // next to 128 accumulator registers more than that spills.)
     using Elem = typename Cfg::Op::Elem;
+    constexpr bool PRE = Cfg::NB * Cfg::Op::ACC_REGS <= 16;
+    constexpr bool PRE_BIAS = PRE && !out_quant<KIND>, PRE_QW = PRE && out_quant<KIND>;
     Elem bias_pre[Cfg::NB][Cfg::Op::ACC_REGS];
-    const bool has_bias = p.bias != nullptr;
+    const bool has_bias = PRE_BIAS && p.bias != nullptr;
     if (has_bias) {
         static_for<Cfg::NB>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
@@ -503,7 +509,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
     uint64_t qw0 = 0;
     if constexpr (out_quant<KIND>) {
         qw0 = p.qwords[0];
-        if (p.q_per_column) {
+        if (PRE_QW && p.q_per_column) {
             static_for<Cfg::NB>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
 #pragma unroll
@@ -535,7 +541,8 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
                 constexpr int j = decltype(jc)::value;
                 __builtin_amdgcn_sched_barrier(0);
                 const int col_b = col0 + j * BLK;
-                const Acc v = tstore_terms<true, !out_quant<KIND>, Cfg>(p, acc[i][j], gi, col_b, lhi, bias_pre[j]);  // (read only where p.bias is set)
+                const Acc v = tstore_terms<true, !out_quant<KIND>, Cfg>(p, acc[i][j], gi, col_b, lhi,
+                                                                      PRE_BIAS ? bias_pre[j] : nullptr);  // (read only where p.bias is set)
 #pragma unroll
                 for (int g = 0; g < Cfg::Op::ACC_REGS / 4; ++g) {
                     const int qc = acc_col<BLK>(4 * g, lhi);  // first of the quad's four columns
@@ -553,7 +560,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
                         uint32_t bits[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const uint64_t qw = out_quant<KIND> ? (p.q_per_column ? qw_pre[j][4 * g + e] : qw0) : 0;
+                            const uint64_t qw = !out_quant<KIND> ? 0 : !p.q_per_column ? qw0 : PRE_QW ? qw_pre[j][4 * g + e] : p.qwords[col_b + qc + e];
                             bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
                         }
                         if (ESZ == 4)
