@@ -281,9 +281,11 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
         int t = env[0] - '0';
         if (t == 3)  // the four-wave form of the 256 x 256 DMA tile is no longer built
             t = 4;
+        if (t == 0)  // nor is the register-staged 256 x 256 tile (it spilled: 315 against 176 us for the 128 x 128 one on
+            t = 1;   // bf16 4096 x 4096 x 4104)
         if (t < 3 || dtl_ok)
             return t;
-        return t == 5 ? 1 : 0;
+        return 1;
     }
     const long t256 = (long)((m + 255) / 256) * ((n + 255) / 256);
     const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128);
@@ -292,7 +294,7 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
     if (scaled)
         return t128 >= 96 ? (dtl_ok ? 5 : 1) : 2;
     if (t256 >= 128)
-        return dtl_ok ? 4 : 0;
+        return dtl_ok ? 4 : 1;
     if (t128 >= 96)
         return dtl_ok ? 5 : 1;
     return 2;

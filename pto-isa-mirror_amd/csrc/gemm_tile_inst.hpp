@@ -42,7 +42,7 @@ hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 #endif
         case 5: return launch_dtl<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>>(p, stream);
         case 6: return launch_dtl<TileCfg<256, 128, 4, 2, PTOAMD_TILE_OP>>(p, stream);
-        case 0: return launch_cfg<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>>(p, stream);
+        case 0:  // (once a register-staged 256 x 256 tile: it kept part of its working set in scratch memory)
         case 1: return launch_cfg<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>>(p, stream);
         default: return launch_cfg<TileCfg<64, 64, 2, 2, PTOAMD_TILE_OP>>(p, stream);
     }
