@@ -400,6 +400,25 @@ constexpr bool acc_out_is_probe = true;
 #else
 constexpr bool acc_out_is_probe = false;
 #endif
+// The byte targets' quantisation word, decoded once: scale, offset and the lower clamp bound (the upper one is 255 above it).
+struct ByteQuant {
+    float scale, offset, lo;
+};
+template <bool VECTOR>
+__device__ __forceinline__ ByteQuant decode_byte_quant(uint64_t word)
+{
+    return ByteQuant{fixpipe_word_scale<VECTOR>(word), (float)(uint32_t)((word >> 37) & 0x1FFu), ((word >> 46) & 1u) ? -128.0f : 0.0f};
+}
+// the same arithmetic as fixpipe_quantize<., true, .> followed by the relu and the narrowing of tstore_bits<OUT_Q8>
+__device__ __forceinline__ uint32_t byte_quant_bits(float acc, const ByteQuant& q, bool relu)
+{
+    const float rounded = rintf(__fadd_rn(__fmul_rn(acc, q.scale), q.offset));
+    const float hi = q.lo + 255.0f;
+    float r = rounded < q.lo ? q.lo : (rounded > hi ? hi : rounded);
+    if (relu)
+        r = r > 0 ? r : 0;
+    return (uint32_t)(int32_t)r & 0xFFu;
+}
 template <int KIND>
 constexpr int out_bytes = (KIND == OUT_F32 || KIND == OUT_I32) ? 4 : (KIND == OUT_Q8 ? 1 : 2);
 template <int KIND>
@@ -505,16 +524,27 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
                 bias_pre[j][r] = reinterpret_cast<const Elem*>(p.bias)[col0 + j * BLK + acc_col<BLK>(r, lhi)];
         });
     }
+    // (byte targets keep the words decoded -- three floats per column instead of a 64-bit word taken apart per element)
+    constexpr bool Q8 = KIND == OUT_Q8;
     uint64_t qw_pre[Cfg::NB][Cfg::Op::ACC_REGS];
+    ByteQuant bq_pre[Cfg::NB][Cfg::Op::ACC_REGS];
     uint64_t qw0 = 0;
+    ByteQuant bq0{};
     if constexpr (out_quant<KIND>) {
         qw0 = p.qwords[0];
+        if (Q8 && !p.q_per_column)
+            bq0 = decode_byte_quant<false>(qw0);
         if (PRE_QW && p.q_per_column) {
             static_for<Cfg::NB>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
 #pragma unroll
-                for (int r = 0; r < Cfg::Op::ACC_REGS; ++r)
-                    qw_pre[j][r] = p.qwords[col0 + j * BLK + acc_col<BLK>(r, lhi)];
+                for (int r = 0; r < Cfg::Op::ACC_REGS; ++r) {
+                    const uint64_t w = p.qwords[col0 + j * BLK + acc_col<BLK>(r, lhi)];
+                    if (Q8)
+                        bq_pre[j][r] = decode_byte_quant<true>(w);
+                    else
+                        qw_pre[j][r] = w;
+                }
             });
         }
     }
@@ -560,7 +590,11 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
                         uint32_t bits[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const uint64_t qw = !out_quant<KIND> ? 0 : !p.q_per_column ? qw0 : PRE_QW ? qw_pre[j][4 * g + e] : p.qwords[col_b + qc + e];
+                            if (Q8 && (PRE_QW || !p.q_per_column)) {
+                                bits[e] = byte_quant_bits((float)v[4 * g + e], p.q_per_column ? bq_pre[j][4 * g + e] : bq0, p.relu != 0);
+                                continue;
+                            }
+                            const uint64_t qw = !out_quant<KIND> ? 0 : !p.q_per_column ? qw0 : (PRE_QW && !Q8) ? qw_pre[j][4 * g + e] : p.qwords[col_b + qc + e];
                             bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
                         }
                         if (ESZ == 4)
