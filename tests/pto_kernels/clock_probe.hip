@@ -146,7 +146,7 @@ int main(int argc, char** argv)
     p.ldb_bytes = (long)pitch;
     p.ldc = n;
     p.out_kind = OUT;
-    p.group_m = 4;
+    p.group_m = getenv("PTOAMD_PROBE_GROUP_M") ? atoi(getenv("PTOAMD_PROBE_GROUP_M")) : 4;  // tile rows walked together (the library's value)
     p.sa = sa;
     p.sb = sb;
     p.scale_ld = (int)(kb / GROUP_BYTES);
