@@ -77,6 +77,10 @@ enum { PTOAMD_MEMCPY_H2H = 0, PTOAMD_MEMCPY_H2D = 1, PTOAMD_MEMCPY_D2H = 2, PTOA
  * ========================================================================================================= */
 int ptoamd_init(int device);                    /* aclInit + aclrtSetDevice: selects the device, checks it is gfx950 */
 int ptoamd_finalize(void);                      /* aclrtResetDevice + aclFinalize */
+/* The dispatchers' environment switches (PTOAMD_TILE, PTOAMD_NO_TAIL_SPLIT, PTOAMD_FORCE_GENERIC,
+ * PTOAMD_B_ND_TRANSPOSE, PTOAMD_GEMV_*) are read once per process; this reads them again.  No counterpart in the
+ * reference (its simulator reads PTO_CPU_MAX_THREADS and the buffer sizes once too, cpu/NPUMemoryModel.hpp:128-135). */
+int ptoamd_reload_options(void);
 const char* ptoamd_last_error(void);            /* text of the calling thread's last failure */
 int ptoamd_device_info(int* compute_units, int* clock_khz, size_t* hbm_bytes, char* arch, size_t arch_len);
 
@@ -175,8 +179,15 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
 /*
  * Block-scaled matmul, TMATMUL_MX (cpu/TMatmul.hpp:169-205, 254-292):
  *   C(i, j) = sum_k A(i, k) * B(k, j) * 2^(sa(i, k/32) - 127) * 2^(sb(k/32, j) - 127)   (+ Cin)
- *   a_type / b_type : both fp8 (PTOAMD_E4M3 | PTOAMD_E5M2) or both fp4 (PTOAMD_E2M1 | PTOAMD_E1M2; E1M2 runs on
- *                     the order-exact generic kernel only)
+ *   a_type / b_type : both fp8 (PTOAMD_E4M3 | PTOAMD_E5M2) or both fp4 (PTOAMD_E2M1 | PTOAMD_E1M2).  A product with an
+ *                     E1M2 operand runs on the E4M3 x E4M3 scaled MFMA, both operands' nibbles widened exactly to E4M3
+ *                     bytes by the loader (b in PTOAMD_B_DN, K a multiple of 128, 8-byte aligned rows); other E1M2
+ *                     shapes take the order-exact generic kernel.
+ *   Numerics of the MFMA kernels: the scaled MFMA aligns the 64 products of a k-step to the largest exponent among
+ *   them and keeps about 13 bits below it before adding, where the reference adds one product at a time in fp32
+ *   (double add, one rounding per k).  Element-wise |C - C_ref| <= 2^-11 * sum_k |a||b| on fp8 data spanning all codes
+ *   (<= 1e-3 of max|C|), within the fp32-sum bound on data of one magnitude; the generic kernel
+ *   (PTOAMD_FORCE_GENERIC=1) reproduces the reference bit for bit.
  *   a  : [M][K] codes row-major (fp4: K/2 bytes per row);  b : PTOAMD_B_DN ([N][K]) or PTOAMD_B_ND ([K][N])
  *   sa : E8M0 bytes in sa_layout (PTOAMD_MX_A_*), logical [M][K/32];  sb : sb_layout (PTOAMD_MX_B_*), [K/32][N]
  *   c_type : PTOAMD_F32 | PTOAMD_BF16 | PTOAMD_F16

@@ -761,8 +761,18 @@ float pto_group_scaling(int alg, float maxabs, unsigned e8m0)
     return s;
 }
 
+/* A half source reaches the quantiser through the half -> float conversion (TQuant.hpp:291: `const float value =
+ * src.data()[...]`), which quietens a signalling NaN; sources passed here as float already are widened by the caller,
+ * so that step is restated for PTO_SRC_F16 (bf16 -> float is a shift and keeps the payload). */
+static float mx_source_value(float v, int src_kind)
+{
+    if (src_kind == PTO_SRC_F16 && isnan(v))
+        return u2f(f2u(v) | 0x00400000u);
+    return v;
+}
+
 /* TQuant.hpp:280-306 */
-static float mx_group_max(const float* src, int rows, int cols, int alg, int axis, int line, int group)
+static float mx_group_max(const float* src, int rows, int cols, int alg, int axis, int line, int group, int src_kind)
 {
     (void)rows;
     float mx = 0.0f;
@@ -770,7 +780,7 @@ static float mx_group_max(const float* src, int rows, int cols, int alg, int axi
     for (int inner = 0; inner < 32; ++inner) {
         const int r = axis == 1 ? line : group * 32 + inner;
         const int c = axis == 1 ? group * 32 + inner : line;
-        const float v = src[(size_t)r * cols + c];
+        const float v = mx_source_value(src[(size_t)r * cols + c], src_kind);
         if (alg == PTO_OCP_FP4) {
             const uint16_t b = (uint16_t)((f2u(v) >> 16) & 0x7FFFu); /* truncated bf16 magnitude bits */
             if (b > mx_bits)
@@ -799,7 +809,7 @@ void pto_tquant_mx(uint8_t* dst, uint8_t* exp, float* mxo, float* scaling, const
     for (int line = 0; line < lines; ++line) {
         for (int g = 0; g < groups; ++g) {
             const int flat = axis == 1 ? line * groups + g : g * lines + line;
-            const float mx = mx_group_max(src, rows, cols, alg, axis, line, g);
+            const float mx = mx_group_max(src, rows, cols, alg, axis, line, g, src_kind);
             const unsigned e = pto_shared_exponent(alg, mx);
             const float sc = pto_group_scaling(alg, mx, e);
             mxo[flat] = mx;
@@ -808,7 +818,7 @@ void pto_tquant_mx(uint8_t* dst, uint8_t* exp, float* mxo, float* scaling, const
             for (int inner = 0; inner < 32; ++inner) {
                 const int r = axis == 1 ? line : g * 32 + inner;
                 const int c = axis == 1 ? g * 32 + inner : line;
-                const float v = src[(size_t)r * cols + c];
+                const float v = mx_source_value(src[(size_t)r * cols + c], src_kind);
                 const size_t idx = (size_t)r * cols + c;
                 if (!fp4) {
                     dst[idx] = (uint8_t)pto_encode_e4m3fn(v * sc, alg == PTO_NV_FP8);

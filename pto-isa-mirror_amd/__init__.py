@@ -44,7 +44,7 @@ EXPORTS = [
     "ptoamd_gemm_mx_ws",
     "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
     "ptoamd_tquant_int8_para", "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_tdequant_para", "ptoamd_mx_scale_relayout",
-    "ptoamd_last_kernel",
+    "ptoamd_last_kernel", "ptoamd_reload_options",
 ]
 
 
@@ -65,12 +65,21 @@ def init(device=0):
     _check(_lib.ptoamd_init(int(device)), "ptoamd_init")
 
 
-def _ptr(t):
+def reload_options():
+    """Re-reads the PTOAMD_* environment switches (the library reads them once per process otherwise)."""
+    _check(_lib.ptoamd_reload_options(), "ptoamd_reload_options")
+
+
+def _ptr(t, strided=False):
+    """Device address of a tensor.  Operands must be contiguous; strided=True also takes a 2-D view with unit column
+    stride, and is passed only where the call forwards the view's row pitch (stride(0)) as a leading dimension."""
     if t is None:
         return C.c_void_p(0)
-    # contiguous, or a 2-D view with unit column stride (its row pitch goes to the library as the leading dimension)
-    assert t.is_cuda and (t.is_contiguous() or (t.dim() == 2 and t.stride(1) == 1)), \
-        "operands must be device tensors, contiguous or row-strided"
+    assert t.is_cuda, "operands must be device tensors"
+    if strided:
+        assert t.is_contiguous() or (t.dim() == 2 and t.stride(1) == 1), "operand must be contiguous or row-strided"
+    else:
+        assert t.is_contiguous(), "operand must be contiguous (this argument has no leading-dimension parameter)"
     return C.c_void_p(t.data_ptr())
 
 
@@ -92,11 +101,11 @@ def gemm(a, b, ab_type, c_type=F32, b_layout=B_DN, c_in=None, relu=False, m=None
     if out is None:
         out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
     if bias is not None:
-        _check(_lib.ptoamd_gemm_bias(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), _ptr(bias), m, n, k,
+        _check(_lib.ptoamd_gemm_bias(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _ptr(c_in), _ptr(bias), m, n, k,
                                      a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu), _stream(stream)),
                "ptoamd_gemm_bias")
         return out
-    _check(_lib.ptoamd_gemm(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), m, n, k, a.stride(0), b.stride(0),
+    _check(_lib.ptoamd_gemm(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _ptr(c_in), m, n, k, a.stride(0), b.stride(0),
                             out.stride(0), b_layout, int(relu), _stream(stream)), "ptoamd_gemm")
     return out
 
@@ -107,7 +116,7 @@ def gemm_fp8(a, b, a_type, b_type, c_type=F32, b_layout=B_DN, c_in=None, bias=No
     n = b.shape[0] if b_layout == B_DN else b.shape[1]
     if out is None:
         out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
-    _check(_lib.ptoamd_gemm_fp8(_ptr(out), c_type, _ptr(a), a_type, _ptr(b), b_type, _ptr(c_in), _ptr(bias), m, n, k,
+    _check(_lib.ptoamd_gemm_fp8(_ptr(out, True), c_type, _ptr(a, True), a_type, _ptr(b, True), b_type, _ptr(c_in), _ptr(bias), m, n, k,
                                 a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu), _stream(stream)), "ptoamd_gemm_fp8")
     return out
 
@@ -117,7 +126,7 @@ def gemm_atomic_add(out, a, b, ab_type, b_layout=B_DN, stream=None):
     m, k = a.shape
     n = out.shape[1]
     c_type = F32 if out.dtype == torch.float32 else I32
-    _check(_lib.ptoamd_gemm_atomic_add(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, m, n, k, a.stride(0), b.stride(0),
+    _check(_lib.ptoamd_gemm_atomic_add(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, m, n, k, a.stride(0), b.stride(0),
                                        out.stride(0), b_layout, _stream(stream)), "ptoamd_gemm_atomic_add")
     return out
 
@@ -130,7 +139,7 @@ def gemm_requant(a, b, ab_type, c_type, quant_words, per_column=False, b_layout=
     n = (b.shape[0] if b_layout == B_DN else b.shape[1]) if n is None else n
     if out is None:
         out = torch.empty((m, n), dtype={I8: torch.int8, U8: torch.uint8, F16: torch.float16, BF16: torch.bfloat16, I16: torch.int16}[c_type], device=a.device)
-    _check(_lib.ptoamd_gemm_requant(_ptr(out), c_type, _ptr(a), _ptr(b), ab_type, _ptr(c_in), _ptr(bias), _ptr(quant_words),
+    _check(_lib.ptoamd_gemm_requant(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _ptr(c_in), _ptr(bias), _ptr(quant_words),
                                     int(per_column), m, n, k, a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu),
                                     _stream(stream)), "ptoamd_gemm_requant")
     return out
@@ -143,7 +152,7 @@ def gemm_w8a8(a, b, scale_a, scale_b, b_layout=B_DN, want_acc=False, stream=None
     if out is None:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
     acc = torch.empty((m, n), dtype=torch.int32, device=a.device) if want_acc else None
-    _check(_lib.ptoamd_gemm_w8a8(_ptr(out), _ptr(acc), _ptr(a), _ptr(b), _ptr(scale_a), _ptr(scale_b), m, n, k,
+    _check(_lib.ptoamd_gemm_w8a8(_ptr(out, True), _ptr(acc), _ptr(a, True), _ptr(b, True), _ptr(scale_a), _ptr(scale_b), m, n, k,
                                  a.stride(0), b.stride(0), out.stride(0), b_layout, _stream(stream)), "ptoamd_gemm_w8a8")
     return (out, acc) if want_acc else out
 
@@ -158,7 +167,7 @@ def gemm_mx_static(a, b, sa, sb, m, n, k, a_type, b_type, out, sa_layout=MX_A_ND
     c_type = {v: key for key, v in _TORCH_OUT.items()}[out.dtype]
     lda = k
     ldb = k if b_layout == B_DN else n
-    _check(_lib.ptoamd_gemm_mx_static(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
+    _check(_lib.ptoamd_gemm_mx_static(_ptr(out, True), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
                                       sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),
            "ptoamd_gemm_mx_static")
     return out
@@ -177,17 +186,17 @@ def gemm_mx(a, b, sa, sb, m, n, k, a_type, b_type, c_type=F32, sa_layout=MX_A_ND
     lda = k
     ldb = k if b_layout == B_DN else n
     if workspace is not None:
-        _check(_lib.ptoamd_gemm_mx_ws(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
+        _check(_lib.ptoamd_gemm_mx_ws(_ptr(out, True), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
                                       sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _ptr(workspace),
                                       C.c_size_t(workspace.numel() * workspace.element_size()), _stream(stream)),
                "ptoamd_gemm_mx_ws")
         return out
     if bias is not None:
-        _check(_lib.ptoamd_gemm_mx_bias(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
+        _check(_lib.ptoamd_gemm_mx_bias(_ptr(out, True), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
                                         sb_layout, _ptr(c_in), _ptr(bias), m, n, k, lda, ldb, out.stride(0), b_layout,
                                         _stream(stream)), "ptoamd_gemm_mx_bias")
         return out
-    _check(_lib.ptoamd_gemm_mx(_ptr(out), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
+    _check(_lib.ptoamd_gemm_mx(_ptr(out, True), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
                                sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),
            "ptoamd_gemm_mx")
     return out
@@ -198,7 +207,7 @@ def gemv_mxfp4(a_bf16, w, sw, n, k, c_type=F32, stream=None, out=None):
     m = a_bf16.shape[0]
     if out is None:
         out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=w.device)
-    _check(_lib.ptoamd_gemv_mxfp4(_ptr(out), c_type, _ptr(a_bf16), _ptr(w), _ptr(sw), m, n, k, a_bf16.stride(0), k,
+    _check(_lib.ptoamd_gemv_mxfp4(_ptr(out, True), c_type, _ptr(a_bf16, True), _ptr(w), _ptr(sw), m, n, k, a_bf16.stride(0), k,
                                   out.stride(0), _stream(stream)), "ptoamd_gemv_mxfp4")
     return out
 
@@ -210,7 +219,8 @@ def tquant_int8(src, scale, offset=None, stream=None, out=None):
     if out is None:
         out = torch.empty((rows, cols), dtype=torch.int8 if offset is None else torch.uint8, device=src.device)
     if scale.dim() == 2:
-        _check(_lib.ptoamd_tquant_int8_para(_ptr(out), _ptr(src), _ptr(scale), _ptr(offset), rows, cols, scale.shape[0],
+        assert offset is None or offset.stride(0) == scale.stride(0), "scale and offset tiles share one row pitch"
+        _check(_lib.ptoamd_tquant_int8_para(_ptr(out), _ptr(src), _ptr(scale, True), _ptr(offset, True), rows, cols, scale.shape[0],
                                             scale.stride(0), _stream(stream)), "ptoamd_tquant_int8_para")
         return out
     _check(_lib.ptoamd_tquant_int8(_ptr(out), _ptr(src), _ptr(scale), _ptr(offset), rows, cols, _stream(stream)),
@@ -248,7 +258,8 @@ def tdequant(src, scale, offset, stream=None, out=None):
     if out is None:
         out = torch.empty((rows, cols), dtype=torch.float32, device=src.device)
     if scale.dim() == 2:
-        _check(_lib.ptoamd_tdequant_para(_ptr(out), _ptr(src), _INT_TYPE[src.dtype], _ptr(scale), _ptr(offset), rows, cols,
+        assert offset.stride(0) == scale.stride(0), "scale and offset tiles share one row pitch"
+        _check(_lib.ptoamd_tdequant_para(_ptr(out), _ptr(src), _INT_TYPE[src.dtype], _ptr(scale, True), _ptr(offset, True), rows, cols,
                                          scale.shape[1], scale.stride(0), _stream(stream)), "ptoamd_tdequant_para")
         return out
     _check(_lib.ptoamd_tdequant(_ptr(out), _ptr(src), _INT_TYPE[src.dtype], _ptr(scale), _ptr(offset), rows, cols,

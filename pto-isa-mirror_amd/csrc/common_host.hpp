@@ -15,6 +15,22 @@ hipError_t ensure_dynamic_lds(const void* kernel, int bytes);
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// The environment switches of the dispatchers, read once per process (and again by ptoamd_reload_options): a launch
+// tests plain fields instead of calling getenv.
+struct Options {
+    int tile = -1;               // PTOAMD_TILE=0..6: run this tile shape; -1 = choose by problem size
+    bool no_tail_split = false;  // PTOAMD_NO_TAIL_SPLIT=1: never split a half-full last round off as smaller tiles
+    int tail_tile = 5;           // PTOAMD_TAIL_TILE=5|6: the tail runs as 128x128 or 256x128 tiles
+    bool force_generic = false;  // PTOAMD_FORCE_GENERIC=1: everything runs on the order-exact generic kernels
+    bool b_nd_transpose = false; // PTOAMD_B_ND_TRANSPOSE=1: a row-major B is re-ordered in global memory, never in the loader
+    bool gemv_sw_cvt = false;    // PTOAMD_GEMV_SW_CVT=1: decode fp4 weights with integer arithmetic
+    bool gemv_no_splitk = false; // PTOAMD_GEMV_NO_SPLITK=1 / PTOAMD_GEMV_NO_WIDE=1: skip those GEMV kernels
+    bool gemv_no_wide = false;
+};
+const Options& options();
+// compute units of the current device (cached per device ordinal)
+int device_compute_units();
+
 // One record per C-ABI launch, written as a JSON line to $PTOAMD_TRACE_DIR/ptoamd_trace_<pid>.jsonl when that variable
 // names a directory (no-op otherwise).  Field names follow the reference simulator's InstructionTraceRecord
 // (include/pto/cpu/trace.hpp:67-87: sequence_id, opcode, input_tiles / output_tiles with address, shape, layout, dtype),

@@ -276,9 +276,8 @@ static bool dma_offsets_fit(int m, int n, long lda_bytes, long ldb_bytes, long k
 static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, bool scale_dma_ok = true)
 {
     const bool dtl_ok = (k_bytes % 128) == 0 && scale_dma_ok;
-    const char* env = getenv("PTOAMD_TILE");
-    if (env && env[0] >= '0' && env[0] <= '6') {
-        int t = env[0] - '0';
+    if (options().tile >= 0) {
+        int t = options().tile;
         if (t == 3)  // the four-wave form of the 256 x 256 DMA tile is no longer built
             t = 4;
         if (t == 0)  // nor is the register-staged 256 x 256 tile (it spilled: 315 against 176 us for the 128 x 128 one on
@@ -300,20 +299,22 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
     return 2;
 }
 
-// Launch on the chosen tile.  When the 256x256 grid is some whole rounds of the 256 CUs plus a last one that is at most
-// half full, the columns of that last round run as 128x128 tiles (two workgroups per CU) in a second launch on the same stream:
-// a tile of the tail then costs about a quarter of a 256x256 tile's time instead of a whole round (MXFP8
-// 4096 x 14336 x 4096, 3.5 rounds: 194 against 200 us).
-// PTOAMD_TILE (an explicit tile) and PTOAMD_NO_TAIL_SPLIT=1 switch the split off.
+// Launch on the chosen tile.  When the 256x256 grid is some whole rounds of the CUs plus a last one that is at most half
+// full, the columns of that last round run as smaller tiles in a second launch on the same stream: 256x128 tiles (at most
+// one workgroup per CU, same wave tile as the large form) or 128x128 tiles (two workgroups per CU); a tile of the tail
+// then costs a half or a quarter of a 256x256 tile's time instead of a whole round (MXFP8 4096 x 14336 x 4096, 3.5
+// rounds of 256 CUs).  PTOAMD_TILE (an explicit tile) and PTOAMD_NO_TAIL_SPLIT=1 switch the split off;
+// PTOAMD_TAIL_TILE=5|6 picks the tail's tile.
 static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStream_t stream)
 {
-    if (tile == 4 && getenv("PTOAMD_TILE") == nullptr && getenv("PTOAMD_NO_TAIL_SPLIT") == nullptr) {
+    if (tile == 4 && options().tile < 0 && !options().no_tail_split) {
+        const int cus = device_compute_units();
         const int tiles_m = (p.m + 255) / 256, tiles_n = (p.n + 255) / 256;
         int whole = tiles_n;  // tile columns that make whole rounds
-        while (whole > 0 && ((long)tiles_m * whole) % 256 != 0)
+        while (whole > 0 && ((long)tiles_m * whole) % cus != 0)
             --whole;
         const long tail_tiles = (long)tiles_m * (tiles_n - whole);
-        if (whole > 0 && whole < tiles_n && tail_tiles <= 128) {  // a last round at most half full
+        if (whole > 0 && whole < tiles_n && tail_tiles <= cus / 2) {  // a last round at most half full
             const int n1 = whole * 256;
             TileGemmParams head = p;
             head.n = n1;
@@ -337,17 +338,13 @@ static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStr
                 tail.col_scale = p.col_scale + n1;
             if (p.qwords && p.q_per_column)
                 tail.qwords = p.qwords + n1;
-            return launch_gemm_tile(5, op, tail, stream);
+            return launch_gemm_tile(options().tail_tile, op, tail, stream);
         }
     }
     return launch_gemm_tile(tile, op, p, stream);
 }
 
-static bool force_generic()
-{
-    const char* env = getenv("PTOAMD_FORCE_GENERIC");
-    return env && env[0] == '1';
-}
+static bool force_generic() { return options().force_generic; }
 
 static const char* tile_kernel_name(int tile, int op)
 {
@@ -548,7 +545,7 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
     // temporary, one launch).  With many row-tiles every element of B would be scattered into LDS that many times, and
     // the DMA tiles cannot do it at all: then B is re-ordered once in global memory and read K-contiguous from there.
     const bool b_in_kernel = b_layout == PTOAMD_B_ND && m <= 1024 && (ebytes == 1 || ebytes == 2) && (n % (16 / ebytes)) == 0 &&
-                             (ldb_b % 16) == 0 && getenv("PTOAMD_B_ND_TRANSPOSE") == nullptr;
+                             (ldb_b % 16) == 0 && !options().b_nd_transpose;
     if (b_layout == PTOAMD_B_ND && !b_in_kernel) {  // TLOAD of an ND B panel: re-order once so the MFMA path reads K-contiguous rows
         PTOAMD_HIP_CHECK(bt.alloc((size_t)n * k_bytes));
         const int rc = ebytes == 2 ? transpose_b<uint16_t>(bt.ptr, b, k, n, ldb, stream)
@@ -605,7 +602,7 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
     const uint8_t* b_kmajor = reinterpret_cast<const uint8_t*>(b);
     long ldb_kmajor = ldb;
     const bool b_in_kernel = b_layout == PTOAMD_B_ND && m <= 1024 && (n % 16) == 0 && (ldb % 16) == 0 &&
-                             getenv("PTOAMD_B_ND_TRANSPOSE") == nullptr;  // (same rule as ptoamd_gemm)
+                             !options().b_nd_transpose;  // (same rule as ptoamd_gemm)
     if (b_layout == PTOAMD_B_ND && !b_in_kernel) {
         PTOAMD_HIP_CHECK(bt.alloc((size_t)n * k));
         const int rc = transpose_b<uint8_t>(bt.ptr, b, k, n, ldb, stream);

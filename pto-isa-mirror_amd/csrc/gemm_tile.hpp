@@ -394,12 +394,6 @@ __device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_
     }
     return f32_to_bf16_bits(__fmul_rn(__fmul_rn((float)v, rs), cs));
 }
-// (the timing build of the DMA kernel borrows acc_out for its time stamps: no raw accumulators are written then)
-#ifdef PTOAMD_CLOCK_PROBE
-constexpr bool acc_out_is_probe = true;
-#else
-constexpr bool acc_out_is_probe = false;
-#endif
 // The byte targets' quantisation word, decoded once: scale, offset and the lower clamp bound (the upper one is 255 above it).
 struct ByteQuant {
     float scale, offset, lo;
@@ -432,7 +426,7 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
     const int gi = row_b + l32;
     const float rs = (KIND == OUT_W8A8_BF16 && (FULL || gi < p.m)) ? p.row_scale[gi] : 1.0f;
     const Acc v = tstore_terms<FULL, !out_quant<KIND>, Cfg>(p, acc, gi, col_b, lhi);
-    const bool raw = KIND == OUT_W8A8_BF16 && p.acc_out != nullptr && !acc_out_is_probe;
+    const bool raw = KIND == OUT_W8A8_BF16 && p.acc_out != nullptr;
 #pragma unroll
     for (int r = 0; r < Cfg::Op::ACC_REGS; ++r) {
         const int gj = col_b + acc_col<Cfg::BLK>(r, lhi);
@@ -630,7 +624,7 @@ __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::
     const bool full = row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n;
     const int esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : (p.out_kind == OUT_Q8 ? 1 : 2);
     const bool aligned = (((long)p.ldc * esz) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
-    const bool raw_acc = p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr && !acc_out_is_probe;
+    const bool raw_acc = p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr;
     if (stage != nullptr && full && aligned && !p.atomic_add && !raw_acc) {
         if (p.out_kind >= OUT_QF16) {
             tstore_staged<OUT_QF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);

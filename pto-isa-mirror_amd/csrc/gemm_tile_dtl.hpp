@@ -87,9 +87,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     static_assert(KS % 2 == 0, "fragment register sets alternate per k-step");
     static_assert((NT / 8) % 16 == 0, "the swizzle of a lane's row must not depend on the piece index");
     extern __shared__ __align__(16) uint8_t smem[];
-#ifdef PTOAMD_CLOCK_PROBE
-    const long wall_entry = wall_clock64();
-#endif
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps the tile bookkeeping in scalar registers
@@ -126,11 +123,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     const uint32_t lds_wave_base = __builtin_amdgcn_readfirstlane(lds_address(smem) + wave * 1024);
     // DMA number q (0 .. LA + LB - 1) of slab kt into ring buffer buf
     auto tload_piece = [&](int kt, int buf, int q) __attribute__((always_inline)) {
-#if defined(PTOAMD_CLOCK_PROBE) && defined(PTOAMD_PROBE_DMA_EVERY)
-        // timing experiment (results are wrong): after the first two slabs issue no DMA (0) or every n-th piece only
-        if (kt > 1 && (PTOAMD_PROBE_DMA_EVERY == 0 || q % (PTOAMD_PROBE_DMA_EVERY ? PTOAMD_PROBE_DMA_EVERY : 1) != 0))
-            return;
-#endif
         const uint32_t dst = lds_wave_base + buf * Cfg::STAGE_BYTES;
         if (q < LA)
             lds_dma16_off(p.a + (long)kt * 128, goff_a[q], dst + q * (NT * 16));
@@ -329,9 +321,6 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     for (int q = 0; q < NREAD; ++q)
         textract_piece(0, 0, 0, q);
     read_scales(0);
-#ifdef PTOAMD_CLOCK_PROBE
-    const long clk0 = __builtin_readcyclecounter(), wall0 = wall_clock64();
-#endif
 
     // One slab.  `more` = slab kt+1 exists (read its first fragments in the last k-step), `dma` = slab kt+2 exists
     // (start its DMA into the buffer this slab frees); both are literal at the call sites so the branches fold.
@@ -363,17 +352,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
             kstep(std::integral_constant<int, s + 1>{}, s, true, cur, s + 1, more, kt + 1, cur ^ 1);
         });
         // every wave is done reading slab kt, and its DMAs of slab kt+1 (issued one slab ago) have landed
-#if defined(PTOAMD_CLOCK_PROBE) && defined(PTOAMD_PROBE_NO_BARRIER)  // timing experiment (results are wrong)
-        __builtin_amdgcn_sched_barrier(0);
-#else
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
-#endif
-#if defined(PTOAMD_CLOCK_PROBE) && defined(PTOAMD_PROBE_NO_SCALE_READS)
-        if (false)
-#else
         if (SC_AHEAD && more)
-#endif
             read_scales(kt + 1);
         kstep(std::integral_constant<int, 0>{}, KS - 1, more, cur ^ 1, 0, dma, kt + 2, cur);
     };
@@ -386,23 +367,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     }
     slab(kt, false, false);
 
-#ifdef PTOAMD_CLOCK_PROBE
-    // core clocks of the K loop and 100 MHz stamps of entry / loop start / loop end / exit, per workgroup (acc_out
-    // doubles as the probe's output here)
-    const long clk1 = __builtin_readcyclecounter(), wall1 = wall_clock64();
-#endif
     // ---- TSTORE.  No wave reads the ring after the last slab's barrier (its fragment reads were issued before it) and
     // no DMA is in flight, so each wave may reuse a piece of it for the staged store without another barrier.
     tstore<Cfg>(p, acc, m0 + wm * Cfg::WTM, n0 + wn * Cfg::WTN, l32, lhi, smem + wave * StagedStore<Cfg>::WAVE_BYTES);
-#ifdef PTOAMD_CLOCK_PROBE
-    if (p.acc_out != nullptr) {
-        __builtin_amdgcn_s_waitcnt(0x0070);  // this wave's stores have left
-        if (lane == 0 && wave == 0) {
-            long* o = reinterpret_cast<long*>(p.acc_out) + blockIdx.x * 8;
-            o[0] = clk1 - clk0; o[1] = wall_entry; o[2] = wall0; o[3] = wall1; o[4] = wall_clock64();
-        }
-    }
-#endif
 }
 
 }  // namespace ptoamd

@@ -622,8 +622,8 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
     p.m = m; p.n = n; p.k = k; p.lda = lda; p.ldw_bytes = ldw / 2; p.ldc = ldc;
     p.out_bf16 = c_type == PTOAMD_BF16;
     p.n_groups = (n + 15) / 16;
-    const char* fg = getenv("PTOAMD_FORCE_GENERIC");
-    const bool stream_ok = !(fg && fg[0] == '1') && k % GEMV_CHUNK == 0 && (reinterpret_cast<uintptr_t>(a_bf16) & 15u) == 0 &&
+    const Options& opt = options();
+    const bool stream_ok = !opt.force_generic && k % GEMV_CHUNK == 0 && (reinterpret_cast<uintptr_t>(a_bf16) & 15u) == 0 &&
                            (reinterpret_cast<uintptr_t>(w) & 15u) == 0 && (reinterpret_cast<uintptr_t>(sw) & 15u) == 0 &&
                            (lda % 8) == 0 && (p.ldw_bytes % 16) == 0;
     if (!stream_ok) {
@@ -633,16 +633,11 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
         set_last_kernel("gemv_mxfp4_generic");
         return PTOAMD_OK;
     }
-    int dev = 0, cus = 256;
-    PTOAMD_HIP_CHECK(hipGetDevice(&dev));
-    PTOAMD_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    const char* sw_cvt = getenv("PTOAMD_GEMV_SW_CVT");
-    const bool swc = sw_cvt && sw_cvt[0] == '1';
-    const char* no_sk = getenv("PTOAMD_GEMV_NO_SPLITK");
-    const char* no_wide = getenv("PTOAMD_GEMV_NO_WIDE");
-    const bool sk_ok = k % SK_SLICE == 0 && (reinterpret_cast<uintptr_t>(sw) & 3u) == 0 && !(no_sk && no_sk[0] == '1');
+    const int cus = device_compute_units();
+    const bool swc = opt.gemv_sw_cvt;
+    const bool sk_ok = k % SK_SLICE == 0 && (reinterpret_cast<uintptr_t>(sw) & 3u) == 0 && !opt.gemv_no_splitk;
     // loader-wave form: K in chunks of 2048; rows are addressed with 32-bit lane offsets
-    if (sk_ok && k % WD_CHUNK == 0 && (long)lda * 2 * 16 < (1L << 31) && p.ldw_bytes * 16 < (1L << 31) && !(no_wide && no_wide[0] == '1')) {
+    if (sk_ok && k % WD_CHUNK == 0 && (long)lda * 2 * 16 < (1L << 31) && p.ldw_bytes * 16 < (1L << 31) && !opt.gemv_no_wide) {
         const int spw = (p.n_groups + cus - 1) / cus;    // strips per workgroup
         const int grid = (p.n_groups + spw - 1) / spw;
         const void* fn = swc ? reinterpret_cast<const void*>(gemv_mxfp4_splitk_wide_kernel<false>)

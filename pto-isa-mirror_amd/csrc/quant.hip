@@ -18,9 +18,10 @@ static_assert(PTOAMD_OCP_MXFP8 == MX_OCP_FP8 && PTOAMD_NV_MXFP8 == MX_NV_FP8 && 
 // elements), so a group is 8 or 4 neighbouring lanes and a wave reads 1 KiB per load instruction; every thread handles
 // UNITS such pieces, one block-wide span apart, with all its loads in flight before the first is used.
 // FP4 codes come from the packed hardware conversion (v_cvt_scalef32_pk_fp4_f32, round to nearest even, saturating): on
-// finite input it is EncodeE2M1Magic (TQuant.hpp:155-176) -- the magic-number add there is a round-to-nearest-even onto
-// the same grid with the same clamp -- and the two cases where that function does not depend on the value alone (an
-// infinite or NaN scaling) are resolved per group before the conversion is consulted.  The bf16 source's re-rounding of
+// finite and infinite input it is EncodeE2M1Magic (TQuant.hpp:155-176) -- the magic-number add there is a
+// round-to-nearest-even onto the same grid with the same clamp; NaN elements are given that function's code (0x7) in
+// software after the conversion, and the two cases where the code does not depend on the value alone (an infinite or
+// NaN scaling) are resolved per group last.  The bf16 source's re-rounding of
 // the scaled value (TQuant.hpp:68-76) is the identity here: the scaling is a power of two, so the product of a bf16
 // value is a bf16 value again unless it is subnormal, and then it is far below the smallest code either way.
 template <int ALG, typename T, bool SRC_BF16>
@@ -54,11 +55,11 @@ __global__ void __launch_bounds__(256) tquant_mx_rows_kernel(uint8_t* dst, uint8
         uint32_t run = 0;
 #pragma unroll
         for (int i = 0; i < EPL; ++i)
-            run = max_step<ALG>(run, v[i]);
+            run = max_step<ALG>(run, v[i], (int)(threadIdx.x & (LPG - 1)) * EPL + i);
 #pragma unroll
         for (int off = 1; off < LPG; off <<= 1)
             run = max_merge<ALG>(run, (uint32_t)__shfl_xor((int)run, off, LPG));
-        const float maxabs = max_value<ALG>(run, u2f(0x7FC00000u));
+        const float maxabs = max_value<ALG>(run);
         const uint32_t e = shared_exponent<ALG>(maxabs);
         const float sc = group_scaling<ALG>(maxabs, e);
         const long g = unit / LPG;
@@ -75,6 +76,13 @@ __global__ void __launch_bounds__(256) tquant_mx_rows_kernel(uint8_t* dst, uint8
                 constexpr int i = decltype(ic)::value;
                 packed = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(packed, __fmul_rn(v[2 * i], sc), __fmul_rn(v[2 * i + 1], sc), 1.0f, i);
             });
+            // a NaN element encodes as +6 (0x7) whatever its sign (TQuant.hpp:157-159); what the packed conversion makes
+            // of a NaN is not relied on
+            uint32_t nan_nibbles = 0;
+#pragma unroll
+            for (int i = 0; i < EPL; ++i)
+                nan_nibbles |= (v[i] != v[i]) ? (0xFu << (4 * i)) : 0u;
+            packed = (packed & ~nan_nibbles) | (0x77777777u & nan_nibbles);
             const uint32_t sb = f2u(sc);  // StoreMxEncodedValue's two special scalings (TQuant.hpp:349-372)
             if ((sb & 0x7FFFFFFFu) == 0x7F800000u)
                 packed = (sb >> 31) ? 0xFFFFFFFFu : 0x77777777u;
@@ -145,13 +153,13 @@ __global__ void tquant_mx_cols_kernel(uint8_t* dst, uint8_t* exp, float* mx, flo
     const T* p = src + (long)g * 32 * cols + cp * 2;
     uint32_t run[2] = {0, 0};
     for (int r = 0; r < 32; ++r) {
-        run[0] = max_step<ALG>(run[0], widen<T>(p[(long)r * cols]));
-        run[1] = max_step<ALG>(run[1], widen<T>(p[(long)r * cols + 1]));
+        run[0] = max_step<ALG>(run[0], widen<T>(p[(long)r * cols]), r);
+        run[1] = max_step<ALG>(run[1], widen<T>(p[(long)r * cols + 1]), r);
     }
     float sc[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const float maxabs = max_value<ALG>(run[j], u2f(0x7FC00000u));
+        const float maxabs = max_value<ALG>(run[j]);
         const uint32_t e = shared_exponent<ALG>(maxabs);
         sc[j] = group_scaling<ALG>(maxabs, e);
         const long gi = (long)g * cols + cp * 2 + j;

@@ -30,6 +30,53 @@ void set_last_kernel(const char* name)
     ++g_launches;
 }
 
+// ---- environment switches ---------------------------------------------------------------------------------------------
+namespace {
+Options g_options;
+std::once_flag g_options_once;
+bool env_is_1(const char* name)
+{
+    const char* v = getenv(name);
+    return v != nullptr && v[0] == '1';
+}
+void read_options()
+{
+    Options o;
+    const char* t = getenv("PTOAMD_TILE");
+    if (t != nullptr && t[0] >= '0' && t[0] <= '6')
+        o.tile = t[0] - '0';
+    o.no_tail_split = getenv("PTOAMD_NO_TAIL_SPLIT") != nullptr;
+    const char* tt = getenv("PTOAMD_TAIL_TILE");
+    if (tt != nullptr && (tt[0] == '5' || tt[0] == '6'))
+        o.tail_tile = tt[0] - '0';
+    o.force_generic = env_is_1("PTOAMD_FORCE_GENERIC");
+    o.b_nd_transpose = getenv("PTOAMD_B_ND_TRANSPOSE") != nullptr;
+    o.gemv_sw_cvt = env_is_1("PTOAMD_GEMV_SW_CVT");
+    o.gemv_no_splitk = env_is_1("PTOAMD_GEMV_NO_SPLITK");
+    o.gemv_no_wide = env_is_1("PTOAMD_GEMV_NO_WIDE");
+    g_options = o;
+}
+}  // namespace
+const Options& options()
+{
+    std::call_once(g_options_once, read_options);
+    return g_options;
+}
+int device_compute_units()
+{
+    static int cus[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return 256;
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
 // ---- launch trace -----------------------------------------------------------------------------------------------------
 namespace {
 struct TraceSink {
@@ -145,6 +192,15 @@ int ptoamd_init(int device)
         set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
         return PTOAMD_E_NODEVICE;
     }
+    (void)options();
+    (void)device_compute_units();
+    return PTOAMD_OK;
+}
+
+int ptoamd_reload_options(void)
+{
+    (void)options();   // the first read has happened
+    read_options();    // not synchronised with launches running on other host threads: call it between launches
     return PTOAMD_OK;
 }
 

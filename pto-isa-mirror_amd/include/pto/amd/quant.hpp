@@ -61,17 +61,9 @@ PTO_INST void tquant_mx(TileOut& dst, TileSrc& src, TileExp* exp, TileMax* mx, T
     for (int g = threadIdx.x; g < vr * groups_per_row; g += PTO_AMD_THREADS) {
         const int r = g / groups_per_row, c0 = (g - r * groups_per_row) * 32;
         uint32_t run = 0;
-        float first_nan = 0.0f;
-        bool seen_nan = false;
-        for (int i = 0; i < 32; ++i) {
-            const float v = to_float(*reinterpret_cast<const S*>(src.Storage() + src.ByteOffset(r, c0 + i)));
-            if (!seen_nan && v != v) {
-                first_nan = v;
-                seen_nan = true;
-            }
-            run = ptoamd::max_step<ALG>(run, v);
-        }
-        const float maxabs = ptoamd::max_value<ALG>(run, first_nan);
+        for (int i = 0; i < 32; ++i)
+            run = ptoamd::max_step<ALG>(run, to_float(*reinterpret_cast<const S*>(src.Storage() + src.ByteOffset(r, c0 + i))), i);
+        const float maxabs = ptoamd::max_value<ALG>(run);
         const uint32_t e = ptoamd::shared_exponent<ALG>(maxabs);
         const float sc = ptoamd::group_scaling<ALG>(maxabs, e);
         if (exp)
@@ -112,8 +104,8 @@ PTO_INST void tquant_mx_cols(TileOut& dst, TileSrc& src, TileExp* exp, TileMax* 
         for (int j = 0; j < 2; ++j) {
             uint32_t run = 0;
             for (int r = 0; r < 32; ++r)
-                run = ptoamd::max_step<ALG>(run, at(g * 32 + r, c0 + j));
-            const float maxabs = ptoamd::max_value<ALG>(run, ptoamd::u2f(0x7FC00000u));
+                run = ptoamd::max_step<ALG>(run, at(g * 32 + r, c0 + j), r);
+            const float maxabs = ptoamd::max_value<ALG>(run);
             const uint32_t e = ptoamd::shared_exponent<ALG>(maxabs);
             sc[j] = ptoamd::group_scaling<ALG>(maxabs, e);
             const int gi = g * vc + c0 + j;

@@ -88,29 +88,36 @@ __device__ __forceinline__ float group_scaling(float maxabs, uint32_t e8m0)
 }
 
 // ComputeMxGroupMax's per-element step (TQuant.hpp:280-306).  The running value is kept as bits: for OCP-FP4 it is
-// the maximum of truncated-bf16 magnitude patterns, otherwise max(fabs) where NaN never wins (NV-FP4: NaN wins).
+// the maximum of truncated-bf16 magnitude patterns, otherwise max(fabs) where NaN never wins.  NV-FP4 returns the first
+// NaN of the group as it stands (sign and payload): a NaN at position pos (0 .. 31 in group order) is carried as
+// bit 31 | (31 - pos) << 26 | sign << 23 | mantissa, which is larger than every magnitude pattern and larger for an
+// earlier position, so one unsigned max over the group -- in any order, across lanes -- leaves the first NaN.
 template <int ALG>
-__device__ __forceinline__ uint32_t max_step(uint32_t run, float v)
+__device__ __forceinline__ uint32_t max_step(uint32_t run, float v, int pos = 0)
 {
     const uint32_t ab = f2u(v) & 0x7FFFFFFFu;
     if (ALG == MX_OCP_FP4) {
         const uint32_t t = ab & 0x7FFF0000u;
         return t > run ? t : run;
     }
-    if (ab > 0x7F800000u)                               // NaN
-        return ALG == MX_NV_FP4 ? 0xFFFFFFFFu : run;  // sentinel: the group maximum is NaN
-    return (run != 0xFFFFFFFFu && ab > run) ? ab : run;
+    if (ab > 0x7F800000u) {  // NaN
+        if (ALG != MX_NV_FP4)
+            return run;
+        const uint32_t tag = 0x80000000u | ((uint32_t)(31 - pos) << 26) | ((f2u(v) >> 31) << 23) | (ab & 0x007FFFFFu);
+        return tag > run ? tag : run;
+    }
+    return ab > run ? ab : run;
 }
 template <int ALG>
 __device__ __forceinline__ uint32_t max_merge(uint32_t a, uint32_t b)
 {
-    return a > b ? a : b;  // bit patterns of non-negative floats order like the floats; the NaN sentinel is largest
+    return a > b ? a : b;  // bit patterns of non-negative floats order like the floats; a tagged NaN is larger than all
 }
 template <int ALG>
-__device__ __forceinline__ float max_value(uint32_t run, float first_nan)
+__device__ __forceinline__ float max_value(uint32_t run)
 {
-    if (ALG == MX_NV_FP4 && run == 0xFFFFFFFFu)
-        return first_nan;
+    if (ALG == MX_NV_FP4 && (run >> 31))
+        return u2f(0x7F800000u | ((run & 0x00800000u) << 8) | (run & 0x007FFFFFu));
     return u2f(run);
 }
 

@@ -70,8 +70,14 @@ def check_f32_drain(got, ref, absdot, k, label, max_rel=1e-4, eps=None):
 
 
 class tile_env:
+    """Sets PTOAMD_* switches for the enclosed launches (the library reads them once, so it is told to read again)."""
+
     def __init__(self, **kw):
         self.kw = kw
+
+    @staticmethod
+    def _reload():
+        ge.load_package().reload_options()
 
     def __enter__(self):
         self.old = {k: os.environ.get(k) for k in self.kw}
@@ -80,6 +86,7 @@ class tile_env:
                 os.environ.pop(k, None)
             else:
                 os.environ[k] = str(v)
+        self._reload()
 
     def __exit__(self, *a):
         for k, v in self.old.items():
@@ -87,6 +94,7 @@ class tile_env:
                 os.environ.pop(k, None)
             else:
                 os.environ[k] = v
+        self._reload()
 
 
 # ------------------------------------------------------------------------------------------- TMATMUL, fp16 / bf16
@@ -1047,7 +1055,13 @@ def test_config5_mxfp4_decode_full_size(pa, oracle):
 
 # ------------------------------------------------------------------------------------------- TQUANT / TDEQUANT
 def _eq_f32(a, b):
-    return np.array_equal(a.view(np.uint32) & 0xFFBFFFFF, b.view(np.uint32) & 0xFFBFFFFF)
+    """Bit equality of two float32 arrays; where both hold a NaN, the quiet bit (22) alone may differ (the host's and the
+    GPU's max / multiply quieten a signalling NaN differently), every other element must match in all 32 bits."""
+    ua, ub = np.ascontiguousarray(a).view(np.uint32).copy(), np.ascontiguousarray(b).view(np.uint32).copy()
+    both_nan = np.isnan(a) & np.isnan(b)
+    ua[both_nan] &= 0xFFBFFFFF
+    ub[both_nan] &= 0xFFBFFFFF
+    return np.array_equal(ua, ub)
 
 
 @pytest.mark.parametrize("alg", [0, 1, 2, 3])
@@ -1121,6 +1135,44 @@ def test_tquant_mxfp8_every_bf16_pattern_and_edge_groups(pa, oracle, alg):
     assert np.array_equal(exp, re)
     bad = np.argwhere(codes != rc)
     assert bad.size == 0, (bad[:5], codes[codes != rc][:5], rc[codes != rc][:5])
+    assert _eq_f32(mx, rm) and _eq_f32(sc, rs)
+
+
+@pytest.mark.parametrize("alg", [2, 3])
+def test_tquant_mxfp4_nan_and_infinity_edge_groups(pa, oracle, alg):
+    """The MXFP4 quantiser's packed hardware conversion against the oracle's magic-number encoder on the groups where a
+    NaN or an infinity decides the code: NaNs of either sign in otherwise finite groups (quiet ones make the whole group's
+    scaling NaN; one whose payload sits in the low 16 bits truncates to a bf16 infinity in the OCP group maximum, so the
+    scaling stays finite and the NaN element itself is encoded: 0x7 whatever its sign), infinities, and both together;
+    f32 sources and the same groups as a bf16 source."""
+    r = np.random.default_rng(70 + alg)
+    g = (r.standard_normal((12, 32)) * 2).astype(np.float32)
+    gb = g.view(np.uint32)
+    gb[0, 5] = 0x7FC00000
+    gb[1, 6] = 0xFFC00000
+    gb[2, 7] = 0x7F800001; gb[2, 8] = 0xFF800001          # payload in the low half only: finite OCP scaling, NaN elements
+    gb[3, 0] = 0xFF80FFFF; gb[3, 31] = 0x7F800400
+    g[4, 3] = np.inf
+    g[5, 4] = -np.inf
+    g[6, 1] = np.inf; gb[6, 2] = 0xFF800001
+    g[7, 9] = -np.inf; gb[7, 10] = 0x7FC00000
+    g[8] = 0.0; gb[8, 30] = 0xFF800001
+    g[9] = r.standard_normal(32) * 1e30
+    g[10] = r.standard_normal(32) * 1e-30; gb[10, 0] = 0xFF812345
+    g[11] = 6.0; g[11, ::2] = -6.0; gb[11, 1] = 0xFF800002
+    src = np.ascontiguousarray(np.tile(g, (1, 4)))
+    codes, exp, mx, sc = (host(t) for t in pa.tquant_mx(dev(src), alg, 1))
+    rc, re, rm, rs = oracle.tquant_mx(src, alg, 1)
+    assert np.array_equal(exp, re)
+    bad = np.argwhere(codes != rc)
+    assert bad.size == 0, (bad[:5], codes[codes != rc][:5], rc[codes != rc][:5])
+    assert _eq_f32(mx, rm) and _eq_f32(sc, rs)
+    # the same groups through a bf16 source (its NaNs keep their payload's high bits, so they are all of the first kind)
+    srcb = torch.from_numpy(src.view(np.int32) >> 16).to(torch.int16).view(torch.bfloat16)
+    as_f32 = (srcb.view(torch.int16).numpy().astype(np.uint16).astype(np.uint32) << 16).view(np.float32)
+    codes, exp, mx, sc = (host(t) for t in pa.tquant_mx(srcb.to(DEV), alg, 1))
+    rc, re, rm, rs = oracle.tquant_mx(as_f32, alg, 1, ob.SRC_BF16)
+    assert np.array_equal(exp, re) and np.array_equal(codes, rc)
     assert _eq_f32(mx, rm) and _eq_f32(sc, rs)
 
 
