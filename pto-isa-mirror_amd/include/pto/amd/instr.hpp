@@ -3,10 +3,18 @@
 // TMATMUL / _ACC / _BIAS / TGEMV* cpu/TMatmul.hpp:77-113,207-252; TSTORE cpu/TStore.hpp:41-79,
 // cpu/common.hpp:187-198 (relu then static_cast).  Wrapper signatures: common/pto_instr.hpp:257-268,377-447,952-1010.
 //
-// Ordering: every instruction that writes LDS ends with a workgroup barrier, and starts with one (earlier readers of
-// the bytes it overwrites are done); instructions that only read LDS need no barrier of their own.
+// Ordering: every instruction that writes LDS starts with a workgroup barrier (earlier readers of the bytes it overwrites
+// are done) and ends with one, with one exception: a TLOAD that can run as LDS-DMA (a fully valid boxed Mat tile from a
+// 16-byte aligned ND / DN global tensor) only issues its copies and marks the tile pending; the first instruction that
+// reads the tile waits for the copies and for the other waves (acquire).  Between the TLOAD and that read the core is
+// free to run other tile instructions -- the TMATMULs of the previous panel -- which is how a PTO program's
+// double-buffered L1 panels overlap copy-in and MFMA on this backend.  Instructions that only read LDS need no barrier
+// of their own.
 #pragma once
+#include <utility>
+
 #include "device_types.hpp"
+#include "lds_dma.hpp"
 #include "tile.hpp"
 
 namespace pto {
@@ -29,12 +37,78 @@ constexpr bool is_number = std::is_integral_v<T> || std::is_same_v<T, float> || 
 template <typename T>
 constexpr bool is_packed4 = std::is_same_v<T, float4_e2m1x2_t> || std::is_same_v<T, float4_e1m2x2_t>;
 
+// a Mat tile whose asynchronous TLOAD may still be in flight: wait for this wave's copies, then for every wave's
+template <typename TileData>
+PTO_INST void acquire(TileData& t)
+{
+    if constexpr (TileData::Loc == TileType::Mat) {
+        if (t.pend_) {  // the same value in every thread of the core
+            dma_wait();
+            __syncthreads();
+            t.pend_ = 0;
+        }
+    }
+}
+
+// ---- TLOAD as LDS-DMA -------------------------------------------------------------------------------------------------
+// A boxed Mat tile is stored as swizzled lines (rows for the A-side layouts, columns for the B-side ones).  When the
+// global tensor delivers those lines contiguously -- ND for row lines, DN for column lines -- every 16-byte chunk of
+// the tile is one lane of a global_load_lds_dwordx4: chunk position q of the tile's storage (line q / C, position
+// q % C) is fetched from the line's logical chunk (q % C) ^ swizzle(line), because the DMA writes lanes linearly and the
+// swizzle therefore has to be applied on the global side.  Returns false (nothing done) when the operands do not
+// qualify; the caller then takes the element-wise path.
+template <typename TileData, typename GlobalData>
+PTO_INST bool tload_dma(TileData& dst, GlobalData& src)
+{
+    using T = typename TileData::DType;
+    if constexpr (TileData::MatLines && TileData::LineBytes % 16 == 0 && sizeof(T) == sizeof(typename GlobalData::DType) &&
+                  ((GlobalData::layout == Layout::ND && TileData::LinesAreRows) ||
+                   (GlobalData::layout == Layout::DN && !TileData::LinesAreRows))) {
+        constexpr bool nd = GlobalData::layout == Layout::ND;
+        // ND: element (r, c) at r * stride[3] + c * stride[4]; DN: the same with the unit stride on the rows
+        const int64_t line_stride = src.GetStride(nd ? 3 : 4), unit_stride = src.GetStride(nd ? 4 : 3);
+        const int64_t gbytes = line_stride * (int64_t)sizeof(T);
+        const uintptr_t gaddr = reinterpret_cast<uintptr_t>(src.data());
+        const bool ok = src.GetShape(0) == 1 && src.GetShape(1) == 1 && src.GetShape(2) == 1 && unit_stride == 1 &&
+                        src.GetShape(3) >= TileData::Rows && src.GetShape(4) >= TileData::Cols &&
+                        dst.GetValidRow() == TileData::Rows && dst.GetValidCol() == TileData::Cols && (gbytes & 15) == 0 &&
+                        (gaddr & 15u) == 0 && gbytes > 0 &&
+                        (int64_t)(TileData::Lines - 1) * gbytes + TileData::LineBytes <= (int64_t)0xFFFFFFFFll;
+        if (!ok)
+            return false;
+        acquire(dst);     // an earlier asynchronous load of the same tile has landed before it is overwritten
+        __syncthreads();  // earlier readers of the tile (TMATMULs through windows, TMOVs) are done
+        constexpr int C = TileData::LineBytes / 16, total = TileData::Lines * C;
+        constexpr int iters = (total + PTO_AMD_THREADS - 1) / PTO_AMD_THREADS;
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const uint32_t lds0 = lds_address_of(dst.Storage()) + wave * 1024u;
+        const uint32_t gb32 = (uint32_t)gbytes;
+#pragma unroll
+        for (int i = 0; i < iters; ++i) {
+            const uint32_t q = threadIdx.x + i * PTO_AMD_THREADS;
+            if (total % PTO_AMD_THREADS == 0 || q < (uint32_t)total) {
+                const uint32_t line = q / C, pos = q % C;
+                const uint32_t chunk = pos ^ ((line >> TileData::Swz::sh) & TileData::Swz::mask);
+                lds_dma16_off(reinterpret_cast<const uint8_t*>(src.data()), line * gb32 + chunk * 16u,
+                              lds0 + (uint32_t)i * (PTO_AMD_THREADS * 16u));
+            }
+        }
+        dst.pend_ = 1;
+        return true;
+    } else {
+        return false;
+    }
+}
+
 // ---- generic element movement between global memory and an LDS tile ------------------------------------------------
 template <typename TileData, typename GlobalData>
 PTO_INST void tload_lds(TileData& dst, GlobalData& src)
 {
     using T = typename TileData::DType;
     static_assert(sizeof(T) == sizeof(typename GlobalData::DType), "TLOAD: tile and global element sizes differ");
+    if (tload_dma(dst, src))
+        return;
+    acquire(dst);
     const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
     const auto* g = reinterpret_cast<const T*>(src.data());
     uint8_t* base = dst.Storage();
@@ -65,6 +139,7 @@ PTO_INST void tstore_lds(GlobalData& dst, TileData& src)
     using T = typename TileData::DType;
     using G = typename GlobalData::DType;
     static_assert(atomic == AtomicType::AtomicNone, "TSTORE AtomicAdd from an LDS tile is not implemented on this backend");
+    acquire(src);
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
     auto* g = reinterpret_cast<G*>(dst.data());
     const uint8_t* base = src.Storage();
@@ -90,13 +165,57 @@ PTO_INST void tstore_lds(GlobalData& dst, TileData& src)
     }
 }
 
+// A Left / Right tile as a window onto the boxed Mat tile it is extracted from: nothing moves, the tile records where
+// its lines live.  Possible when the Mat tile stores the lines the matrix unit wants (rows for Left, columns for Right),
+// the offset along a line is a whole number of 16-byte chunks, and the window lies inside the source's valid region with
+// the destination fully valid (a copy would zero-fill what lies outside; a window cannot).  Returns false when the
+// extraction has to copy.
+template <typename DstTile, typename SrcTile>
+PTO_INST bool textract_window(DstTile& dst, SrcTile& src, int row0, int col0)
+{
+    using T = typename DstTile::DType;
+    if constexpr (SrcTile::MatLines && !is_packed4<T> &&
+                  ((DstTile::Loc == TileType::Left && SrcTile::LinesAreRows) || (DstTile::Loc == TileType::Right && !SrcTile::LinesAreRows))) {
+        constexpr bool left = DstTile::Loc == TileType::Left;
+        const uint32_t kb0 = (uint32_t)(left ? col0 : row0) * (uint32_t)sizeof(T);
+        const bool ok = (kb0 & 15u) == 0 && row0 >= 0 && col0 >= 0 && row0 + DstTile::Rows <= src.GetValidRow() &&
+                        col0 + DstTile::Cols <= src.GetValidCol() && dst.GetValidRow() == DstTile::Rows &&
+                        dst.GetValidCol() == DstTile::Cols;
+        if (!ok)
+            return false;
+        acquire(src);
+        dst.lds_ = src.lds_;
+        dst.pitch_ = SrcTile::LineBytes;
+        dst.sh_ = SrcTile::Swz::sh;
+        dst.mask_ = SrcTile::Swz::mask;
+        dst.line0_ = (uint32_t)(left ? row0 : col0);
+        dst.kb0_ = kb0;
+        return true;
+    } else {
+        return false;
+    }
+}
+
 // dst(r, c) = src(r + row0, c + col0) over dst's static extent, zero outside src's valid region: the zero fill is what
 // lets TMATMUL walk the padded K of Left / Right tiles
-template <typename DstTile, typename SrcTile>
+// (WINDOW_OK: the caller does not go on to modify the destination, as the relu forms do)
+template <bool WINDOW_OK = true, typename DstTile, typename SrcTile>
 PTO_INST void textract_lds(DstTile& dst, SrcTile& src, int row0, int col0)
 {
     using T = typename DstTile::DType;
     static_assert(std::is_same_v<T, typename SrcTile::DType>, "TMOV / TEXTRACT: element types differ");
+    if constexpr (DstTile::Loc == TileType::Left || DstTile::Loc == TileType::Right) {
+        if constexpr (WINDOW_OK) {
+            if (textract_window(dst, src, row0, col0))
+                return;
+        }
+        dst.BindOwnLines();  // a copy goes to the tile's own bytes in L0A / L0B
+        if (!dst.own_ok_) {
+            report(1);  // the TASSIGN address (plus the tile's size) lies outside the region: nothing is copied
+            return;
+        }
+    }
+    acquire(src);
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
     const uint8_t* s = src.Storage();
     uint8_t* d = dst.Storage();
@@ -147,64 +266,66 @@ PTO_INST void textract_lds(DstTile& dst, SrcTile& src, int row0, int col0)
 }
 
 // ---- the contraction ------------------------------------------------------------------------------------------------
-// One 32 x 32 block per MFMA chain: lane (l32, lhi) feeds row l32 of the Left block and column l32 of the Right block;
-// its k-slots inside a step are lhi * (STEP / 2) .. + STEP / 2 - 1.
+// One 32 x 32 block per MFMA chain.  Lane (l32, lhi) feeds line l32 of an operand block (a row of Left, a column of
+// Right); its k-slots inside a step are lhi * (STEP / 2) .. + STEP / 2 - 1, read as one fragment of 4, 8 or 16 bytes.
+// The Right fragment goes in as the instruction's first operand, so the result block arrives transposed: the lane holds
+// row l32 of C and four consecutive columns per register quad.
 template <typename T>
 struct Mfma;
 template <>
 struct Mfma<_Float16> {
     static constexpr int STEP = 16;
+    using Frag = f16x8;
     template <typename Acc>
-    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const f16x8*>(a), *reinterpret_cast<const f16x8*>(b), c, 0, 0, 0);
-    }
+    PTO_INST static Acc run(Frag a, Frag b, Acc c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(b, a, c, 0, 0, 0); }
 };
 template <>
 struct Mfma<__bf16> {
     static constexpr int STEP = 16;
+    using Frag = bf16x8;
     template <typename Acc>
-    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(a), *reinterpret_cast<const bf16x8*>(b), c, 0, 0, 0);
-    }
+    PTO_INST static Acc run(Frag a, Frag b, Acc c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, a, c, 0, 0, 0); }
 };
 template <>
 struct Mfma<int8_t> {
     static constexpr int STEP = 32;
+    using Frag = i32x4v;
     template <typename Acc>
-    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
-    {
-        return __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const i32x4v*>(a), *reinterpret_cast<const i32x4v*>(b), c, 0, 0, 0);
-    }
+    PTO_INST static Acc run(Frag a, Frag b, Acc c) { return __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, c, 0, 0, 0); }
 };
 template <>
 struct Mfma<float> {
     static constexpr int STEP = 2;
+    using Frag = float;
     template <typename Acc>
-    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x2f32(*reinterpret_cast<const float*>(a), *reinterpret_cast<const float*>(b), c, 0, 0, 0);
-    }
+    PTO_INST static Acc run(Frag a, Frag b, Acc c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(b, a, c, 0, 0, 0); }
 };
 template <>
 struct Mfma<float8_e4m3_t> {
     static constexpr int STEP = 16;
+    using Frag = long;
     template <typename Acc>
-    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(*reinterpret_cast<const long*>(a), *reinterpret_cast<const long*>(b), c, 0, 0, 0);
-    }
+    PTO_INST static Acc run(Frag a, Frag b, Acc c) { return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(b, a, c, 0, 0, 0); }
 };
 template <>
 struct Mfma<float8_e5m2_t> {
     static constexpr int STEP = 16;
+    using Frag = long;
     template <typename Acc>
-    PTO_INST static Acc run(const uint8_t* a, const uint8_t* b, Acc c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(*reinterpret_cast<const long*>(a), *reinterpret_cast<const long*>(b), c, 0, 0, 0);
-    }
+    PTO_INST static Acc run(Frag a, Frag b, Acc c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(b, a, c, 0, 0, 0); }
 };
+
+// compile-time loop with literal indices (register arrays stay in registers)
+template <int... Is, class F>
+PTO_INST void static_for_impl(std::integer_sequence<int, Is...>, F&& f)
+{
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+PTO_INST void static_for(F&& f)
+{
+    static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
+}
 
 template <bool INIT, typename TileRes, typename TileLeftT, typename TileRightT>
 PTO_INST void tmatmul(TileRes& c, TileLeftT& a, TileRightT& b)
@@ -218,34 +339,77 @@ PTO_INST void tmatmul(TileRes& c, TileLeftT& a, TileRightT& b)
     static_assert(std::is_integral_v<typename TileRes::DType> == std::is_integral_v<T>,
                   "TMATMUL: int8 operands accumulate in int32, floating operands in float");
     using M = Mfma<T>;
+    using Frag = typename M::Frag;
     static_assert(TileLeftT::Cols % M::STEP == 0, "TMATMUL: the static K of the tiles must be a multiple of the MFMA k-step");
     const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int kpad = min((a.GetValidCol() + M::STEP - 1) / M::STEP * M::STEP, TileLeftT::Cols);
     const uint8_t* pa = a.Storage();
     const uint8_t* pb = b.Storage();
-    constexpr int RB = TileRes::RB, CB = TileRes::CB;
+    if constexpr (INIT) {
 #pragma unroll
-    for (int slot = 0; slot < TileRes::NBLK; ++slot) {
-        const int blk = slot * WAVES + wave;
-        if (blk < RB * CB) {
-            const int bi = blk / CB, bj = blk - bi * CB;
-            const int arow = min(bi * 32 + l32, TileLeftT::Rows - 1);
-            const int bcol = min(bj * 32 + l32, TileRightT::Cols - 1);
-            typename TileRes::Vec16 acc = c.regs[slot];
-            if constexpr (INIT)
-                acc = typename TileRes::Vec16(0);
-            for (int k0 = 0; k0 < kpad; k0 += M::STEP) {
-                const int k = k0 + lhi * (M::STEP / 2);
-                acc = M::run(pa + a.ByteOffset(arow, k), pb + b.ByteOffset(k, bcol), acc);
+        for (int slot = 0; slot < TileRes::NBLK; ++slot)
+            c.regs[slot] = typename TileRes::Vec16(0);
+    }
+    if constexpr (TileRes::BLOCKED) {
+        // The wave owns MB x NB neighbouring blocks: per k-step it reads MB Left and NB Right fragments and issues
+        // MB * NB MFMAs.  A lane's line is the same in every k-step, so the line part of the address is computed once.
+        constexpr int MB = TileRes::MB, NB = TileRes::NB;
+        const int wr = wave / TileRes::grid.wc, wc = wave % TileRes::grid.wc;
+        uint32_t aline[MB], bline[NB];
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+            aline[i] = (uint32_t)min((wr * MB + i) * 32 + l32, TileLeftT::Rows - 1);
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+            bline[j] = (uint32_t)min((wc * NB + j) * 32 + l32, TileRightT::Cols - 1);
+        auto kstep = [&](int k0) __attribute__((always_inline)) {
+            const int k = k0 + lhi * (M::STEP / 2);
+            Frag fa[MB], fb[NB];
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+                fb[j] = *reinterpret_cast<const Frag*>(pb + b.ByteOffset(k, (int)bline[j]));
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+                fa[i] = *reinterpret_cast<const Frag*>(pa + a.ByteOffset((int)aline[i], k));
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+                    c.regs[i * NB + j] = M::run(fa[i], fb[j], c.regs[i * NB + j]);
+        };
+        if constexpr (TileLeftT::ValidCol != DYNAMIC) {  // the padded K is known: a straight line of k-steps
+            constexpr int kpad = (TileLeftT::ValidCol + M::STEP - 1) / M::STEP * M::STEP < TileLeftT::Cols
+                                     ? (TileLeftT::ValidCol + M::STEP - 1) / M::STEP * M::STEP
+                                     : TileLeftT::Cols;
+            static_for<kpad / M::STEP>([&](auto sc) { kstep(decltype(sc)::value * M::STEP); });
+        } else {
+            const int kpad = min((a.GetValidCol() + M::STEP - 1) / M::STEP * M::STEP, TileLeftT::Cols);
+            for (int k0 = 0; k0 < kpad; k0 += M::STEP)
+                kstep(k0);
+        }
+    } else {
+        const int kpad = min((a.GetValidCol() + M::STEP - 1) / M::STEP * M::STEP, TileLeftT::Cols);
+#pragma unroll
+        for (int slot = 0; slot < TileRes::NBLK; ++slot) {
+            int bi, bj;
+            if (TileRes::block_of(slot, wave, bi, bj)) {
+                const int arow = min(bi * 32 + l32, TileLeftT::Rows - 1);
+                const int bcol = min(bj * 32 + l32, TileRightT::Cols - 1);
+                typename TileRes::Vec16 acc = c.regs[slot];
+                for (int k0 = 0; k0 < kpad; k0 += M::STEP) {
+                    const int k = k0 + lhi * (M::STEP / 2);
+                    acc = M::run(*reinterpret_cast<const Frag*>(pa + a.ByteOffset(arow, k)),
+                                 *reinterpret_cast<const Frag*>(pb + b.ByteOffset(k, bcol)), acc);
+                }
+                c.regs[slot] = acc;
             }
-            c.regs[slot] = acc;
         }
     }
 }
 
 // Block-scaled contraction on v_mfma_scale_f32_32x32x64_f8f6f4: a k-step is two MX blocks of 32; lane (l32, lhi) feeds
-// bytes [16 lhi, 16 lhi + 16) of each block of its row / column and the E8M0 scale of block lhi.
+// bytes [16 lhi, 16 lhi + 16) of each block of its row / column and the E8M0 scale of block lhi.  As in tmatmul the Right
+// operand (with its scale) goes first, so the accumulator block arrives transposed.
 template <typename T>
 struct MxFormat;
 template <>
@@ -314,12 +478,10 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kpad = min((a.GetValidCol() + 63) / 64 * 64, TileRightT::Rows);
     const uint8_t *pa = a.Storage(), *pb = b.Storage(), *psa = as.Storage(), *psb = bs.Storage();
-    constexpr int CB = TileRes::CB;
 #pragma unroll
     for (int slot = 0; slot < TileRes::NBLK; ++slot) {
-        const int blk = slot * WAVES + wave;
-        if (blk < TileRes::RB * CB) {
-            const int bi = blk / CB, bj = blk - bi * CB;
+        int bi, bj;
+        if (TileRes::block_of(slot, wave, bi, bj)) {
             const int arow = min(bi * 32 + l32, TileLeftT::Rows - 1);
             const int bcol = min(bj * 32 + l32, TileRightT::Cols - 1);
             typename TileRes::Vec16 acc = c.regs[slot];
@@ -338,7 +500,7 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
                     const uint2 eb[4] = {fp4x8_to_e4m3<TB>(b0.x), fp4x8_to_e4m3<TB>(b0.y), fp4x8_to_e4m3<TB>(b1.x), fp4x8_to_e4m3<TB>(b1.y)};
                     av = i32x8v{(int)ea[0].x, (int)ea[0].y, (int)ea[1].x, (int)ea[1].y, (int)ea[2].x, (int)ea[2].y, (int)ea[3].x, (int)ea[3].y};
                     bv = i32x8v{(int)eb[0].x, (int)eb[0].y, (int)eb[1].x, (int)eb[1].y, (int)eb[2].x, (int)eb[2].y, (int)eb[3].x, (int)eb[3].y};
-                    acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 0, 0, 0, sa, 0, sb);
+                    acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, acc, 0, 0, 0, sb, 0, sa);
                 } else {
                     if constexpr (is_packed4<TA>) {  // fp4: the lane's 16 bytes are the whole MX block lhi
                         const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(arow, k0 + 32 * lhi));
@@ -353,7 +515,7 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
                         av = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
                         bv = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
                     }
-                    acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, MxFormat<TA>::code, MxFormat<TB>::code, 0, sa, 0, sb);
+                    acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, acc, MxFormat<TB>::code, MxFormat<TA>::code, 0, sb, 0, sa);
                 }
             }
             c.regs[slot] = acc;
@@ -367,18 +529,21 @@ PTO_INST void for_each_acc(TileRes& c, F&& f)
 {
     const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    constexpr int CB = TileRes::CB;
 #pragma unroll
     for (int slot = 0; slot < TileRes::NBLK; ++slot) {
-        const int blk = slot * WAVES + wave;
-        if (blk < TileRes::RB * CB) {
-            const int bi = blk / CB, bj = blk - bi * CB;
+        int bi, bj;
+        if (TileRes::block_of(slot, wave, bi, bj)) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                f(slot, r, bi * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3), bj * 32 + l32);
+                f(slot, r, bi * 32 + l32, bj * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3));
         }
     }
 }
+
+template <typename G>
+struct alignas(4 * sizeof(G)) Quad {
+    G v[4];
+};
 
 template <typename TileRes, typename GlobalData, AtomicType atomic, ReluPreMode relu>
 PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
@@ -386,6 +551,50 @@ PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
     using G = typename GlobalData::DType;
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
     auto* g = reinterpret_cast<G*>(dst.data());
+    // Row-major destination with unit column stride: a lane's register quad is four consecutive columns of one row, so
+    // it leaves as one 8- or 16-byte store where the quad is whole and aligned.
+    if constexpr (GlobalData::layout == Layout::ND && atomic == AtomicType::AtomicNone && (sizeof(G) == 2 || sizeof(G) == 4)) {
+        const int64_t ld = dst.GetStride(3);
+        const bool vec_ok = dst.GetShape(0) == 1 && dst.GetShape(1) == 1 && dst.GetShape(2) == 1 && dst.GetStride(4) == 1 &&
+                            (ld & 3) == 0 && (reinterpret_cast<uintptr_t>(g) & (4 * sizeof(G) - 1)) == 0 && vr <= dst.GetShape(3);
+        if (vec_ok) {
+            const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+            const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+            for (int slot = 0; slot < TileRes::NBLK; ++slot) {
+                int bi, bj;
+                if (TileRes::block_of(slot, wave, bi, bj)) {
+                    const int row = bi * 32 + l32;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int col = bj * 32 + 8 * q + 4 * lhi;
+                        if (row < vr && col + 3 < vc) {
+                            Quad<G> out;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                auto v = src.regs[slot][4 * q + e];
+                                if constexpr (relu == ReluPreMode::NormalRelu)
+                                    v = v > 0 ? v : 0;
+                                out.v[e] = convert<G>(v);
+                            }
+                            *reinterpret_cast<Quad<G>*>(g + (int64_t)row * ld + col) = out;
+                        } else if (row < vr) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                if (col + e < vc) {
+                                    auto v = src.regs[slot][4 * q + e];
+                                    if constexpr (relu == ReluPreMode::NormalRelu)
+                                        v = v > 0 ? v : 0;
+                                    g[(int64_t)row * ld + col + e] = convert<G>(v);
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+            return;
+        }
+    }
     for_each_acc(src, [&](int slot, int r, int row, int col) {
         if (row < vr && col < vc) {
             auto v = src.regs[slot][r];
@@ -561,7 +770,7 @@ PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, WaitEvents&...)
     if constexpr (SrcTileData::Loc == TileType::Acc) {
         amd::tmov_acc<0, reluMode>(dst, src, 0, 0, [](int) { return (uint64_t)0; });
     } else {
-        amd::textract_lds(dst, src, 0, 0);
+        amd::textract_lds<reluMode == ReluPreMode::NoRelu>(dst, src, 0, 0);
         if constexpr (reluMode == ReluPreMode::NormalRelu)
             amd::trelu_lds(dst);
     }
@@ -600,7 +809,7 @@ PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, uint16_t index
     if constexpr (SrcTileData::Loc == TileType::Acc) {
         amd::tmov_acc<0, reluMode>(dst, src, indexRow, indexCol, [](int) { return (uint64_t)0; });
     } else {
-        amd::textract_lds(dst, src, indexRow, indexCol);
+        amd::textract_lds<reluMode == ReluPreMode::NoRelu>(dst, src, indexRow, indexCol);
         if constexpr (reluMode == ReluPreMode::NormalRelu)
             amd::trelu_lds(dst);
     }

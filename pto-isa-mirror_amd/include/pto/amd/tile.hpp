@@ -2,12 +2,22 @@
 // valid-shape accessors), cpu/TAssign.hpp:21-36 (address binding).
 //
 // Where a tile lives on gfx950:
-//   Mat (L1), Vec (UB), Bias, Scaling, ScaleLeft/Right : LDS, plain row-major [Rows][Cols]
-//   Left  (L0A) : LDS, [Rows = M][Cols = K], k contiguous, 16-byte chunks XOR-swizzled by row (MFMA fragment reads)
-//   Right (L0B) : LDS, stored transposed [Cols = N][Rows = K], k contiguous, same swizzle
-//   Acc   (L0C) : registers; the tile is cut into 32 x 32 MFMA blocks, block b belongs to wave b % WAVES
-// BLayout / SLayout / fractal size are accepted for source compatibility; the internal layouts above are the backend's
-// own (they are invisible in global-memory results).
+//   Vec (UB), Bias, Scaling, ScaleLeft/Right, Mat without a box layout : LDS, plain row-major [Rows][Cols]
+//   Mat (L1) with a box layout : LDS, "lines" of contiguous elements with the 16-byte chunks of a line XOR-swizzled by
+//                the line index: SLayout::RowMajor boxes (NZ, the A-side panels) keep rows as lines, [Rows][Cols];
+//                SLayout::ColMajor boxes (ZN, the B-side panels) keep columns as lines, [Cols][Rows].  Either way a
+//                GEMM panel is stored K-contiguous, which is what a 16-byte global -> LDS copy delivers and what an
+//                MFMA fragment read wants (packed fp4 Mat tiles stay plain row-major)
+//   Left  (L0A) : lines = rows, [M][K]; Right (L0B) : lines = columns, [N][K]; same swizzle.  A Left / Right tile is
+//                either a window onto the Mat tile it was extracted from (no bytes move: the matrix unit is fed from
+//                LDS through registers, there is no separate L0 memory to fill) or, when the extraction cannot be a
+//                window (unaligned offsets, ragged valid regions, a transposing or re-pairing move), a copy in the
+//                L0A / L0B region.  A window is valid until its Mat tile is next written.
+//   Acc   (L0C) : registers; the tile is cut into 32 x 32 MFMA blocks; when the block grid divides over a grid of
+//                waves each wave owns a rectangle of blocks (so an operand fragment feeds several MFMAs), otherwise
+//                block b belongs to wave b % WAVES
+// BLayout / SLayout / fractal size select among these; the internal layouts are the backend's own (they are invisible
+// in global-memory results).
 #pragma once
 #include "base.hpp"
 
@@ -72,17 +82,87 @@ struct ElemTraits<float4_e1m2x2_t> {
     static constexpr int bytes2 = 1;
 };
 
-// register storage of an accumulator tile
+// ---- swizzled line storage ---------------------------------------------------------------------------------------------
+// A line of LINE_BYTES bytes holds 16-byte chunks; chunk c of line l is stored at chunk position c ^ ((l >> sh) & mask).
+// sh / mask are chosen so that 16 consecutive lines read at one chunk index -- what a quarter wave of ds_read_b128 does
+// when it fetches MFMA fragments -- touch 16 different 16-byte slots of the 256 bytes that span all LDS banks:
+//   2 chunks per line (32 B): 8 lines per 256 B, lines l and l + 8 differ in the chunk bit     sh 3, mask 1
+//   4 chunks (64 B) sh 2, mask 3;   8 chunks (128 B) sh 1, mask 7;   16 or more chunks sh 0, mask 15
+template <int LINE_BYTES>
+struct LineSwizzle {
+    static constexpr int chunks = LINE_BYTES / 16;
+    static constexpr bool on = LINE_BYTES % 16 == 0 && chunks >= 2 && (chunks & (chunks - 1)) == 0;
+    static constexpr uint32_t sh = !on ? 0 : (chunks >= 16 ? 0 : (chunks == 8 ? 1 : (chunks == 4 ? 2 : 3)));
+    static constexpr uint32_t mask = !on ? 0 : (chunks >= 16 ? 15 : (uint32_t)chunks - 1);
+};
+PTO_INST uint32_t line_offset(uint32_t line, uint32_t kbyte, uint32_t pitch, uint32_t sh, uint32_t mask)
+{
+    return line * pitch + ((((kbyte >> 4) ^ ((line >> sh) & mask)) << 4) | (kbyte & 15u));
+}
+
+// how the accumulator blocks of an RB x CB block grid are dealt to the waves: a WR x WC grid of waves, each owning
+// (RB / WR) x (CB / WC) neighbouring blocks, with the split that needs the fewest operand fragments per k-step;
+// WR = 0 when no split divides the grid (blocks are then dealt round-robin)
+struct WaveGrid {
+    int wr, wc;
+};
+constexpr WaveGrid pick_wave_grid(int rb, int cb, int waves)
+{
+    WaveGrid best{0, 0};
+    int best_cost = 1 << 30;
+    for (int wr = 1; wr <= waves; ++wr) {
+        if (waves % wr != 0)
+            continue;
+        const int wc = waves / wr;
+        if (rb % wr != 0 || cb % wc != 0)
+            continue;
+        const int cost = rb / wr + cb / wc;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = WaveGrid{wr, wc};
+        }
+    }
+    return best;
+}
+
+// register storage of an accumulator tile.  Blocks are kept transposed: lane (l32, lhi) of the owning wave holds row
+// l32 of the block and, in register r, column 8 (r / 4) + 4 lhi + r % 4 -- four consecutive columns per register quad,
+// so a drain to row-major memory writes 8 or 16 contiguous bytes per lane and quad.
 template <typename T, int Rows, int Cols>
 struct AccStorage {
-    static constexpr int RB = (Rows + 31) / 32, CB = (Cols + 31) / 32, NBLK = (RB * CB + WAVES - 1) / WAVES;
+    static constexpr int RB = (Rows + 31) / 32, CB = (Cols + 31) / 32;
+    static constexpr WaveGrid grid = pick_wave_grid(RB, CB, WAVES);
+    static constexpr bool BLOCKED = grid.wr != 0;
+    static constexpr int MB = BLOCKED ? RB / grid.wr : 1, NB = BLOCKED ? CB / grid.wc : 1;
+    static constexpr int NBLK = BLOCKED ? MB * NB : (RB * CB + WAVES - 1) / WAVES;
     using Reg = std::conditional_t<std::is_integral_v<T>, int32_t, float>;
     typedef Reg Vec16 __attribute__((ext_vector_type(16)));
     Vec16 regs[NBLK];
+    // block (bi, bj) held in slot `slot` of wave `wave`; false when the slot is empty (round-robin dealing only)
+    PTO_INST static bool block_of(int slot, int wave, int& bi, int& bj)
+    {
+        if constexpr (BLOCKED) {
+            bi = (wave / grid.wc) * MB + slot / NB;
+            bj = (wave % grid.wc) * NB + slot % NB;
+            return true;
+        } else {
+            const int blk = slot * WAVES + wave;
+            bi = blk / CB;
+            bj = blk - bi * CB;
+            return blk < RB * CB;
+        }
+    }
 };
 struct LdsStorage {
     uint32_t lds_ = 0;   // byte offset of the tile in the arena
     uint32_t addr_ = 0;  // the TASSIGN address (offset inside the tile's region)
+    uint32_t pend_ = 0;  // Mat tiles: an asynchronous TLOAD into the tile may still be in flight
+};
+// Left / Right tiles: where the lines live (the tile's own storage, or a window onto a Mat tile)
+struct WindowStorage : LdsStorage {
+    uint32_t pitch_ = 0, sh_ = 0, mask_ = 0;  // line pitch in bytes and the swizzle of the storage the lines live in
+    uint32_t line0_ = 0, kb0_ = 0;            // first line / first byte along a line of the window
+    uint32_t own_ok_ = 1;                     // the tile's own storage lies inside its region (needed by copies only)
 };
 
 }  // namespace amd
@@ -91,7 +171,8 @@ template <TileType Loc_, typename Element_, const int Rows_, const int Cols_, co
           const int RowValid_ = Rows_, const int ColValid_ = Cols_, const SLayout SFractal_ = SLayout::NoneBox,
           const int SFractalSize_ = TileConfig::fractalABSize, auto PadVal_ = PadValue::Null,
           const CompactMode Compact_ = CompactMode::Null>
-struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_, Rows_, Cols_>, amd::LdsStorage> {
+struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_, Rows_, Cols_>,
+                                 std::conditional_t<Loc_ == TileType::Left || Loc_ == TileType::Right, amd::WindowStorage, amd::LdsStorage>> {
     using DType = Element_;
     static constexpr TileType Loc = Loc_;
     static constexpr int Rows = Rows_, Cols = Cols_, ValidRow = RowValid_, ValidCol = ColValid_;
@@ -118,10 +199,37 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
             vcol_ = a;
     }
     PTO_INST Tile(int r, int c) : vrow_(r), vcol_(c) { BindDefault(); }
+    // ---- storage layout (static part) ----
+    static constexpr bool is_packed4 = amd::ElemTraits<Element_>::bytes2 == 1;
+    // Mat tiles with a box layout are stored as swizzled lines; lines are rows for SLayout::RowMajor boxes, columns for
+    // SLayout::ColMajor boxes
+    static constexpr bool MatLines = Loc_ == TileType::Mat && SFractal_ != SLayout::NoneBox && !is_packed4;
+    static constexpr bool Lined = MatLines || Loc_ == TileType::Left || Loc_ == TileType::Right;
+    static constexpr bool LinesAreRows = Loc_ == TileType::Left || (MatLines && SFractal_ == SLayout::RowMajor);
+    static constexpr int Lines = LinesAreRows ? Rows_ : Cols_;
+    static constexpr int LineBytes = (LinesAreRows ? Cols_ : Rows_) * amd::ElemTraits<Element_>::bytes2 / 2;
+    using Swz = amd::LineSwizzle<LineBytes>;
+
     PTO_INST void BindDefault()
     {
         if constexpr (Loc_ != TileType::Acc)
             this->lds_ = amd::Region<Loc_>::base;
+        if constexpr (Loc_ == TileType::Left || Loc_ == TileType::Right) {
+            this->own_ok_ = Bytes <= amd::Region<Loc_>::size;
+            BindOwnLines();
+        }
+    }
+    // the lines are the tile's own storage (not a window onto a Mat tile)
+    PTO_INST void BindOwnLines()
+    {
+        if constexpr (Loc_ == TileType::Left || Loc_ == TileType::Right) {
+            this->lds_ = amd::Region<Loc_>::base + this->addr_;
+            this->pitch_ = LineBytes;
+            this->sh_ = Swz::sh;
+            this->mask_ = Swz::mask;
+            this->line0_ = 0;
+            this->kb0_ = 0;
+        }
     }
     static constexpr size_t GetSizeInBytes() { return Bytes; }
     PTO_INST int GetValidRow() const { return vrow_; }
@@ -131,32 +239,20 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
     PTO_INST uint32_t ByteOffset(int r, int c) const
     {
         constexpr int b2 = amd::ElemTraits<Element_>::bytes2;
-        if constexpr (Loc_ == TileType::Left)
-            return KContiguous<Cols_>(r, c);
-        else if constexpr (Loc_ == TileType::Right)
-            return KContiguous<Rows_>(c, r);
-        else
+        if constexpr (Loc_ == TileType::Left || Loc_ == TileType::Right) {
+            const uint32_t line = (uint32_t)(LinesAreRows ? r : c) + this->line0_;
+            const uint32_t kb = (uint32_t)((LinesAreRows ? c : r) * b2 / 2) + this->kb0_;
+            return amd::line_offset(line, kb, this->pitch_, this->sh_, this->mask_);
+        } else if constexpr (MatLines) {
+            return amd::line_offset((uint32_t)(LinesAreRows ? r : c), (uint32_t)((LinesAreRows ? c : r) * b2 / 2), LineBytes, Swz::sh,
+                                    Swz::mask);
+        } else {
             return (uint32_t)(((int64_t)r * Cols_ + c) * b2 / 2);
+        }
     }
     // which nibble of that byte holds element (r, c) of a packed fp4 tile: pairs run along k for Left / Right tiles,
     // along a row otherwise
     PTO_INST static int Nibble(int r, int c) { return Loc_ == TileType::Right ? (r & 1) : (c & 1); }
-    // [row][KC] with k contiguous; 16-byte chunk index XORed with the row when the row holds a power-of-two number of
-    // chunks (<= 8 of its low bits), so 32 rows read at one k land in different banks
-    template <int KC>
-    PTO_INST static uint32_t KContiguous(int row, int k)
-    {
-        constexpr int b2 = amd::ElemTraits<Element_>::bytes2;
-        constexpr int row_bytes = KC * b2 / 2, chunks = row_bytes / 16;
-        constexpr bool swz = row_bytes % 16 == 0 && chunks >= 2 && (chunks & (chunks - 1)) == 0;
-        const int kb = k * b2 / 2;
-        if constexpr (swz) {
-            constexpr int mask = chunks < 8 ? chunks - 1 : 7;
-            return (uint32_t)(row * row_bytes + ((((kb >> 4) ^ (row & mask))) << 4) + (kb & 15));
-        } else {
-            return (uint32_t)(row * row_bytes + kb);
-        }
-    }
     // the tile's on-chip address as TASSIGN bound it (what the reference's data() pointer stands for)
     PTO_INST uint64_t data() const
     {
@@ -251,7 +347,19 @@ PTO_INST uint64_t GetScaleAddr(uint64_t addr) { return addr >> 4; }
 template <typename T, typename AddrType>
 PTO_INST void TASSIGN(T& obj, AddrType addr)
 {
-    if constexpr (T::Loc != TileType::Acc) {
+    if constexpr (T::Loc == TileType::Left || T::Loc == TileType::Right) {
+        // a Left / Right tile needs its own bytes only when an extraction has to copy; one that does not fit its region
+        // can still be a window onto a Mat tile, so the range check is deferred to the copy
+        using R = amd::Region<T::Loc>;
+        uint32_t a = (uint32_t)(uint64_t)addr;
+        if ((a & 15u) != 0) {
+            amd::report(1);
+            a = 0;
+        }
+        obj.addr_ = a;
+        obj.own_ok_ = a + T::Bytes <= R::size;
+        obj.BindOwnLines();
+    } else if constexpr (T::Loc != TileType::Acc) {
         using R = amd::Region<T::Loc>;
         uint32_t a = (uint32_t)(uint64_t)addr;
         if (a + T::Bytes > R::size || (a & 15u) != 0) {
@@ -266,7 +374,9 @@ PTO_INST void TASSIGN(T& obj, AddrType addr)
 template <std::size_t Addr, typename T>
 PTO_INST std::enable_if_t<is_tile_data_v<T>> TASSIGN(T& obj)
 {
-    if constexpr (T::Loc != TileType::Acc) {
+    if constexpr (T::Loc == TileType::Left || T::Loc == TileType::Right) {
+        static_assert(Addr % 16 == 0, "TASSIGN: address not 16-byte aligned");
+    } else if constexpr (T::Loc != TileType::Acc) {
         static_assert(Addr + T::Bytes <= amd::Region<T::Loc>::size && Addr % 16 == 0,
                       "TASSIGN: address outside the tile's on-chip region or not 16-byte aligned");
     }
