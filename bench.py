@@ -140,6 +140,60 @@ def config5(pa, ev, gen, steps, warmup):
                 frac_of_peak=nbytes / ker / 1e6 / PEAK_HBM_GBPS)
 
 
+def _pto_lib(name):
+    """A library of kernels written in the PTO tile ISA against the header layer (pto-isa-mirror_amd/kernels/<name>.hip)."""
+    import ctypes as C
+    path = os.path.join(ge.PKG_DIR, "lib", f"libpto_{name}.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `make -C pto-isa-mirror_amd`")
+    return C, C.CDLL(path)
+
+
+def pto_api_bf16(pa, ev, gen, steps, warmup):
+    """configs[1] through the reference's own programming interface: the GEMM of kernels/gemm_performance.hip is a core
+    program of TASSIGN / TLOAD / TEXTRACT / TMATMUL(_ACC) / TSTORE calls, compiled against include/pto."""
+    C, lib = _pto_lib("gemm_performance")
+    m = n = k = 4096
+    a = randn_bf16((m, k), gen, 0.02)
+    b = randn_bf16((n, k), gen, 0.02)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+
+    def step():
+        rc = lib.pto_gemm_performance(0, C.c_void_p(out.data_ptr()), C.c_void_p(a.data_ptr()), C.c_void_p(b.data_ptr()),
+                                      C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, rc
+
+    wall, ker = time_launches(ev, step, steps, warmup)
+    ref = pa.gemm(a, b, pa.BF16, pa.BF16, pa.B_DN)
+    torch.cuda.synchronize()
+    assert lib.pto_gemm_performance_status() == 0 and torch.equal(out, ref), "the PTO-style GEMM and the launcher disagree"
+    flops = 2 * m * n * k
+    return dict(config="configs[1] bf16 4096^3 -> bf16 written in the PTO tile ISA (TLOAD / TEXTRACT / TMATMUL_ACC / TSTORE, "
+                       "256 x 256 tiles, K panels of 64)", kernel="GemmPerformance<bf16, 256, 256, 64> (header layer)", ms=ker,
+                wall_ms=wall, tflops=flops / ker / 1e9, bound="mfma", frac_of_peak=flops / ker / 1e9 / PEAK_TFLOPS["bf16"])
+
+
+def pto_api_config1(pa, ev, gen, steps, warmup):
+    """configs[0] through the tile ISA (kernels/gemm_tiled.hip): 128 x 128 tiles as BASELINE.json words it, and 64 x 64."""
+    C, lib = _pto_lib("gemm_tiled")
+    a = (torch.rand((512, 512), generator=gen, device=DEV) * 2 - 1).to(torch.float16)
+    b = (torch.rand((512, 512), generator=gen, device=DEV) * 2 - 1).to(torch.float16)
+    out = torch.empty((512, 512), dtype=torch.float32, device=DEV)
+    res = {}
+    for case in (0, 1):
+        def step():
+            rc = lib.pto_gemm_tiled(case, C.c_void_p(out.data_ptr()), C.c_void_p(a.data_ptr()), C.c_void_p(b.data_ptr()),
+                                    C.c_void_p(torch.cuda.current_stream().cuda_stream))
+            assert rc == 0, rc
+        res[case] = time_launches(ev, step, steps, warmup)
+    flops = 2 * 512 ** 3
+    wall, ker = res[0]
+    return dict(config="configs[0] fp16 512^3 -> fp32, B row-major, written in the PTO tile ISA (TLOAD / TMOV / TMATMUL_ACC / "
+                       "TSTORE, 128 x 128 tiles, K slabs of 64, 16 cores)", kernel="RunTiledGemm<f16, 128, 128, 64> (header layer)",
+                ms=ker, wall_ms=wall, tflops=flops / ker / 1e9, bound="latency",
+                frac_of_peak=flops / ker / 1e9 / PEAK_TFLOPS["f16"], ms_with_64x64_tiles=res[1][1])
+
+
 def _elementwise(name, kernel, nbytes, wall, ker):
     return dict(config=name, kernel=kernel, ms=ker, wall_ms=wall, gbps=nbytes / ker / 1e6, bound="hbm",
                 frac_of_peak=nbytes / ker / 1e6 / PEAK_HBM_GBPS, algorithmic_bytes=nbytes)
@@ -241,9 +295,10 @@ def main():
                     help="untimed run-in of the same launches before the warmup steps, for the GPU clock to settle")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-config measurements after the headline")
-    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4, 5, 6, 7, 8], default=None,
+    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10], default=None,
                     help="measure just BASELINE.json configs[N] (a per_config entry) and print it: for profiling one kernel; "
-                         "5-8 are the elementwise kernels (TQUANT MXFP8, TQUANT MXFP4, TQUANT INT8, TDEQUANT)")
+                         "5-8 are the elementwise kernels (TQUANT MXFP8, TQUANT MXFP4, TQUANT INT8, TDEQUANT), 9 and 10 "
+                         "configs[1] and configs[0] written in the PTO tile ISA")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic, to scale rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -265,7 +320,7 @@ def main():
     gen = torch.Generator(device=DEV).manual_seed(1)
     if args.only is not None:
         fn = {0: config1, 2: config3, 3: config4, 4: config5, 5: quant_mxfp8, 6: quant_mxfp4, 7: quant_int8,
-              8: dequant_int8}[args.only]
+              8: dequant_int8, 9: pto_api_bf16, 10: pto_api_config1}[args.only]
         print(json.dumps(fn(pa, ev, gen, args.steps, args.warmup)))
         return
 
@@ -291,7 +346,8 @@ def main():
     }
     if not args.no_extra:
         per = []
-        for fn in (config1, config3, config4, config5, quant_mxfp8, quant_mxfp4, quant_int8, dequant_int8):
+        for fn in (config1, config3, config4, config5, pto_api_bf16, pto_api_config1, quant_mxfp8, quant_mxfp4, quant_int8,
+                   dequant_int8):
             per.append(fn(pa, ev, gen, 50, 5))
             torch.cuda.empty_cache()
         line["per_config"] = per

@@ -32,6 +32,14 @@
 #ifndef PTO_AMD_L0S_BYTES
 #define PTO_AMD_L0S_BYTES (4 * 1024)
 #endif
+// Staging bytes of the fix-pipe (behind the regions above): where TSTORE of an accumulator tile turns the matrix unit's
+// register layout into whole rows before they leave for global memory.  A wave stages one 32 x 32 block at a time in a
+// band of 32 rows x (row bytes + 16); with fewer bytes than WAVES such bands of the output type, TSTORE writes each
+// lane's register quads directly (8 or 16 bytes per row and store instead of 64 or 128).  0 by default: the default
+// split of the other regions already fills the CU's 160 KiB.
+#ifndef PTO_AMD_STAGE_BYTES
+#define PTO_AMD_STAGE_BYTES 0
+#endif
 
 // A PTO kernel entry is written `__global__ AICORE void f(...)`; here it is a device function run by pto::amd::launch.
 // (PTO_AMD_CHECK_REFERENCE_SOURCE: a device-only syntax pass over an unmodified reference kernel file, whose

@@ -220,6 +220,33 @@ PTO_INST void textract_lds(DstTile& dst, SrcTile& src, int row0, int col0)
     const uint8_t* s = src.Storage();
     uint8_t* d = dst.Storage();
     __syncthreads();
+    // Transposing move of a whole window: the source keeps the other direction contiguous (a row-major B panel on its way
+    // to a Right tile, a column-major A panel to a Left tile).  One thread gathers the 16 / sizeof(T) elements of a
+    // destination chunk from consecutive source lines -- neighbouring lanes read neighbouring elements of one line -- and
+    // writes the chunk with one 16-byte store.
+    if constexpr ((DstTile::Loc == TileType::Left || DstTile::Loc == TileType::Right) && SrcTile::MatLines && !is_packed4<T> &&
+                  (sizeof(T) == 1 || sizeof(T) == 2) && DstTile::LinesAreRows != SrcTile::LinesAreRows && DstTile::LineBytes % 16 == 0) {
+        if (row0 >= 0 && col0 >= 0 && row0 + DstTile::Rows <= vr && col0 + DstTile::Cols <= vc && dst.GetValidRow() == DstTile::Rows &&
+            dst.GetValidCol() == DstTile::Cols) {
+            constexpr int EPC = 16 / (int)sizeof(T), chunks = DstTile::LineBytes / 16, units = DstTile::Lines * chunks;
+            for (int u = threadIdx.x; u < units; u += PTO_AMD_THREADS) {
+                const int line = u % DstTile::Lines, kc = u / DstTile::Lines;
+                uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) {
+                    const int kk = kc * EPC + e;
+                    const int r = DstTile::LinesAreRows ? line : kk, c = DstTile::LinesAreRows ? kk : line;
+                    const uint8_t* sp = s + src.ByteOffset(r + row0, c + col0);
+                    const uint32_t v = sizeof(T) == 2 ? (uint32_t)*reinterpret_cast<const uint16_t*>(sp) : (uint32_t)*sp;
+                    w[e * (int)sizeof(T) / 4] |= v << (8 * ((e * (int)sizeof(T)) % 4));
+                }
+                const int r0 = DstTile::LinesAreRows ? line : kc * EPC, c0 = DstTile::LinesAreRows ? kc * EPC : line;
+                *reinterpret_cast<uint4*>(d + dst.ByteOffset(r0, c0)) = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+            __syncthreads();
+            return;
+        }
+    }
     if constexpr (is_packed4<T>) {
         // two fp4 codes per byte: one thread builds one destination byte from the two source nibbles it needs (the
         // pairing direction of source and destination may differ: a Right tile pairs along k, a Mat tile along a row)
@@ -560,6 +587,43 @@ PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
         if (vec_ok) {
             const int lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
             const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            // Whole tile, whole blocks, 16-byte aligned rows, and a staging band per wave: every block goes through LDS
+            // and leaves as whole rows (64 or 128 contiguous bytes per row and store instruction).  The band is private
+            // to the wave, so no workgroup barrier is involved.
+            constexpr int row_bytes = 32 * (int)sizeof(G), pitch = row_bytes + 16, band = 32 * pitch;
+            if constexpr (TileRes::Rows % 32 == 0 && TileRes::Cols % 32 == 0 && (uint32_t)(WAVES * band) <= (uint32_t)PTO_AMD_STAGE_BYTES) {
+                if (vr == TileRes::Rows && vc == TileRes::Cols && ((ld * (int64_t)sizeof(G)) & 15) == 0 &&
+                    (reinterpret_cast<uintptr_t>(g) & 15u) == 0) {
+                    uint8_t* stage = lds_arena() + STAGE_BASE + wave * band;
+                    constexpr int lanes_per_row = row_bytes / 16, rows_per_pass = 64 / lanes_per_row;
+                    const int rrow = lane / lanes_per_row, rchunk = lane % lanes_per_row;
+#pragma unroll
+                    for (int slot = 0; slot < TileRes::NBLK; ++slot) {
+                        int bi, bj;
+                        TileRes::block_of(slot, wave, bi, bj);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            Quad<G> out;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                auto v = src.regs[slot][4 * q + e];
+                                if constexpr (relu == ReluPreMode::NormalRelu)
+                                    v = v > 0 ? v : 0;
+                                out.v[e] = convert<G>(v);
+                            }
+                            *reinterpret_cast<Quad<G>*>(stage + l32 * pitch + (8 * q + 4 * lhi) * (int)sizeof(G)) = out;
+                        }
+#pragma unroll
+                        for (int pass = 0; pass < 32 / rows_per_pass; ++pass) {
+                            const int r = pass * rows_per_pass + rrow;
+                            const i32x4v v = *reinterpret_cast<const i32x4v*>(stage + r * pitch + rchunk * 16);
+                            uint8_t* gp = reinterpret_cast<uint8_t*>(g + (int64_t)(bi * 32 + r) * ld + bj * 32) + rchunk * 16;
+                            __builtin_nontemporal_store(v, reinterpret_cast<i32x4v*>(gp));
+                        }
+                    }
+                    return;
+                }
+            }
 #pragma unroll
             for (int slot = 0; slot < TileRes::NBLK; ++slot) {
                 int bi, bj;

@@ -53,8 +53,9 @@ struct Region {
                                      : L == TileType::Scaling ? PTO_AMD_FB_BYTES
                                                               : PTO_AMD_L0S_BYTES / 2;
 };
-constexpr uint32_t LDS_TOTAL = PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES +
-                               PTO_AMD_BIAS_BYTES + PTO_AMD_FB_BYTES + PTO_AMD_L0S_BYTES;
+constexpr uint32_t STAGE_BASE = PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES +
+                                PTO_AMD_BIAS_BYTES + PTO_AMD_FB_BYTES + PTO_AMD_L0S_BYTES;
+constexpr uint32_t LDS_TOTAL = STAGE_BASE + PTO_AMD_STAGE_BYTES;
 #ifndef PTO_AMD_CHECK_REFERENCE_SOURCE
 static_assert(LDS_TOTAL <= 160 * 1024, "the on-chip regions must fit the 160 KiB LDS of a CU");
 #endif

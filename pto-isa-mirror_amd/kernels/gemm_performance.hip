@@ -8,6 +8,7 @@
 //   * a core is a workgroup of 512 threads (8 waves), and the L1 region takes most of the CU's 160 KiB of LDS: two panels
 //     of A and two of B;
 //   * Left / Right tiles extracted from those panels are windows onto them, so L0A / L0B need no bytes of their own;
+//   * 20 KiB of fix-pipe staging let TSTORE turn the accumulator blocks into whole 64-byte rows of bf16;
 //   * a core executes its tile instructions in program order, so the copy-in of panel p + 1 is issued *before* the
 //     TMATMULs of panel p (TLOAD only starts the copies; the TEXTRACT of the next iteration waits for them), where the
 //     reference issues it in the same iteration and lets the MTE2 queue run ahead.  The event flags of the reference
@@ -20,6 +21,7 @@
 #define PTO_AMD_BIAS_BYTES (1 * 1024)
 #define PTO_AMD_FB_BYTES (1 * 1024)
 #define PTO_AMD_L0S_BYTES (1 * 1024)
+#define PTO_AMD_STAGE_BYTES (8 * 32 * (64 + 16))  // a band of 32 rows x (64 + 16) bytes per wave: 16-bit results leave as whole rows
 #include <pto/pto-inst.hpp>
 
 using namespace pto;

@@ -1,0 +1,102 @@
+"""The GEMM written in the PTO tile ISA (pto-isa-mirror_amd/kernels/gemm_performance.hip: double-buffered TLOAD of K
+panels, TEXTRACT, TMATMUL / TMATMUL_ACC, one TSTORE per core) against the oracle, through its extern "C" launcher.
+
+The kernels run on the header layer's fast forms -- LDS-DMA TLOAD, Left / Right windows, register-blocked TMATMUL, staged
+TSTORE -- so these are also the parity tests of those forms at full size.  The bars are the ones the C-ABI launcher of
+the same product is held to (tests/test_gpu_parity.py::test_config2_bf16_4096_cubed).
+"""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import __graft_entry__ as ge
+from oracle import binding as ob
+from test_gpu_parity import DEV, bf16_to_f32, check_f32_drain, host, pa, relerr, sel  # noqa: F401  (pa: the package fixture)
+
+pytestmark = pytest.mark.gpu
+
+LIB = os.path.join(ge.PKG_DIR, "lib", "libpto_gemm_performance.so")
+
+
+@pytest.fixture(scope="module")
+def perf():
+    assert os.path.exists(LIB), "build first: make -C pto-isa-mirror_amd"
+    lib = C.CDLL(LIB)
+
+    def run(case, out, a, b):
+        rc = lib.pto_gemm_performance(case, C.c_void_p(out.data_ptr()), C.c_void_p(a.data_ptr()), C.c_void_p(b.data_ptr()),
+                                      C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, f"launch failed with HIP error {rc}"
+        torch.cuda.synchronize()
+        assert lib.pto_gemm_performance_status() == 0
+        return out
+
+    return run
+
+
+def test_f16_1024x1024x512_whole_matrix(pa, oracle, perf):
+    """Case 2: fp16 inputs uniform in [-1, 1], fp32 result, 16 cores of 256 x 256; every output against the oracle."""
+    m, n, k = 1024, 1024, 512
+    r = np.random.default_rng(77)
+    a = r.uniform(-1, 1, (m, k)).astype(np.float16)
+    b = r.uniform(-1, 1, (n, k)).astype(np.float16)   # [N][K]: the DN view of B
+    out = perf(2, torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV), torch.from_numpy(a).to(DEV),
+               torch.from_numpy(b).to(DEV))
+    ref = oracle.matmul_f16(a.view(np.uint16), b.view(np.uint16), b_dn=True)
+    absdot = np.abs(a.astype(np.float64)) @ np.abs(b.astype(np.float64)).T
+    check_f32_drain(host(out), ref, absdot, k, "PTO-style GEMM f16 1024x1024x512")
+
+
+def test_bf16_4096_cubed(pa, oracle, perf):
+    """Cases 0 and 1: configs[1] (bf16 4096^3, A row-major, B column-major, N(0,1) * 0.02) written in the tile ISA.  The
+    fp32 drain is held to both error bars on 4096 sampled outputs and two whole 256 x 256 tiles; the bf16 drain must be
+    the rounding of the fp32 drain bit for bit, everywhere; every output element must have been written."""
+    m = n = k = 4096
+    gen = torch.Generator(device=DEV).manual_seed(2)
+    a = (torch.randn((m, k), generator=gen, device=DEV) * 0.02).to(torch.bfloat16)
+    b = (torch.randn((n, k), generator=gen, device=DEV) * 0.02).to(torch.bfloat16)
+    f = perf(1, torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV), a, b)
+    out = perf(0, torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV), a, b)
+    f_h, out_h = host(f), host(out)
+    assert not np.isnan(f_h).any()
+    assert np.array_equal(out_h, oracle.store_f32(f_h, ob.ST_BF16))
+    rows = np.unique(np.concatenate([[0, 1, 255, 256, 2047, 2048, 4095], np.arange(5, 4096, 72)]))[:64]
+    cols = np.arange(0, 4096, 64) + np.arange(64) % 64
+    blocks = [("samples", rows, cols), ("tile (0, 0)", np.arange(256), np.arange(256)),
+              ("tile (15, 15)", np.arange(3840, 4096), np.arange(3840, 4096)),
+              ("tile (7, 3)", np.arange(1792, 2048), np.arange(768, 1024))]
+    for label, rr, cc in blocks:
+        ar, bc = host(sel(a, rr)), host(sel(b, cc))
+        ref = oracle.matmul_bf16(ar, bc, b_dn=True)
+        absdot = np.abs(bf16_to_f32(ar).astype(np.float64)) @ np.abs(bf16_to_f32(bc).astype(np.float64)).T
+        check_f32_drain(f_h[np.ix_(rr, cc)], ref, absdot, k, f"PTO-style GEMM bf16 4096^3, {label}")
+        assert relerr(bf16_to_f32(out_h[np.ix_(rr, cc)]), ref) <= 1e-2
+    # the same product through the C-ABI launcher: both run k ascending in 16-wide MFMA steps per output element
+    assert relerr(f_h, host(pa.gemm(a, b, pa.BF16, pa.F32, pa.B_DN))) <= 1e-5
+
+
+TILED_LIB = os.path.join(ge.PKG_DIR, "lib", "libpto_gemm_tiled.so")
+
+
+@pytest.mark.parametrize("case", [0, 1])
+def test_configs0_tiled_gemm_in_the_tile_isa(pa, oracle, case):
+    """configs[0] written in the tile ISA (kernels/gemm_tiled.hip): fp16 512^3 -> fp32, A and B row-major, K slabs of 64,
+    128 x 128 (case 0) or 64 x 64 (case 1) tiles of C per core.  B's slab is transposed by the TMOV into the Right tile.
+    Every output against the oracle's sequential fp32 sum."""
+    lib = C.CDLL(TILED_LIB)
+    r = np.random.default_rng(1234)
+    a = r.uniform(-1, 1, (512, 512)).astype(np.float16)
+    b = r.uniform(-1, 1, (512, 512)).astype(np.float16)   # [K][N]
+    da, db = torch.from_numpy(a).to(DEV), torch.from_numpy(b).to(DEV)
+    out = torch.full((512, 512), float("nan"), dtype=torch.float32, device=DEV)
+    rc = lib.pto_gemm_tiled(case, C.c_void_p(out.data_ptr()), C.c_void_p(da.data_ptr()), C.c_void_p(db.data_ptr()),
+                            C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert lib.pto_gemm_tiled_status() == 0
+    ref = oracle.matmul_f16(a.view(np.uint16), b.view(np.uint16), b_dn=False)
+    absdot = np.abs(a.astype(np.float64)) @ np.abs(b.astype(np.float64))
+    check_f32_drain(host(out), ref, absdot, 512, f"PTO-style tiled GEMM f16 512^3, case {case}")
