@@ -47,7 +47,8 @@ enum {
     PTOAMD_E5M2 = 7, /* float8_e5m2_t                      reference: MXTypes.hpp:345 */
     PTOAMD_E2M1 = 8, /* float4_e2m1x2_t, two per byte, even element in the low nibble   MXTypes.hpp:341,350-372 */
     PTOAMD_E1M2 = 9, /* float4_e1m2x2_t                    MXTypes.hpp:342 */
-    PTOAMD_I16 = 10
+    PTOAMD_I16 = 10,
+    PTOAMD_HIF8 = 11 /* hifloat8_t, one byte per element     reference: include/pto/cpu/Hifloat8.hpp:138-215 */
 };
 
 /* memory layout of the B operand ([K, N] logical) — reference Layout::ND / Layout::DN (common/type.hpp:163-165) */
@@ -116,8 +117,15 @@ int ptoamd_event_elapsed_ms(float* ms, void* start, void* stop);
  *   a       : row-major, leading dimension lda (elements)
  *   b       : b_layout PTOAMD_B_ND ([K][N], ldb >= N) or PTOAMD_B_DN ([N][K], ldb >= K)
  *   c_in    : optional accumulator input (TMATMUL_ACC), same type as the accumulator (f32 / i32), ld = ldc; may be NULL
- *   relu    : TSTORE's ReluPreMode::NormalRelu
+ *   relu    : flags: PTOAMD_RELU (1) = TSTORE's ReluPreMode::NormalRelu; PTOAMD_SATURATE_INF (2), quantising drains only
+ * No alignment is asked of a, b or the leading dimensions beyond that of an element: rows of 16 bytes or more run on the
+ * MFMA tiles whatever their alignment (the LDS-DMA tiles when rows are 16-byte aligned and K is a whole number of
+ * 128-byte slabs, the register-staged tiles otherwise; a row-major B is transposed on its way into LDS by the latter).
+ * PTOAMD_F32 and PTOAMD_HIF8 operands (hif8 x hif8 only, cpu/TMatmul.hpp:38) run on the order-exact kernel: one thread
+ * per output, k ascending, fmaf -- the simulator's arithmetic bit for bit.  No entry point of this group allocates.
  */
+#define PTOAMD_RELU 1
+#define PTOAMD_SATURATE_INF 2 /* bit 48 of the reference's task cookie (cpu/common.hpp:146): see ptoamd_gemm_requant */
 int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, int m, int n, int k,
                 int lda, int ldb, int ldc, int b_layout, int relu, void* stream);
 
@@ -130,6 +138,17 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
 int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                      int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream);
 
+/*
+ * ptoamd_gemm_bias with a caller-owned workspace for a row-major B (PTOAMD_B_ND): B is re-ordered into the workspace once
+ * ([N][K], ptoamd_gemm_workspace_bytes(n, k, ab_type, b_layout) bytes, 256-byte aligned) and the product then runs on the
+ * fastest tiles, where ptoamd_gemm transposes B inside the loader of the register-staged tiles for every tile row of C --
+ * the better choice for small M, the slower one for large M.  workspace == NULL is ptoamd_gemm_bias.  No counterpart in
+ * the reference (its TLOAD re-orders an ND panel into L1 per tile, cpu/TLoad.hpp:287-321).
+ */
+size_t ptoamd_gemm_workspace_bytes(int n, int k, int ab_type, int b_layout);
+int ptoamd_gemm_ws(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias, int m, int n,
+                   int k, int lda, int ldb, int ldc, int b_layout, int relu, void* workspace, size_t workspace_bytes, void* stream);
+
 /* TMATMUL / _ACC / _BIAS on a mixed fp8 pair (cpu/TMatmul.hpp:31-49 admits all four E4M3 / E5M2 pairings of Left and Right):
  * as ptoamd_gemm_bias with separate operand types; bias may be NULL. */
 int ptoamd_gemm_fp8(void* c, int c_type, const void* a, int a_type, const void* b, int b_type, const void* c_in, const void* bias,
@@ -140,6 +159,9 @@ int ptoamd_gemm_fp8(void* c, int c_type, const void* a, int a_type, const void* 
  * word (TSTORE(dst, src, preQuantScalar)) or one word per column (TSTORE_FP with a Scaling tile):
  *   r = acc(i, j) * scale(word);  s8 / u8: clamp(rint(r + offset(word)), byte range chosen by the word's sign bit);
  *   f16: clamp to +-65504 (finite values only for float accumulators);  bf16: the product rounded to bfloat16;
+ *   with PTOAMD_SATURATE_INF in `relu` (the fix-pipe's saturation control, cpu/common.hpp:146,157-171) the f16 and bf16
+ *   targets of a float accumulator turn a NaN product into 0 and clamp an infinite one like a finite one
+ *   (+-65504 / +-FLT_MAX);
  *   s16 (int32 accumulators only, the SHIFTS322S16 mode): (int16)(acc >> (bits 32..35 of the word + 1)), wrapping as
  *   the reference does;  then relu, then the store.
  * Cin and bias are added to the accumulator before the quantisation.

@@ -56,6 +56,8 @@ class Oracle:
         L.pto_encode_e2m1_magic.argtypes = [C.c_float]
         L.pto_shared_exponent.restype = C.c_uint
         L.pto_shared_exponent.argtypes = [C.c_int, C.c_float]
+        L.pto_hif8_to_f64.restype = C.c_double
+        L.pto_hif8_to_f64.argtypes = [C.c_uint]
         L.pto_group_scaling.restype = C.c_float
         L.pto_group_scaling.argtypes = [C.c_int, C.c_float, C.c_uint]
         L.pto_tile_offset.restype = C.c_int64
@@ -175,6 +177,15 @@ class Oracle:
         out = np.empty((m, n), self._ST_DT[dst_kind])
         self.lib.pto_store_f32(_p(out), dst_kind, _p(acc), m, n, n, n, int(relu))
         return out
+
+    def hif8_table(self):
+        """The 256 HiFloat8 values as float64."""
+        return np.array([self.lib.pto_hif8_to_f64(c) for c in range(256)], np.float64)
+
+    def matmul_hif8(self, a, b, b_dn=False):
+        """hif8 x hif8 TMATMUL: every code is an exact float, then the f32 product (sequential fma, k ascending)."""
+        t = self.hif8_table().astype(np.float32)
+        return self.matmul_f32(t[np.asarray(a, np.uint8)], t[np.asarray(b, np.uint8)], b_dn=b_dn)
 
     def store_quant(self, acc, dst_kind, words, per_column, relu=False, saturate_inf=0):
         words = _c(words, np.uint64)
@@ -330,7 +341,20 @@ class RefLib:
         assert rc == 0, rc
         return out
 
-    def store_quant(self, acc, dst, words, per_column, relu=False):
+    def hif8_table(self):
+        out = np.empty(256, np.float64)
+        self.lib.ref_hif8_table(_p(out))
+        return out
+
+    def store_quant(self, acc, dst, words, per_column, relu=False, saturate_inf=0):
+        """saturate_inf sets bit 48 of the simulator's task cookie for the call (cpu/common.hpp:146)."""
+        self.lib.ref_set_task_cookie(C.c_uint64((1 << 48) if saturate_inf else 0))
+        try:
+            return self._store_quant(acc, dst, words, per_column, relu)
+        finally:
+            self.lib.ref_set_task_cookie(C.c_uint64(0))
+
+    def _store_quant(self, acc, dst, words, per_column, relu=False):
         words = _c(words, np.uint64)
         m, n = acc.shape
         key = ("i32" if acc.dtype == np.int32 else "f32") + "_" + dst

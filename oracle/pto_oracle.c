@@ -748,6 +748,38 @@ unsigned pto_shared_exponent(int alg, float maxabs)
     return (e + (round_up ? 1u : 0u)) & 0xFFu;
 }
 
+/* cpu/Hifloat8.hpp:65-135 (decodeHiF8Mathematically): sign, a prefix code giving the number of exponent bits (4, 3, 2, 1
+ * or 0, sign-magnitude with an implicit leading one) and mantissa bits (1, 2, 3, 3, 3); payloads 1..7 are 2^(p - 23);
+ * 0x00 is zero, 0x80 NaN, 0x6F / 0xEF the infinities. */
+double pto_hif8_to_f64(unsigned code)
+{
+    const double sign = (code & 0x80u) ? -1.0 : 1.0;
+    const unsigned p = code & 0x7Fu;
+    if ((p >> 3) == 0) {
+        if ((p & 7u) == 0)
+            return (code & 0x80u) ? (double)NAN : 0.0;
+        return sign * ldexp(1.0, (int)(p & 7u) - 23);
+    }
+    int ebits, rest_bits;
+    unsigned rest;
+    if ((p >> 5) == 3) { ebits = 4; rest = p & 0x1Fu; rest_bits = 5; }
+    else if ((p >> 5) == 2) { ebits = 3; rest = p & 0x1Fu; rest_bits = 5; }
+    else if ((p >> 5) == 1) { ebits = 2; rest = p & 0x1Fu; rest_bits = 5; }
+    else if ((p >> 4) == 1) { ebits = 1; rest = p & 0x0Fu; rest_bits = 4; }
+    else { ebits = 0; rest = p & 0x07u; rest_bits = 3; }
+    const int mbits = rest_bits - ebits;
+    const unsigned raw_e = rest >> mbits, raw_m = rest & ((1u << mbits) - 1u);
+    double e = 0.0;
+    if (ebits > 0) {
+        const unsigned sbit = raw_e & (1u << (ebits - 1));
+        const double mag = (double)((1u << (ebits - 1)) | (raw_e - sbit));
+        e = sbit ? -mag : mag;
+    }
+    if (ebits == 4 && e == 15.0 && raw_m == 1)
+        return sign * (double)INFINITY;
+    return sign * ldexp(1.0 + (double)raw_m / (double)(1u << mbits), (int)e);
+}
+
 /* TQuant.hpp:226-252, 336-347 */
 float pto_group_scaling(int alg, float maxabs, unsigned e8m0)
 {

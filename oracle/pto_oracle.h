@@ -103,6 +103,7 @@ unsigned pto_encode_e4m3fn(float v, int nv);
 unsigned pto_encode_e2m1_magic(float v);
 unsigned pto_shared_exponent(int alg, float maxabs);
 float pto_group_scaling(int alg, float maxabs, unsigned e8m0);
+double pto_hif8_to_f64(unsigned code); /* cpu/Hifloat8.hpp:65-135 */
 /* src is [rows, cols] row-major, already widened to float from src_kind (which only matters for the fp4 bf16
  * re-rounding).  axis 1: groups of 32 along a row; exp/max/scaling are [rows][cols/32].  axis 0: groups of 32
  * along a column; exp/max/scaling are [rows/32][cols].  dst: bytes (fp8) or packed nibbles, row-major (fp4). */

@@ -479,6 +479,17 @@ int ref_store_i32_i16(int16_t* out, const int32_t* acc, int m, int n, const uint
                   RunStoreQuant<int16_t, int32_t, false>(out, acc, m, n, q, per_col);
 }
 
+// the fix-pipe's control bits as the simulator reads them (get_task_cookie, common/cpu_stub.hpp:606-612); bit 48 is the
+// saturate-inf control of quantize_element (cpu/common.hpp:146).  Per calling thread.
+void ref_set_task_cookie(uint64_t cookie) { pto::cpu_sim::set_task_cookie(cookie); }
+
+// static_cast<double>(hifloat8_t::FromRaw(code)) for all 256 codes (cpu/Hifloat8.hpp)
+void ref_hif8_table(double* out256)
+{
+    for (int c = 0; c < 256; ++c)
+        out256[c] = static_cast<double>(hifloat8_t::FromRaw(static_cast<uint8_t>(c)));
+}
+
 // ---- TQUANT / TDEQUANT; shape_id selects one of the compiled static shapes -------------------
 // shape ids: 0 = 4x32, 1 = 2x128, 2 = 2x256, 3 = 16x64, 4 = 8x512, 5 = 64x64, 6 = 32x96
 #define PTO_REF_SHAPES(X) X(0, 4, 32) X(1, 2, 128) X(2, 2, 256) X(3, 16, 64) X(4, 8, 512) X(5, 64, 64) X(6, 32, 96)

@@ -16,7 +16,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libptoamd.so")
 
 # element types (include/ptoamd.h)
-F32, F16, BF16, I32, I8, U8, E4M3, E5M2, E2M1, E1M2, I16 = range(11)
+F32, F16, BF16, I32, I8, U8, E4M3, E5M2, E2M1, E1M2, I16, HIF8 = range(12)
+RELU, SATURATE_INF = 1, 2  # flags of the `relu` argument
 B_ND, B_DN = 0, 1
 MX_A_ZZ, MX_A_ND, MX_A_DN, MX_B_NN, MX_B_ND, MX_B_DN = range(6)
 OCP_MXFP8, NV_MXFP8, OCP_MXFP4, NV_MXFP4 = range(4)
@@ -34,13 +35,14 @@ _lib = C.CDLL(LIB_PATH)
 _lib.ptoamd_last_error.restype = C.c_char_p
 _lib.ptoamd_last_kernel.restype = C.c_char_p
 _lib.ptoamd_gemm_mx_workspace_bytes.restype = C.c_size_t
+_lib.ptoamd_gemm_workspace_bytes.restype = C.c_size_t
 
 EXPORTS = [
     "ptoamd_init", "ptoamd_finalize", "ptoamd_last_error", "ptoamd_device_info", "ptoamd_malloc", "ptoamd_free",
     "ptoamd_malloc_host", "ptoamd_free_host", "ptoamd_memcpy", "ptoamd_memcpy_async", "ptoamd_memset",
     "ptoamd_stream_create", "ptoamd_stream_destroy", "ptoamd_stream_synchronize", "ptoamd_event_create",
     "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
-    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_fp8", "ptoamd_gemm_requant", "ptoamd_gemm_atomic_add", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
+    "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_ws", "ptoamd_gemm_workspace_bytes", "ptoamd_gemm_fp8", "ptoamd_gemm_requant", "ptoamd_gemm_atomic_add", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
     "ptoamd_gemm_mx_ws",
     "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
     "ptoamd_tquant_int8_para", "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_tdequant_para", "ptoamd_mx_scale_relayout",
@@ -91,15 +93,25 @@ def _stream(stream):
 _TORCH_OUT = {F32: torch.float32, F16: torch.float16, BF16: torch.bfloat16, I32: torch.int32}
 
 
+def gemm_workspace_bytes(n, k, ab_type, b_layout):
+    return int(_lib.ptoamd_gemm_workspace_bytes(n, k, ab_type, b_layout))
+
+
 def gemm(a, b, ab_type, c_type=F32, b_layout=B_DN, c_in=None, relu=False, m=None, n=None, k=None, stream=None, out=None,
-         bias=None):
+         bias=None, workspace=None):
     """TLOAD -> TMATMUL / TMATMUL_ACC / TMATMUL_BIAS -> TSTORE.  a: [m, k]; b: [n, k] (B_DN) or [k, n] (B_ND), raw-typed
-    tensors; bias: [n] of the accumulator type."""
+    tensors; bias: [n] of the accumulator type; workspace: a uint8 device tensor of gemm_workspace_bytes(...) bytes into
+    which a row-major b is re-ordered (without one it is transposed inside the loader)."""
     m = a.shape[0] if m is None else m
     k = a.shape[1] if k is None else k
     n = (b.shape[0] if b_layout == B_DN else b.shape[1]) if n is None else n
     if out is None:
         out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
+    if workspace is not None:
+        _check(_lib.ptoamd_gemm_ws(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _ptr(c_in), _ptr(bias), m, n, k,
+                                   a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu), _ptr(workspace),
+                                   C.c_size_t(workspace.numel() * workspace.element_size()), _stream(stream)), "ptoamd_gemm_ws")
+        return out
     if bias is not None:
         _check(_lib.ptoamd_gemm_bias(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _ptr(c_in), _ptr(bias), m, n, k,
                                      a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu), _stream(stream)),

@@ -22,7 +22,7 @@ struct Options {
     bool no_tail_split = false;  // PTOAMD_NO_TAIL_SPLIT=1: never split a half-full last round off as smaller tiles
     int tail_tile = 5;           // PTOAMD_TAIL_TILE=5|6: the tail runs as 128x128 or 256x128 tiles
     bool force_generic = false;  // PTOAMD_FORCE_GENERIC=1: everything runs on the order-exact generic kernels
-    bool b_nd_transpose = false; // PTOAMD_B_ND_TRANSPOSE=1: a row-major B is re-ordered in global memory, never in the loader
+    bool b_nd_in_loader = false; // PTOAMD_B_ND_IN_LOADER=1: a row-major B is transposed by the loader even when a workspace is given
     bool gemv_sw_cvt = false;    // PTOAMD_GEMV_SW_CVT=1: decode fp4 weights with integer arithmetic
     bool gemv_no_splitk = false; // PTOAMD_GEMV_NO_SPLITK=1 / PTOAMD_GEMV_NO_WIDE=1: skip those GEMV kernels
     bool gemv_no_wide = false;

@@ -105,7 +105,7 @@ struct GenericParams {
     int m, n, k;
     long lda, sbk, sbn;  // element strides: A row pitch; B(k, j) = b[k * sbk + j * sbn]
     int ldc;
-    int a_type, b_type, out_kind, relu;
+    int a_type, b_type, out_kind, relu;  // relu: bit 0 relu, bit 1 saturate-inf (as TileGemmParams)
     int sa_layout, sb_layout, mx;
     const uint64_t* qwords;  // OUT_Q8 / OUT_QF16: fix-pipe quantisation words
     int q_per_column;
@@ -122,6 +122,7 @@ __device__ __forceinline__ float load_elem_f32(const void* p, long idx, int type
         case PTOAMD_E5M2: return e5m2_to_f32(reinterpret_cast<const uint8_t*>(p)[idx]);
         case PTOAMD_E2M1: return e2m1_to_f32((reinterpret_cast<const uint8_t*>(p)[idx >> 1] >> ((idx & 1) * 4)) & 0xFu);
         case PTOAMD_E1M2: return e1m2_to_f32((reinterpret_cast<const uint8_t*>(p)[idx >> 1] >> ((idx & 1) * 4)) & 0xFu);
+        case PTOAMD_HIF8: return hif8_to_f32(reinterpret_cast<const uint8_t*>(p)[idx]);
         default: return (float)reinterpret_cast<const int8_t*>(p)[idx];
     }
 }
@@ -131,9 +132,12 @@ template <bool SRC_INT>
 __device__ __forceinline__ void store_quant(const GenericParams& p, long o, float acc, int gj)
 {
     const uint64_t w = p.qwords[p.q_per_column ? gj : 0];
+    const bool sat_inf = !SRC_INT && (p.relu & 2) != 0;
     if (p.out_kind == OUT_QBF16) {
         float r = __fmul_rn(acc, p.q_per_column ? fixpipe_word_scale<true>(w) : fixpipe_word_scale<false>(w));
-        if (p.relu)
+        if (sat_inf)
+            r = fixpipe_saturate_inf<false>(r);
+        if (p.relu & 1)
             r = r > 0 ? r : 0;
         reinterpret_cast<uint16_t*>(p.c)[o] = f32_to_bf16_bits(r);
         return;
@@ -144,7 +148,9 @@ __device__ __forceinline__ void store_quant(const GenericParams& p, long o, floa
         r = p.q_per_column ? fixpipe_quantize<true, true, SRC_INT>(acc, w) : fixpipe_quantize<false, true, SRC_INT>(acc, w);
     else
         r = p.q_per_column ? fixpipe_quantize<true, false, SRC_INT>(acc, w) : fixpipe_quantize<false, false, SRC_INT>(acc, w);
-    if (p.relu)
+    if (!byte && sat_inf)
+        r = fixpipe_saturate_inf<true>(r);
+    if (p.relu & 1)
         r = r > 0 ? r : 0;
     if (byte)
         reinterpret_cast<uint8_t*>(p.c)[o] = (uint8_t)(int32_t)r;
@@ -158,7 +164,7 @@ __device__ __forceinline__ void store_out(const GenericParams& p, long o, float 
         store_quant<false>(p, o, v, gj);
         return;
     }
-    if (p.relu)
+    if (p.relu & 1)
         v = v > 0 ? v : 0;
     switch (p.out_kind) {
         case OUT_F32:
@@ -192,7 +198,7 @@ __global__ void gemm_generic_kernel(const GenericParams p)
         int32_t v = (int32_t)acc;
         if (p.out_kind == OUT_QS16) {
             int32_t r = fixpipe_shift_s16(v, p.qwords[p.q_per_column ? gj : 0]);
-            if (p.relu)
+            if (p.relu & 1)
                 r = r > 0 ? r : 0;
             reinterpret_cast<int16_t*>(p.c)[o] = (int16_t)r;
             return;
@@ -201,7 +207,7 @@ __global__ void gemm_generic_kernel(const GenericParams p)
             store_quant<true>(p, o, (float)v, gj);
             return;
         }
-        if (p.relu)
+        if (p.relu & 1)
             v = v > 0 ? v : 0;
         if (p.out_kind == OUT_I32) {
             if (p.atomic_add)
@@ -273,9 +279,11 @@ static bool dma_offsets_fit(int m, int n, long lda_bytes, long ldb_bytes, long k
     return last <= (long)UINT32_MAX;
 }
 
-static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, bool scale_dma_ok = true)
+// dma_ok: what the DMA tiles need besides whole slabs -- 16-byte aligned operand rows, 32-bit lane offsets, and for the
+// block-scaled types scale rows they can stream.
+static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, bool dma_ok = true)
 {
-    const bool dtl_ok = (k_bytes % 128) == 0 && scale_dma_ok;
+    const bool dtl_ok = (k_bytes % 128) == 0 && dma_ok;
     if (options().tile >= 0) {
         int t = options().tile;
         if (t == 3)  // the four-wave form of the 256 x 256 DMA tile is no longer built
@@ -357,19 +365,6 @@ static const char* tile_kernel_name(int tile, int op)
     return buf;
 }
 
-// Temporary device buffers (transposed B, re-laid scales) are stream-ordered allocations released after the launch.
-struct StreamTemp {
-    void* ptr = nullptr;
-    hipStream_t stream;
-    explicit StreamTemp(hipStream_t s) : stream(s) {}
-    hipError_t alloc(size_t bytes) { return hipMallocAsync(&ptr, bytes, stream); }
-    ~StreamTemp()
-    {
-        if (ptr)
-            (void)hipFreeAsync(ptr, stream);
-    }
-};
-
 template <typename T>
 static int transpose_b(void* dst, const void* src, int k, int n, long ldb, hipStream_t stream)
 {
@@ -449,12 +444,28 @@ int ptoamd_gemm(void* c, int c_type, const void* a, const void* b, int ab_type, 
 
 static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                        const uint64_t* qwords, int q_per_column, int m, int n, int k, int lda, int ldb, int ldc, int b_layout,
-                       int relu, void* stream_, int atomic_add = 0, int b_type = -1);
+                       int relu, void* stream_, int atomic_add = 0, int b_type = -1, void* ws = nullptr, size_t ws_bytes = 0);
 
 int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                      int m, int n, int k, int lda, int ldb, int ldc, int b_layout, int relu, void* stream_)
 {
     return gemm_common(c, c_type, a, b, ab_type, c_in, bias, nullptr, 0, m, n, k, lda, ldb, ldc, b_layout, relu, stream_);
+}
+
+size_t ptoamd_gemm_workspace_bytes(int n, int k, int ab_type, int b_layout)
+{
+    if (n <= 0 || k <= 0 || b_layout != PTOAMD_B_ND)
+        return 0;
+    return (size_t)n * (size_t)k * (size_t)(elem_bits(ab_type) / 8);
+}
+
+int ptoamd_gemm_ws(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias, int m, int n,
+                   int k, int lda, int ldb, int ldc, int b_layout, int relu, void* workspace, size_t workspace_bytes, void* stream_)
+{
+    PTOAMD_REQUIRE(workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, PTOAMD_E_ALIGNMENT,
+                   "ptoamd_gemm_ws: the workspace must be 256-byte aligned");
+    return gemm_common(c, c_type, a, b, ab_type, c_in, bias, nullptr, 0, m, n, k, lda, ldb, ldc, b_layout, relu, stream_, 0, -1,
+                       workspace, workspace ? workspace_bytes : 0);
 }
 
 int ptoamd_gemm_fp8(void* c, int c_type, const void* a, int a_type, const void* b, int b_type, const void* c_in, const void* bias,
@@ -488,7 +499,7 @@ int ptoamd_gemm_atomic_add(void* c, int c_type, const void* a, const void* b, in
 
 static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias,
                        const uint64_t* qwords, int q_per_column, int m, int n, int k, int lda, int ldb, int ldc, int b_layout,
-                       int relu, void* stream_, int atomic_add, int b_type)
+                       int relu, void* stream_, int atomic_add, int b_type, void* ws, size_t ws_bytes)
 {
     // b_type: -1 = as ab_type; otherwise the second type of a mixed fp8 pair (ab_type is then A's)
     if (b_type < 0)
@@ -505,11 +516,14 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
     PTOAMD_REQUIRE(b_layout == PTOAMD_B_ND || b_layout == PTOAMD_B_DN, PTOAMD_E_INVALID, "ptoamd_gemm: unknown b_layout");
     PTOAMD_REQUIRE(lda >= k && ldc >= n && ldb >= (b_layout == PTOAMD_B_DN ? k : n), PTOAMD_E_INVALID,
                    "ptoamd_gemm: leading dimension smaller than the row length");
+    PTOAMD_REQUIRE((relu & ~(PTOAMD_RELU | PTOAMD_SATURATE_INF)) == 0, PTOAMD_E_INVALID, "ptoamd_gemm: unknown bits in the relu / flags argument");
     const bool is_int = ab_type == PTOAMD_I8;
     const bool is_float = ab_type == PTOAMD_F16 || ab_type == PTOAMD_BF16 || ab_type == PTOAMD_F32 ||
-                          ab_type == PTOAMD_E4M3 || ab_type == PTOAMD_E5M2;
+                          ab_type == PTOAMD_E4M3 || ab_type == PTOAMD_E5M2 || ab_type == PTOAMD_HIF8;
     PTOAMD_REQUIRE(is_int || is_float, PTOAMD_E_UNSUPPORTED,
-                   "ptoamd_gemm: operand type %d is not a TMATMUL input type (s8, f16, bf16, f32, e4m3, e5m2)", ab_type);
+                   "ptoamd_gemm: operand type %d is not a TMATMUL input type (s8, f16, bf16, f32, e4m3, e5m2, hif8)", ab_type);
+    PTOAMD_REQUIRE((ab_type == PTOAMD_HIF8) == (b_type == PTOAMD_HIF8), PTOAMD_E_UNSUPPORTED,
+                   "ptoamd_gemm: hif8 pairs with hif8 only");
     int out_kind;
     if (qwords != nullptr) {
         PTOAMD_REQUIRE(c_type != PTOAMD_I16 || is_int, PTOAMD_E_UNSUPPORTED,
@@ -525,9 +539,20 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
     }
     const int ebytes = elem_bits(ab_type) / 8;
     const long k_bytes = (long)k * ebytes, lda_b = (long)lda * ebytes, ldb_b = (long)ldb * ebytes;
-    const bool tile_ok = !force_generic() && ab_type != PTOAMD_F32 && aligned16(a) && aligned16(b) && (lda_b % 16) == 0 &&
-                         (k_bytes % 16) == 0 &&
-                         (b_layout == PTOAMD_B_DN ? (ldb_b % 16) == 0 : true);
+    const uintptr_t emask = (uintptr_t)ebytes - 1;
+    // The register-staged MFMA tiles take rows at any alignment and of any length from 16 bytes up (the row's last chunk
+    // is masked), so only f32 / hif8 operands, rows shorter than 16 bytes and misaligned elements go to the order-exact
+    // kernel.  B row-major: with a workspace it is re-ordered there once and the fastest tiles run; without one the
+    // register-staged tiles transpose it on its way into LDS.  Nothing is allocated either way.
+    const bool mfma_type = ab_type != PTOAMD_F32 && ab_type != PTOAMD_HIF8;
+    const bool elems_ok = (reinterpret_cast<uintptr_t>(a) & emask) == 0 && (reinterpret_cast<uintptr_t>(b) & emask) == 0;
+    const size_t ws_need = b_layout == PTOAMD_B_ND ? (size_t)n * (size_t)k_bytes : 0;
+    const bool b_via_ws = b_layout == PTOAMD_B_ND && ws != nullptr && (ebytes == 1 || ebytes == 2) && !options().b_nd_in_loader;
+    PTOAMD_REQUIRE(!b_via_ws || ws_need <= ws_bytes, PTOAMD_E_INVALID,
+                   "ptoamd_gemm_ws: re-ordering B needs %zu bytes of workspace, %zu available", ws_need, ws_bytes);
+    const bool b_in_kernel = b_layout == PTOAMD_B_ND && !b_via_ws && (ebytes == 1 || ebytes == 2) && (long)n * ebytes >= 16;
+    const bool tile_ok = !force_generic() && mfma_type && elems_ok && k_bytes >= 16 &&
+                         (b_layout == PTOAMD_B_DN || b_via_ws || b_in_kernel);
     if (!tile_ok) {
         GenericParams g{};
         g.a = a; g.b = b; g.c = c; g.c_in = c_in; g.bias = bias;
@@ -538,21 +563,13 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
         g.qwords = qwords; g.q_per_column = q_per_column; g.atomic_add = atomic_add;
         return launch_generic(g, stream);
     }
-    StreamTemp bt(stream);
     const uint8_t* b_kmajor = reinterpret_cast<const uint8_t*>(b);
     long ldb_kmajor = ldb_b;
-    // A row-major B with few output row-tiles is transposed on its way into LDS by the register-staged tiles (no
-    // temporary, one launch).  With many row-tiles every element of B would be scattered into LDS that many times, and
-    // the DMA tiles cannot do it at all: then B is re-ordered once in global memory and read K-contiguous from there.
-    const bool b_in_kernel = b_layout == PTOAMD_B_ND && m <= 1024 && (ebytes == 1 || ebytes == 2) && (n % (16 / ebytes)) == 0 &&
-                             (ldb_b % 16) == 0 && !options().b_nd_transpose;
-    if (b_layout == PTOAMD_B_ND && !b_in_kernel) {  // TLOAD of an ND B panel: re-order once so the MFMA path reads K-contiguous rows
-        PTOAMD_HIP_CHECK(bt.alloc((size_t)n * k_bytes));
-        const int rc = ebytes == 2 ? transpose_b<uint16_t>(bt.ptr, b, k, n, ldb, stream)
-                                   : transpose_b<uint8_t>(bt.ptr, b, k, n, ldb, stream);
+    if (b_via_ws) {  // TLOAD of an ND B panel: re-order once so the MFMA path reads K-contiguous rows
+        const int rc = ebytes == 2 ? transpose_b<uint16_t>(ws, b, k, n, ldb, stream) : transpose_b<uint8_t>(ws, b, k, n, ldb, stream);
         if (rc != PTOAMD_OK)
             return rc;
-        b_kmajor = reinterpret_cast<const uint8_t*>(bt.ptr);
+        b_kmajor = reinterpret_cast<const uint8_t*>(ws);
         ldb_kmajor = k_bytes;
     }
     TileGemmParams p{};
@@ -569,7 +586,9 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
                    : ab_type == PTOAMD_E4M3 ? (b_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E4E5)
                                             : (b_type == PTOAMD_E5M2 ? TOP_FP8_E5E5 : TOP_FP8_E5E4);
     p.b_nd = b_in_kernel; p.b_esz = ebytes;
-    const int tile = pick_tile(m, n, k_bytes, false, false, !b_in_kernel && dma_offsets_fit(m, n, lda_b, ldb_kmajor, k_bytes));
+    const bool dma_ok = !b_in_kernel && aligned16(a) && aligned16(b_kmajor) && (lda_b % 16) == 0 && (ldb_kmajor % 16) == 0 &&
+                        dma_offsets_fit(m, n, lda_b, ldb_kmajor, k_bytes);
+    const int tile = pick_tile(m, n, k_bytes, false, false, dma_ok);
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;
@@ -587,8 +606,9 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
     PTOAMD_REQUIRE(b_layout == PTOAMD_B_ND || b_layout == PTOAMD_B_DN, PTOAMD_E_INVALID, "ptoamd_gemm_w8a8: unknown b_layout");
     PTOAMD_REQUIRE(lda >= k && ldc >= n && ldb >= (b_layout == PTOAMD_B_DN ? k : n), PTOAMD_E_INVALID,
                    "ptoamd_gemm_w8a8: leading dimension smaller than the row length");
-    const bool tile_ok = !force_generic() && aligned16(a) && aligned16(b) && (lda % 16) == 0 && (k % 16) == 0 &&
-                         (b_layout == PTOAMD_B_DN ? (ldb % 16) == 0 : true);
+    // (rows at any alignment, any K from 16 up: see ptoamd_gemm; a row-major B is transposed by the register-staged loader)
+    const bool b_in_kernel = b_layout == PTOAMD_B_ND && n >= 16;
+    const bool tile_ok = !force_generic() && k >= 16 && (b_layout == PTOAMD_B_DN || b_in_kernel);
     if (!tile_ok) {
         GenericParams g{};
         g.a = a; g.b = b; g.c = out_bf16; g.acc_out = acc_out; g.row_scale = scale_a; g.col_scale = scale_b;
@@ -598,27 +618,15 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
         g.a_type = g.b_type = PTOAMD_I8; g.out_kind = OUT_W8A8_BF16;
         return launch_generic(g, stream);
     }
-    StreamTemp bt(stream);
-    const uint8_t* b_kmajor = reinterpret_cast<const uint8_t*>(b);
-    long ldb_kmajor = ldb;
-    const bool b_in_kernel = b_layout == PTOAMD_B_ND && m <= 1024 && (n % 16) == 0 && (ldb % 16) == 0 &&
-                             !options().b_nd_transpose;  // (same rule as ptoamd_gemm)
-    if (b_layout == PTOAMD_B_ND && !b_in_kernel) {
-        PTOAMD_HIP_CHECK(bt.alloc((size_t)n * k));
-        const int rc = transpose_b<uint8_t>(bt.ptr, b, k, n, ldb, stream);
-        if (rc != PTOAMD_OK)
-            return rc;
-        b_kmajor = reinterpret_cast<const uint8_t*>(bt.ptr);
-        ldb_kmajor = k;
-    }
     TileGemmParams p{};
     p.a = reinterpret_cast<const uint8_t*>(a);
-    p.b = b_kmajor;
+    p.b = reinterpret_cast<const uint8_t*>(b);
     p.c = out_bf16; p.acc_out = acc_out; p.row_scale = scale_a; p.col_scale = scale_b;
-    p.m = m; p.n = n; p.k_bytes = k; p.lda_bytes = lda; p.ldb_bytes = ldb_kmajor; p.ldc = ldc;
+    p.m = m; p.n = n; p.k_bytes = k; p.lda_bytes = lda; p.ldb_bytes = ldb; p.ldc = ldc;
     p.out_kind = OUT_W8A8_BF16; p.group_m = 4;
     p.b_nd = b_in_kernel; p.b_esz = 1;
-    const int tile = pick_tile(m, n, k, false, false, !b_in_kernel && dma_offsets_fit(m, n, lda, ldb_kmajor, k));
+    const bool dma_ok = !b_in_kernel && aligned16(a) && aligned16(b) && (lda % 16) == 0 && (ldb % 16) == 0 && dma_offsets_fit(m, n, lda, ldb, k);
+    const int tile = pick_tile(m, n, k, false, false, dma_ok);
     PTOAMD_HIP_CHECK(launch_tiles(tile, TOP_I8, p, stream));
     set_last_kernel(tile_kernel_name(tile, TOP_I8));
     return PTOAMD_OK;

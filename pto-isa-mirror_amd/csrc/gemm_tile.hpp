@@ -33,7 +33,7 @@ struct TileGemmParams {
     long lda_bytes, ldb_bytes;
     int ldc;
     int scale_ld;           // MX: bytes per scale row (k / 32)
-    int relu;
+    int relu;               // bit 0: relu; bit 1: the fix-pipe's saturate-inf control (half / bfloat16 quantising drains)
     int out_kind;           // OutKind
     int group_m;            // tile-order grouping for L2 reuse
     int b_nd;               // register-staged tiles only: b is [k][ldb_bytes] (rows of N), transposed on the way into LDS
@@ -324,7 +324,7 @@ __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int 
     const Elem* cin = reinterpret_cast<const Elem*>(p.c_in);
     // one branch per block when no term applies (the common case): a 16x16 block has four registers, and three
     // separate tests per block cost more than the block's conversions
-    if (cin == nullptr && p.bias == nullptr && !(RELU && p.relu))
+    if (cin == nullptr && p.bias == nullptr && !(RELU && (p.relu & 1)))
         return v;
     if (cin != nullptr) {
 #pragma unroll
@@ -344,7 +344,7 @@ __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int 
                 v[r] += reinterpret_cast<const Elem*>(p.bias)[gj];
         }
     }
-    if (RELU && p.relu) {
+    if (RELU && (p.relu & 1)) {
 #pragma unroll
         for (int r = 0; r < Cfg::Op::ACC_REGS; ++r)
             v[r] = v[r] > 0 ? v[r] : 0;
@@ -355,9 +355,10 @@ __device__ __forceinline__ Acc tstore_terms(const TileGemmParams& p, Acc v, int 
 // bits of one output element (1- and 2-byte kinds in the low part); W8A8: ((float)acc * scale_a[i]) * scale_b[j] -> bf16,
 // each step rounded to f32; the quantising kinds: fix-pipe word `qw`, then relu
 template <int KIND, class V>
-__device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_t qw = 0, bool q_vector = false, bool relu = false,
+__device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_t qw = 0, bool q_vector = false, int relu_flags = 0,
                                                 int q16_kind = OUT_QF16)
 {
+    const bool relu = (relu_flags & 1) != 0, sat_inf = (relu_flags & 2) != 0;
     if (KIND == OUT_F32)
         return __builtin_bit_cast(uint32_t, (float)v);
     if (KIND == OUT_I32)
@@ -383,11 +384,15 @@ __device__ __forceinline__ uint32_t tstore_bits(V v, float rs, float cs, uint64_
         }
         if (q16_kind == OUT_QBF16) {
             float r = __fmul_rn((float)v, q_vector ? fixpipe_word_scale<true>(qw) : fixpipe_word_scale<false>(qw));
+            if (!src_int && sat_inf)
+                r = fixpipe_saturate_inf<false>(r);
             if (relu)
                 r = r > 0 ? r : 0;
             return f32_to_bf16_bits(r);
         }
         float r = q_vector ? fixpipe_quantize<true, false, src_int>((float)v, qw) : fixpipe_quantize<false, false, src_int>((float)v, qw);
+        if (!src_int && sat_inf)
+            r = fixpipe_saturate_inf<true>(r);
         if (relu)
             r = r > 0 ? r : 0;
         return (uint32_t)f32_to_f16_bits(r);
@@ -434,7 +439,7 @@ __device__ __forceinline__ void tstore_block(const TileGemmParams& p, const Acc&
             const long o = (long)gi * p.ldc + gj;
             const float cs = KIND == OUT_W8A8_BF16 ? p.col_scale[gj] : 1.0f;
             const uint64_t qw = out_quant<KIND> ? p.qwords[p.q_per_column ? gj : 0] : 0;
-            const uint32_t bits = tstore_bits<KIND>(v[r], rs, cs, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
+            const uint32_t bits = tstore_bits<KIND>(v[r], rs, cs, qw, p.q_per_column != 0, p.relu, p.out_kind);
             if (KIND == OUT_F32 && p.atomic_add)
                 atomicAdd(reinterpret_cast<float*>(p.c) + o, __builtin_bit_cast(float, bits));
             else if (KIND == OUT_I32 && p.atomic_add)
@@ -585,11 +590,11 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             if (Q8 && (PRE_QW || !p.q_per_column)) {
-                                bits[e] = byte_quant_bits((float)v[4 * g + e], p.q_per_column ? bq_pre[j][4 * g + e] : bq0, p.relu != 0);
+                                bits[e] = byte_quant_bits((float)v[4 * g + e], p.q_per_column ? bq_pre[j][4 * g + e] : bq0, (p.relu & 1) != 0);
                                 continue;
                             }
                             const uint64_t qw = !out_quant<KIND> ? 0 : !p.q_per_column ? qw0 : (PRE_QW && !Q8) ? qw_pre[j][4 * g + e] : p.qwords[col_b + qc + e];
-                            bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu != 0, p.out_kind);
+                            bits[e] = tstore_bits<KIND>(v[4 * g + e], rs, 1.0f, qw, p.q_per_column != 0, p.relu, p.out_kind);
                         }
                         if (ESZ == 4)
                             *reinterpret_cast<uint4*>(dst) = make_uint4(bits[0], bits[1], bits[2], bits[3]);
@@ -655,6 +660,35 @@ __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::
     });
 }
 
+// 16 bytes of a row starting at `g`, of which only the first `rem` belong to the row (rem >= 16: a whole chunk, at any
+// alignment; rem <= 0: nothing, zeros).  A partial chunk is read as the 16 bytes ending at the row's end -- the row is at
+// least 16 bytes long -- and shifted down by the bytes that precede the chunk.
+__device__ __forceinline__ uint4 load_unaligned16(const uint8_t* g)
+{
+    uint32_t w[4];
+    __builtin_memcpy(w, g, 16);  // one global_load_dwordx4: the target takes vector memory accesses at any alignment
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+__device__ __forceinline__ uint4 load_chunk_tail(const uint8_t* g, int rem)
+{
+    if (rem >= 16)
+        return load_unaligned16(g);
+    if (rem <= 0)
+        return make_uint4(0, 0, 0, 0);
+    const uint4 w = load_unaligned16(g + rem - 16);
+    const uint64_t lo = ((uint64_t)w.y << 32) | w.x, hi = ((uint64_t)w.w << 32) | w.z;
+    const int sh = (16 - rem) * 8;  // 8 .. 120 bits
+    uint64_t rlo, rhi;
+    if (sh >= 64) {
+        rlo = hi >> (sh - 64);
+        rhi = 0;
+    } else {
+        rlo = (lo >> sh) | (hi << (64 - sh));
+        rhi = hi >> sh;
+    }
+    return make_uint4((uint32_t)rlo, (uint32_t)(rlo >> 32), (uint32_t)rhi, (uint32_t)(rhi >> 32));
+}
+
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmParams p)
 {
@@ -715,7 +749,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
             const int c = tid + i * NT;
             const int k_lo = c % epc, nc = (c / epc) % (BN / epc), k_hi = c / BN;
             const int krow = k_hi * epc + k_lo;
-            const bool inside = n0 + nc * epc < p.n;  // (N is a multiple of EPC: a chunk is inside or outside as a whole)
+            const int cols_left = p.n - (n0 + nc * epc);  // columns of B from this chunk's first one on
+            const bool inside = cols_left > 0;
             gb[i] = p.b + (long)krow * p.ldb_bytes + (long)(inside ? n0 + nc * epc : 0) * p.b_esz;
             sb_off[i] = Cfg::A_BYTES + nc * epc * 128 + k_lo * p.b_esz;
             b_koff[i] = inside ? krow * p.b_esz : (1 << 30);
@@ -726,23 +761,56 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
     const int k_slabs = (p.k_bytes + 127) / 128;
 
     uint4 ra[LA], rb[LB];
-    auto tload = [&](int kt) {
+    // Rows need no alignment: a chunk is read with a 16-byte load at whatever address it starts (the part supports
+    // unaligned global accesses).  Two forms of the slab load, chosen per slab by a workgroup-uniform test, so that the
+    // common one stays as lean as it was:
+    //   whole   every chunk of the slab lies inside its row, or outside it as a whole (rows of whole 16-byte chunks);
+    //   ragged  the row's last chunk holds fewer than 16 of the row's bytes (K * esz % 16 != 0; B row-major: N * esz % 16
+    //           != 0): that chunk is read as the 16 bytes that END at the row's end and shifted down, so nothing past the
+    //           row is touched (the bytes after a matrix's last row may not be mapped) and the lanes beyond K are zero.
+    const bool ragged_k = (p.k_bytes & 15) != 0;
+    const bool ragged_n = p.b_nd && (((long)p.n * p.b_esz) & 15) != 0;
+    auto tload_whole = [&](int kt) {
         const bool live = kt * 128 + ld_chunk * 16 < p.k_bytes;  // partial last slab: missing chunks are zero
 #pragma unroll
         for (int i = 0; i < LA; ++i) {
             if (expands_fp4<Op> && a_exp)
                 ra[i] = live ? expand_fp4_to_e4m3(*reinterpret_cast<const uint2*>(ga[i] + (long)kt * 64), a_exp) : make_uint4(0, 0, 0, 0);
             else
-                ra[i] = live ? *reinterpret_cast<const uint4*>(ga[i] + (long)kt * 128) : make_uint4(0, 0, 0, 0);
+                ra[i] = live ? load_unaligned16(ga[i] + (long)kt * 128) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < LB; ++i) {
             if (expands_fp4<Op> && b_exp)  // (B is [N][K] here: the host sends row-major packed B elsewhere)
                 rb[i] = live ? expand_fp4_to_e4m3(*reinterpret_cast<const uint2*>(gb[i] + (long)kt * 64), b_exp) : make_uint4(0, 0, 0, 0);
             else
-                rb[i] = kt * 128 + b_koff[i] < p.k_bytes ? *reinterpret_cast<const uint4*>(gb[i] + kt * b_slab_stride)
-                                                         : make_uint4(0, 0, 0, 0);
+                rb[i] = kt * 128 + b_koff[i] < p.k_bytes ? load_unaligned16(gb[i] + kt * b_slab_stride) : make_uint4(0, 0, 0, 0);
         }
+    };
+    auto tload_ragged = [&](int kt) {
+        const int rem = p.k_bytes - (kt * 128 + ld_chunk * 16);  // bytes of the row from this chunk on; <= 0: none
+#pragma unroll
+        for (int i = 0; i < LA; ++i)
+            ra[i] = load_chunk_tail(ga[i] + (long)kt * 128, rem);
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            if (!p.b_nd) {
+                rb[i] = load_chunk_tail(gb[i] + (long)kt * 128, rem);
+            } else {  // a chunk of B's row k runs along N and ends with the row's columns
+                const int epc = 16 / p.b_esz;
+                const int nc = ((tid + i * NT) / epc) % (BN / epc);
+                const int cols_left = p.n - (n0 + nc * epc);
+                rb[i] = kt * 128 + b_koff[i] < p.k_bytes ? load_chunk_tail(gb[i] + kt * b_slab_stride, min(cols_left, epc) * p.b_esz)
+                                                         : make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+    // (the fp4-expanding loads read 8-byte half chunks of rows that are whole slabs: never ragged)
+    auto tload = [&](int kt) {
+        if (ragged_n || (ragged_k && (kt + 1) * 128 > p.k_bytes))
+            tload_ragged(kt);
+        else
+            tload_whole(kt);
     };
     auto stage = [&](int buf) {
         uint8_t* base = smem + buf * Cfg::STAGE_BYTES;

@@ -1,5 +1,6 @@
 // Host runtime of the gfx950 backend: the counterpart of the fake aclrt* runtime the reference's tests and demos use
 // (include/pto/common/cpu_stub.hpp:73-120, 524-555), on the HIP runtime.
+#include <dlfcn.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -50,7 +51,7 @@ void read_options()
     if (tt != nullptr && (tt[0] == '5' || tt[0] == '6'))
         o.tail_tile = tt[0] - '0';
     o.force_generic = env_is_1("PTOAMD_FORCE_GENERIC");
-    o.b_nd_transpose = getenv("PTOAMD_B_ND_TRANSPOSE") != nullptr;
+    o.b_nd_in_loader = getenv("PTOAMD_B_ND_IN_LOADER") != nullptr;
     o.gemv_sw_cvt = env_is_1("PTOAMD_GEMV_SW_CVT");
     o.gemv_no_splitk = env_is_1("PTOAMD_GEMV_NO_SPLITK");
     o.gemv_no_wide = env_is_1("PTOAMD_GEMV_NO_WIDE");
@@ -105,6 +106,36 @@ TraceSink& trace_sink()
     static TraceSink sink;
     return sink;
 }
+
+// Marker ranges for profilers (PTOAMD_ROCTX=1): every C-ABI launch is bracketed by a roctx range named after the PTO
+// instruction chain it stands for, so `rocprofv3 --marker-trace --kernel-trace` shows PTO opcodes next to the kernels.
+// The marker library is looked up at run time (rocprofiler-sdk's, else roctracer's); without it the switch does nothing.
+struct Roctx {
+    int (*push)(const char*) = nullptr;
+    int (*pop)() = nullptr;
+    Roctx()
+    {
+        const char* on = getenv("PTOAMD_ROCTX");
+        if (on == nullptr || on[0] != '1')
+            return;
+        for (const char* name : {"librocprofiler-sdk-roctx.so", "librocprofiler-sdk-roctx.so.1", "libroctx64.so", "libroctx64.so.4"}) {
+            void* h = dlopen(name, RTLD_NOW | RTLD_GLOBAL);
+            if (h == nullptr)
+                continue;
+            push = reinterpret_cast<int (*)(const char*)>(dlsym(h, "roctxRangePushA"));
+            pop = reinterpret_cast<int (*)()>(dlsym(h, "roctxRangePop"));
+            if (push != nullptr && pop != nullptr)
+                return;
+            push = nullptr;
+            pop = nullptr;
+        }
+    }
+};
+Roctx& roctx()
+{
+    static Roctx r;
+    return r;
+}
 const char* dtype_name(int t)
 {
     static const char* names[] = {"f32", "f16", "bf16", "i32", "i8", "u8", "e4m3", "e5m2", "e2m1x2", "e1m2x2", "i16"};
@@ -115,6 +146,11 @@ const char* dtype_name(int t)
 TraceScope::TraceScope(const char* opcode, const char* pipeline, long m, long n, long k)
     : on_(trace_sink().enabled), opcode_(opcode), pipeline_(pipeline), m_(m), n_(n), k_(k), launches_before_(g_launches)
 {
+    if (roctx().push != nullptr) {
+        char label[96];
+        snprintf(label, sizeof label, "PTO %s %ldx%ldx%ld", opcode, m, n, k);
+        roctx().push(label);
+    }
 }
 TraceScope& TraceScope::in(const void* address, long rows, long cols, const char* layout, int dtype)
 {
@@ -130,6 +166,8 @@ TraceScope& TraceScope::out(const void* address, long rows, long cols, const cha
 }
 TraceScope::~TraceScope()
 {
+    if (roctx().pop != nullptr)
+        roctx().pop();
     if (!on_ || g_launches == launches_before_)
         return;  // tracing off, or the call was rejected before anything ran
     TraceSink& sink = trace_sink();

@@ -242,6 +242,7 @@ PTO_INST RecordEvent TCVT(TileDataD& dst, TileDataS& src, RoundMode mode, Satura
     using D = typename TileDataD::DType;
     using S = typename TileDataS::DType;
     static_assert(TileDataD::Loc != TileType::Acc && TileDataS::Loc != TileType::Acc, "TCVT works on on-chip buffer tiles");
+    PTO_AMD_TRACE_INSTR(1, TR_TCVT, dst, src);
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
     const uint8_t* s = src.Storage();
     uint8_t* d = dst.Storage();
@@ -279,6 +280,7 @@ template <typename TileData, PadValue PadVal = PadValue::Zero, std::enable_if_t<
           typename... WaitEvents>
 PTO_INST RecordEvent TFILLPAD(TileData& dst, TileData& src, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TFILLPAD, dst, src);
     amd::tfillpad_lds<PadVal>(dst, src);
     return {};
 }
@@ -292,6 +294,7 @@ PTO_INST RecordEvent TFILLPAD(DstTileData& dst, SrcTileData& src, WaitEvents&...
         static_assert(DstTileData::Cols >= SrcTileData::Cols && DstTileData::Rows >= SrcTileData::Rows, "TFILLPAD_EXPAND: the destination is at least as large as the source");
     else
         static_assert(DstTileData::Cols == SrcTileData::Cols && DstTileData::Rows == SrcTileData::Rows, "TFILLPAD: source and destination have the same static shape");
+    PTO_AMD_TRACE_INSTR(1, TR_TFILLPAD, dst, src);
     amd::tfillpad_lds<DstTileData::PadVal>(dst, src);
     return {};
 }
@@ -316,8 +319,10 @@ PTO_INST RecordEvent TRESHAPE(TileDataOut& dst, TileDataIn& src, WaitEvents&...)
                   "TRESHAPE: cannot reshape between boxed and non-boxed layouts");
     static_assert(TileDataIn::Loc != TileType::Acc && TileDataIn::Loc != TileType::Left && TileDataIn::Loc != TileType::Right,
                   "TRESHAPE works on row-major on-chip buffer tiles (Mat / Vec / Bias / Scaling) on this backend");
+    PTO_AMD_TRACE_INSTR(1, TR_TRESHAPE, dst, src);
     dst.lds_ = src.lds_;
     dst.addr_ = src.addr_;
+    dst.pend_ = src.pend_;
     return {};
 }
 

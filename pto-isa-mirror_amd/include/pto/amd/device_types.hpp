@@ -89,6 +89,18 @@ __device__ __forceinline__ float fixpipe_quantize(float acc, uint64_t word)
     return r;
 }
 
+// The fix-pipe's saturation control (bit 48 of the task cookie, cpu/common.hpp:146,157-171): with it set, the half and
+// bfloat16 targets turn a NaN product into 0 and clamp an infinite one to the largest finite value of the target's
+// range like any other (without it, non-finite products pass through).  `r` is acc * scale of a float accumulator.
+template <bool TO_F16>
+__device__ __forceinline__ float fixpipe_saturate_inf(float r)
+{
+    if (r != r)
+        return 0.0f;
+    const float hi = TO_F16 ? 65504.0f : 3.402823466e38f;
+    return r < -hi ? -hi : (r > hi ? hi : r);
+}
+
 // the int16 shift mode of the fix-pipe (cpu/common.hpp:174-180): arithmetic shift right by bits 32..35 of the word plus
 // one; the reference narrows to int16 before it clamps, so the value wraps
 __device__ __forceinline__ int32_t fixpipe_shift_s16(int32_t acc, uint64_t word)
@@ -109,6 +121,41 @@ __device__ __forceinline__ float e5m2_to_f32(uint32_t c)
 {
     // E5M2 is the upper byte of an IEEE half
     return f16_bits_to_f32((uint16_t)(c << 8));
+}
+// HiFloat8 (reference: include/pto/cpu/Hifloat8.hpp:65-135): sign, then a prefix code that says how many of the remaining
+// bits are exponent (4, 3, 2, 1 or 0; sign-magnitude with an implicit leading one) and how many mantissa (1, 2, 3, 3, 3);
+// payloads 1 .. 7 are the powers of two 2^-22 .. 2^-16, 0x00 is zero, 0x80 NaN, 0x6F / 0xEF the infinities.  Every value is
+// exact in float (and in bfloat16).
+__device__ __forceinline__ float hif8_to_f32(uint32_t c)
+{
+    const uint32_t sign = (c & 0x80u) << 24, p = c & 0x7Fu;
+    if ((p >> 3) == 0) {
+        if (p == 0)
+            return sign ? u2f(0x7FC00000u) : 0.0f;
+        return u2f(sign | ((p + 104u) << 23));  // 2^(p - 23)
+    }
+    int ebits, mbits;
+    if ((p >> 5) != 0) {
+        ebits = (int)(p >> 5) + 1;  // prefixes 01, 10, 11 -> 2, 3, 4 exponent bits out of 5
+        mbits = 5 - ebits;
+    } else if ((p >> 4) == 1) {
+        ebits = 1;
+        mbits = 3;
+    } else {
+        ebits = 0;
+        mbits = 3;
+    }
+    const uint32_t rest = p & ((1u << (ebits + mbits)) - 1u);
+    const uint32_t raw_e = rest >> mbits, raw_m = rest & ((1u << mbits) - 1u);
+    int e = 0;
+    if (ebits > 0) {
+        const uint32_t sbit = raw_e & (1u << (ebits - 1));
+        const int mag = (int)((1u << (ebits - 1)) | (raw_e - sbit));
+        e = sbit ? -mag : mag;
+    }
+    if (ebits == 4 && e == 15 && raw_m == 1)
+        return u2f(sign | 0x7F800000u);
+    return u2f(sign | ((uint32_t)(e + 127) << 23) | (raw_m << (23 - mbits)));
 }
 __device__ __forceinline__ float e2m1_to_f32(uint32_t c)
 {

@@ -16,6 +16,7 @@
 #include "device_types.hpp"
 #include "lds_dma.hpp"
 #include "tile.hpp"
+#include "trace.hpp"
 
 namespace pto {
 namespace amd {
@@ -730,6 +731,7 @@ template <typename TileData, typename GlobalData, typename... WaitEvents>
 PTO_INST RecordEvent TLOAD(TileData& dst, GlobalData& src, WaitEvents&...)
 {
     static_assert(TileData::Loc != TileType::Acc, "TLOAD targets an on-chip buffer tile, not an accumulator");
+    PTO_AMD_TRACE_INSTR(1, TR_TLOAD, dst, src);
     amd::tload_lds(dst, src);
     return {};
 }
@@ -739,6 +741,7 @@ template <typename TileData, typename GlobalData, AtomicType atomicType = Atomic
           ReluPreMode reluPreMode = ReluPreMode::NoRelu, typename... WaitEvents>
 PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TSTORE, dst, src);
     if constexpr (TileData::Loc == TileType::Acc)
         amd::tstore_acc<TileData, GlobalData, atomicType, reluPreMode>(dst, src);
     else
@@ -752,6 +755,7 @@ template <typename TileData, typename GlobalData, AtomicType atomicType = Atomic
           ReluPreMode reluPreMode = ReluPreMode::NoRelu>
 PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, uint64_t preQuantScalar)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TSTORE, dst, src);
     static_assert(TileData::Loc == TileType::Acc && atomicType == AtomicType::AtomicNone, "quantising TSTORE drains an accumulator tile");
     amd::tstore_acc_quant<false, TileData, GlobalData, reluPreMode>(dst, src, [&](int) { return preQuantScalar; });
     return {};
@@ -761,6 +765,7 @@ template <typename TileData, typename GlobalData, typename FpTileData, AtomicTyp
           typename = std::enable_if_t<is_tile_data_v<FpTileData> && FpTileData::Loc == TileType::Scaling>>
 PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, FpTileData& fp)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TSTORE_FP, dst, src, fp);
     static_assert(TileData::Loc == TileType::Acc && atomicType == AtomicType::AtomicNone, "quantising TSTORE drains an accumulator tile");
     static_assert(sizeof(typename FpTileData::DType) == 8, "the Scaling tile holds one 64-bit quantisation word per column");
     const uint8_t* words = fp.Storage();
@@ -831,6 +836,7 @@ template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode, type
 PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, WaitEvents&...)
 {
     static_assert(DstTileData::Loc != TileType::Acc, "TMOV into an accumulator tile is not implemented on this backend");
+    PTO_AMD_TRACE_INSTR(1, TR_TMOV, dst, src);
     if constexpr (SrcTileData::Loc == TileType::Acc) {
         amd::tmov_acc<0, reluMode>(dst, src, 0, 0, [](int) { return (uint64_t)0; });
     } else {
@@ -850,6 +856,7 @@ template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode = Rel
           std::enable_if_t<all_events_v<WaitEvents...>, int> = 0>
 PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, uint64_t preQuantScalar, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TMOV, dst, src);
     static_assert(SrcTileData::Loc == TileType::Acc, "the quantising TMOV drains an accumulator tile");
     amd::tmov_acc<1, reluMode>(dst, src, 0, 0, [&](int) { return preQuantScalar; });
     return {};
@@ -858,6 +865,7 @@ template <typename DstTileData, typename SrcTileData, typename FpTileData, ReluP
           std::enable_if_t<is_tile_data_v<FpTileData> && FpTileData::Loc == TileType::Scaling && all_events_v<WaitEvents...>, int> = 0>
 PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, FpTileData& fp, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TMOV, dst, src, fp);
     static_assert(SrcTileData::Loc == TileType::Acc, "the quantising TMOV drains an accumulator tile");
     static_assert(sizeof(typename FpTileData::DType) == 8, "the Scaling tile holds one 64-bit quantisation word per column");
     const uint8_t* words = fp.Storage();
@@ -869,6 +877,7 @@ template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode = Rel
           std::enable_if_t<all_events_v<WaitEvents...>, int> = 0>
 PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, uint16_t indexRow = 0, uint16_t indexCol = 0, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TEXTRACT, dst, src);
     static_assert(DstTileData::Loc != TileType::Acc, "TEXTRACT into an accumulator tile is not implemented on this backend");
     if constexpr (SrcTileData::Loc == TileType::Acc) {
         amd::tmov_acc<0, reluMode>(dst, src, indexRow, indexCol, [](int) { return (uint64_t)0; });
@@ -883,6 +892,7 @@ template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode = Rel
           std::enable_if_t<all_events_v<WaitEvents...>, int> = 0>
 PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, uint64_t preQuantScalar, uint16_t indexRow, uint16_t indexCol, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TEXTRACT, dst, src);
     static_assert(SrcTileData::Loc == TileType::Acc, "the quantising TEXTRACT drains an accumulator tile");
     amd::tmov_acc<1, reluMode>(dst, src, indexRow, indexCol, [&](int) { return preQuantScalar; });
     return {};
@@ -891,6 +901,7 @@ template <typename DstTileData, typename SrcTileData, typename FpTileData, ReluP
           std::enable_if_t<is_tile_data_v<FpTileData> && FpTileData::Loc == TileType::Scaling && all_events_v<WaitEvents...>, int> = 0>
 PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, FpTileData& fp, uint16_t indexRow, uint16_t indexCol, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TEXTRACT, dst, src, fp);
     static_assert(SrcTileData::Loc == TileType::Acc, "the quantising TEXTRACT drains an accumulator tile");
     static_assert(sizeof(typename FpTileData::DType) == 8, "the Scaling tile holds one 64-bit quantisation word per column");
     const uint8_t* words = fp.Storage();
@@ -900,55 +911,97 @@ PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, FpTileData& fp
 }
 
 // ---- TMATMUL family ------------------------------------------------------------------------------------------------
+namespace amd {
+template <typename TileRes>
+PTO_INST void copy_acc(TileRes& out, TileRes& in)
+{
+    if (&out != &in) {
+#pragma unroll
+        for (int s = 0; s < TileRes::NBLK; ++s)
+            out.regs[s] = in.regs[s];
+    }
+}
+// bias (1 x N, any LDS tile) is added after the K loop, per column (reference: cpu/TMatmul.hpp:219-230)
+template <typename TileRes, typename TileBias>
+PTO_INST void add_bias_row(TileRes& c, TileBias& bias)
+{
+    using B = typename TileBias::DType;
+    const uint8_t* pb = bias.Storage();
+    const int vc = c.GetValidCol();
+    for_each_acc(c, [&](int slot, int r, int, int col) {
+        if (col < vc)
+            c.regs[slot][r] += static_cast<typename TileRes::Reg>(*reinterpret_cast<const B*>(pb + bias.ByteOffset(0, col)));
+    });
+}
+}  // namespace amd
+
 template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
 PTO_INST RecordEvent TMATMUL(TileRes& cMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TMATMUL, cMatrix, aMatrix, bMatrix);
     amd::tmatmul<true>(cMatrix, aMatrix, bMatrix);
     return {};
 }
 template <AccPhase Phase, typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
 PTO_INST RecordEvent TMATMUL(TileRes& cMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TMATMUL, cMatrix, aMatrix, bMatrix);
     amd::tmatmul<true>(cMatrix, aMatrix, bMatrix);
     return {};
 }
 template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
 PTO_INST RecordEvent TMATMUL_ACC(TileRes& cOutMatrix, TileRes& cInMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, WaitEvents&...)
 {
-    if (&cOutMatrix != &cInMatrix) {
-#pragma unroll
-        for (int s = 0; s < TileRes::NBLK; ++s)
-            cOutMatrix.regs[s] = cInMatrix.regs[s];
-    }
+    PTO_AMD_TRACE_INSTR(1, TR_TMATMUL_ACC, cOutMatrix, cInMatrix, aMatrix, bMatrix);
+    amd::copy_acc(cOutMatrix, cInMatrix);
     amd::tmatmul<false>(cOutMatrix, aMatrix, bMatrix);
     return {};
 }
 template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
 PTO_INST RecordEvent TMATMUL_ACC(TileRes& cMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TMATMUL_ACC, cMatrix, cMatrix, aMatrix, bMatrix);
     amd::tmatmul<false>(cMatrix, aMatrix, bMatrix);
     return {};
 }
-// bias (1 x N, any LDS tile) is added after the K loop, per column (reference: cpu/TMatmul.hpp:219-230)
 template <typename TileRes, typename TileLeftT, typename TileRightT, typename TileBias, typename... WaitEvents>
 PTO_INST RecordEvent TMATMUL_BIAS(TileRes& cMatrix, TileLeftT& aMatrix, TileRightT& bMatrix, TileBias& biasData, WaitEvents&...)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TMATMUL_BIAS, cMatrix, aMatrix, bMatrix, biasData);
     amd::tmatmul<true>(cMatrix, aMatrix, bMatrix);
-    using B = typename TileBias::DType;
-    const uint8_t* pb = biasData.Storage();
-    const int vc = cMatrix.GetValidCol();
-    amd::for_each_acc(cMatrix, [&](int slot, int r, int, int col) {
-        if (col < vc)
-            cMatrix.regs[slot][r] += static_cast<typename TileRes::Reg>(*reinterpret_cast<const B*>(pb + biasData.ByteOffset(0, col)));
-    });
+    amd::add_bias_row(cMatrix, biasData);
     return {};
 }
 // ---- TMATMUL_MX / TGEMV_MX (fp8 E4M3 / E5M2 or fp4 E2M1 operands; reference: cpu/TMatmul.hpp:169-205,254-326) ------------------
+// (a trace record names the accumulator and the two operand tiles; the scale tiles follow their operands)
+namespace amd {
+template <TraceOpOrInt OP, typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT>
+PTO_INST void tmatmul_mx_plain(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRightT& b, TileRightScaleT& bs)
+{
+    PTO_AMD_TRACE_INSTR(1, PTO_AMD_TRACE_OP(OP), c, a, b);
+    tmatmul_mx<true>(c, a, as, b, bs);
+}
+template <TraceOpOrInt OP, typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT>
+PTO_INST void tmatmul_mx_acc(TileRes& cOut, TileRes& cIn, TileLeftT& a, TileLeftScaleT& as, TileRightT& b, TileRightScaleT& bs)
+{
+    PTO_AMD_TRACE_INSTR(1, PTO_AMD_TRACE_OP(OP), cOut, cIn, a, b);
+    copy_acc(cOut, cIn);
+    tmatmul_mx<false>(cOut, a, as, b, bs);
+}
+template <TraceOpOrInt OP, typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT, typename TileBias>
+PTO_INST void tmatmul_mx_bias(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRightT& b, TileRightScaleT& bs, TileBias& bias)
+{
+    static_assert(std::is_same_v<typename TileBias::DType, float> && TileBias::Rows == 1, "TMATMUL_MX: bias is one row of float");
+    PTO_AMD_TRACE_INSTR(1, PTO_AMD_TRACE_OP(OP), c, a, b, bias);
+    tmatmul_mx<true>(c, a, as, b, bs);
+    add_bias_row(c, bias);
+}
+}  // namespace amd
 template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT,
           typename = std::enable_if_t<TileLeftScaleT::Loc == TileType::ScaleLeft>>
 PTO_INST RecordEvent TMATMUL_MX(TileRes& cMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale, TileRightT& bMatrix, TileRightScaleT& bScale)
 {
-    amd::tmatmul_mx<true>(cMatrix, aMatrix, aScale, bMatrix, bScale);
+    amd::tmatmul_mx_plain<PTO_AMD_TR(TR_TMATMUL_MX)>(cMatrix, aMatrix, aScale, bMatrix, bScale);
     return {};
 }
 template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT,
@@ -956,12 +1009,7 @@ template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typenam
 PTO_INST RecordEvent TMATMUL_MX(TileRes& cOutMatrix, TileRes& cInMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale,
                                 TileRightT& bMatrix, TileRightScaleT& bScale)
 {
-    if (&cOutMatrix != &cInMatrix) {
-#pragma unroll
-        for (int s = 0; s < TileRes::NBLK; ++s)
-            cOutMatrix.regs[s] = cInMatrix.regs[s];
-    }
-    amd::tmatmul_mx<false>(cOutMatrix, aMatrix, aScale, bMatrix, bScale);
+    amd::tmatmul_mx_acc<PTO_AMD_TR(TR_TMATMUL_MX)>(cOutMatrix, cInMatrix, aMatrix, aScale, bMatrix, bScale);
     return {};
 }
 template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT, typename TileBias,
@@ -969,36 +1017,55 @@ template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typenam
 PTO_INST RecordEvent TMATMUL_MX(TileRes& cMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale, TileRightT& bMatrix,
                                 TileRightScaleT& bScale, TileBias& biasData)
 {
-    static_assert(std::is_same_v<typename TileBias::DType, float> && TileBias::Rows == 1, "TMATMUL_MX: bias is one row of float");
-    amd::tmatmul_mx<true>(cMatrix, aMatrix, aScale, bMatrix, bScale);
-    const uint8_t* pb = biasData.Storage();
-    const int vc = cMatrix.GetValidCol();
-    amd::for_each_acc(cMatrix, [&](int slot, int r, int, int col) {
-        if (col < vc)
-            cMatrix.regs[slot][r] += *reinterpret_cast<const float*>(pb + biasData.ByteOffset(0, col));
-    });
+    amd::tmatmul_mx_bias<PTO_AMD_TR(TR_TMATMUL_MX)>(cMatrix, aMatrix, aScale, bMatrix, bScale, biasData);
     return {};
 }
-template <typename TileRes, typename... Rest>
-PTO_INST RecordEvent TGEMV_MX(TileRes& cMatrix, Rest&... rest)
+template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT,
+          typename = std::enable_if_t<TileLeftScaleT::Loc == TileType::ScaleLeft>>
+PTO_INST RecordEvent TGEMV_MX(TileRes& cMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale, TileRightT& bMatrix, TileRightScaleT& bScale)
 {
-    return TMATMUL_MX(cMatrix, rest...);
+    amd::tmatmul_mx_plain<PTO_AMD_TR(TR_TGEMV_MX)>(cMatrix, aMatrix, aScale, bMatrix, bScale);
+    return {};
+}
+template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT,
+          typename = std::enable_if_t<TileLeftScaleT::Loc == TileType::ScaleLeft>>
+PTO_INST RecordEvent TGEMV_MX(TileRes& cOutMatrix, TileRes& cInMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale, TileRightT& bMatrix,
+                              TileRightScaleT& bScale)
+{
+    amd::tmatmul_mx_acc<PTO_AMD_TR(TR_TGEMV_MX)>(cOutMatrix, cInMatrix, aMatrix, aScale, bMatrix, bScale);
+    return {};
+}
+template <typename TileRes, typename TileLeftT, typename TileLeftScaleT, typename TileRightT, typename TileRightScaleT, typename TileBias,
+          typename = std::enable_if_t<TileLeftScaleT::Loc == TileType::ScaleLeft && TileBias::Loc == TileType::Bias>>
+PTO_INST RecordEvent TGEMV_MX(TileRes& cMatrix, TileLeftT& aMatrix, TileLeftScaleT& aScale, TileRightT& bMatrix, TileRightScaleT& bScale,
+                              TileBias& biasData)
+{
+    amd::tmatmul_mx_bias<PTO_AMD_TR(TR_TGEMV_MX)>(cMatrix, aMatrix, aScale, bMatrix, bScale, biasData);
+    return {};
 }
 
 template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
 PTO_INST RecordEvent TGEMV(TileRes& c, TileLeftT& a, TileRightT& b, WaitEvents&...)
 {
-    return TMATMUL(c, a, b);
+    PTO_AMD_TRACE_INSTR(1, TR_TGEMV, c, a, b);
+    amd::tmatmul<true>(c, a, b);
+    return {};
 }
 template <typename TileRes, typename TileLeftT, typename TileRightT, typename... WaitEvents>
 PTO_INST RecordEvent TGEMV_ACC(TileRes& cOut, TileRes& cIn, TileLeftT& a, TileRightT& b, WaitEvents&...)
 {
-    return TMATMUL_ACC(cOut, cIn, a, b);
+    PTO_AMD_TRACE_INSTR(1, TR_TGEMV_ACC, cOut, cIn, a, b);
+    amd::copy_acc(cOut, cIn);
+    amd::tmatmul<false>(cOut, a, b);
+    return {};
 }
 template <typename TileRes, typename TileLeftT, typename TileRightT, typename TileBias, typename... WaitEvents>
 PTO_INST RecordEvent TGEMV_BIAS(TileRes& c, TileLeftT& a, TileRightT& b, TileBias& bias, WaitEvents&...)
 {
-    return TMATMUL_BIAS(c, a, b, bias);
+    PTO_AMD_TRACE_INSTR(1, TR_TGEMV_BIAS, c, a, b, bias);
+    amd::tmatmul<true>(c, a, b);
+    amd::add_bias_row(c, bias);
+    return {};
 }
 
 }  // namespace pto

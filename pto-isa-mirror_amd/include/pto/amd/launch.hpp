@@ -3,8 +3,16 @@
 // launch of the reference's NPU tests and LaunchKernelMultiCore of its CPU simulator (common/cpu_stub.hpp:367-427).
 #pragma once
 #include <atomic>
+#ifdef PTO_AMD_TRACE
+#include <stdio.h>
+#include <stdlib.h>
+#include <unistd.h>
+
+#include <vector>
+#endif
 
 #include "tile.hpp"
+#include "trace.hpp"
 
 namespace pto {
 namespace amd {
@@ -14,6 +22,54 @@ __attribute__((global)) __launch_bounds__(PTO_AMD_THREADS) void core_entry(Args.
 {
     Kernel(args...);
 }
+
+#ifdef PTO_AMD_TRACE
+// After a traced launch: wait for it, read the records of the traced core and append them as JSON lines (field names of
+// the reference's InstructionTraceRecord, cpu/trace.hpp:80-88) to $PTOAMD_TRACE_DIR/ptoamd_instr_trace_<pid>.jsonl.
+inline int write_instruction_trace(hipStream_t stream)
+{
+    hipError_t e = hipStreamSynchronize(stream);
+    if (e != hipSuccess)
+        return (int)e;
+    unsigned int count = 0;
+    if ((e = hipMemcpyFromSymbol(&count, HIP_SYMBOL(g_trace_count), sizeof count)) != hipSuccess)
+        return (int)e;
+    const unsigned int kept = count < PTO_AMD_TRACE_MAX ? count : PTO_AMD_TRACE_MAX;
+    std::vector<TraceRecord> rec(kept);
+    if (kept > 0 && (e = hipMemcpyFromSymbol(rec.data(), HIP_SYMBOL(g_trace), kept * sizeof(TraceRecord))) != hipSuccess)
+        return (int)e;
+    const char* dir = getenv("PTOAMD_TRACE_DIR");
+    if (dir == nullptr || *dir == 0)
+        return 0;
+    char path[1024];
+    snprintf(path, sizeof path, "%s/ptoamd_instr_trace_%ld.jsonl", dir, (long)getpid());
+    FILE* f = fopen(path, "a");
+    if (f == nullptr)
+        return 0;
+    for (unsigned int i = 0; i < kept; ++i) {
+        const TraceRecord& r = rec[i];
+        fprintf(f, "{\"block_idx\": %u, \"subblock_id\": 0, \"sequence_id\": %u, \"opcode\": \"%s\"", r.block_idx, i, trace_op_name(r.opcode));
+        for (int side = 0; side < 2; ++side) {
+            fprintf(f, ", \"%s\": [", side == 0 ? "output_tiles" : "input_tiles");
+            bool first = true;
+            for (int k = 0; k < 4; ++k) {
+                const TraceOperand& o = r.operands[k];
+                if (!o.used || (k < r.n_out) != (side == 0))
+                    continue;
+                fprintf(f, "%s{\"address\": %llu, \"shape\": [%d, %d], \"layout\": \"%s\", \"dtype\": \"%s\"}", first ? "" : ", ",
+                        (unsigned long long)o.address, o.rows, o.cols, trace_place_name(o.place), trace_dtype_name(o.dtype));
+                first = false;
+            }
+            fprintf(f, "]");
+        }
+        fprintf(f, "}\n");
+    }
+    if (count > kept)
+        fprintf(f, "{\"dropped_records\": %u}\n", count - kept);
+    fclose(f);
+    return 0;
+}
+#endif
 
 // returns hipSuccess (0) or the HIP error of the launch
 template <auto Kernel, typename... Args>
@@ -33,8 +89,18 @@ inline int launch(int blocks, void* stream, Args... args)
             return (int)e;
         configured.fetch_or(bit, std::memory_order_release);
     }
+#ifdef PTO_AMD_TRACE
+    const unsigned int zero = 0;
+    if (const hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_trace_count), &zero, sizeof zero); e != hipSuccess)
+        return (int)e;
+#endif
     hipLaunchKernelGGL(entry, dim3(blocks), dim3(PTO_AMD_THREADS), LDS_TOTAL, static_cast<hipStream_t>(stream), args...);
-    return (int)hipGetLastError();
+    const int rc = (int)hipGetLastError();
+#ifdef PTO_AMD_TRACE
+    if (rc == 0)
+        return write_instruction_trace(static_cast<hipStream_t>(stream));
+#endif
+    return rc;
 }
 
 // the sticky status word of this translation unit's cores (0 = no constraint violated); synchronises the device

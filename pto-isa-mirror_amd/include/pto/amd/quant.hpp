@@ -138,6 +138,7 @@ template <auto quant_type, typename TileDataOut, typename TileDataSrc, typename 
           typename = std::enable_if_t<quant_type == QuantType::INT8_SYM || quant_type == QuantType::INT8_ASYM>>
 PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataPara& scale, TileDataPara* offset = nullptr)
 {
+    PTO_AMD_TRACE_INSTR(1, TR_TQUANT, dst, src, scale);
     amd::tquant_int8<quant_type == QuantType::INT8_ASYM>(dst, src, scale, offset);
     return {};
 }
@@ -149,6 +150,7 @@ template <auto quant_type, typename TileDataOut, typename TileDataSrc, typename 
 PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataExp* exp, TileDataMax* max, TileDataScaling* scaling)
 {
     constexpr int alg = (quant_type == QuantType::MXFP8 ? 0 : 2) + (scale_alg == QuantScaleAlg::NV ? 1 : 0);
+    PTO_AMD_TRACE_INSTR(1, TR_TQUANT, dst, src);
     amd::tquant_mx<alg>(dst, src, exp, max, scaling);
     return {};
 }
@@ -164,6 +166,7 @@ PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataExp* exp
 {
     static_assert(quant_type == QuantType::MXFP8, "TQUANT: the NZ store mode is defined for MXFP8");
     static_assert(store_mode == VecStoreMode::NZ, "TQUANT: this overload is the NZ store mode");
+    PTO_AMD_TRACE_INSTR(1, TR_TQUANT, dst, src);
     amd::tquant_mx<0>(dst, src, exp, max, scaling);
     const int rows = src.GetValidRow(), groups = src.GetValidCol() / 32;
     if (exp == nullptr || exp_zz == nullptr || rows % 16 != 0 || groups % 2 != 0) {
@@ -189,6 +192,7 @@ PTO_INST RecordEvent TQUANT(TileDataOut& dst, TileDataSrc& src, TileDataExp* exp
     static_assert(std::is_same_v<decltype(mx_alg), MxQuantAlg>, "TQUANT<grp_axis, mx_alg>: mx_alg is an MxQuantAlg");
     constexpr int alg = static_cast<int>(mx_alg);
     static_assert(alg >= 0 && alg <= 3, "TQUANT: the HiFloat4 algorithm is not implemented on this backend");
+    PTO_AMD_TRACE_INSTR(1, TR_TQUANT, dst, src);
     if constexpr (grp_axis == 1)
         amd::tquant_mx<alg>(dst, src, exp, max, scaling);
     else
@@ -202,6 +206,7 @@ PTO_INST RecordEvent TDEQUANT(TileDataDst& dst, TileDataSrc& src, TileDataPara& 
 {
     using D = typename TileDataDst::DType;
     static_assert(std::is_same_v<D, float>, "TDEQUANT writes a float tile on this backend");
+    PTO_AMD_TRACE_INSTR(1, TR_TDEQUANT, dst, src, scale, offset);
     const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
     __syncthreads();
     for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {

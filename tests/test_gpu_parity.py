@@ -149,8 +149,8 @@ def test_row_major_b_is_transposed_inside_the_kernel(pa, oracle, tile, kind, m, 
         got = host(pa.gemm(da, db, ta, tc, pa.B_ND, n=n))
         assert pa.last_kernel().startswith(TILE_NAMES[tile])
         same = host(pa.gemm(da, bt, ta, tc, pa.B_DN))
-        with tile_env(PTOAMD_B_ND_TRANSPOSE=1):
-            via_copy = host(pa.gemm(da, db, ta, tc, pa.B_ND, n=n))
+        ws = torch.empty(pa.gemm_workspace_bytes(n, da.shape[1], ta, pa.B_ND), dtype=torch.uint8, device=DEV)
+        via_copy = host(pa.gemm(da, db, ta, tc, pa.B_ND, n=n, workspace=ws))  # B re-ordered into a caller workspace
     assert np.array_equal(got.view(np.uint32), same.view(np.uint32))
     assert np.array_equal(got.view(np.uint32), via_copy.view(np.uint32))
     if kind == "i8":
@@ -380,9 +380,6 @@ def test_w8a8_fused_dequant(pa, oracle):
     assert np.array_equal(host(out_nd), ref_out)
     out_nd, acc_nd = pa.gemm_w8a8(dev(a), b_nd, dev(sa), dev(sb), b_layout=pa.B_ND, want_acc=True)
     assert np.array_equal(host(out_nd), ref_out) and np.array_equal(host(acc_nd), ref_acc)
-    with tile_env(PTOAMD_B_ND_TRANSPOSE=1):
-        out_nd = pa.gemm_w8a8(dev(a), b_nd, dev(sa), dev(sb), b_layout=pa.B_ND)
-    assert np.array_equal(host(out_nd), ref_out)
 
 
 def test_config3_w8a8_full_size(pa, oracle):
@@ -1212,3 +1209,156 @@ def test_errors_are_loud(pa):
     with pytest.raises(pa.PtoAmdError):
         pa.gemv_mxfp4(torch.zeros((17, 256), dtype=torch.bfloat16, device=DEV), torch.zeros((16, 128), dtype=torch.uint8, device=DEV),
                       torch.zeros((16, 8), dtype=torch.uint8, device=DEV), 16, 256)
+
+
+# ------------------------------------------------------------------------------------------- rows at any alignment
+@pytest.mark.parametrize("kind,m,k,n,b_dn,pad,skew", [
+    ("f16", 40, 50, 60, False, 0, 0),      # the reference's tmatmul case 1: K * 2 = 100 bytes, B row-major with N * 2 = 120
+    ("bf16", 40, 50, 60, False, 0, 0),
+    ("f16", 1, 110, 50, False, 0, 0),      # its GEMV shape
+    ("f16", 26, 100, 94, False, 3, 1),     # its bias shape, padded pitches and operands that start on odd elements
+    ("i8", 33, 70, 100, True, 7, 3),       # K = 70 bytes, pitch 77, operands 3 bytes off alignment
+    ("i8", 130, 257, 33, True, 0, 1),
+    ("i8", 64, 100, 72, False, 5, 0),      # B row-major with N = 72 bytes, pitch 77
+    ("e4m3", 48, 90, 40, True, 2, 0),
+    ("bf16", 300, 1033, 260, True, 1, 0),  # several slabs, a 2-byte tail
+])
+def test_unaligned_rows_stay_on_the_mfma_tiles(pa, oracle, kind, m, k, n, b_dn, pad, skew):
+    """Rows whose length or pitch is not a multiple of 16 bytes, and operands that start anywhere, run on the
+    register-staged MFMA tiles (unaligned 16-byte loads, the row's last chunk read up to the row's end and shifted): the
+    shapes of the reference's own tmatmul tests among them.  Integer results are exact; float results meet the fp32 bars."""
+    r = np.random.default_rng(m * 7 + k * 3 + n)
+    lda = k + pad
+    ldb = (k if b_dn else n) + pad
+    brows = n if b_dn else k
+    if kind == "i8":
+        dt, ta, tc = np.int8, pa.I8, pa.I32
+        a_full = r.integers(-128, 128, m * lda + skew).astype(np.int8)
+        b_full = r.integers(-128, 128, brows * ldb + skew).astype(np.int8)
+    elif kind == "e4m3":
+        dt, ta, tc = np.uint8, pa.E4M3, pa.F32
+        a_full = r.integers(0, 0x78, m * lda + skew).astype(np.uint8)
+        b_full = r.integers(0, 0x78, brows * ldb + skew).astype(np.uint8)
+    else:
+        dt, ta, tc = np.uint16, (pa.F16 if kind == "f16" else pa.BF16), pa.F32
+        conv = (lambda x: x.astype(np.float16).view(np.uint16)) if kind == "f16" else bf16_bits
+        a_full = conv(r.uniform(-1, 1, m * lda + skew).astype(np.float32))
+        b_full = conv(r.uniform(-1, 1, brows * ldb + skew).astype(np.float32))
+    a = a_full[skew:].reshape(m, lda)[:, :k]
+    b = b_full[skew:].reshape(brows, ldb)[:, :(k if b_dn else n)]
+    tdt = {np.int8: torch.int8, np.uint8: torch.uint8, np.uint16: (torch.float16 if kind == "f16" else torch.bfloat16)}[dt]
+
+    def on_device(full, rows, ld, cols):
+        t = torch.from_numpy(np.ascontiguousarray(full)).to(DEV)
+        t = t.view(tdt) if dt == np.uint16 else t
+        return t[skew:].view(rows, ld)[:, :cols]  # a row-strided view that starts `skew` elements into its buffer
+
+    da, db = on_device(a_full, m, lda, k), on_device(b_full, brows, ldb, k if b_dn else n)
+    got = host(pa.gemm(da, db, ta, tc, pa.B_DN if b_dn else pa.B_ND, m=m, n=n, k=k))
+    assert pa.last_kernel().startswith("tile"), pa.last_kernel()
+    a_c, b_c = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    if kind == "i8":
+        assert np.array_equal(got, oracle.matmul_i8(a_c, b_c, b_dn=b_dn))
+        return
+    if kind == "e4m3":
+        ref = oracle.matmul_fp8(a_c, b_c, b_dn=b_dn)
+        fa, fb = _mx_unpack(oracle, a_c, ob.E4M3), _mx_unpack(oracle, b_c, ob.E4M3)
+        check_f32_drain(got, ref, np.abs(fa) @ (np.abs(fb).T if b_dn else np.abs(fb)), k, f"unaligned e4m3 {m}x{n}x{k}", max_rel=1e-3,
+                        eps=2.0 ** -11)
+        return
+    ref = (oracle.matmul_f16 if kind == "f16" else oracle.matmul_bf16)(a_c, b_c, b_dn=b_dn)
+    fa = a_c.view(np.float16).astype(np.float64) if kind == "f16" else bf16_to_f32(a_c).astype(np.float64)
+    fb = b_c.view(np.float16).astype(np.float64) if kind == "f16" else bf16_to_f32(b_c).astype(np.float64)
+    check_f32_drain(got, ref, np.abs(fa) @ (np.abs(fb).T if b_dn else np.abs(fb)), k, f"unaligned {kind} {m}x{n}x{k}")
+
+
+def test_unaligned_k_large_int8_product(pa, oracle):
+    """int8 2048 x 2048 x 8200 (K is 8 bytes past a multiple of 16, every second row misaligned): an MFMA tile runs it;
+    512 sampled outputs are exact."""
+    m, n, k = 2048, 2048, 8200
+    gen = torch.Generator(device=DEV).manual_seed(8200)
+    a = torch.randint(-128, 128, (m, k), generator=gen, device=DEV, dtype=torch.int8)
+    b = torch.randint(-128, 128, (n, k), generator=gen, device=DEV, dtype=torch.int8)
+    got = host(pa.gemm(a, b, pa.I8, pa.I32, pa.B_DN))
+    assert pa.last_kernel().startswith("tile"), pa.last_kernel()
+    rows = np.array([0, 1, 127, 128, 1023, 2046, 2047, 77])
+    cols = np.arange(0, 2048, 32) + np.arange(64) % 32
+    ref = oracle.matmul_i8(host(sel(a, rows)), host(sel(b, cols)), b_dn=True)
+    assert np.array_equal(got[np.ix_(rows, cols)], ref)
+
+
+def test_row_major_b_through_a_workspace(pa, oracle):
+    """ptoamd_gemm_ws: a row-major B re-ordered into the caller's workspace, then the LDS-DMA tiles; bit-identical to the
+    product with the same B given column-major, and a workspace that is too small is refused."""
+    m, n, k = 2048, 2048, 1024
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    a = (torch.randn((m, k), generator=gen, device=DEV) * 0.1).to(torch.bfloat16)
+    b = (torch.randn((k, n), generator=gen, device=DEV) * 0.1).to(torch.bfloat16)
+    ws = torch.empty(pa.gemm_workspace_bytes(n, k, pa.BF16, pa.B_ND), dtype=torch.uint8, device=DEV)
+    assert ws.numel() == n * k * 2 and pa.gemm_workspace_bytes(n, k, pa.BF16, pa.B_DN) == 0
+    got = pa.gemm(a, b, pa.BF16, pa.F32, pa.B_ND, workspace=ws)
+    assert "dtl" in pa.last_kernel(), pa.last_kernel()
+    same = pa.gemm(a, b.t().contiguous(), pa.BF16, pa.F32, pa.B_DN)
+    assert torch.equal(got, same)
+    in_loader = pa.gemm(a, b, pa.BF16, pa.F32, pa.B_ND)   # no workspace: the register-staged loader transposes, nothing is allocated
+    assert pa.last_kernel().startswith("tile") and "dtl" not in pa.last_kernel()
+    assert relerr(host(in_loader), host(same)) <= 1e-5
+    with pytest.raises(pa.PtoAmdError, match="workspace"):
+        pa.gemm(a, b, pa.BF16, pa.F32, pa.B_ND, workspace=ws[: ws.numel() // 2])
+
+
+def test_hif8_tmatmul_is_order_exact(pa, oracle):
+    """hif8 x hif8 (the one non-MX 8-bit float pair of cpu/TMatmul.hpp:38 besides E4M3 / E5M2): every code decodes to an
+    exact float and the product runs on the order-exact kernel, bit for bit the simulator's fma chain; every code appears."""
+    r = np.random.default_rng(88)
+    m, k, n = 24, 96, 40
+    a = r.integers(0, 256, (m, k)).astype(np.uint8)
+    b = r.integers(0, 256, (k, n)).astype(np.uint8)
+    a[0, :] = np.arange(96)
+    a[1, :] = np.arange(96, 192)
+    a[2, :64] = np.arange(192, 256)
+    for x in (a, b):   # keep NaN and the infinities to one row / column each, so that the other sums stay finite
+        x[(x == 0x80) | ((x & 0x7F) == 0x6F)] = 0x33
+    a[2, 70], a[2, 71], a[2, 72] = 0x80, 0x6F, 0xEF
+    table = oracle.hif8_table()
+    assert np.isnan(table[0x80]) and table[0x6F] == np.inf and table[0xEF] == -np.inf and table[0x01] == 2.0 ** -22
+    ref = oracle.matmul_hif8(a, b)
+    got = host(pa.gemm(dev(a), dev(b), pa.HIF8, pa.F32, pa.B_ND))
+    assert pa.last_kernel() == "generic"
+    nan = np.isnan(ref)
+    assert np.array_equal(nan, np.isnan(got)) and np.array_equal(got[~nan].view(np.uint32), ref[~nan].view(np.uint32))
+    with pytest.raises(pa.PtoAmdError):   # hif8 pairs with hif8 only
+        pa.gemm_fp8(dev(a), dev(np.ascontiguousarray(b.T)), pa.HIF8, pa.E4M3)
+
+
+@pytest.mark.parametrize("tile", [None, 1, 2])
+@pytest.mark.parametrize("per_col", [False, True])
+def test_requant_saturate_inf_flag(pa, oracle, tile, per_col):
+    """PTOAMD_SATURATE_INF: the fix-pipe's saturation control on the f16 and bf16 drains of a float accumulator that holds
+    infinities, NaNs and values past the half range; with the flag off they pass through as the reference's do."""
+    r = np.random.default_rng(5 + int(per_col))
+    m, n, k = 128, 128, 64
+    a = r.uniform(-1, 1, (m, k)).astype(np.float16)
+    b = r.uniform(-1, 1, (n, k)).astype(np.float16)
+    a[0, 0] = np.inf          # row 0: +-inf accumulators
+    a[1, 0] = np.inf; a[1, 1] = -np.inf   # row 1: inf - inf = NaN wherever both columns of b are of one sign ... and inf elsewhere
+    a[2, :] = 60000.0         # row 2: finite sums far past 65504
+    b[:, 0] = np.where(b[:, 0] == 0, 0.5, b[:, 0])
+    mk = _word_vector if per_col else _word_scalar
+    words = np.array([mk(r.uniform(0.5, 2.0)) for _ in range(n)], np.uint64)
+    acc = oracle.matmul_f16(a.view(np.uint16), b.view(np.uint16), b_dn=True)
+    assert np.isinf(acc[0]).all() and np.isnan(acc[1]).any() and (np.abs(acc[2]) > 7e4).any()
+    env = tile_env(PTOAMD_TILE=tile) if tile is not None else tile_env(PTOAMD_FORCE_GENERIC=1)
+    with env:
+        gpu_acc = host(pa.gemm(dev(a), dev(b), pa.F16, pa.F32, pa.B_DN))
+        for c_type, st in ((pa.F16, ob.ST_F16), (pa.BF16, ob.ST_BF16)):
+            for flags in (0, pa.SATURATE_INF, pa.SATURATE_INF | pa.RELU):
+                got = host(pa.gemm_requant(dev(a), dev(b), pa.F16, c_type, dev(words.view(np.int64)), per_col, relu=flags))
+                want = oracle.store_quant(gpu_acc, st, words, per_col, relu=bool(flags & pa.RELU), saturate_inf=int(bool(flags & pa.SATURATE_INF)))
+                g16, w16 = got.view(np.uint16), want.view(np.uint16)
+                nan_mask = 0x7C00 if c_type == pa.F16 else 0x7F80
+                both_nan = ((g16 & 0x7FFF) > nan_mask) & ((w16 & 0x7FFF) > nan_mask)
+                assert np.array_equal(np.where(both_nan, 0, g16), np.where(both_nan, 0, w16)), (c_type, flags)
+                if (flags & pa.SATURATE_INF) and c_type == pa.F16:
+                    assert not both_nan.any() and ((g16 & 0x7FFF) < nan_mask).all()   # nothing non-finite is left
+                    # (bfloat16: the clamp is to +-FLT_MAX, which the conversion then rounds to infinity, as the reference's does)

@@ -422,3 +422,46 @@ def test_case_runner_and_launch_trace(tmp_path):
     assert [r["opcode"] for r in quant] == ["TQUANT_MXFP8", "TQUANT_MXFP8", "TMATMUL_MX"]
     assert quant[0]["pipeline"] == "vector" and quant[0]["kernel"] == "tquant_mx_rows"
     assert [t["layout"] for t in quant[2]["input_tiles"][2:4]] == ["MX_A_ND", "MX_B_DN"]
+
+
+def test_instruction_trace_of_a_pto_kernel(tmp_path, monkeypatch):
+    """A kernel source compiled with -DPTO_AMD_TRACE leaves one record per executed tile instruction, in execution order,
+    with the operands' place, shape and dtype: the single-tile matmul of case 1 is TLOAD, TLOAD, TMOV, TMOV, TMATMUL,
+    TSTORE; the split-K program of case 3 repeats its body five times, with TMATMUL first and TMATMUL_ACC after."""
+    import json
+
+    path = os.path.join(HERE, "pto_kernels", "build", "libptokernels_trace.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: run __graft_entry__.build() (make -C tests/pto_kernels)")
+    lib = ctypes.CDLL(path)
+    lib.pto_kernels_launch.argtypes = [ctypes.c_int] + [ctypes.c_void_p] * 5
+    lib.pto_kernels_launch.restype = ctypes.c_int
+    lib.pto_kernels_status.restype = ctypes.c_int
+    monkeypatch.setenv("PTOAMD_TRACE_DIR", str(tmp_path))
+    r = np.random.default_rng(3)
+    a = r.integers(1, 5, (40, 50)).astype(np.float16)
+    b = r.integers(1, 5, (50, 60)).astype(np.float16)
+    out = run(lib, 1, ((40, 60), torch.float32), a, b)
+    assert np.array_equal(out.cpu().numpy(), a.astype(np.float32) @ b.astype(np.float32))  # the traced build computes the same
+    files = sorted(os.listdir(tmp_path))
+    assert len(files) == 1 and files[0].startswith("ptoamd_instr_trace_") and files[0].endswith(".jsonl")
+    with open(tmp_path / files[0]) as f:
+        recs = [json.loads(line) for line in f]
+    assert [x["opcode"] for x in recs] == ["TLOAD", "TLOAD", "TMOV", "TMOV", "TMATMUL", "TSTORE"]
+    assert [x["sequence_id"] for x in recs] == list(range(6)) and all(x["block_idx"] == 0 for x in recs)
+    assert recs[0]["output_tiles"] == [{"address": 0, "shape": [40, 50], "layout": "Mat", "dtype": "float16"}]
+    assert recs[0]["input_tiles"][0]["layout"] == "ND" and recs[0]["input_tiles"][0]["shape"] == [40, 50]
+    assert recs[1]["output_tiles"][0]["address"] == 0x8000 and recs[1]["output_tiles"][0]["shape"] == [50, 60]
+    assert [t["layout"] for t in recs[4]["output_tiles"] + recs[4]["input_tiles"]] == ["Acc", "Left", "Right"]
+    assert recs[4]["output_tiles"][0] == {"address": 0, "shape": [40, 60], "layout": "Acc", "dtype": "float32"}
+    assert recs[5]["output_tiles"][0]["layout"] == "ND" and recs[5]["output_tiles"][0]["dtype"] == "float32"
+    assert recs[5]["input_tiles"][0]["layout"] == "Acc"
+    # a loop is recorded as executed: five K slabs
+    os.remove(tmp_path / files[0])
+    a5 = r.integers(1, 5, (5 * 128, 128)).astype(np.float16)
+    b5 = r.integers(1, 5, (5 * 128, 64)).astype(np.float16)
+    run(lib, 3, ((128, 64), torch.float32), a5, b5)
+    with open(tmp_path / sorted(os.listdir(tmp_path))[0]) as f:
+        ops = [json.loads(line)["opcode"] for line in f]
+    body = ["TLOAD", "TLOAD", "TMOV", "TMOV"]
+    assert ops == body + ["TMATMUL"] + (body + ["TMATMUL_ACC"]) * 4 + ["TSTORE"]

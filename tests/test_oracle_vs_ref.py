@@ -338,3 +338,34 @@ def test_scalar_quant_helpers(oracle, reflib):
             a = reflib.lib.ref_extract_m1(word, vm)
             b = oracle.lib.pto_quant_word_scale(word, vm)
             assert (np.isnan(a) and np.isnan(b)) or a == b, (word, vm)
+
+
+def test_hif8_decode_all_codes(oracle, reflib):
+    """HiFloat8: all 256 codes, the oracle's arithmetic decode against the compiled reference's table (cpu/Hifloat8.hpp)."""
+    want, got = reflib.hif8_table(), oracle.hif8_table()
+    assert np.array_equal(np.isnan(want), np.isnan(got))
+    assert np.array_equal(np.nan_to_num(want, nan=0.0).view(np.uint64), np.nan_to_num(got, nan=0.0).view(np.uint64))
+    assert np.array_equal(np.signbit(want), np.signbit(got))
+    assert np.array_equal(want[~np.isnan(want)].astype(np.float32).astype(np.float64), want[~np.isnan(want)])  # exact in f32
+
+
+@pytest.mark.parametrize("per_col", [0, 1])
+@pytest.mark.parametrize("relu", [False, True])
+def test_store_quant_saturate_inf(oracle, reflib, per_col, relu):
+    """The fix-pipe's saturation control (task cookie bit 48, cpu/common.hpp:146,157-164) on non-finite and overflowing
+    products of a float accumulator, half target: off, they pass through; on, NaN becomes 0 and the rest is clamped."""
+    r = _rng(31 + per_col)
+    m, n = 16, 24
+    acc = (r.standard_normal((m, n)) * 3000).astype(np.float32)
+    acc[0, :4] = [np.inf, -np.inf, np.nan, 1e30]
+    acc[3, 5:9] = [-1e30, 7e4, -7e4, np.nan]
+    acc.ravel()[11::17] = np.inf
+    mk = _word_vector if per_col else _word_scalar
+    words = np.array([mk(r.uniform(0.5, 40.0)) for _ in range(n)], np.uint64)
+    for sat in (0, 1):
+        want = reflib.store_quant(acc, "f16", words, per_col, relu, saturate_inf=sat)
+        got = oracle.store_quant(acc, ob.ST_F16, words, per_col, relu, saturate_inf=sat)
+        both_nan = ((want & 0x7FFF) > 0x7C00) & ((got & 0x7FFF) > 0x7C00)
+        assert np.array_equal(np.where(both_nan, 0, want), np.where(both_nan, 0, got)), sat
+    assert not np.array_equal(reflib.store_quant(acc, "f16", words, per_col, relu, saturate_inf=0),
+                              reflib.store_quant(acc, "f16", words, per_col, relu, saturate_inf=1))
