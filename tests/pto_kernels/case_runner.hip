@@ -4,6 +4,12 @@
 // comparison with the semantics of the reference's ResultCmp (tests/common/test_common.h:231-309).
 //
 //   case_runner <case>      exit status 0 = match, 1 = mismatch, 2 = usage / runtime error
+//   case_runner --data <dir> --manifest <file> [-l] [-t <suite>[.<case>]]...
+//                           the reference's own case lists (tmatmul, tmatmul_mx, tstore_acc2gm, tdequant), inputs and
+//                           goldens read from <dir>/<suite>/<case>/*.bin, one manifest line per case (written by
+//                           tests/golden/gen_runner_cases.py); -l lists the cases, -t selects a suite or one case (the
+//                           habit of tests/run_cpu.py -t), no -t runs them all.  Every case runs through the C ABI; a
+//                           case whose manifest line names a compiled PTO kernel (k<id>) runs through that as well.
 //
 // Cases:
 //   tmatmul       PTO kernel RunTMATMUL (header layer): f16 40x50x60 -> f32, inputs randint(1, 5)          [tmatmul case1]
@@ -283,8 +289,256 @@ static bool case_quant_gemm(void* stream)
     return ResultCmp(golden, out.data(), 0.001f);
 }
 
+// ---- data-driven cases ------------------------------------------------------------------------------------------------------
+#include <fstream>
+#include <sstream>
+
+struct CaseLine {
+    std::string suite, name, op, at, bt, ct, extra, pto;
+    int m, k, n;
+    float eps;
+};
+
+static int type_code(const std::string& t)
+{
+    static const char* names[] = {"f32", "f16", "bf16", "i32", "i8", "u8", "e4m3", "e5m2", "e2m1", "e1m2", "i16"};
+    for (int i = 0; i < 11; ++i)
+        if (t == names[i])
+            return i;
+    fprintf(stderr, "unknown type %s\n", t.c_str());
+    exit(2);
+}
+static size_t type_bits(int t) { return (t == PTOAMD_F32 || t == PTOAMD_I32) ? 32 : ((t == PTOAMD_F16 || t == PTOAMD_BF16 || t == PTOAMD_I16) ? 16 : ((t == PTOAMD_E2M1 || t == PTOAMD_E1M2) ? 4 : 8)); }
+
+static std::vector<uint8_t> read_bin(const std::string& dir, const CaseLine& c, const char* name, size_t expect_bytes)
+{
+    const std::string path = dir + "/" + c.suite + "/" + c.name + "/" + name + ".bin";
+    std::ifstream f(path, std::ios::binary);
+    if (!f) {
+        fprintf(stderr, "cannot read %s\n", path.c_str());
+        exit(2);
+    }
+    std::vector<uint8_t> v((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    if (expect_bytes != 0 && v.size() != expect_bytes) {
+        fprintf(stderr, "%s holds %zu bytes, the case needs %zu\n", path.c_str(), v.size(), expect_bytes);
+        exit(2);
+    }
+    return v;
+}
+
+static float half_value(uint16_t b)
+{
+    _Float16 h;
+    memcpy(&h, &b, 2);
+    return (float)h;
+}
+static float bf16_value(uint16_t b)
+{
+    const uint32_t w = (uint32_t)b << 16;
+    float f;
+    memcpy(&f, &w, 4);
+    return f;
+}
+// rows x cols elements of type t starting at p (row pitch ld elements) as floats
+static std::vector<float> as_floats(const uint8_t* p, int t, int rows, int cols, int ld)
+{
+    std::vector<float> v((size_t)rows * cols);
+    for (int r = 0; r < rows; ++r)
+        for (int c = 0; c < cols; ++c) {
+            const size_t i = (size_t)r * ld + c;
+            float x;
+            switch (t) {
+                case PTOAMD_F32: x = reinterpret_cast<const float*>(p)[i]; break;
+                case PTOAMD_I32: x = (float)reinterpret_cast<const int32_t*>(p)[i]; break;
+                case PTOAMD_F16: x = half_value(reinterpret_cast<const uint16_t*>(p)[i]); break;
+                case PTOAMD_BF16: x = bf16_value(reinterpret_cast<const uint16_t*>(p)[i]); break;
+                case PTOAMD_I16: x = (float)reinterpret_cast<const int16_t*>(p)[i]; break;
+                case PTOAMD_U8: x = (float)p[i]; break;
+                default: x = (float)reinterpret_cast<const int8_t*>(p)[i]; break;
+            }
+            v[(size_t)r * cols + c] = x;
+        }
+    return v;
+}
+
+static bool check(const CaseLine& c, const char* backend, const DeviceBuffer& out, int ct, int rows, int cols, int ld,
+                  const std::vector<uint8_t>& golden)
+{
+    const auto raw = out.download<uint8_t>((size_t)rows * ld * type_bits(ct) / 8);
+    const auto got = as_floats(raw.data(), ct, rows, cols, ld);
+    const auto want = as_floats(golden.data(), ct, rows, cols, cols);
+    printf("%s.%s [%s] ", c.suite.c_str(), c.name.c_str(), backend);
+    return ResultCmp(want, got.data(), c.eps);
+}
+
+static bool run_data_case(const std::string& dir, const CaseLine& c, void* stream)
+{
+    const int at = type_code(c.at), bt = type_code(c.bt), ct = type_code(c.ct);
+    const int m = c.m, k = c.k, n = c.n;
+    bool ok = true;
+    if (c.op == "gemm" || c.op == "gemm_bias" || c.op == "gemm_splitk" || c.op == "store" || c.op == "store_q") {
+        const int repeats = c.op == "gemm_splitk" ? atoi(c.extra.c_str()) : 1;
+        const auto a = read_bin(dir, c, "x1_gm", (size_t)repeats * m * k * type_bits(at) / 8);
+        const auto b = read_bin(dir, c, "x2_gm", (size_t)repeats * k * n * type_bits(bt) / 8);
+        const auto golden = read_bin(dir, c, "golden", (size_t)m * n * type_bits(ct) / 8);
+        DeviceBuffer da(a.data(), a.size()), db(b.data(), b.size()), dc((size_t)m * n * 4), dc2((size_t)m * n * 4);
+        const size_t abytes = (size_t)m * k * type_bits(at) / 8, bbytes = (size_t)k * n * type_bits(bt) / 8;
+        const DeviceBuffer* result = &dc;
+        if (c.op == "gemm") {
+            RT(ptoamd_gemm(dc.dev, ct, da.dev, db.dev, at, nullptr, m, n, k, k, n, n, PTOAMD_B_ND, 0, stream));
+        } else if (c.op == "gemm_bias") {
+            const auto bias = read_bin(dir, c, "bias_gm", (size_t)n * 4);
+            DeviceBuffer dbias(bias.data(), bias.size());
+            RT(ptoamd_gemm_bias(dc.dev, ct, da.dev, db.dev, at, nullptr, dbias.dev, m, n, k, k, n, n, PTOAMD_B_ND, 0, stream));
+            RT(aclrtSynchronizeStream(stream));
+        } else if (c.op == "gemm_splitk") {  // TMATMUL for the first K slab, TMATMUL_ACC for the others
+            for (int r = 0; r < repeats; ++r) {
+                const DeviceBuffer& dst = (r & 1) ? dc2 : dc;
+                const DeviceBuffer& src = (r & 1) ? dc : dc2;
+                RT(ptoamd_gemm(dst.dev, ct, (uint8_t*)da.dev + r * abytes, (uint8_t*)db.dev + r * bbytes, at, r ? src.dev : nullptr, m, n, k, k, n,
+                               n, PTOAMD_B_ND, 0, stream));
+                result = &dst;
+            }
+        } else if (c.op == "store") {
+            RT(ptoamd_gemm(dc.dev, ct, da.dev, db.dev, at, nullptr, m, n, k, k, n, n, PTOAMD_B_ND, atoi(c.extra.c_str()), stream));
+        } else {
+            uint64_t word = 0;
+            int relu = 0;
+            sscanf(c.extra.c_str(), "%llu:%d", (unsigned long long*)&word, &relu);
+            DeviceBuffer dw(&word, 8);
+            RT(ptoamd_gemm_requant(dc.dev, ct, da.dev, db.dev, at, nullptr, nullptr, (const uint64_t*)dw.dev, 0, m, n, k, k, n, n, PTOAMD_B_ND,
+                                   relu, stream));
+            RT(aclrtSynchronizeStream(stream));
+        }
+        RT(aclrtSynchronizeStream(stream));
+        ok = check(c, ptoamd_last_kernel(), *result, ct, m, n, n, golden) && ok;
+        if (c.pto.size() > 1 && c.pto[0] == 'k') {  // the same case as a kernel written in the tile ISA
+            DeviceBuffer dp((size_t)m * n * 4);
+            std::vector<uint8_t> bias;
+            if (c.op == "gemm_bias")
+                bias = read_bin(dir, c, "bias_gm", (size_t)n * 4);
+            DeviceBuffer dbias(bias.empty() ? a.data() : bias.data(), bias.empty() ? 16 : bias.size());
+            RT(pto_kernels_launch(atoi(c.pto.c_str() + 1), dp.dev, da.dev, db.dev, bias.empty() ? nullptr : dbias.dev, stream));
+            RT(aclrtSynchronizeStream(stream));
+            ok = pto_kernels_status() == 0 && check(c, "pto kernel", dp, ct, m, n, n, golden) && ok;
+        }
+    } else if (c.op == "mx" || c.op == "mx_bias") {
+        int vm = 0, vk = 0, vn = 0;
+        char fa[8] = "", fb[8] = "";
+        sscanf(c.extra.c_str(), "%d:%d:%d:%7[^:]:%7s", &vm, &vk, &vn, fa, fb);
+        const size_t kg = (size_t)k / 32;
+        const auto a = read_bin(dir, c, "x1_gm", (size_t)m * k * type_bits(at) / 8);
+        const auto b = read_bin(dir, c, "x2_gm", (size_t)n * k * type_bits(bt) / 8);
+        const auto sa = read_bin(dir, c, "x1_mx_gm", (size_t)m * kg), sb = read_bin(dir, c, "x2_mx_gm", (size_t)n * kg);
+        const auto golden = read_bin(dir, c, "golden", (size_t)vm * vn * 4);
+        DeviceBuffer da(a.data(), a.size()), db(b.data(), b.size()), dsa(sa.data(), sa.size()), dsb(sb.data(), sb.size()), dc((size_t)m * n * 4);
+        const int la = strcmp(fa, "zz") == 0 ? PTOAMD_MX_A_ZZ : PTOAMD_MX_A_ND, lb = strcmp(fb, "nn") == 0 ? PTOAMD_MX_B_NN : PTOAMD_MX_B_DN;
+        if (c.op == "mx") {
+            RT(ptoamd_gemm_mx(dc.dev, PTOAMD_F32, da.dev, db.dev, at, bt, (const uint8_t*)dsa.dev, (const uint8_t*)dsb.dev, la, lb, nullptr, m, n, k,
+                              k, k, n, PTOAMD_B_DN, stream));
+            RT(aclrtSynchronizeStream(stream));
+        } else {
+            const auto bias = read_bin(dir, c, "bias_gm", (size_t)n * 4);
+            DeviceBuffer dbias(bias.data(), bias.size());
+            RT(ptoamd_gemm_mx_bias(dc.dev, PTOAMD_F32, da.dev, db.dev, at, bt, (const uint8_t*)dsa.dev, (const uint8_t*)dsb.dev, la, lb, nullptr,
+                                   (const float*)dbias.dev, m, n, k, k, k, n, PTOAMD_B_DN, stream));
+            RT(aclrtSynchronizeStream(stream));
+        }
+        ok = check(c, ptoamd_last_kernel(), dc, PTOAMD_F32, vm, vn, n, golden);
+    } else if (c.op == "dequant") {
+        const auto src = read_bin(dir, c, "x1_gm", (size_t)m * n * type_bits(at) / 8);
+        const auto scale = read_bin(dir, c, "x2_gm", (size_t)m * 4), off = read_bin(dir, c, "bias_gm", (size_t)m * 4);
+        const auto golden = read_bin(dir, c, "golden", (size_t)m * n * 4);
+        DeviceBuffer ds(src.data(), src.size()), dsc(scale.data(), scale.size()), dof(off.data(), off.size()), dc((size_t)m * n * 4);
+        RT(ptoamd_tdequant((float*)dc.dev, ds.dev, at, (const float*)dsc.dev, (const float*)dof.dev, m, n, stream));
+        RT(aclrtSynchronizeStream(stream));
+        ok = check(c, ptoamd_last_kernel(), dc, PTOAMD_F32, m, n, n, golden);
+    } else {
+        fprintf(stderr, "unknown op %s\n", c.op.c_str());
+        exit(2);
+    }
+    printf("%s.%s: %s\n", c.suite.c_str(), c.name.c_str(), ok ? "PASS" : "FAIL");
+    return ok;
+}
+
+static int run_data_cases(int argc, char** argv)
+{
+    std::string dir, manifest;
+    std::vector<std::string> select;
+    bool list = false;
+    for (int i = 1; i < argc; ++i) {
+        const std::string a = argv[i];
+        if (a == "--data" && i + 1 < argc)
+            dir = argv[++i];
+        else if (a == "--manifest" && i + 1 < argc)
+            manifest = argv[++i];
+        else if (a == "-t" && i + 1 < argc)
+            select.push_back(argv[++i]);
+        else if (a == "-l")
+            list = true;
+        else {
+            fprintf(stderr, "usage: case_runner --data <dir> --manifest <file> [-l] [-t <suite>[.<case>]]...\n");
+            return 2;
+        }
+    }
+    std::ifstream mf(manifest);
+    if (!mf) {
+        fprintf(stderr, "cannot read the manifest %s\n", manifest.c_str());
+        return 2;
+    }
+    std::vector<CaseLine> cases;
+    for (std::string text; std::getline(mf, text);) {
+        if (text.empty() || text[0] == '#')
+            continue;
+        std::istringstream in(text);
+        CaseLine c;
+        in >> c.suite >> c.name >> c.op >> c.m >> c.k >> c.n >> c.at >> c.bt >> c.ct >> c.extra >> c.eps >> c.pto;
+        if (!in) {
+            fprintf(stderr, "bad manifest line: %s\n", text.c_str());
+            return 2;
+        }
+        cases.push_back(c);
+    }
+    auto wanted = [&](const CaseLine& c) {
+        if (select.empty())
+            return true;
+        for (const auto& s : select)
+            if (s == c.suite || s == c.suite + "." + c.name)
+                return true;
+        return false;
+    };
+    if (list) {
+        for (const auto& c : cases)
+            if (wanted(c))
+                printf("%s.%s\n", c.suite.c_str(), c.name.c_str());
+        return 0;
+    }
+    aclInit(nullptr);
+    RT(aclrtSetDevice(0));
+    aclrtStream stream;
+    RT(aclrtCreateStream(&stream));
+    int ran = 0, failed = 0;
+    for (const auto& c : cases)
+        if (wanted(c)) {
+            ++ran;
+            failed += run_data_case(dir, c, stream) ? 0 : 1;
+        }
+    aclrtDestroyStream(stream);
+    aclrtResetDevice(0);
+    aclFinalize();
+    printf("%d cases run, %d failed\n", ran, failed);
+    if (ran == 0) {
+        fprintf(stderr, "no case matches the selection\n");
+        return 2;
+    }
+    return failed ? 1 : 0;
+}
+
 int main(int argc, char** argv)
 {
+    if (argc > 1 && (strcmp(argv[1], "--data") == 0 || strcmp(argv[1], "--manifest") == 0 || strcmp(argv[1], "-l") == 0 ||
+                     strcmp(argv[1], "-t") == 0))
+        return run_data_cases(argc, argv);
     if (argc != 2) {
         fprintf(stderr, "usage: case_runner tmatmul|tmatmul_i8|tmatmul_mx|gemm|gemm_mx|quant_gemm\n");
         return 2;

@@ -465,3 +465,45 @@ def test_instruction_trace_of_a_pto_kernel(tmp_path, monkeypatch):
         ops = [json.loads(line)["opcode"] for line in f]
     body = ["TLOAD", "TLOAD", "TMOV", "TMOV"]
     assert ops == body + ["TMATMUL"] + (body + ["TMATMUL_ACC"]) * 4 + ["TSTORE"]
+
+
+def _expand_runner_cases(tmp_path):
+    """tests/golden/runner_cases.npz -> <tmp>/<suite>/<case>/<name>.bin, the files the runner reads."""
+    data = np.load(os.path.join(HERE, "golden", "runner_cases.npz"), allow_pickle=False)
+    for key in data.files:
+        suite, case, name = key.split("/")
+        os.makedirs(tmp_path / suite / case, exist_ok=True)
+        data[key].tofile(tmp_path / suite / case / f"{name}.bin")
+    return os.path.join(HERE, "golden", "runner_cases.txt")
+
+
+def test_case_runner_reference_case_lists(tmp_path):
+    """The framework-free runner over the reference's own case lists (tmatmul case1-4 / gemm / bias, tmatmul_mx case1-19,
+    tstore_acc2gm, tdequant): inputs and goldens come from files (goldens made by the oracle), every case runs through the
+    C ABI, those with a compiled PTO kernel through that too, and the comparison is the reference's ResultCmp.  -l lists,
+    -t selects a suite or a case, an unknown selection is exit status 2."""
+    if not os.path.exists(RUNNER):
+        raise RuntimeError(f"{RUNNER} is missing: run __graft_entry__.build()")
+    manifest = _expand_runner_cases(tmp_path)
+    base = [RUNNER, "--data", str(tmp_path), "--manifest", manifest]
+    listed = subprocess.run(base + ["-l"], capture_output=True, text=True, timeout=60)
+    names = listed.stdout.split()
+    assert listed.returncode == 0 and len(names) == 50
+    assert {"tmatmul.case1", "tmatmul.case_bias_5", "tmatmul_mx.case19", "tstore_acc2gm.case_relu_21", "tdequant.case2"} <= set(names)
+    res = subprocess.run(base, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stdout[-4000:] + res.stderr[-2000:]
+    assert "50 cases run, 0 failed" in res.stdout
+    for name in names:
+        assert f"{name}: PASS" in res.stdout, name
+    assert res.stdout.count("[pto kernel]") == 6  # tmatmul case1, 2, 3, gemm_1, bf16_1, bias_1 also ran as tile-ISA kernels
+    one = subprocess.run(base + ["-t", "tmatmul_mx.case2"], capture_output=True, text=True, timeout=60)
+    assert one.returncode == 0 and "1 cases run, 0 failed" in one.stdout
+    suite = subprocess.run(base + ["-t", "tdequant"], capture_output=True, text=True, timeout=60)
+    assert suite.returncode == 0 and "2 cases run, 0 failed" in suite.stdout
+    assert subprocess.run(base + ["-t", "no_such_suite"], capture_output=True, timeout=60).returncode == 2
+    # a wrong golden is a failure, not a pass: flip one case's golden and run it alone
+    path = tmp_path / "tmatmul" / "case1" / "golden.bin"
+    g = np.fromfile(path, np.float32)
+    (g + 1.0).astype(np.float32).tofile(path)
+    bad = subprocess.run(base + ["-t", "tmatmul.case1"], capture_output=True, text=True, timeout=60)
+    assert bad.returncode == 1 and "tmatmul.case1: FAIL" in bad.stdout
