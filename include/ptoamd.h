@@ -76,7 +76,11 @@ enum { PTOAMD_MEMCPY_H2H = 0, PTOAMD_MEMCPY_H2D = 1, PTOAMD_MEMCPY_D2H = 2, PTOA
 /* =========================================================================================================
  * 1. Host runtime  (replaces the fake aclrt* runtime, include/pto/common/cpu_stub.hpp:73-120, 524-555)
  * ========================================================================================================= */
-int ptoamd_init(int device);                    /* aclInit + aclrtSetDevice: selects the device, checks it is gfx950 */
+/* aclInit + aclrtSetDevice: selects the device and checks it is gfx950.  It also does, for that device, everything a
+ * first launch would otherwise do lazily (launch attributes of every kernel, the device address of the static scratch
+ * array): after ptoamd_init(device) the entry points below issue kernel launches and nothing else, which is what a
+ * caller that captures them into a HIP graph needs.  Without it the first call per kernel and device sets up lazily. */
+int ptoamd_init(int device);
 int ptoamd_finalize(void);                      /* aclrtResetDevice + aclFinalize */
 /* The dispatchers' environment switches (PTOAMD_TILE, PTOAMD_NO_TAIL_SPLIT, PTOAMD_FORCE_GENERIC,
  * PTOAMD_B_ND_TRANSPOSE, PTOAMD_GEMV_*) are read once per process; this reads them again.  No counterpart in the

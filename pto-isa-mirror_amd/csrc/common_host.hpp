@@ -13,6 +13,12 @@ void set_last_kernel(const char* name);
 // sets hipFuncAttributeMaxDynamicSharedMemorySize once per (kernel, current device); thread-safe
 hipError_t ensure_dynamic_lds(const void* kernel, int bytes);
 
+// Everything a first launch would otherwise set up lazily, done for the current device: the dynamic-LDS attribute of
+// every tile and GEMV kernel and the device address of the library's static scratch array.  After it, no entry point
+// calls anything but kernel launches (a requirement of callers that capture launches into a HIP graph).
+int prepare_gemm_kernels();
+int prepare_gemv_kernels();
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 // The environment switches of the dispatchers, read once per process (and again by ptoamd_reload_options): a launch

@@ -402,6 +402,14 @@ static int static_scratch(uint8_t** ptr)
     return PTOAMD_OK;
 }
 
+int prepare_gemm_kernels()
+{
+    for (int op : {TOP_BF16, TOP_F16, TOP_I8, TOP_FP8_E4E4, TOP_FP8_E5E5, TOP_FP8_E4E5, TOP_FP8_E5E4, TOP_FP4})
+        PTOAMD_HIP_CHECK(launch_gemm_tile(TILE_PREPARE_ALL, op, TileGemmParams{}, nullptr));
+    uint8_t* unused = nullptr;
+    return static_scratch(&unused);
+}
+
 }  // namespace ptoamd
 
 using namespace ptoamd;

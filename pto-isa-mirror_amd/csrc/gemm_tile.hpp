@@ -17,6 +17,9 @@
 
 namespace ptoamd {
 
+// tile id that asks a launcher to give all its kernels their launch attributes on the current device and launch nothing
+constexpr int TILE_PREPARE_ALL = -1000;
+
 struct TileGemmParams {
     const uint8_t* a;       // [m][lda_bytes]
     const uint8_t* b;       // [n][ldb_bytes]

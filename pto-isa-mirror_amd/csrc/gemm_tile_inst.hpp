@@ -10,7 +10,7 @@ template <class Cfg>
 static hipError_t launch_cfg(const TileGemmParams& p, hipStream_t stream)
 {
     const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_kernel<Cfg>), Cfg::LDS_BYTES);
-    if (e != hipSuccess)
+    if (e != hipSuccess || p.m <= 0)  // m = 0: only make the kernel ready to launch on the current device
         return e;
     const int tiles = ((p.m + Cfg::BM - 1) / Cfg::BM) * ((p.n + Cfg::BN - 1) / Cfg::BN);
     hipLaunchKernelGGL(gemm_tile_kernel<Cfg>, dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
@@ -21,7 +21,7 @@ template <class Cfg>
 static hipError_t launch_dtl(const TileGemmParams& p, hipStream_t stream)
 {
     const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_dtl_kernel<Cfg>), Cfg::LDS_BYTES);
-    if (e != hipSuccess)
+    if (e != hipSuccess || p.m <= 0)
         return e;
     const int tiles = ((p.m + Cfg::BM - 1) / Cfg::BM) * ((p.n + Cfg::BN - 1) / Cfg::BN);
     hipLaunchKernelGGL(gemm_tile_dtl_kernel<Cfg>, dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
@@ -30,6 +30,15 @@ static hipError_t launch_dtl(const TileGemmParams& p, hipStream_t stream)
 
 hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 {
+    if (tile == TILE_PREPARE_ALL) {  // every kernel of this unit gets its launch attributes on the current device
+        TileGemmParams none{};
+        for (int t : {4, 5, 6, 1, 2}) {
+            const hipError_t e = PTOAMD_TILE_FN(t, none, stream);
+            if (e != hipSuccess)
+                return e;
+        }
+        return hipSuccess;
+    }
     switch (tile) {
         // (tile id 3 was a four-wave form of the 256 x 256 tile, 128 x 128 per wave: never faster than the eight-wave form
         // and a third of this translation unit's compile time; the id now selects tile 4)

@@ -349,7 +349,12 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
 }
 
 // ---- split-K kernel with loader waves (k % 2048 == 0) ----------------------------------------------------------
-// Same arithmetic and k-assignment as the split-K kernel above.  Two things hold that kernel back: its 512-byte row
+// Same products and the same partition of K into 512-wide slices as the split-K kernel above; the ORDER in which a
+// workgroup adds its chunks is rotated (see K below), so the fp32 sums agree with that kernel's to rounding (1e-5
+// relative in the tests), not bit for bit.  The order is a function of blockIdx.x and of the grid, which follows the
+// device's compute-unit count: results are deterministic on one device and launch shape, and not reproducible bit for
+// bit across devices with different CU counts.  A caller that needs one order everywhere sets PTOAMD_GEMV_NO_WIDE=1
+// (the split-K kernel above: its order of additions depends on k alone).  Two things hold that kernel back: its 512-byte row
 // pieces (an LDS-DMA that covers 1 KiB of one row streams about a fifth faster, non-temporal another 13 %: a weight byte
 // is read once and stays out of the memory-side cache), and that a wave which both computes and issues its own DMAs
 // sits in the issue whenever the CU's memory queue is full, its matrix pipe idle, while the queue runs dry during its
@@ -597,6 +602,15 @@ __global__ void gemv_mxfp4_generic_kernel(const GemvParams p)
         reinterpret_cast<uint16_t*>(p.out)[(long)gi * p.ldc + gj] = f32_to_bf16_bits(acc);
     else
         reinterpret_cast<float*>(p.out)[(long)gi * p.ldc + gj] = acc;
+}
+
+int prepare_gemv_kernels()
+{
+    PTOAMD_HIP_CHECK(ensure_dynamic_lds(reinterpret_cast<const void*>(gemv_mxfp4_splitk_wide_kernel<false>), WD_LDS));
+    PTOAMD_HIP_CHECK(ensure_dynamic_lds(reinterpret_cast<const void*>(gemv_mxfp4_splitk_wide_kernel<true>), WD_LDS));
+    PTOAMD_HIP_CHECK(ensure_dynamic_lds(reinterpret_cast<const void*>(gemv_mxfp4_splitk_kernel<false>), SK_LDS));
+    PTOAMD_HIP_CHECK(ensure_dynamic_lds(reinterpret_cast<const void*>(gemv_mxfp4_splitk_kernel<true>), SK_LDS));
+    return PTOAMD_OK;
 }
 
 }  // namespace ptoamd

@@ -232,7 +232,10 @@ int ptoamd_init(int device)
     }
     (void)options();
     (void)device_compute_units();
-    return PTOAMD_OK;
+    int rc = prepare_gemm_kernels();
+    if (rc == PTOAMD_OK)
+        rc = prepare_gemv_kernels();
+    return rc;
 }
 
 int ptoamd_reload_options(void)

@@ -24,6 +24,11 @@ namespace amd {
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef int i32x4v __attribute__((ext_vector_type(4)));
+// staging accesses: one wave writes its band as register quads and reads it back as 16-byte row chunks with no workgroup
+// barrier in between, so the two access types must be allowed to alias and the compiler may not move one across the other
+typedef int i32x4s __attribute__((ext_vector_type(4), may_alias));
+typedef int i32x2s __attribute__((ext_vector_type(2), may_alias));
+typedef int i32x2v_plain __attribute__((ext_vector_type(2)));
 
 template <typename D, typename S>
 PTO_INST D convert(S v)
@@ -573,6 +578,15 @@ struct alignas(4 * sizeof(G)) Quad {
     G v[4];
 };
 
+template <typename G>
+PTO_INST void stage_quad(uint8_t* at, const Quad<G>& q)
+{
+    if constexpr (sizeof(G) == 2)
+        *reinterpret_cast<i32x2s*>(at) = __builtin_bit_cast(i32x2v_plain, q);
+    else
+        *reinterpret_cast<i32x4s*>(at) = __builtin_bit_cast(i32x4v, q);
+}
+
 template <typename TileRes, typename GlobalData, AtomicType atomic, ReluPreMode relu>
 PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
 {
@@ -592,6 +606,53 @@ PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
             // and leaves as whole rows (64 or 128 contiguous bytes per row and store instruction).  The band is private
             // to the wave, so no workgroup barrier is involved.
             constexpr int row_bytes = 32 * (int)sizeof(G), pitch = row_bytes + 16, band = 32 * pitch;
+            // 16-bit outputs, two blocks side by side in one wave: the pair is staged 16 rows at a time, so that a row
+            // leaves as 128 contiguous bytes (a whole cache line per row, where 64-byte halves from two instructions
+            // cost extra write traffic).  Same band size or less: 16 rows of 128 + 16 bytes.
+            constexpr bool pair = sizeof(G) == 2 && TileRes::BLOCKED && TileRes::NB % 2 == 0;
+            constexpr int pair_pitch = 128 + 16, pair_band = 16 * pair_pitch;
+            if constexpr (pair && TileRes::Rows % 32 == 0 && TileRes::Cols % 32 == 0 &&
+                          (uint32_t)(WAVES * pair_band) <= (uint32_t)PTO_AMD_STAGE_BYTES) {
+                if (vr == TileRes::Rows && vc == TileRes::Cols && ((ld * (int64_t)sizeof(G)) & 15) == 0 &&
+                    (reinterpret_cast<uintptr_t>(g) & 15u) == 0) {
+                    uint8_t* stage = lds_arena() + STAGE_BASE + wave * pair_band;
+#pragma unroll
+                    for (int slot = 0; slot < TileRes::NBLK; slot += 2) {
+                        int bi, bj;
+                        TileRes::block_of(slot, wave, bi, bj);
+#pragma unroll
+                        for (int half = 0; half < 2; ++half) {
+                            if ((l32 >> 4) == half) {
+#pragma unroll
+                                for (int blk = 0; blk < 2; ++blk) {
+#pragma unroll
+                                    for (int q = 0; q < 4; ++q) {
+                                        Quad<G> out;
+#pragma unroll
+                                        for (int e = 0; e < 4; ++e) {
+                                            auto v = src.regs[slot + blk][4 * q + e];
+                                            if constexpr (relu == ReluPreMode::NormalRelu)
+                                                v = v > 0 ? v : 0;
+                                            out.v[e] = convert<G>(v);
+                                        }
+                                        stage_quad(stage + (l32 & 15) * pair_pitch + blk * 64 + (8 * q + 4 * lhi) * 2, out);
+                                    }
+                                }
+                            }
+                            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                            for (int pass = 0; pass < 2; ++pass) {
+                                const int idx = lane + 64 * pass, r = idx >> 3, chunk = idx & 7;
+                                const i32x4v v = *reinterpret_cast<const i32x4s*>(stage + r * pair_pitch + chunk * 16);
+                                uint8_t* gp = reinterpret_cast<uint8_t*>(g + (int64_t)(bi * 32 + half * 16 + r) * ld + bj * 32) + chunk * 16;
+                                __builtin_nontemporal_store(v, reinterpret_cast<i32x4v*>(gp));
+                            }
+                            __builtin_amdgcn_wave_barrier();
+                        }
+                    }
+                    return;
+                }
+            }
             if constexpr (TileRes::Rows % 32 == 0 && TileRes::Cols % 32 == 0 && (uint32_t)(WAVES * band) <= (uint32_t)PTO_AMD_STAGE_BYTES) {
                 if (vr == TileRes::Rows && vc == TileRes::Cols && ((ld * (int64_t)sizeof(G)) & 15) == 0 &&
                     (reinterpret_cast<uintptr_t>(g) & 15u) == 0) {
@@ -612,15 +673,17 @@ PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
                                     v = v > 0 ? v : 0;
                                 out.v[e] = convert<G>(v);
                             }
-                            *reinterpret_cast<Quad<G>*>(stage + l32 * pitch + (8 * q + 4 * lhi) * (int)sizeof(G)) = out;
+                            stage_quad(stage + l32 * pitch + (8 * q + 4 * lhi) * (int)sizeof(G), out);
                         }
+                        __builtin_amdgcn_wave_barrier();
 #pragma unroll
                         for (int pass = 0; pass < 32 / rows_per_pass; ++pass) {
                             const int r = pass * rows_per_pass + rrow;
-                            const i32x4v v = *reinterpret_cast<const i32x4v*>(stage + r * pitch + rchunk * 16);
+                            const i32x4v v = *reinterpret_cast<const i32x4s*>(stage + r * pitch + rchunk * 16);
                             uint8_t* gp = reinterpret_cast<uint8_t*>(g + (int64_t)(bi * 32 + r) * ld + bj * 32) + rchunk * 16;
                             __builtin_nontemporal_store(v, reinterpret_cast<i32x4v*>(gp));
                         }
+                        __builtin_amdgcn_wave_barrier();
                     }
                     return;
                 }
@@ -813,6 +876,41 @@ PTO_INST void tmov_acc(DstTile& dst, SrcTile& src, int row0, int col0, WordOf&& 
     });
     __syncthreads();
 }
+// Into an accumulator tile: dst(r, c) = src(r + row0, c + col0) over dst's valid region, element by element with the
+// reference's implicit conversion (cpu/TMov.hpp:28-33, cpu/TExtract.hpp:21-46; the simulator places no restriction on
+// the destination).  From another accumulator of the same shape the move is register to register; from an on-chip
+// buffer tile every lane fetches the elements of the blocks it holds.  Elements outside the valid region keep their value.
+template <ReluPreMode relu, typename DstTile, typename SrcTile>
+PTO_INST void tmov_into_acc(DstTile& dst, SrcTile& src, int row0, int col0)
+{
+    using Reg = typename DstTile::Reg;
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    if constexpr (SrcTile::Loc == TileType::Acc) {
+        static_assert(DstTile::Rows == SrcTile::Rows && DstTile::Cols == SrcTile::Cols,
+                      "accumulator to accumulator moves keep the tile shape (registers do not change lanes)");
+        for_each_acc(dst, [&](int slot, int r, int row, int col) {
+            if (row < vr && col < vc) {
+                Reg v = static_cast<Reg>(src.regs[slot][r]);
+                if constexpr (relu == ReluPreMode::NormalRelu)
+                    v = v > 0 ? v : 0;
+                dst.regs[slot][r] = v;
+            }
+        });
+    } else {
+        using S = typename SrcTile::DType;
+        acquire(src);
+        __syncthreads();  // writers of the source tile are done
+        const uint8_t* ps = src.Storage();
+        for_each_acc(dst, [&](int slot, int r, int row, int col) {
+            if (row < vr && col < vc) {
+                Reg v = static_cast<Reg>(*reinterpret_cast<const S*>(ps + src.ByteOffset(row + row0, col + col0)));
+                if constexpr (relu == ReluPreMode::NormalRelu)
+                    v = v > 0 ? v : 0;
+                dst.regs[slot][r] = v;
+            }
+        });
+    }
+}
 // relu over the valid region of an LDS tile (TMOV's relu form between buffer tiles, cpu/TMov.hpp:37-54)
 template <typename TileData>
 PTO_INST void trelu_lds(TileData& t)
@@ -835,9 +933,10 @@ template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode, type
           std::enable_if_t<all_events_v<WaitEvents...>, int> = 0>
 PTO_INST RecordEvent TMOV(DstTileData& dst, SrcTileData& src, WaitEvents&...)
 {
-    static_assert(DstTileData::Loc != TileType::Acc, "TMOV into an accumulator tile is not implemented on this backend");
     PTO_AMD_TRACE_INSTR(1, TR_TMOV, dst, src);
-    if constexpr (SrcTileData::Loc == TileType::Acc) {
+    if constexpr (DstTileData::Loc == TileType::Acc) {
+        amd::tmov_into_acc<reluMode>(dst, src, 0, 0);
+    } else if constexpr (SrcTileData::Loc == TileType::Acc) {
         amd::tmov_acc<0, reluMode>(dst, src, 0, 0, [](int) { return (uint64_t)0; });
     } else {
         amd::textract_lds<reluMode == ReluPreMode::NoRelu>(dst, src, 0, 0);
@@ -878,8 +977,11 @@ template <typename DstTileData, typename SrcTileData, ReluPreMode reluMode = Rel
 PTO_INST RecordEvent TEXTRACT(DstTileData& dst, SrcTileData& src, uint16_t indexRow = 0, uint16_t indexCol = 0, WaitEvents&...)
 {
     PTO_AMD_TRACE_INSTR(1, TR_TEXTRACT, dst, src);
-    static_assert(DstTileData::Loc != TileType::Acc, "TEXTRACT into an accumulator tile is not implemented on this backend");
-    if constexpr (SrcTileData::Loc == TileType::Acc) {
+    static_assert(DstTileData::Loc != TileType::Acc || SrcTileData::Loc != TileType::Acc,
+                  "TEXTRACT between accumulator tiles would move registers across lanes: go through a Vec tile");
+    if constexpr (DstTileData::Loc == TileType::Acc) {
+        amd::tmov_into_acc<reluMode>(dst, src, indexRow, indexCol);
+    } else if constexpr (SrcTileData::Loc == TileType::Acc) {
         amd::tmov_acc<0, reluMode>(dst, src, indexRow, indexCol, [](int) { return (uint64_t)0; });
     } else {
         amd::textract_lds<reluMode == ReluPreMode::NoRelu>(dst, src, indexRow, indexCol);

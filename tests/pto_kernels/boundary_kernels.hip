@@ -290,6 +290,53 @@ __global__ AICORE void RunTSTORE_ATOMIC(__gm__ OutT* out, __gm__ T* a, __gm__ T*
     TSTORE<AccT, GlobalOut, AtomicType::AtomicAdd>(outGlobal, cTile);
 }
 
+// ---- TMOV / TEXTRACT into an accumulator tile ---------------------------------------------------------------------------
+// MODE 0: C0 [M][N] comes in through a Vec tile, TMOV places it in the accumulator, TMATMUL_ACC adds A B onto it.
+// MODE 1: TEXTRACT<NormalRelu> takes the accumulator's start value from offset (8, 16) of a larger [M + 8][N + 16] Vec tile.
+// MODE 2: accumulator to accumulator: C1 = A B, TMOV(C2, C1), C2 += A B.
+template <typename OutT, typename T, int M, int K, int N, int MODE>
+__global__ AICORE void RunTMOV_INTO_ACC(__gm__ OutT* out, __gm__ T* a, __gm__ T* b, __gm__ OutT* c0)
+{
+    GlobalTensor<T, Shape<1, 1, 1, M, K>, Stride<M * K, M * K, M * K, K, 1>> aGlobal(a);
+    GlobalTensor<T, Shape<1, 1, 1, K, N>, Stride<K * N, K * N, K * N, N, 1>> bGlobal(b);
+    GlobalTensor<OutT, Shape<1, 1, 1, M, N>, Stride<M * N, M * N, M * N, N, 1>> outGlobal(out);
+    constexpr int Mp = CeilAlign<int>(M, 16), Kp = CeilAlign<int>(K, sizeof(T) == 1 ? 32 : 16), Np = CeilAlign<int>(N, sizeof(T) == 1 ? 32 : 16);
+    Tile<TileType::Mat, T, Mp, Kp, BLayout::ColMajor, M, K, SLayout::RowMajor, 512> aMat;
+    Tile<TileType::Mat, T, Kp, Np, BLayout::ColMajor, K, N, SLayout::RowMajor, 512> bMat;
+    TASSIGN(aMat, 0x0);
+    TASSIGN(bMat, 0x4000);
+    TileLeft<T, Mp, Kp, M, K> aTile;
+    TileRight<T, Kp, Np, K, N> bTile;
+    TileAcc<OutT, Mp, Np, M, N> cTile, c1Tile;
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(cTile, 0x0);
+    TASSIGN(c1Tile, 0x4000);
+    TLOAD(aMat, aGlobal);
+    TLOAD(bMat, bGlobal);
+    TMOV(aTile, aMat);
+    TMOV(bTile, bMat);
+    if constexpr (MODE == 0) {
+        GlobalTensor<OutT, Shape<1, 1, 1, M, N>, Stride<M * N, M * N, M * N, N, 1>> c0Global(c0);
+        Tile<TileType::Vec, OutT, Mp, Np, BLayout::RowMajor, M, N> c0Tile;
+        TASSIGN(c0Tile, 0x0);
+        TLOAD(c0Tile, c0Global);
+        TMOV(cTile, c0Tile);
+    } else if constexpr (MODE == 1) {
+        constexpr int R = M + 8, C = N + 16, Rp = CeilAlign<int>(R, 16), Cp = CeilAlign<int>(C, 16);
+        GlobalTensor<OutT, Shape<1, 1, 1, R, C>, Stride<R * C, R * C, R * C, C, 1>> c0Global(c0);
+        Tile<TileType::Vec, OutT, Rp, Cp, BLayout::RowMajor, R, C> c0Tile;
+        TASSIGN(c0Tile, 0x0);
+        TLOAD(c0Tile, c0Global);
+        TEXTRACT<decltype(cTile), decltype(c0Tile), ReluPreMode::NormalRelu>(cTile, c0Tile, 8, 16);
+    } else {
+        TMATMUL(c1Tile, aTile, bTile);
+        TMOV(cTile, c1Tile);
+    }
+    TMATMUL_ACC(cTile, aTile, bTile);
+    TSTORE(outGlobal, cTile);
+}
+
 // ---- 5-D global tensors: gather through TLOAD, scatter through TSTORE ----------------------------------------------------
 // ND: Shape<2,3,4,8,16> with padded strides is a 192 x 16 logical matrix; DN: the same shape is 8 x 384.
 // `packed` receives the logical matrix row-major; `scattered` (same 5-D geometry as the source) receives it back.
@@ -526,6 +573,7 @@ extern "C" int pto_boundary_launch_cvt(int id, void* dst, void* src, int mode, i
 //   30 / 31: 5-D global tensor half ND / DN (out = packed, src1 = scattered)     32: float ND
 //   40..44: fix-pipe TMOV / TEXTRACT modes 0..4 on a half 48x64x96 product (src2 = quant words)
 //   45: mode 1 on an int8 48x64x96 product (int32 accumulator -> int8)
+//   46-49: TMOV / TEXTRACT into an accumulator tile (from a Vec tile, with relu at an offset, from another accumulator; int32)
 //   50: TRESHAPE     60: TASSIGN at the address in `arg`     70: TQUANT<MXFP8> of an f32 A, TMOV ND -> NZ, TMATMUL_MX
 extern "C" int pto_boundary_launch(int id, void* out, void* src0, void* src1, void* src2, unsigned arg, void* stream)
 {
@@ -549,6 +597,10 @@ extern "C" int pto_boundary_launch(int id, void* out, void* src0, void* src1, vo
     case 43: return run<&RunTMOV_FIXPIPE<int8_t, float, half, 48, 64, 96, 3>>(stream, 1, (int8_t*)out, (half*)src0, (half*)src1, (uint64_t*)src2);
     case 44: return run<&RunTMOV_FIXPIPE<float, float, half, 48, 64, 96, 4>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (uint64_t*)src2);
     case 45: return run<&RunTMOV_FIXPIPE<int8_t, int32_t, int8_t, 48, 64, 96, 1>>(stream, 1, (int8_t*)out, (int8_t*)src0, (int8_t*)src1, (uint64_t*)src2);
+    case 46: return run<&RunTMOV_INTO_ACC<float, half, 40, 50, 60, 0>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)src2);
+    case 47: return run<&RunTMOV_INTO_ACC<float, half, 40, 50, 60, 1>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)src2);
+    case 48: return run<&RunTMOV_INTO_ACC<float, half, 40, 50, 60, 2>>(stream, 1, (float*)out, (half*)src0, (half*)src1, (float*)src2);
+    case 49: return run<&RunTMOV_INTO_ACC<int32_t, int8_t, 24, 64, 40, 0>>(stream, 1, (int32_t*)out, (int8_t*)src0, (int8_t*)src1, (int32_t*)src2);
     case 50: return run<&RunTRESHAPE>(stream, 1, (float*)out, (float*)src0);
     case 60: return run<&RunTASSIGN_OUT_OF_RANGE>(stream, 1, (float*)out, (float*)src0, (uint32_t)arg);
     case 70: return run<&RunQUANT_TMATMUL_MX<32, 128, 64>>(stream, 1, (float*)out, (float*)src0, (E4*)src1, (float8_e8m0_t*)src2);

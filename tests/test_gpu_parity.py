@@ -947,10 +947,21 @@ def test_mxfp4_gemm_large_takes_the_256_tile(pa, oracle):
     b, sb = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
     out = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E2M1, pa.E2M1, pa.F32)
     assert pa.last_kernel() == "tile256x256w8_dtl_fp4_e2m1"
-    rows, cols = np.array([0, 31, 32, 255, 256, 1027, 2047]), np.arange(0, n, 131)
-    ref = oracle.matmul_mx(host(sel(a, rows)), host(sel(b, cols)), host(sel(sa, rows)), host(sel(sb, cols)), len(rows), k, len(cols),
-                           ob.E2M1, ob.E2M1)
-    assert relerr(host(out)[np.ix_(rows, cols)], ref) <= 2e-2
+    table = oracle.mx_decode_table(ob.E2M1)
+    out_h = host(out)
+
+    def magnitudes(codes, scales):
+        nib = np.stack([codes & 0xF, codes >> 4], -1).reshape(codes.shape[0], -1)
+        return np.abs(table[nib]) * np.repeat(2.0 ** (scales.astype(np.float64) - 127), 32, 1)
+    rows = np.unique(np.concatenate([[0, 31, 32, 255, 256, 1027, 2047], np.arange(5, m, 33)]))[:64]
+    cols = np.arange(0, n, 64) + np.arange(64) % 64
+    # both error bars of an fp32 drain on 64 x 64 sampled outputs and on two whole 256 x 256 tiles
+    for label, rr, cc in (("samples", rows, cols), ("tile (0, 0)", np.arange(256), np.arange(256)),
+                          ("tile (7, 15)", np.arange(m - 256, m), np.arange(n - 256, n))):
+        ar, bc, sar, sbc = host(sel(a, rr)), host(sel(b, cc)), host(sel(sa, rr)), host(sel(sb, cc))
+        ref = oracle.matmul_mx(ar, bc, sar, sbc, len(rr), k, len(cc), ob.E2M1, ob.E2M1)
+        check_f32_drain(out_h[np.ix_(rr, cc)], ref, magnitudes(ar, sar) @ magnitudes(bc, sbc).T, k,
+                        f"MXFP4 2048x4096x2048, {label}")
     with tile_env(PTOAMD_TILE=5):
         other = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E2M1, pa.E2M1, pa.F32)
     assert relerr(host(other), host(out)) <= 1e-5
@@ -1040,9 +1051,16 @@ def test_config5_mxfp4_decode_full_size(pa, oracle):
     w, sw = pa.tquant_mx(xw, pa.OCP_MXFP4, want_aux=False)
     out = pa.gemv_mxfp4(a, w, sw, n, k, pa.F32)
     assert pa.last_kernel() == "gemv_mxfp4_splitk_wide"
-    cols = np.arange(0, n, 97)
-    ref = _gemv_reference(oracle, host(a), host(sel(w, cols)), host(sel(sw, cols)), len(cols), k)
-    assert relerr(host(out)[:, cols], ref) <= 2e-2
+    out_h, a_h = host(out), host(a)
+    table = oracle.mx_decode_table(ob.E2M1)
+    # both error bars of an fp32 drain: every 97th weight row, and two whole strips of 256 weight rows
+    for label, cols in (("samples", np.arange(0, n, 97)), ("first 256 outputs", np.arange(256)), ("last 256 outputs", np.arange(n - 256, n))):
+        wc, swc = host(sel(w, cols)), host(sel(sw, cols))
+        ref = _gemv_reference(oracle, a_h, wc, swc, len(cols), k)
+        nib = np.stack([wc & 0xF, wc >> 4], -1).reshape(len(cols), k)
+        wabs = np.abs(table[nib]) * np.repeat(2.0 ** (swc.astype(np.float64) - 127), 32, 1)
+        check_f32_drain(out_h[:, cols], ref, np.abs(bf16_to_f32(a_h).astype(np.float64)) @ wabs.T, k,
+                        f"configs[4] MXFP4 GEMV 16x28672x8192, {label}")
     # linear in the activations: (2^-3 * A) W = 2^-3 (A W) exactly, and rows do not mix
     out2 = pa.gemv_mxfp4((a.float() * 0.125).to(torch.bfloat16), w, sw, n, k, pa.F32)
     assert torch.equal(out2, out * 0.125)

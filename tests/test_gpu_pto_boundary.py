@@ -455,6 +455,30 @@ def test_tmov_and_textract_fixpipe_forms(lib, oracle):
     assert np.array_equal(got, oracle.store_quant(oracle.matmul_i8(ai, bi), ob.ST_I8, word, per_column=False))
 
 
+def test_tmov_and_textract_into_an_accumulator_tile(lib, oracle):
+    """The start value of an accumulator comes from a Vec tile (TMOV), from an offset of a larger Vec tile with relu
+    (TEXTRACT), or from another accumulator (reference: cpu/TMov.hpp:21-35 moves between any two tile kinds); the
+    product is then added onto it by TMATMUL_ACC, so the result is the oracle's matmul with that start value."""
+    r = np.random.default_rng(46)
+    m, k, n = 40, 50, 60
+    # small integers: every partial sum is exact, so the MFMA's order of additions cannot show
+    a, b = f16_bits(r.integers(-4, 5, (m, k))), f16_bits(r.integers(-4, 5, (k, n)))
+    c0 = r.integers(-100, 100, (m, n)).astype(np.float32)
+    got = launch(lib, 46, torch.zeros((m, n), dtype=torch.float32, device=DEV), dev(a), dev(b), dev(c0)).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), oracle.matmul_f16(a, b, cin=c0).view(np.uint32))
+    big = r.integers(-100, 100, (m + 8, n + 16)).astype(np.float32)
+    got = launch(lib, 47, torch.zeros((m, n), dtype=torch.float32, device=DEV), dev(a), dev(b), dev(big)).cpu().numpy()
+    start = np.maximum(big[8:, 16:], 0).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), oracle.matmul_f16(a, b, cin=np.ascontiguousarray(start)).view(np.uint32))
+    got = launch(lib, 48, torch.zeros((m, n), dtype=torch.float32, device=DEV), dev(a), dev(b), dev(c0)).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), oracle.matmul_f16(a, b, cin=oracle.matmul_f16(a, b)).view(np.uint32))
+    m, k, n = 24, 64, 40
+    ai, bi = r.integers(-128, 128, (m, k)).astype(np.int8), r.integers(-128, 128, (k, n)).astype(np.int8)
+    ci = r.integers(-10 ** 6, 10 ** 6, (m, n)).astype(np.int32)
+    got = launch(lib, 49, torch.zeros((m, n), dtype=torch.int32, device=DEV), dev(ai), dev(bi), dev(ci)).cpu().numpy()
+    assert np.array_equal(got, oracle.matmul_i8(ai, bi, cin=ci))
+
+
 def test_treshape_aliases_the_storage(lib):
     src = np.arange(1024, dtype=np.float32).reshape(16, 64)
     got = launch(lib, 50, torch.zeros((8, 128), dtype=torch.float32, device=DEV), dev(src)).cpu().numpy()

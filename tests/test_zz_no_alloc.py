@@ -46,11 +46,13 @@ def test_static_scratch_entry_matches_the_workspace_entry_twice_in_a_row(pa, ora
     outs = [torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV) for (m, n, _, _) in shapes]
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats(DEV)["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info(DEV)[0]   # the driver's own count: sees a hipMalloc made behind torch's back
     for (m, n, k, typ), (_, (a, b, sa, sb)), out in zip(shapes, cases, outs):   # back to back on one stream
         pa.gemm_mx_static(a, b, sa, sb, m, n, k, typ, typ, out, sa_layout=pa.MX_A_ZZ, sb_layout=pa.MX_B_NN)
         assert pa.last_kernel().startswith("tile"), pa.last_kernel()
     torch.cuda.synchronize()
     assert torch.cuda.memory_stats(DEV)["allocation.all.allocated"] == before   # nothing went through torch's allocator either
+    assert torch.cuda.mem_get_info(DEV)[0] == free_before                        # and the device's free memory did not move
     for (m, n, k, typ), ((a, b, sa, sb), _), out, ref_ws in zip(shapes, cases, outs, want):
         got = out.cpu().numpy()
         assert np.array_equal(got.view(np.uint32), ref_ws.cpu().numpy().view(np.uint32)), (m, n, k)
