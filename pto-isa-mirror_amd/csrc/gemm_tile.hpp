@@ -692,7 +692,9 @@ __device__ __forceinline__ uint4 load_chunk_tail(const uint8_t* g, int rem)
     return make_uint4((uint32_t)rlo, (uint32_t)(rlo >> 32), (uint32_t)rhi, (uint32_t)(rhi >> 32));
 }
 
-template <class Cfg>
+// RAGGED: some row of A or B does not end on a 16-byte chunk boundary (see the loader below).  A compile-time form, so
+// that the kernel for whole chunks carries neither the tail-masking code nor a branch in its K loop.
+template <class Cfg, bool RAGGED>
 __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmParams p)
 {
     using Op = typename Cfg::Op;
@@ -765,8 +767,8 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
 
     uint4 ra[LA], rb[LB];
     // Rows need no alignment: a chunk is read with a 16-byte load at whatever address it starts (the part supports
-    // unaligned global accesses).  Two forms of the slab load, chosen per slab by a workgroup-uniform test, so that the
-    // common one stays as lean as it was:
+    // unaligned global accesses).  Two forms of the slab load; the ragged one exists in the RAGGED kernel only and is
+    // chosen there per slab by a workgroup-uniform test:
     //   whole   every chunk of the slab lies inside its row, or outside it as a whole (rows of whole 16-byte chunks);
     //   ragged  the row's last chunk holds fewer than 16 of the row's bytes (K * esz % 16 != 0; B row-major: N * esz % 16
     //           != 0): that chunk is read as the 16 bytes that END at the row's end and shifted down, so nothing past the
@@ -810,10 +812,13 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_kernel(const TileGemmP
     };
     // (the fp4-expanding loads read 8-byte half chunks of rows that are whole slabs: never ragged)
     auto tload = [&](int kt) {
-        if (ragged_n || (ragged_k && (kt + 1) * 128 > p.k_bytes))
-            tload_ragged(kt);
-        else
-            tload_whole(kt);
+        if constexpr (RAGGED) {
+            if (ragged_n || (ragged_k && (kt + 1) * 128 > p.k_bytes)) {
+                tload_ragged(kt);
+                return;
+            }
+        }
+        tload_whole(kt);
     };
     auto stage = [&](int buf) {
         uint8_t* base = smem + buf * Cfg::STAGE_BYTES;

@@ -9,11 +9,18 @@ namespace ptoamd {
 template <class Cfg>
 static hipError_t launch_cfg(const TileGemmParams& p, hipStream_t stream)
 {
-    const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_kernel<Cfg>), Cfg::LDS_BYTES);
-    if (e != hipSuccess || p.m <= 0)  // m = 0: only make the kernel ready to launch on the current device
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_kernel<Cfg, false>), Cfg::LDS_BYTES);
+    if (e == hipSuccess)
+        e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_kernel<Cfg, true>), Cfg::LDS_BYTES);
+    if (e != hipSuccess || p.m <= 0)  // m = 0: only make the kernels ready to launch on the current device
         return e;
     const int tiles = ((p.m + Cfg::BM - 1) / Cfg::BM) * ((p.n + Cfg::BN - 1) / Cfg::BN);
-    hipLaunchKernelGGL(gemm_tile_kernel<Cfg>, dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
+    // rows that do not end on a 16-byte chunk boundary take the kernel with the tail-masking loader
+    const bool ragged = (p.k_bytes & 15) != 0 || (p.b_nd && (((long)p.n * p.b_esz) & 15) != 0);
+    if (ragged)
+        hipLaunchKernelGGL((gemm_tile_kernel<Cfg, true>), dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
+    else
+        hipLaunchKernelGGL((gemm_tile_kernel<Cfg, false>), dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
     return hipGetLastError();
 }
 

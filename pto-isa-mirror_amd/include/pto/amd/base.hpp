@@ -34,9 +34,10 @@
 #endif
 // Staging bytes of the fix-pipe (behind the regions above): where TSTORE of an accumulator tile turns the matrix unit's
 // register layout into whole rows before they leave for global memory.  A wave stages one 32 x 32 block at a time in a
-// band of 32 rows x (row bytes + 16); with fewer bytes than WAVES such bands of the output type, TSTORE writes each
-// lane's register quads directly (8 or 16 bytes per row and store instead of 64 or 128).  0 by default: the default
-// split of the other regions already fills the CU's 160 KiB.
+// band of 32 rows x (row bytes + 16) -- for 16-bit outputs with two blocks side by side in the wave, 16 rows of the
+// pair at a time in 16 x (128 + 16) bytes, so that every row leaves as a whole 128-byte line; with fewer bytes than
+// WAVES such bands of the output type, TSTORE writes each lane's register quads directly (8 or 16 bytes per row and
+// store).  0 by default: the default split of the other regions already fills the CU's 160 KiB.
 #ifndef PTO_AMD_STAGE_BYTES
 #define PTO_AMD_STAGE_BYTES 0
 #endif
