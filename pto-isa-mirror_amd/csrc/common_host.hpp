@@ -26,7 +26,7 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 struct Options {
     int tile = -1;               // PTOAMD_TILE=0..6: run this tile shape; -1 = choose by problem size
     bool no_tail_split = false;  // PTOAMD_NO_TAIL_SPLIT=1: never split a half-full last round off as smaller tiles
-    int tail_tile = 5;           // PTOAMD_TAIL_TILE=5|6: the tail runs as 128x128 or 256x128 tiles
+    int tail_tile = 0;           // PTOAMD_TAIL_TILE=5|6|7: the tail's tile; 0 = 256x128 ring-3 tiles (block-scaled) or 128x128
     bool force_generic = false;  // PTOAMD_FORCE_GENERIC=1: everything runs on the order-exact generic kernels
     bool b_nd_in_loader = false; // PTOAMD_B_ND_IN_LOADER=1: a row-major B is transposed by the loader even when a workspace is given
     bool gemv_sw_cvt = false;    // PTOAMD_GEMV_SW_CVT=1: decode fp4 weights with integer arithmetic

@@ -38,9 +38,9 @@ hipError_t launch_gemm_tile(int tile, int op, const TileGemmParams& p, hipStream
 
 void tile_shape(int tile, int* bm, int* bn)
 {
-    static const int bms[7] = {256, 128, 64, 256, 256, 128, 256};
-    static const int bns[7] = {256, 128, 64, 256, 256, 128, 128};
-    const int t = tile < 0 || tile > 6 ? 2 : tile;
+    static const int bms[8] = {256, 128, 64, 256, 256, 128, 256, 256};
+    static const int bns[8] = {256, 128, 64, 256, 256, 128, 128, 128};
+    const int t = tile < 0 || tile > 7 ? 2 : tile;
     *bm = bms[t];
     *bn = bns[t];
 }
@@ -267,8 +267,9 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 // Which tile shape to run: the largest whose grid still fills most of the 256 CUs.  PTOAMD_TILE=0|1|2 overrides,
 // PTOAMD_FORCE_GENERIC=1 sends everything to the order-exact kernel (used by the parity tests).
-// Tiles 0-2 stage slabs through registers (any K that is a multiple of 16 bytes); tiles 3-6 DMA slabs straight into
-// LDS and need K to be a whole number of 128-byte slabs.  Measured on MI355X: the 8-wave 256x256 DMA tile (4) is the
+// Tiles 0-2 stage slabs through registers (any K); tiles 3-7 DMA slabs straight into LDS and need K to be a whole
+// number of 128-byte slabs (7: the 256 x 128 tile with a ring of three slabs, block-scaled types only -- for the other
+// types the id selects tile 6).  Measured on MI355X: the 8-wave 256x256 DMA tile (4) is the
 // fastest for every operand type once the grid fills the chip (the block-scaled types included: their scales come
 // through LDS, which leaves the 32-byte fp8 fragments just enough registers); smaller grids take the 128x128 DMA tile.
 // The DMA tiles address an operand as a wave-uniform 64-bit base plus a 32-bit per-lane byte offset: the last row's offset
@@ -296,13 +297,19 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
     }
     const long t256 = (long)((m + 255) / 256) * ((n + 255) / 256);
     const long t128 = (long)((m + 127) / 128) * ((n + 127) / 128);
-    if (scaled && dtl_ok && t256 >= 128)
+    const long t256x128 = (long)((m + 255) / 256) * ((n + 127) / 128);
+    const int cus = device_compute_units();
+    // Block-scaled types between half and three quarters of a round of 256 x 256 tiles: the 256 x 128 tile with the
+    // three-slab ring puts a workgroup on (nearly) every CU (MXFP4 2048 x 4096 x 4096: 22.5 against 24.9 us)
+    if (scaled && dtl_ok && t256 >= cus / 2 && t256 < 3 * cus / 4 && t256x128 <= cus)
+        return 7;
+    if (scaled && dtl_ok && t256 >= cus / 2)
         return 4;  // half the copy-in bytes per MFMA of the 128x128 tile
     if (scaled)
-        return t128 >= 96 ? (dtl_ok ? 5 : 1) : 2;
-    if (t256 >= 128)
+        return t128 >= 3 * cus / 8 ? (dtl_ok ? 5 : 1) : 2;
+    if (t256 >= cus / 2)
         return dtl_ok ? 4 : 1;
-    if (t128 >= 96)
+    if (t128 >= 3 * cus / 8)
         return dtl_ok ? 5 : 1;
     return 2;
 }
@@ -312,7 +319,7 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
 // one workgroup per CU, same wave tile as the large form) or 128x128 tiles (two workgroups per CU); a tile of the tail
 // then costs a half or a quarter of a 256x256 tile's time instead of a whole round (MXFP8 4096 x 14336 x 4096, 3.5
 // rounds of 256 CUs).  PTOAMD_TILE (an explicit tile) and PTOAMD_NO_TAIL_SPLIT=1 switch the split off;
-// PTOAMD_TAIL_TILE=5|6 picks the tail's tile.
+// PTOAMD_TAIL_TILE=5|6|7 picks the tail's tile (default: 7 for the block-scaled types, 5 otherwise).
 static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStream_t stream)
 {
     if (tile == 4 && options().tile < 0 && !options().no_tail_split) {
@@ -346,7 +353,9 @@ static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStr
                 tail.col_scale = p.col_scale + n1;
             if (p.qwords && p.q_per_column)
                 tail.qwords = p.qwords + n1;
-            return launch_gemm_tile(options().tail_tile, op, tail, stream);
+            // block-scaled types: the 256 x 128 tile with the three-slab ring unless a tail tile was asked for
+            const bool scaled_op = op >= TOP_FP8_E4E4;
+            return launch_gemm_tile(options().tail_tile > 0 ? options().tail_tile : (scaled_op ? 7 : 5), op, tail, stream);
         }
     }
     return launch_gemm_tile(tile, op, p, stream);
@@ -358,8 +367,8 @@ static const char* tile_kernel_name(int tile, int op)
 {
     static const char* ops[TOP_COUNT] = {"bf16", "f16", "i8", "fp8_e4m3_e4m3", "fp8_e5m2_e5m2", "fp8_e4m3_e5m2",
                                          "fp8_e5m2_e4m3", "fp4_e2m1"};
-    static const char* tiles[7] = {"tile256x256", "tile128x128", "tile64x64", "tile256x256w4_dtl", "tile256x256w8_dtl",
-                                   "tile128x128_dtl", "tile256x128_dtl"};
+    static const char* tiles[8] = {"tile256x256", "tile128x128", "tile64x64", "tile256x256w4_dtl", "tile256x256w8_dtl",
+                                   "tile128x128_dtl", "tile256x128_dtl", "tile256x128r3_dtl"};
     static thread_local char buf[64];
     snprintf(buf, sizeof buf, "%s_%s", tiles[tile], ops[op]);
     return buf;

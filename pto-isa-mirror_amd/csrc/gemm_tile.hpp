@@ -282,9 +282,11 @@ __device__ __forceinline__ int frag_chunk(int s, int lhi, int f)
     return 4 * s + 2 * f + lhi;
 }
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, class Op_>
+// RING_: slabs the operand ring of the direct-to-LDS kernel holds (2: the copy-in of slab kt + 2 starts when slab kt is
+// done with its buffer; 3: that of slab kt + 3, one more slab of time for it to land, for tiles whose slab is short).
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, class Op_, int RING_ = 2>
 struct TileCfg {
-    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, RING = RING_;
     using Op = Op_;
     static constexpr int THREADS = WAVES_M * WAVES_N * 64;
     static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;  // per-wave output tile
@@ -296,7 +298,8 @@ struct TileCfg {
     // the direct-to-LDS kernel of a block-scaled operand type keeps two buffers of 16 scale bytes per tile row behind
     // the operand ring
     static constexpr int SCALE_BYTES = Op::SCALED ? 2 * (BM + BN) * 16 : 0;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES + SCALE_BYTES;
+    static constexpr int LDS_BYTES = RING * STAGE_BYTES + SCALE_BYTES;
+    static_assert(LDS_BYTES <= 160 * 1024, "the ring and the scale buffers fit the CU's LDS");
     static constexpr int LA = BM * 8 / THREADS, LB = BN * 8 / THREADS;  // 16-byte chunks per thread per slab
     static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "wave tiles are made of 32x32 blocks");
     static_assert(BLK == 32 || Op::FRAG_BYTES == 16, "the 16x16 instructions take 16-byte fragments");

@@ -62,9 +62,12 @@ __device__ __forceinline__ void sched_kstep()
 #ifndef PTOAMD_DMA_PHASES_16
 #define PTOAMD_DMA_PHASES_16 8
 #endif
-template <int NDMA, int KS, int BLK = 32>
+// (ONE_PHASE: rings deeper than two slabs have a whole slab of slack and issue everything in phase 0)
+template <int NDMA, int KS, int BLK = 32, bool ONE_PHASE = false>
 __host__ __device__ constexpr int dma_phase_begin(int phase)
 {
+    if (ONE_PHASE)
+        return phase >= 1 ? NDMA : 0;
     constexpr int share32[] = {PTOAMD_DMA_PHASES};
     constexpr int share16[] = {PTOAMD_DMA_PHASES_16};
     constexpr int n = BLK == 16 ? sizeof(share16) / sizeof(share16[0]) : sizeof(share32) / sizeof(share32[0]);
@@ -83,7 +86,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     using Op = typename Cfg::Op;
     using Acc = typename Op::Acc;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, LA = Cfg::LA, LB = Cfg::LB;
-    constexpr int NT = Cfg::THREADS, FR = Op::FRAG_BYTES / 16, KS = Cfg::KSTEPS;
+    constexpr int NT = Cfg::THREADS, FR = Op::FRAG_BYTES / 16, KS = Cfg::KSTEPS, RING = Cfg::RING;
     static_assert(KS % 2 == 0, "fragment register sets alternate per k-step");
     static_assert((NT / 8) % 16 == 0, "the swizzle of a lane's row must not depend on the piece index");
     extern __shared__ __align__(16) uint8_t smem[];
@@ -165,7 +168,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
             scb_n[j][w] = 0x7F7F7F7Fu;
     }
     const uint8_t* sc_src[NSW];
-    const uint32_t lds_scales = lds_address(smem) + 2 * Cfg::STAGE_BYTES;
+    const uint32_t lds_scales = lds_address(smem) + RING * Cfg::STAGE_BYTES;
     if (has_scales) {
 #pragma unroll
         for (int w = 0; w < NSW; ++w) {
@@ -190,7 +193,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // with E8M0 127 once, in the prologue.)
     auto read_scales = [&](int kt) __attribute__((always_inline)) {
         if (Op::SCALED) {
-            const uint8_t* base = smem + 2 * Cfg::STAGE_BYTES + ((kt / SPG) & 1) * (SROWS * 16) + (kt % SPG) * GPS;
+            const uint8_t* base = smem + RING * Cfg::STAGE_BYTES + ((kt / SPG) & 1) * (SROWS * 16) + (kt % SPG) * GPS;
 #pragma unroll
             for (int w = 0; w < SW; ++w) {
 #pragma unroll
@@ -248,7 +251,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // (s + 1) & 1, from buffer rbuf step rs) and, in a slab's last step, the DMAs of slab dkt spread between them.
     auto kstep = [&](auto phase, int s, bool reads, int rbuf, int rs, bool dmas, int dkt, int dbuf) __attribute__((always_inline)) {
         constexpr int PH = decltype(phase)::value;
-        constexpr int DQ0 = dma_phase_begin<NDMA, KS, BLK>(PH), DN = dma_phase_begin<NDMA, KS, BLK>(PH + 1) - DQ0;
+        constexpr int DQ0 = dma_phase_begin<NDMA, KS, BLK, (Cfg::RING > 2)>(PH), DN = dma_phase_begin<NDMA, KS, BLK, (Cfg::RING > 2)>(PH + 1) - DQ0;
         constexpr int DSPAN = (BLK == 16 && PH > 0) ? NMMA / 2 : NMMA;  // MFMAs the phase's DMAs are spread over
         const int set = SETS == 2 ? (s & 1) : 0;
         const int nset = SETS == 2 ? (set ^ 1) : 0;
@@ -304,13 +307,28 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     tload_scales(0);
     if (Op::SCALED && !has_scales) {
         for (int o = tid * 16; o < 2 * SROWS * 16; o += NT * 16)
-            *reinterpret_cast<uint4*>(smem + 2 * Cfg::STAGE_BYTES + o) = make_uint4(0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu);
+            *reinterpret_cast<uint4*>(smem + RING * Cfg::STAGE_BYTES + o) = make_uint4(0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu, 0x7F7F7F7Fu);
     }
     // slab 1's first DMAs go out now but only slab 0 (and the scales) are waited for: the counter retires loads in
     // order, so "at most N1 outstanding" means everything issued before slab 1's pieces has landed; slab 1 is covered
     // by the first slab's barrier
-    constexpr int N1 = dma_phase_begin<NDMA, KS, BLK>(1);
-    if (k_slabs > 1) {
+    constexpr int N1 = dma_phase_begin<NDMA, KS, BLK, (Cfg::RING > 2)>(1);
+    // A deeper ring starts slabs 1 .. RING - 1 whole as well (it is built for the types whose slab goes out in one
+    // phase), so that from the first slab on the copy-in runs RING - 1 slabs ahead.  At the barrier of slab kt the ring
+    // may leave WAITN DMAs in flight: those of the slabs after kt + 1, but no more than were issued after the scale
+    // chunk that is read at that barrier (requested SPG - 1 slabs earlier).
+    static_assert(RING == 2 || N1 == NDMA, "rings deeper than two slabs issue a slab's DMAs in one phase");
+    constexpr int WAITN = RING == 2 ? 0 : ((RING - 2 < SPG - 1 || !Op::SCALED) ? RING - 2 : SPG - 1) * NDMA;
+    static_assert(WAITN < 64 && (RING - 1) * NDMA < 64, "vmcnt is a 6-bit count");
+    if (RING > 2 && k_slabs >= RING) {
+        static_for<RING - 1>([&](auto sc) { tload(decltype(sc)::value + 1, decltype(sc)::value + 1); });
+        constexpr int W0 = (RING - 1) * NDMA;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (W0 & 15) | ((W0 >> 4) << 14));  // slab 0 and the scales have landed
+    } else if (RING > 2) {
+        for (int s1 = 1; s1 < k_slabs; ++s1)
+            tload(s1, s1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+    } else if (k_slabs > 1) {
         static_for<N1>([&](auto qc) { tload_piece(1, 1, decltype(qc)::value); });
         __builtin_amdgcn_s_waitcnt(0x0F70 | (N1 & 15) | ((N1 >> 4) << 14));  // vmcnt(N1)
     } else {
@@ -325,8 +343,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // One slab.  `more` = slab kt+1 exists (read its first fragments in the last k-step), `dma` = slab kt+2 exists
     // (start its DMA into the buffer this slab frees); both are literal at the call sites so the branches fold.
     // (always_inline: out of line, a lambda takes the accumulators by reference and they live in scratch memory)
-    auto slab = [&](int kt, bool more, bool dma) __attribute__((always_inline)) {
-        const int cur = kt & 1;
+    // `cur` / `nxt`: ring buffers of slab kt and kt + 1; slab kt + RING - 1 ... goes into the buffer slab kt frees.
+    // `steady`: slabs kt + 1 .. kt + RING - 1 are all in flight or landed (the barrier may then leave WAITN DMAs pending).
+    auto slab = [&](int kt, int cur, bool more, bool dma, auto steady) __attribute__((always_inline)) {
+        const int nxt = RING == 2 ? (cur ^ 1) : (cur + 1 == RING ? 0 : cur + 1);
         if (Op::SCALED) {
             // The request for the next scale chunk sits here, at the top of the slab, and not between two k-steps: a
             // branch between them splits the slab into basic blocks, and the compiler then sinks the first k-step's
@@ -349,23 +369,41 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         }
         static_for<KS - 1>([&](auto sc) {
             constexpr int s = decltype(sc)::value;
-            kstep(std::integral_constant<int, s + 1>{}, s, true, cur, s + 1, more, kt + 1, cur ^ 1);
+            kstep(std::integral_constant<int, s + 1>{}, s, true, cur, s + 1, more, kt + 1, nxt);
         });
-        // every wave is done reading slab kt, and its DMAs of slab kt+1 (issued one slab ago) have landed
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        // every wave is done reading slab kt, and its DMAs of slab kt+1 (issued RING - 1 slabs ago) have landed
+        constexpr int WN = decltype(steady)::value ? WAITN : 0;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (WN & 15) | ((WN >> 4) << 14));  // vmcnt(WN)
         __syncthreads();
         if (SC_AHEAD && more)
             read_scales(kt + 1);
-        kstep(std::integral_constant<int, 0>{}, KS - 1, more, cur ^ 1, 0, dma, kt + 2, cur);
+        kstep(std::integral_constant<int, 0>{}, KS - 1, more, nxt, 0, dma, kt + RING, cur);
     };
-    int kt = 0;
-    for (; kt + 2 < k_slabs; ++kt)
-        slab(kt, true, true);
-    if (kt + 1 < k_slabs) {
-        slab(kt, true, false);
-        ++kt;
+    int kt = 0, cur = 0;
+    if constexpr (RING == 2) {
+        for (; kt + 2 < k_slabs; ++kt)
+            slab(kt, kt & 1, true, true, std::true_type{});
+        if (kt + 1 < k_slabs) {
+            slab(kt, kt & 1, true, false, std::false_type{});
+            ++kt;
+        }
+        slab(kt, kt & 1, false, false, std::false_type{});
+    } else {
+        const auto advance = [&]() {
+            ++kt;
+            cur = cur + 1 == RING ? 0 : cur + 1;
+        };
+        while (kt + RING < k_slabs) {
+            slab(kt, cur, true, true, std::true_type{});
+            advance();
+        }
+        // the last RING slabs (or fewer): nothing more to start; the barrier waits for everything in flight
+        while (kt + 1 < k_slabs) {
+            slab(kt, cur, true, false, std::false_type{});
+            advance();
+        }
+        slab(kt, cur, false, false, std::false_type{});
     }
-    slab(kt, false, false);
 
     // ---- TSTORE.  No wave reads the ring after the last slab's barrier (its fragment reads were issued before it) and
     // no DMA is in flight, so each wave may reuse a piece of it for the staged store without another barrier.

@@ -39,7 +39,7 @@ hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 {
     if (tile == TILE_PREPARE_ALL) {  // every kernel of this unit gets its launch attributes on the current device
         TileGemmParams none{};
-        for (int t : {4, 5, 6, 1, 2}) {
+        for (int t : {4, 5, 6, 7, 1, 2}) {
             const hipError_t e = PTOAMD_TILE_FN(t, none, stream);
             if (e != hipSuccess)
                 return e;
@@ -58,6 +58,11 @@ hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 #endif
         case 5: return launch_dtl<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>>(p, stream);
         case 6: return launch_dtl<TileCfg<256, 128, 4, 2, PTOAMD_TILE_OP>>(p, stream);
+#ifdef PTOAMD_TILE_RING3  // block-scaled types: the 256 x 128 tile with a ring of three slabs
+        case 7: return launch_dtl<TileCfg<256, 128, 4, 2, PTOAMD_TILE_OP, 3>>(p, stream);
+#else
+        case 7: return launch_dtl<TileCfg<256, 128, 4, 2, PTOAMD_TILE_OP>>(p, stream);
+#endif
         case 0:  // (once a register-staged 256 x 256 tile: it kept part of its working set in scratch memory)
         case 1: return launch_cfg<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>>(p, stream);
         default: return launch_cfg<TileCfg<64, 64, 2, 2, PTOAMD_TILE_OP>>(p, stream);

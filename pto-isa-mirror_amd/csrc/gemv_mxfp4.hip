@@ -367,8 +367,11 @@ __global__ void __launch_bounds__(SK_WAVES * 64) gemv_mxfp4_splitk_kernel(const 
 //   stage   one strip of 16 weight rows x one chunk: row r is one piece of 1 KiB at r KiB (16-byte chunk c at position
 //           c ^ r, applied on the global side, so that the 16 rows a 16-lane group reads at one chunk index fall into
 //           16 different bank groups), then 16 x 64 scale bytes.  A ring of six stages: the loaders run up to six ahead.
-//   sync    two workgroup barriers per stage: (A) every loader's pieces of stage t have landed, (B) every compute wave
-//           has its fragments of stage t in registers, so the loaders refill the slot with stage t + 6.
+//   sync    one workgroup barrier per stage t: every loader's pieces of stage t have landed, and every compute wave has
+//           its fragments of stage t - 1 in registers, so after it the loaders refill that slot with stage t + 5 while
+//           the compute waves read stage t.  (Two barriers per stage -- landed / consumed -- ran 0.2 us slower; with
+//           no synchronisation at all, results wrong, the launch takes 23.8 instead of 24.6 us: what is left is the
+//           memory system's, not the barriers'.)
 constexpr int WD_CHUNK = 2048;                       // k per chunk
 constexpr int WD_WBYTES = 16 * (WD_CHUNK / 2);       // 16 KiB
 constexpr int WD_SBYTES = 16 * (WD_CHUNK / 32);      // 1 KiB
@@ -511,21 +514,23 @@ __global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvP
                             default: PTOAMD_WAIT_VM(5 * WD_VM_PER_STAGE); break;
                         }
                     }
-                    wg_barrier();   // (A)
+                    // The one barrier of a stage: every loader's pieces of this stage have landed, and every compute
+                    // wave has the previous stage's fragments in registers (it waited for those reads before its
+                    // MFMAs), so the loaders refill the previous stage's slot right away while the compute waves read
+                    // this one.
+                    wg_barrier();
                     const uint8_t* buf = smem + (consumed % WD_RING) * WD_STAGE;
-                    uint4 sc4, wv[4];
-                    if (!loader) {
+                    ++consumed;
+                    if (loader) {
+                        if (consumed > 1)
+                            issue_next();
+                    } else {
+                        uint4 sc4, wv[4];
                         sc4 = *reinterpret_cast<const uint4*>(buf + sread);
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
                             wv[j] = *reinterpret_cast<const uint4*>(buf + (wread ^ (64 * j)));
                         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    }
-                    wg_barrier();   // (B)
-                    ++consumed;
-                    if (loader) {
-                        issue_next();
-                    } else {
                         const uint32_t sc[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {

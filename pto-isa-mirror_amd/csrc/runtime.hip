@@ -44,11 +44,11 @@ void read_options()
 {
     Options o;
     const char* t = getenv("PTOAMD_TILE");
-    if (t != nullptr && t[0] >= '0' && t[0] <= '6')
+    if (t != nullptr && t[0] >= '0' && t[0] <= '7')
         o.tile = t[0] - '0';
     o.no_tail_split = getenv("PTOAMD_NO_TAIL_SPLIT") != nullptr;
     const char* tt = getenv("PTOAMD_TAIL_TILE");
-    if (tt != nullptr && (tt[0] == '5' || tt[0] == '6'))
+    if (tt != nullptr && tt[0] >= '5' && tt[0] <= '7')
         o.tail_tile = tt[0] - '0';
     o.force_generic = env_is_1("PTOAMD_FORCE_GENERIC");
     o.b_nd_in_loader = getenv("PTOAMD_B_ND_IN_LOADER") != nullptr;

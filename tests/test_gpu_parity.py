@@ -771,7 +771,43 @@ def test_mx_block_scales_select_the_right_group(pa, oracle):
         assert relerr(got, ref) <= 2e-2, g
 
 
-@pytest.mark.parametrize("tile", [4, 5, 6])
+@pytest.mark.parametrize("typ", [ob.E4M3, ob.E2M1])
+def test_mx_three_slab_ring_tile_every_k_length(pa, oracle, typ):
+    """Tile 7 (256 x 128, ring of three slabs).  The DMA tiles stream scale rows of whole 16-byte chunks, so K is a
+    multiple of 512: 4, 8, 12, 20 fp8 slabs or 2, 4, 6, 10 fp4 slabs -- fewer slabs than ring buffers, one more, many.
+    Same slabs and k-steps as the two-slab 128 x 128 tile, so the results must agree bit for bit, and hold the oracle's bar."""
+    r = np.random.default_rng(77 + typ)
+    m, n = 300, 200   # ragged in both directions: two row tiles, two column tiles
+    for k in (512, 1024, 1536, 2560):
+        a, b, sa, sb = _mx_inputs(r, typ, m, n, k)
+        ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, typ, typ)
+        with tile_env(PTOAMD_TILE=7):
+            got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[typ], PA_T[typ], pa.F32))
+            assert pa.last_kernel().startswith("tile256x128r3_dtl"), pa.last_kernel()
+        with tile_env(PTOAMD_TILE=5):
+            other = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[typ], PA_T[typ], pa.F32))
+        assert np.array_equal(got.view(np.uint32), other.view(np.uint32)), k
+        assert relerr(got, ref) <= 2e-2, k
+
+
+def test_three_slab_ring_tile_one_to_five_slabs_without_scales(pa, oracle):
+    """The same tile on a plain fp8 TMATMUL (no scale arrays, any whole number of 128-byte slabs): 1, 2, 3, 4 and 5
+    slabs cover a ring that is never full, exactly full, and wrapped."""
+    r = np.random.default_rng(78)
+    m, n = 260, 130
+    for k in (128, 256, 384, 512, 640):
+        a, b, _, _ = _mx_inputs(r, ob.E4M3, m, n, k)
+        ref = oracle.matmul_fp8(a, b, b_dn=True)
+        with tile_env(PTOAMD_TILE=7):
+            got = host(pa.gemm_fp8(dev(a), dev(b), pa.E4M3, pa.E4M3, pa.F32))
+            assert pa.last_kernel().startswith("tile256x128r3_dtl"), pa.last_kernel()
+        with tile_env(PTOAMD_TILE=5):
+            other = host(pa.gemm_fp8(dev(a), dev(b), pa.E4M3, pa.E4M3, pa.F32))
+        assert np.array_equal(got.view(np.uint32), other.view(np.uint32)), k
+        assert relerr(got, ref) <= 2e-2, k
+
+
+@pytest.mark.parametrize("tile", [4, 5, 6, 7])
 @pytest.mark.parametrize("typ", [ob.E4M3, ob.E2M1])
 def test_mx_scale_chunks_across_slabs(pa, oracle, typ, tile):
     """The DMA tiles fetch scales as 16-byte chunks per row (4 fp8 slabs / 2 fp4 slabs) into two alternating LDS
@@ -939,14 +975,16 @@ def test_config4_mxfp8_full_size(pa, oracle):
     assert torch.equal(g2, g1 * 2)
 
 
-def test_mxfp4_gemm_large_takes_the_256_tile(pa, oracle):
-    """MXFP4 x MXFP4 at a grid that fills the chip: 2048 x 4096 x 2048, operands quantised by TQUANT<MXFP4> (OCP)."""
-    m, n, k = 2048, 4096, 2048
+@pytest.mark.parametrize("m,kernel", [(4096, "tile256x256w8_dtl_fp4_e2m1"), (2048, "tile256x128r3_dtl_fp4_e2m1")])
+def test_mxfp4_gemm_large_takes_the_256_tile(pa, oracle, m, kernel):
+    """MXFP4 x MXFP4, operands quantised by TQUANT<MXFP4> (OCP): 4096 x 4096 x 2048 is one round of 256 x 256 tiles;
+    2048 x 4096 x 2048 would be half a round of them and runs as 256 x 128 tiles with the three-slab ring."""
+    n, k = 4096, 2048
     gen = torch.Generator(device=DEV).manual_seed(44)
     a, sa = pa.tquant_mx(torch.randn((m, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
     b, sb = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
     out = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E2M1, pa.E2M1, pa.F32)
-    assert pa.last_kernel() == "tile256x256w8_dtl_fp4_e2m1"
+    assert pa.last_kernel() == kernel
     table = oracle.mx_decode_table(ob.E2M1)
     out_h = host(out)
 
@@ -957,11 +995,11 @@ def test_mxfp4_gemm_large_takes_the_256_tile(pa, oracle):
     cols = np.arange(0, n, 64) + np.arange(64) % 64
     # both error bars of an fp32 drain on 64 x 64 sampled outputs and on two whole 256 x 256 tiles
     for label, rr, cc in (("samples", rows, cols), ("tile (0, 0)", np.arange(256), np.arange(256)),
-                          ("tile (7, 15)", np.arange(m - 256, m), np.arange(n - 256, n))):
+                          ("last tile", np.arange(m - 256, m), np.arange(n - 256, n))):
         ar, bc, sar, sbc = host(sel(a, rr)), host(sel(b, cc)), host(sel(sa, rr)), host(sel(sb, cc))
         ref = oracle.matmul_mx(ar, bc, sar, sbc, len(rr), k, len(cc), ob.E2M1, ob.E2M1)
         check_f32_drain(out_h[np.ix_(rr, cc)], ref, magnitudes(ar, sar) @ magnitudes(bc, sbc).T, k,
-                        f"MXFP4 2048x4096x2048, {label}")
+                        f"MXFP4 {m}x4096x2048, {label}")
     with tile_env(PTOAMD_TILE=5):
         other = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E2M1, pa.E2M1, pa.F32)
     assert relerr(host(other), host(out)) <= 1e-5
