@@ -85,6 +85,14 @@ def _ptr(t, strided=False):
     return C.c_void_p(t.data_ptr())
 
 
+def _cin(c_in, out):
+    """The accumulator input is read at the output's row pitch (the C ABI has one ldc for both)."""
+    if c_in is None:
+        return C.c_void_p(0)
+    assert c_in.dim() == 2 and c_in.stride(0) == out.stride(0), "c_in must have the output's row pitch"
+    return _ptr(c_in, True)
+
+
 def _stream(stream):
     s = stream if stream is not None else torch.cuda.current_stream()
     return C.c_void_p(s.cuda_stream)
@@ -108,16 +116,16 @@ def gemm(a, b, ab_type, c_type=F32, b_layout=B_DN, c_in=None, relu=False, m=None
     if out is None:
         out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
     if workspace is not None:
-        _check(_lib.ptoamd_gemm_ws(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _ptr(c_in), _ptr(bias), m, n, k,
+        _check(_lib.ptoamd_gemm_ws(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _cin(c_in, out), _ptr(bias), m, n, k,
                                    a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu), _ptr(workspace),
                                    C.c_size_t(workspace.numel() * workspace.element_size()), _stream(stream)), "ptoamd_gemm_ws")
         return out
     if bias is not None:
-        _check(_lib.ptoamd_gemm_bias(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _ptr(c_in), _ptr(bias), m, n, k,
+        _check(_lib.ptoamd_gemm_bias(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _cin(c_in, out), _ptr(bias), m, n, k,
                                      a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu), _stream(stream)),
                "ptoamd_gemm_bias")
         return out
-    _check(_lib.ptoamd_gemm(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _ptr(c_in), m, n, k, a.stride(0), b.stride(0),
+    _check(_lib.ptoamd_gemm(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _cin(c_in, out), m, n, k, a.stride(0), b.stride(0),
                             out.stride(0), b_layout, int(relu), _stream(stream)), "ptoamd_gemm")
     return out
 
@@ -128,7 +136,7 @@ def gemm_fp8(a, b, a_type, b_type, c_type=F32, b_layout=B_DN, c_in=None, bias=No
     n = b.shape[0] if b_layout == B_DN else b.shape[1]
     if out is None:
         out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=a.device)
-    _check(_lib.ptoamd_gemm_fp8(_ptr(out, True), c_type, _ptr(a, True), a_type, _ptr(b, True), b_type, _ptr(c_in), _ptr(bias), m, n, k,
+    _check(_lib.ptoamd_gemm_fp8(_ptr(out, True), c_type, _ptr(a, True), a_type, _ptr(b, True), b_type, _cin(c_in, out), _ptr(bias), m, n, k,
                                 a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu), _stream(stream)), "ptoamd_gemm_fp8")
     return out
 
@@ -151,7 +159,7 @@ def gemm_requant(a, b, ab_type, c_type, quant_words, per_column=False, b_layout=
     n = (b.shape[0] if b_layout == B_DN else b.shape[1]) if n is None else n
     if out is None:
         out = torch.empty((m, n), dtype={I8: torch.int8, U8: torch.uint8, F16: torch.float16, BF16: torch.bfloat16, I16: torch.int16}[c_type], device=a.device)
-    _check(_lib.ptoamd_gemm_requant(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _ptr(c_in), _ptr(bias), _ptr(quant_words),
+    _check(_lib.ptoamd_gemm_requant(_ptr(out, True), c_type, _ptr(a, True), _ptr(b, True), ab_type, _cin(c_in, out), _ptr(bias), _ptr(quant_words),
                                     int(per_column), m, n, k, a.stride(0), b.stride(0), out.stride(0), b_layout, int(relu),
                                     _stream(stream)), "ptoamd_gemm_requant")
     return out
@@ -180,7 +188,7 @@ def gemm_mx_static(a, b, sa, sb, m, n, k, a_type, b_type, out, sa_layout=MX_A_ND
     lda = k
     ldb = k if b_layout == B_DN else n
     _check(_lib.ptoamd_gemm_mx_static(_ptr(out, True), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
-                                      sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),
+                                      sb_layout, _cin(c_in, out), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),
            "ptoamd_gemm_mx_static")
     return out
 
@@ -199,17 +207,17 @@ def gemm_mx(a, b, sa, sb, m, n, k, a_type, b_type, c_type=F32, sa_layout=MX_A_ND
     ldb = k if b_layout == B_DN else n
     if workspace is not None:
         _check(_lib.ptoamd_gemm_mx_ws(_ptr(out, True), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
-                                      sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _ptr(workspace),
+                                      sb_layout, _cin(c_in, out), m, n, k, lda, ldb, out.stride(0), b_layout, _ptr(workspace),
                                       C.c_size_t(workspace.numel() * workspace.element_size()), _stream(stream)),
                "ptoamd_gemm_mx_ws")
         return out
     if bias is not None:
         _check(_lib.ptoamd_gemm_mx_bias(_ptr(out, True), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
-                                        sb_layout, _ptr(c_in), _ptr(bias), m, n, k, lda, ldb, out.stride(0), b_layout,
+                                        sb_layout, _cin(c_in, out), _ptr(bias), m, n, k, lda, ldb, out.stride(0), b_layout,
                                         _stream(stream)), "ptoamd_gemm_mx_bias")
         return out
     _check(_lib.ptoamd_gemm_mx(_ptr(out, True), c_type, _ptr(a), _ptr(b), a_type, b_type, _ptr(sa), _ptr(sb), sa_layout,
-                               sb_layout, _ptr(c_in), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),
+                               sb_layout, _cin(c_in, out), m, n, k, lda, ldb, out.stride(0), b_layout, _stream(stream)),
            "ptoamd_gemm_mx")
     return out
 

@@ -498,8 +498,10 @@ struct StagedStore {
     static_assert((32 * Cfg::WTN / 16) % 64 == 0, "a band is a whole number of 64-lane reads, down to one-byte outputs");
 };
 
-// `stage` is the calling wave's private LDS region of StagedStore<Cfg>::WAVE_BYTES bytes; the wave's tile lies inside
-// the matrix and its rows of C start on 16-byte boundaries (checked by the caller)
+// `stage` is the calling wave's private LDS region of StagedStore<Cfg>::WAVE_BYTES bytes.  The wave tile's columns lie
+// inside the matrix (checked by the caller); its last rows may lie past row m - 1: they are computed on clamped row
+// indices and not stored.  Rows of C need no alignment: a row piece leaves as 16-byte stores at whatever address it
+// starts (the part takes unaligned vector stores; on 16-byte aligned rows they are whole 128-byte lines).
 template <int KIND, class Cfg, class Acc>
 __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0,
                                               int l32, int lhi, uint8_t* stage)
@@ -557,7 +559,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
     if constexpr (KIND == OUT_W8A8_BF16) {
 #pragma unroll
         for (int i = 0; i < Cfg::MB; ++i)  // the row scales likewise: one load latency instead of one per block row
-            rs_pre[i] = p.row_scale[row0 + i * BLK + l32];
+            rs_pre[i] = p.row_scale[min(row0 + i * BLK + l32, p.m - 1)];
         static_for<Cfg::NB>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
 #pragma unroll
@@ -570,7 +572,7 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
         static_for<BPB>([&](auto hc) {
             constexpr int i = band * BPB + decltype(hc)::value;
             const int srow = decltype(hc)::value * BLK + l32;  // row inside the band
-            const int gi = row0 + i * BLK + l32;
+            const int gi = min(row0 + i * BLK + l32, p.m - 1);
             const float rs = KIND == OUT_W8A8_BF16 ? rs_pre[i] : 1.0f;
             static_for<Cfg::NB>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
@@ -617,11 +619,12 @@ __device__ __forceinline__ void tstore_staged(const TileGemmParams& p, Acc (&acc
         for (int it = 0; it < ITERS; ++it) {
             const int q = it * 64 + lane, row = q / CHUNKS, ch = q % CHUNKS;
             const uint4 v = *reinterpret_cast<const uint4*>(stage + row * ROW_BYTES + ch * 16);
-            typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
+            typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4), aligned(1)));
             nt_u32x4* dst = reinterpret_cast<nt_u32x4*>(reinterpret_cast<uint8_t*>(p.c) +
                                                         ((long)(row0 + band * 32 + row) * p.ldc + col0) * ESZ + ch * 16);
             const nt_u32x4 vv = {v.x, v.y, v.z, v.w};
-            __builtin_nontemporal_store(vv, dst);  // C is not read again by this kernel: keep it out of the L2's way (plain stores end TSTORE
+            if (row0 + band * 32 + row < p.m)
+                __builtin_nontemporal_store(vv, dst);  // C is not read again by this kernel: keep it out of the L2's way (plain stores end TSTORE
                                                    // 0.3 us sooner, but their write-backs cost the next launch 1 us)
         }
     });
@@ -632,11 +635,10 @@ template <class Cfg, class Acc>
 __device__ __forceinline__ void tstore(const TileGemmParams& p, Acc (&acc)[Cfg::MB][Cfg::NB], int row0, int col0, int l32,
                                        int lhi, uint8_t* stage = nullptr)
 {
-    const bool full = row0 + Cfg::WTM <= p.m && col0 + Cfg::WTN <= p.n;
-    const int esz = (p.out_kind == OUT_F32 || p.out_kind == OUT_I32) ? 4 : (p.out_kind == OUT_Q8 ? 1 : 2);
-    const bool aligned = (((long)p.ldc * esz) & 15) == 0 && (reinterpret_cast<uintptr_t>(p.c) & 15) == 0;
+    // the staged form takes wave tiles whose columns are all inside the matrix (rows past m - 1 are skipped row by row)
+    const bool cols_inside = row0 < p.m && col0 + Cfg::WTN <= p.n;
     const bool raw_acc = p.out_kind == OUT_W8A8_BF16 && p.acc_out != nullptr;
-    if (stage != nullptr && full && aligned && !p.atomic_add && !raw_acc) {
+    if (stage != nullptr && cols_inside && !p.atomic_add && !raw_acc) {
         if (p.out_kind >= OUT_QF16) {
             tstore_staged<OUT_QF16, Cfg>(p, acc, row0, col0, l32, lhi, stage);
         } else if (p.out_kind == OUT_Q8) {

@@ -771,6 +771,37 @@ def test_mx_block_scales_select_the_right_group(pa, oracle):
         assert relerr(got, ref) <= 2e-2, g
 
 
+@pytest.mark.parametrize("tile", [2, 4, 5])
+@pytest.mark.parametrize("c_type", ["bf16", "f32"])
+def test_staged_store_rows_at_any_alignment_and_ragged_row_tiles(pa, oracle, tile, c_type):
+    """TSTORE through the LDS staging on rows of C that start at odd addresses (pitch of 267 elements, first element one
+    past an aligned address) and on tiles whose last rows lie past m - 1: the output must equal, bit for bit, the one
+    written to a dense aligned matrix, with the pitch's spare column and the row past the end untouched; and an
+    accumulator input read at the same odd pitch must be added."""
+    r = np.random.default_rng(90 + tile)
+    m, n, k = 300, 266, 256   # column tiles all whole for the 64- and 128-wide wave tiles up to column 256; the rest is edge
+    ct = pa.BF16 if c_type == "bf16" else pa.F32
+    dt = torch.bfloat16 if c_type == "bf16" else torch.float32
+    a, b = bf16_bits(r.standard_normal((m, k))), bf16_bits(r.standard_normal((n, k)))
+    cin = r.standard_normal((m, n)).astype(np.float32)
+    da, db = dev(a).view(torch.bfloat16), dev(b).view(torch.bfloat16)
+    with tile_env(PTOAMD_TILE=tile):
+        dense = pa.gemm(da, db, pa.BF16, ct, pa.B_DN, c_in=dev(cin))
+        big = torch.full(((m + 1) * 267 + 1,), 7.0, dtype=dt, device=DEV)
+        view = big[1:1 + m * 267].view(m, 267)[:, :n]
+        cin_big = torch.zeros((m, 267), dtype=torch.float32, device=DEV)
+        cin_big[:, :n] = dev(cin)
+        pa.gemm(da, db, pa.BF16, ct, pa.B_DN, c_in=cin_big[:, :n], out=view)
+    torch.cuda.synchronize()
+    assert torch.equal(view, dense)
+    rest = big.clone()
+    rest[1:1 + m * 267].view(m, 267)[:, :n] = 7.0
+    assert bool((rest == 7.0).all())   # nothing outside the m x n window was written
+    ref = oracle.matmul_bf16(a, b, cin=cin, b_dn=True)
+    got = host(dense) if c_type == "f32" else bf16_to_f32(host(dense))
+    assert relerr(got, ref) <= (1e-2 if c_type == "bf16" else 1e-4)
+
+
 @pytest.mark.parametrize("typ", [ob.E4M3, ob.E2M1])
 def test_mx_three_slab_ring_tile_every_k_length(pa, oracle, typ):
     """Tile 7 (256 x 128, ring of three slabs).  The DMA tiles stream scale rows of whole 16-byte chunks, so K is a
