@@ -264,6 +264,8 @@ static int elem_bits(int type)
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static long ws_row_bytes(long k_bytes) { return (k_bytes + 15) / 16 * 16; }  // row pitch of a transposed B in a workspace
+static bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
 // Which tile shape to run: the largest whose grid still fills most of the 256 CUs.  PTOAMD_TILE=0|1|2 overrides,
 // PTOAMD_FORCE_GENERIC=1 sends everything to the order-exact kernel (used by the parity tests).
@@ -282,11 +284,16 @@ static bool dma_offsets_fit(int m, int n, long lda_bytes, long ldb_bytes, long k
 
 // dma_ok: what the DMA tiles need besides whole slabs -- 16-byte aligned operand rows, 32-bit lane offsets, and for the
 // block-scaled types scale rows they can stream.
-static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, bool dma_ok = true)
+// The plain types' tiles 4 and 5 also take a K that is not a whole number of slabs (at least one slab long).
+// (ragged_k_ok: the operand type has them -- bf16, f16, int8)
+static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, bool dma_ok = true, bool ragged_k_ok = false)
 {
-    const bool dtl_ok = (k_bytes % 128) == 0 && dma_ok;
+    const bool ragged_k = (k_bytes % 128) != 0;
+    const bool dtl_ok = dma_ok && (!ragged_k || (ragged_k_ok && k_bytes > 128));
     if (options().tile >= 0) {
         int t = options().tile;
+        if (ragged_k && t > 5)  // tiles 6 and 7 exist for whole slabs only
+            t = 5;
         if (t == 3)  // the four-wave form of the 256 x 256 DMA tile is no longer built
             t = 4;
         if (t == 0)  // nor is the register-staged 256 x 256 tile (it spilled: 315 against 176 us for the 128 x 128 one on
@@ -375,11 +382,11 @@ static const char* tile_kernel_name(int tile, int op)
 }
 
 template <typename T>
-static int transpose_b(void* dst, const void* src, int k, int n, long ldb, hipStream_t stream)
+static int transpose_b(void* dst, const void* src, int k, int n, long ldb, long ld_dst, hipStream_t stream)
 {
     dim3 block(32, 8), grid((n + 31) / 32, (k + 31) / 32);
     hipLaunchKernelGGL(transpose_kernel<T>, grid, block, 0, stream, reinterpret_cast<T*>(dst),
-                       reinterpret_cast<const T*>(src), k, n, ldb, (long)k);
+                       reinterpret_cast<const T*>(src), k, n, ldb, ld_dst);
     PTOAMD_HIP_CHECK(hipGetLastError());
     return PTOAMD_OK;
 }
@@ -473,7 +480,7 @@ size_t ptoamd_gemm_workspace_bytes(int n, int k, int ab_type, int b_layout)
 {
     if (n <= 0 || k <= 0 || b_layout != PTOAMD_B_ND)
         return 0;
-    return (size_t)n * (size_t)k * (size_t)(elem_bits(ab_type) / 8);
+    return (size_t)n * (size_t)ws_row_bytes((long)k * (elem_bits(ab_type) / 8));
 }
 
 int ptoamd_gemm_ws(void* c, int c_type, const void* a, const void* b, int ab_type, const void* c_in, const void* bias, int m, int n,
@@ -563,7 +570,7 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
     // register-staged tiles transpose it on its way into LDS.  Nothing is allocated either way.
     const bool mfma_type = ab_type != PTOAMD_F32 && ab_type != PTOAMD_HIF8;
     const bool elems_ok = (reinterpret_cast<uintptr_t>(a) & emask) == 0 && (reinterpret_cast<uintptr_t>(b) & emask) == 0;
-    const size_t ws_need = b_layout == PTOAMD_B_ND ? (size_t)n * (size_t)k_bytes : 0;
+    const size_t ws_need = b_layout == PTOAMD_B_ND ? (size_t)n * (size_t)ws_row_bytes(k_bytes) : 0;
     const bool b_via_ws = b_layout == PTOAMD_B_ND && ws != nullptr && (ebytes == 1 || ebytes == 2) && !options().b_nd_in_loader;
     PTOAMD_REQUIRE(!b_via_ws || ws_need <= ws_bytes, PTOAMD_E_INVALID,
                    "ptoamd_gemm_ws: re-ordering B needs %zu bytes of workspace, %zu available", ws_need, ws_bytes);
@@ -583,11 +590,14 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
     const uint8_t* b_kmajor = reinterpret_cast<const uint8_t*>(b);
     long ldb_kmajor = ldb_b;
     if (b_via_ws) {  // TLOAD of an ND B panel: re-order once so the MFMA path reads K-contiguous rows
-        const int rc = ebytes == 2 ? transpose_b<uint16_t>(ws, b, k, n, ldb, stream) : transpose_b<uint8_t>(ws, b, k, n, ldb, stream);
+        // rows of the re-ordered copy start on 16-byte boundaries whatever K is
+        const long pitch = ws_row_bytes(k_bytes);
+        const int rc = ebytes == 2 ? transpose_b<uint16_t>(ws, b, k, n, ldb, pitch / 2, stream)
+                                   : transpose_b<uint8_t>(ws, b, k, n, ldb, pitch, stream);
         if (rc != PTOAMD_OK)
             return rc;
         b_kmajor = reinterpret_cast<const uint8_t*>(ws);
-        ldb_kmajor = k_bytes;
+        ldb_kmajor = pitch;
     }
     TileGemmParams p{};
     p.a = reinterpret_cast<const uint8_t*>(a);
@@ -603,9 +613,10 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
                    : ab_type == PTOAMD_E4M3 ? (b_type == PTOAMD_E4M3 ? TOP_FP8_E4E4 : TOP_FP8_E4E5)
                                             : (b_type == PTOAMD_E5M2 ? TOP_FP8_E5E5 : TOP_FP8_E5E4);
     p.b_nd = b_in_kernel; p.b_esz = ebytes;
-    const bool dma_ok = !b_in_kernel && aligned16(a) && aligned16(b_kmajor) && (lda_b % 16) == 0 && (ldb_kmajor % 16) == 0 &&
+    // (LDS-DMA needs dword-aligned global addresses, no more: rows at 4-byte alignment run 114 against 100 us on bf16 4096^3)
+    const bool dma_ok = !b_in_kernel && aligned4(a) && aligned4(b_kmajor) && (lda_b % 4) == 0 && (ldb_kmajor % 4) == 0 &&
                         dma_offsets_fit(m, n, lda_b, ldb_kmajor, k_bytes);
-    const int tile = pick_tile(m, n, k_bytes, false, false, dma_ok);
+    const int tile = pick_tile(m, n, k_bytes, false, false, dma_ok, op == TOP_BF16 || op == TOP_F16 || op == TOP_I8);
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
     set_last_kernel(tile_kernel_name(tile, op));
     return PTOAMD_OK;
@@ -642,8 +653,8 @@ int ptoamd_gemm_w8a8(void* out_bf16, int32_t* acc_out, const int8_t* a, const in
     p.m = m; p.n = n; p.k_bytes = k; p.lda_bytes = lda; p.ldb_bytes = ldb; p.ldc = ldc;
     p.out_kind = OUT_W8A8_BF16; p.group_m = 4;
     p.b_nd = b_in_kernel; p.b_esz = 1;
-    const bool dma_ok = !b_in_kernel && aligned16(a) && aligned16(b) && (lda % 16) == 0 && (ldb % 16) == 0 && dma_offsets_fit(m, n, lda, ldb, k);
-    const int tile = pick_tile(m, n, k, false, false, dma_ok);
+    const bool dma_ok = !b_in_kernel && aligned4(a) && aligned4(b) && (lda % 4) == 0 && (ldb % 4) == 0 && dma_offsets_fit(m, n, lda, ldb, k);
+    const int tile = pick_tile(m, n, k, false, false, dma_ok, true);
     PTOAMD_HIP_CHECK(launch_tiles(tile, TOP_I8, p, stream));
     set_last_kernel(tile_kernel_name(tile, TOP_I8));
     return PTOAMD_OK;

@@ -80,9 +80,16 @@ __host__ __device__ constexpr int dma_phase_begin(int phase)
     return eighths * NDMA / 8;
 }
 
-template <class Cfg>
+// RAGGED: K is not a whole number of 128-byte slabs (and at least one).  The last slab's copy-in then goes lane by
+// lane: a chunk that lies inside its row is DMAed as always, the chunk the row ends in is read through registers as the
+// 16 bytes that END at the row's end (nothing past a row is touched) and written to the lane's LDS position with the
+// bytes past K zero, and chunks past K are written as zeros -- so the MFMAs run over a whole slab and the products
+// beyond K vanish.  A compile-time form: the kernel for whole slabs carries none of it.  Its slabs go out in one DMA
+// phase, so that a slab is requested in exactly one place.
+template <class Cfg, bool RAGGED = false>
 __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileGemmParams p)
 {
+    static_assert(!RAGGED || (Cfg::RING == 2 && !Cfg::Op::SCALED), "the ragged-K form exists for the two-slab ring of the plain types");
     using Op = typename Cfg::Op;
     using Acc = typename Op::Acc;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, MB = Cfg::MB, NB = Cfg::NB, LA = Cfg::LA, LB = Cfg::LB;
@@ -121,7 +128,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
 #pragma unroll
     for (int i = 0; i < LB; ++i)
         goff_b[i] = (uint32_t)((long)min(n0 + ld_row + i * (NT / 8), p.n - 1) * p.ldb_bytes + ld_chunk * 16);
-    const int k_slabs = p.k_bytes / 128;
+    const int k_slabs = RAGGED ? (p.k_bytes + 127) / 128 : p.k_bytes / 128;
 
     const uint32_t lds_wave_base = __builtin_amdgcn_readfirstlane(lds_address(smem) + wave * 1024);
     // DMA number q (0 .. LA + LB - 1) of slab kt into ring buffer buf
@@ -132,7 +139,27 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         else
             lds_dma16_off(p.b + (long)kt * 128, goff_b[q - LA], dst + Cfg::A_BYTES + (q - LA) * (NT * 16));
     };
+    // the same for the last slab of a ragged K (see RAGGED above)
+    auto tload_piece_last = [&](int buf, int q) __attribute__((always_inline)) {
+        const int kt = k_slabs - 1;
+        const int rem = p.k_bytes - kt * 128 - ld_chunk * 16;  // bytes of the lane's row from its chunk on
+        const bool is_a = q < LA;
+        const int piece = is_a ? q : q - LA;
+        const int lds_off = buf * Cfg::STAGE_BYTES + (is_a ? 0 : Cfg::A_BYTES) + piece * (NT * 16);
+        const uint8_t* base = (is_a ? p.a : p.b) + (long)kt * 128;
+        const uint32_t goff = is_a ? goff_a[piece] : goff_b[piece];
+        if (rem >= 16)
+            lds_dma16_off(base, goff, lds_wave_base + lds_off);
+        else
+            *reinterpret_cast<uint4*>(smem + lds_off + tid * 16) = load_chunk_tail(base + goff, rem);
+    };
     auto tload = [&](int kt, int buf) __attribute__((always_inline)) {
+        if (RAGGED && kt == k_slabs - 1) {
+#pragma unroll
+            for (int q = 0; q < LA + LB; ++q)
+                tload_piece_last(buf, q);
+            return;
+        }
 #pragma unroll
         for (int q = 0; q < LA + LB; ++q)
             tload_piece(kt, buf, q);
@@ -249,9 +276,10 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     };
     // One k-step: the MFMAs of step s (register set s & 1), with the fragment reads of the next step (register set
     // (s + 1) & 1, from buffer rbuf step rs) and, in a slab's last step, the DMAs of slab dkt spread between them.
-    auto kstep = [&](auto phase, int s, bool reads, int rbuf, int rs, bool dmas, int dkt, int dbuf) __attribute__((always_inline)) {
+    auto kstep = [&](auto phase, int s, bool reads, int rbuf, int rs, bool dmas, int dkt, int dbuf, auto lastdma) __attribute__((always_inline)) {
         constexpr int PH = decltype(phase)::value;
-        constexpr int DQ0 = dma_phase_begin<NDMA, KS, BLK, (Cfg::RING > 2)>(PH), DN = dma_phase_begin<NDMA, KS, BLK, (Cfg::RING > 2)>(PH + 1) - DQ0;
+        constexpr bool LASTDMA = decltype(lastdma)::value;  // the DMAs of this k-step are those of a ragged K's last slab
+        constexpr int DQ0 = dma_phase_begin<NDMA, KS, BLK, (Cfg::RING > 2 || RAGGED)>(PH), DN = dma_phase_begin<NDMA, KS, BLK, (Cfg::RING > 2 || RAGGED)>(PH + 1) - DQ0;
         constexpr int DSPAN = (BLK == 16 && PH > 0) ? NMMA / 2 : NMMA;  // MFMAs the phase's DMAs are spread over
         const int set = SETS == 2 ? (s & 1) : 0;
         const int nset = SETS == 2 ? (set ^ 1) : 0;
@@ -295,7 +323,12 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
             if (dmas) {
                 constexpr int xa = x < DSPAN ? x : DSPAN, xb = x + 1 < DSPAN ? x + 1 : DSPAN;
                 constexpr int q0 = DQ0 + xa * DN / DSPAN, q1 = DQ0 + xb * DN / DSPAN;
-                static_for<q1 - q0>([&](auto qc) { tload_piece(dkt, dbuf, q0 + decltype(qc)::value); });
+                static_for<q1 - q0>([&](auto qc) {
+                    if constexpr (LASTDMA)
+                        tload_piece_last(dbuf, q0 + decltype(qc)::value);
+                    else
+                        tload_piece(dkt, dbuf, q0 + decltype(qc)::value);
+                });
             }
         });
         if constexpr (SETS == 2 && !HYBRID)
@@ -312,7 +345,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // slab 1's first DMAs go out now but only slab 0 (and the scales) are waited for: the counter retires loads in
     // order, so "at most N1 outstanding" means everything issued before slab 1's pieces has landed; slab 1 is covered
     // by the first slab's barrier
-    constexpr int N1 = dma_phase_begin<NDMA, KS, BLK, (Cfg::RING > 2)>(1);
+    constexpr int N1 = dma_phase_begin<NDMA, KS, BLK, (Cfg::RING > 2 || RAGGED)>(1);
     // A deeper ring starts slabs 1 .. RING - 1 whole as well (it is built for the types whose slab goes out in one
     // phase), so that from the first slab on the copy-in runs RING - 1 slabs ahead.  At the barrier of slab kt the ring
     // may leave WAITN DMAs in flight: those of the slabs after kt + 1, but no more than were issued after the scale
@@ -327,6 +360,9 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     } else if (RING > 2) {
         for (int s1 = 1; s1 < k_slabs; ++s1)
             tload(s1, s1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+    } else if (RAGGED && k_slabs > 1) {
+        tload(1, 1);  // (one phase: N1 = NDMA; slab 1 may be the ragged last one, whose register-loaded chunks are not DMAs)
         __builtin_amdgcn_s_waitcnt(0x0F70);
     } else if (k_slabs > 1) {
         static_for<N1>([&](auto qc) { tload_piece(1, 1, decltype(qc)::value); });
@@ -345,7 +381,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
     // (always_inline: out of line, a lambda takes the accumulators by reference and they live in scratch memory)
     // `cur` / `nxt`: ring buffers of slab kt and kt + 1; slab kt + RING - 1 ... goes into the buffer slab kt frees.
     // `steady`: slabs kt + 1 .. kt + RING - 1 are all in flight or landed (the barrier may then leave WAITN DMAs pending).
-    auto slab = [&](int kt, int cur, bool more, bool dma, auto steady) __attribute__((always_inline)) {
+    auto slab = [&](int kt, int cur, bool more, bool dma, auto steady, auto lastdma) __attribute__((always_inline)) {
         const int nxt = RING == 2 ? (cur ^ 1) : (cur + 1 == RING ? 0 : cur + 1);
         if (Op::SCALED) {
             // The request for the next scale chunk sits here, at the top of the slab, and not between two k-steps: a
@@ -369,7 +405,7 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         }
         static_for<KS - 1>([&](auto sc) {
             constexpr int s = decltype(sc)::value;
-            kstep(std::integral_constant<int, s + 1>{}, s, true, cur, s + 1, more, kt + 1, nxt);
+            kstep(std::integral_constant<int, s + 1>{}, s, true, cur, s + 1, more, kt + 1, nxt, std::false_type{});
         });
         // every wave is done reading slab kt, and its DMAs of slab kt+1 (issued RING - 1 slabs ago) have landed
         constexpr int WN = decltype(steady)::value ? WAITN : 0;
@@ -377,32 +413,39 @@ __global__ void __launch_bounds__(Cfg::THREADS) gemm_tile_dtl_kernel(const TileG
         __syncthreads();
         if (SC_AHEAD && more)
             read_scales(kt + 1);
-        kstep(std::integral_constant<int, 0>{}, KS - 1, more, nxt, 0, dma, kt + RING, cur);
+        kstep(std::integral_constant<int, 0>{}, KS - 1, more, nxt, 0, dma, kt + RING, cur, lastdma);
     };
     int kt = 0, cur = 0;
     if constexpr (RING == 2) {
-        for (; kt + 2 < k_slabs; ++kt)
-            slab(kt, kt & 1, true, true, std::true_type{});
+        // (ragged K: the slab that requests the last one is peeled off the loop)
+        for (; kt + (RAGGED ? 3 : 2) < k_slabs; ++kt)
+            slab(kt, kt & 1, true, true, std::true_type{}, std::false_type{});
+        if constexpr (RAGGED) {
+            if (kt + 2 < k_slabs) {
+                slab(kt, kt & 1, true, true, std::true_type{}, std::true_type{});
+                ++kt;
+            }
+        }
         if (kt + 1 < k_slabs) {
-            slab(kt, kt & 1, true, false, std::false_type{});
+            slab(kt, kt & 1, true, false, std::false_type{}, std::false_type{});
             ++kt;
         }
-        slab(kt, kt & 1, false, false, std::false_type{});
+        slab(kt, kt & 1, false, false, std::false_type{}, std::false_type{});
     } else {
         const auto advance = [&]() {
             ++kt;
             cur = cur + 1 == RING ? 0 : cur + 1;
         };
         while (kt + RING < k_slabs) {
-            slab(kt, cur, true, true, std::true_type{});
+            slab(kt, cur, true, true, std::true_type{}, std::false_type{});
             advance();
         }
         // the last RING slabs (or fewer): nothing more to start; the barrier waits for everything in flight
         while (kt + 1 < k_slabs) {
-            slab(kt, cur, true, false, std::false_type{});
+            slab(kt, cur, true, false, std::false_type{}, std::false_type{});
             advance();
         }
-        slab(kt, cur, false, false, std::false_type{});
+        slab(kt, cur, false, false, std::false_type{}, std::false_type{});
     }
 
     // ---- TSTORE.  No wave reads the ring after the last slab's barrier (its fragment reads were issued before it) and

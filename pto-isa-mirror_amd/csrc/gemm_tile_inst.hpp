@@ -24,16 +24,35 @@ static hipError_t launch_cfg(const TileGemmParams& p, hipStream_t stream)
     return hipGetLastError();
 }
 
-template <class Cfg>
+// RAGGED_K: this tile also exists in the form that takes a K extent of any length (the plain types' 256 x 256 and
+// 128 x 128 tiles); the launcher picks it when K is not a whole number of 128-byte slabs.
+template <class Cfg, bool RAGGED_K = false>
 static hipError_t launch_dtl(const TileGemmParams& p, hipStream_t stream)
 {
-    const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_dtl_kernel<Cfg>), Cfg::LDS_BYTES);
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_dtl_kernel<Cfg, false>), Cfg::LDS_BYTES);
+    if constexpr (RAGGED_K) {
+        if (e == hipSuccess)
+            e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_dtl_kernel<Cfg, true>), Cfg::LDS_BYTES);
+    }
     if (e != hipSuccess || p.m <= 0)
         return e;
     const int tiles = ((p.m + Cfg::BM - 1) / Cfg::BM) * ((p.n + Cfg::BN - 1) / Cfg::BN);
-    hipLaunchKernelGGL(gemm_tile_dtl_kernel<Cfg>, dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
+    if (p.k_bytes % 128 != 0) {
+        if constexpr (RAGGED_K) {
+            hipLaunchKernelGGL((gemm_tile_dtl_kernel<Cfg, true>), dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
+            return hipGetLastError();
+        }
+        return hipErrorInvalidValue;  // the dispatcher sends such a K to this form only where it exists
+    }
+    hipLaunchKernelGGL((gemm_tile_dtl_kernel<Cfg, false>), dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
     return hipGetLastError();
 }
+
+#ifdef PTOAMD_TILE_RAGGED_K
+#define PTOAMD_RK true
+#else
+#define PTOAMD_RK false
+#endif
 
 hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 {
@@ -51,12 +70,12 @@ hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
         // and a third of this translation unit's compile time; the id now selects tile 4)
 #ifdef PTOAMD_TILE_OP16  // the large eight-wave tile runs on the 16x16 instructions where the operand type has them
         case 3:
-        case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP16>>(p, stream);
+        case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP16>, PTOAMD_RK>(p, stream);
 #else
         case 3:
-        case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>>(p, stream);
+        case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>, PTOAMD_RK>(p, stream);
 #endif
-        case 5: return launch_dtl<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>>(p, stream);
+        case 5: return launch_dtl<TileCfg<128, 128, 2, 2, PTOAMD_TILE_OP>, PTOAMD_RK>(p, stream);
         case 6: return launch_dtl<TileCfg<256, 128, 4, 2, PTOAMD_TILE_OP>>(p, stream);
 #ifdef PTOAMD_TILE_RING3  // block-scaled types: the 256 x 128 tile with a ring of three slabs
         case 7: return launch_dtl<TileCfg<256, 128, 4, 2, PTOAMD_TILE_OP, 3>>(p, stream);

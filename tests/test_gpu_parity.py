@@ -192,11 +192,15 @@ TILE_NAMES = ("tile256x256_", "tile128x128_", "tile64x64_", "tile256x256w4_dtl",
 ALL_TILES = [1, 2, 4, 5, 6]  # (ids 0 and 3, a register-staged and a four-wave 256 x 256 tile, are no longer built: they select 1 and 4)
 
 
-def expect_tile(pa, tile, k_bytes):
-    """Tiles 3-6 need whole 128-byte K slabs; otherwise the dispatcher falls back to the register-staged tile."""
+def expect_tile(pa, tile, k_bytes, ragged_k_form=False):
+    """The DMA tiles need whole 128-byte K slabs -- except tiles 4 and 5 of bf16 / f16 / int8 (ragged_k_form), which
+    take any K longer than one slab; otherwise the dispatcher falls back to the register-staged tile."""
     name = pa.last_kernel()
     if tile >= 3 and k_bytes % 128:
-        assert name.startswith("tile128x128_"), name
+        if ragged_k_form and k_bytes > 128:
+            assert name.startswith(TILE_NAMES[tile if tile in (4, 5) else 5]), name
+        else:
+            assert name.startswith("tile128x128_"), name
     else:
         assert name.startswith(TILE_NAMES[tile]), name
 
@@ -210,7 +214,7 @@ def test_bf16_gemm_every_tile_shape(pa, oracle, tile, m, n, k):
     ref = oracle.matmul_bf16(a, b, b_dn=True)
     with tile_env(PTOAMD_TILE=tile):
         got32 = host(pa.gemm(dev(a).view(torch.bfloat16), dev(b).view(torch.bfloat16), pa.BF16, pa.F32, pa.B_DN))
-        expect_tile(pa, tile, 2 * k)
+        expect_tile(pa, tile, 2 * k, ragged_k_form=True)
         got16 = host(pa.gemm(dev(a).view(torch.bfloat16), dev(b).view(torch.bfloat16), pa.BF16, pa.BF16, pa.B_DN))
     absdot = np.abs(bf16_to_f32(a).astype(np.float64)) @ np.abs(bf16_to_f32(b).astype(np.float64)).T
     check_f32_drain(got32, ref, absdot, k, f"bf16 {m}x{n}x{k} tile {tile}")
@@ -1359,6 +1363,45 @@ def test_unaligned_rows_stay_on_the_mfma_tiles(pa, oracle, kind, m, k, n, b_dn, 
     check_f32_drain(got, ref, np.abs(fa) @ (np.abs(fb).T if b_dn else np.abs(fb)), k, f"unaligned {kind} {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("tile", [4, 5])
+@pytest.mark.parametrize("kind,k", [("i8", 132), ("i8", 260), ("i8", 388), ("i8", 516), ("i8", 1300), ("i8", 376),
+                                    ("bf16", 66), ("bf16", 130), ("bf16", 194), ("bf16", 1034), ("f16", 322)])
+def test_dma_tiles_take_a_ragged_k(pa, oracle, kind, k, tile):
+    """K that is not a whole number of 128-byte slabs on the LDS-DMA tiles (rows 4-byte aligned): 2, 3, 4, 5 and 11
+    slabs, tails of 4 and 120 bytes.  The last slab's chunks past K are zero in LDS whatever lies behind the rows in
+    memory -- the rows are packed, so behind a row lies the next one, and the matrices are followed by NaN / 0x7F bytes.
+    Integer results are exact; float results are compared with the register-staged tile (same slabs, same k-steps) bit
+    for bit and with the oracle."""
+    r = np.random.default_rng(k * 5 + tile)
+    m, n = 300, 260
+    if kind == "i8":
+        a = np.concatenate([r.integers(-128, 128, m * k), np.full(64, 127)]).astype(np.int8)
+        b = np.concatenate([r.integers(-128, 128, n * k), np.full(64, 127)]).astype(np.int8)
+        ta, tc, tdt = pa.I8, pa.I32, torch.int8
+    else:
+        conv = (lambda x: x.astype(np.float16).view(np.uint16)) if kind == "f16" else bf16_bits
+        a = np.concatenate([conv(r.uniform(-1, 1, m * k).astype(np.float32)), np.full(64, 0x7FC0 if kind == "bf16" else 0x7E00, np.uint16)])
+        b = np.concatenate([conv(r.uniform(-1, 1, n * k).astype(np.float32)), np.full(64, 0x7FC0 if kind == "bf16" else 0x7E00, np.uint16)])
+        ta, tc, tdt = (pa.F16 if kind == "f16" else pa.BF16), pa.F32, (torch.float16 if kind == "f16" else torch.bfloat16)
+    da = (dev(a) if kind == "i8" else dev(a).view(tdt))[:m * k].view(m, k)
+    db = (dev(b) if kind == "i8" else dev(b).view(tdt))[:n * k].view(n, k)
+    with tile_env(PTOAMD_TILE=tile):
+        got = host(pa.gemm(da, db, ta, tc, pa.B_DN))
+        assert "_dtl_" in pa.last_kernel(), pa.last_kernel()
+    a2, b2 = a[:m * k].reshape(m, k), b[:n * k].reshape(n, k)
+    if kind == "i8":
+        assert np.array_equal(got, oracle.matmul_i8(a2, b2, b_dn=True))
+        return
+    with tile_env(PTOAMD_TILE=1):
+        other = host(pa.gemm(da, db, ta, tc, pa.B_DN))
+        assert pa.last_kernel().startswith("tile128x128_"), pa.last_kernel()
+    assert not np.isnan(got).any()
+    if tile == 5:   # the 128 x 128 DMA tile and the register-staged one share the 32 x 32 instruction and the k order
+        assert np.array_equal(got.view(np.uint32), other.view(np.uint32))
+    ref = (oracle.matmul_f16 if kind == "f16" else oracle.matmul_bf16)(a2, b2, b_dn=True)
+    assert relerr(got, ref) <= 1e-4
+
+
 def test_unaligned_k_large_int8_product(pa, oracle):
     """int8 2048 x 2048 x 8200 (K is 8 bytes past a multiple of 16, every second row misaligned): an MFMA tile runs it;
     512 sampled outputs are exact."""
@@ -1367,7 +1410,7 @@ def test_unaligned_k_large_int8_product(pa, oracle):
     a = torch.randint(-128, 128, (m, k), generator=gen, device=DEV, dtype=torch.int8)
     b = torch.randint(-128, 128, (n, k), generator=gen, device=DEV, dtype=torch.int8)
     got = host(pa.gemm(a, b, pa.I8, pa.I32, pa.B_DN))
-    assert pa.last_kernel().startswith("tile"), pa.last_kernel()
+    assert pa.last_kernel() == "tile128x128_dtl_i8", pa.last_kernel()   # rows 4-byte aligned: the LDS-DMA tile, ragged-K form
     rows = np.array([0, 1, 127, 128, 1023, 2046, 2047, 77])
     cols = np.arange(0, 2048, 32) + np.arange(64) % 32
     ref = oracle.matmul_i8(host(sel(a, rows)), host(sel(b, cols)), b_dn=True)
@@ -1383,6 +1426,7 @@ def test_row_major_b_through_a_workspace(pa, oracle):
     b = (torch.randn((k, n), generator=gen, device=DEV) * 0.1).to(torch.bfloat16)
     ws = torch.empty(pa.gemm_workspace_bytes(n, k, pa.BF16, pa.B_ND), dtype=torch.uint8, device=DEV)
     assert ws.numel() == n * k * 2 and pa.gemm_workspace_bytes(n, k, pa.BF16, pa.B_DN) == 0
+    assert pa.gemm_workspace_bytes(10, 33, pa.I8, pa.B_ND) == 10 * 48   # rows of the re-ordered copy are padded to 16 bytes
     got = pa.gemm(a, b, pa.BF16, pa.F32, pa.B_ND, workspace=ws)
     assert "dtl" in pa.last_kernel(), pa.last_kernel()
     same = pa.gemm(a, b.t().contiguous(), pa.BF16, pa.F32, pa.B_DN)
