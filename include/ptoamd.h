@@ -123,8 +123,9 @@ int ptoamd_event_elapsed_ms(float* ms, void* start, void* stop);
  *   c_in    : optional accumulator input (TMATMUL_ACC), same type as the accumulator (f32 / i32), ld = ldc; may be NULL
  *   relu    : flags: PTOAMD_RELU (1) = TSTORE's ReluPreMode::NormalRelu; PTOAMD_SATURATE_INF (2), quantising drains only
  * No alignment is asked of a, b or the leading dimensions beyond that of an element: rows of 16 bytes or more run on the
- * MFMA tiles whatever their alignment (the LDS-DMA tiles when rows are 16-byte aligned and K is a whole number of
- * 128-byte slabs, the register-staged tiles otherwise; a row-major B is transposed on its way into LDS by the latter).
+ * MFMA tiles whatever their alignment: the LDS-DMA tiles when rows start on 4-byte boundaries (bf16 / f16 / int8: any K
+ * longer than 128 bytes; fp8: K a whole number of 128-byte slabs), the register-staged tiles otherwise; a row-major B is
+ * transposed on its way into LDS by the latter.  Rows of C need no alignment either.
  * PTOAMD_F32 and PTOAMD_HIF8 operands (hif8 x hif8 only, cpu/TMatmul.hpp:38) run on the order-exact kernel: one thread
  * per output, k ascending, fmaf -- the simulator's arithmetic bit for bit.  No entry point of this group allocates.
  */
@@ -144,7 +145,7 @@ int ptoamd_gemm_bias(void* c, int c_type, const void* a, const void* b, int ab_t
 
 /*
  * ptoamd_gemm_bias with a caller-owned workspace for a row-major B (PTOAMD_B_ND): B is re-ordered into the workspace once
- * ([N][K], ptoamd_gemm_workspace_bytes(n, k, ab_type, b_layout) bytes, 256-byte aligned) and the product then runs on the
+ * ([N][K] with rows padded to 16 bytes, ptoamd_gemm_workspace_bytes(n, k, ab_type, b_layout) bytes, 256-byte aligned) and the product then runs on the
  * fastest tiles, where ptoamd_gemm transposes B inside the loader of the register-staged tiles for every tile row of C --
  * the better choice for small M, the slower one for large M.  workspace == NULL is ptoamd_gemm_bias.  No counterpart in
  * the reference (its TLOAD re-orders an ND panel into L1 per tile, cpu/TLoad.hpp:287-321).
