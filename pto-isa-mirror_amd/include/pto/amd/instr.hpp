@@ -747,8 +747,9 @@ PTO_INST float quant_word_scale(uint64_t word)
 {
     return ptoamd::fixpipe_word_scale<VECTOR>(word);
 }
+// sat_inf: bit 48 of the task cookie, read once per instruction by the caller
 template <bool VECTOR, typename G, typename Reg>
-PTO_INST float quantize_element(Reg acc, uint64_t word)
+PTO_INST float quantize_element(Reg acc, uint64_t word, bool sat_inf = false)
 {
     constexpr bool src_is_int = std::is_integral_v<Reg>;
     static_assert(std::is_same_v<G, int8_t> || std::is_same_v<G, uint8_t> || std::is_same_v<G, _Float16> || std::is_same_v<G, __bf16> ||
@@ -763,12 +764,40 @@ PTO_INST float quantize_element(Reg acc, uint64_t word)
     } else if constexpr (sizeof(G) == 1) {
         r = ptoamd::fixpipe_quantize<VECTOR, true, src_is_int>((float)acc, word);
     } else if constexpr (std::is_same_v<G, _Float16>) {
-        r = ptoamd::fixpipe_quantize<VECTOR, false, src_is_int>((float)acc, word);
+        if (!src_is_int && sat_inf)
+            r = ptoamd::fixpipe_saturate_inf<true>(r);
+        else
+            r = ptoamd::fixpipe_quantize<VECTOR, false, src_is_int>((float)acc, word);
     } else {
-        if (r == r && fabsf(r) != __builtin_inff())
+        if (sat_inf)
+            r = ptoamd::fixpipe_saturate_inf<false>(r);
+        else if (r == r && fabsf(r) != __builtin_inff())
             r = r < -3.402823466e38f ? -3.402823466e38f : (r > 3.402823466e38f ? 3.402823466e38f : r);
     }
     return r;
+}
+
+// The same from an on-chip buffer tile (the reference's TSTORE quantises whatever tile it is given, cpu/TStore.hpp:41-62;
+// its tstore_quant tests drain Vec tiles of float / int32): element by element over the valid region.
+template <bool VECTOR, typename TileData, typename GlobalData, ReluPreMode relu, typename WordOf>
+PTO_INST void tstore_lds_quant(GlobalData& dst, TileData& src, WordOf&& word_of)
+{
+    using T = typename TileData::DType;
+    using G = typename GlobalData::DType;
+    static_assert(std::is_same_v<T, float> || std::is_same_v<T, int32_t>, "the fix-pipe quantises float or int32 values");
+    acquire(src);
+    __syncthreads();  // writers of the tile (and of the Scaling tile the words come from) are done
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    auto* g = reinterpret_cast<G*>(dst.data());
+    const uint8_t* base = src.Storage();
+    const bool sat_inf = (get_task_cookie() >> 48) & 1u;
+    for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
+        const int r = idx / vc, c = idx - r * vc;
+        float v = quantize_element<VECTOR, G>(*reinterpret_cast<const T*>(base + src.ByteOffset(r, c)), word_of(c), sat_inf);
+        if constexpr (relu == ReluPreMode::NormalRelu)
+            v = v > 0 ? v : 0;
+        g[dst.Offset(r, c)] = static_cast<G>(v);
+    }
 }
 
 template <bool VECTOR, typename TileRes, typename GlobalData, ReluPreMode relu, typename WordOf>
@@ -777,9 +806,10 @@ PTO_INST void tstore_acc_quant(GlobalData& dst, TileRes& src, WordOf&& word_of)
     using G = typename GlobalData::DType;
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
     auto* g = reinterpret_cast<G*>(dst.data());
+    const bool sat_inf = (get_task_cookie() >> 48) & 1u;
     for_each_acc(src, [&](int slot, int r, int row, int col) {
         if (row < vr && col < vc) {
-            float v = quantize_element<VECTOR, G>(src.regs[slot][r], word_of(col));
+            float v = quantize_element<VECTOR, G>(src.regs[slot][r], word_of(col), sat_inf);
             if constexpr (relu == ReluPreMode::NormalRelu)
                 v = v > 0 ? v : 0;
             g[dst.Offset(row, col)] = static_cast<G>(v);
@@ -819,21 +849,29 @@ template <typename TileData, typename GlobalData, AtomicType atomicType = Atomic
 PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, uint64_t preQuantScalar)
 {
     PTO_AMD_TRACE_INSTR(1, TR_TSTORE, dst, src);
-    static_assert(TileData::Loc == TileType::Acc && atomicType == AtomicType::AtomicNone, "quantising TSTORE drains an accumulator tile");
-    amd::tstore_acc_quant<false, TileData, GlobalData, reluPreMode>(dst, src, [&](int) { return preQuantScalar; });
+    static_assert(atomicType == AtomicType::AtomicNone, "the quantising TSTORE does not add atomically");
+    if constexpr (TileData::Loc == TileType::Acc)
+        amd::tstore_acc_quant<false, TileData, GlobalData, reluPreMode>(dst, src, [&](int) { return preQuantScalar; });
+    else
+        amd::tstore_lds_quant<false, TileData, GlobalData, reluPreMode>(dst, src, [&](int) { return preQuantScalar; });
     return {};
 }
+// (the words come from a Scaling tile, or -- as the reference's tstore_quant tests have it -- from a one-row Vec tile of
+// 64-bit elements)
 template <typename TileData, typename GlobalData, typename FpTileData, AtomicType atomicType = AtomicType::AtomicNone,
           ReluPreMode reluPreMode = ReluPreMode::NoRelu,
-          typename = std::enable_if_t<is_tile_data_v<FpTileData> && FpTileData::Loc == TileType::Scaling>>
+          typename = std::enable_if_t<is_tile_data_v<FpTileData> && (FpTileData::Loc == TileType::Scaling || FpTileData::Loc == TileType::Vec) &&
+                                      sizeof(typename FpTileData::DType) == 8>>
 PTO_INST RecordEvent TSTORE(GlobalData& dst, TileData& src, FpTileData& fp)
 {
     PTO_AMD_TRACE_INSTR(1, TR_TSTORE_FP, dst, src, fp);
-    static_assert(TileData::Loc == TileType::Acc && atomicType == AtomicType::AtomicNone, "quantising TSTORE drains an accumulator tile");
-    static_assert(sizeof(typename FpTileData::DType) == 8, "the Scaling tile holds one 64-bit quantisation word per column");
+    static_assert(atomicType == AtomicType::AtomicNone, "the quantising TSTORE does not add atomically");
     const uint8_t* words = fp.Storage();
-    amd::tstore_acc_quant<true, TileData, GlobalData, reluPreMode>(
-        dst, src, [&](int col) { return *reinterpret_cast<const uint64_t*>(words + fp.ByteOffset(0, col)); });
+    const auto word_of = [&](int col) { return *reinterpret_cast<const uint64_t*>(words + fp.ByteOffset(0, col)); };
+    if constexpr (TileData::Loc == TileType::Acc)
+        amd::tstore_acc_quant<true, TileData, GlobalData, reluPreMode>(dst, src, word_of);
+    else
+        amd::tstore_lds_quant<true, TileData, GlobalData, reluPreMode>(dst, src, word_of);
     return {};
 }
 
@@ -857,6 +895,7 @@ PTO_INST void tmov_acc(DstTile& dst, SrcTile& src, int row0, int col0, WordOf&& 
     using D = typename DstTile::DType;
     const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
     uint8_t* d = dst.Storage();
+    const bool sat_inf = QUANT != 0 && ((get_task_cookie() >> 48) & 1u);
     __syncthreads();
     for_each_acc(src, [&](int slot, int r, int row, int col) {
         const int dr = row - row0, dc = col - col0;
@@ -867,7 +906,7 @@ PTO_INST void tmov_acc(DstTile& dst, SrcTile& src, int row0, int col0, WordOf&& 
                     v = v > 0 ? v : 0;
                 *reinterpret_cast<D*>(d + dst.ByteOffset(dr, dc)) = convert<D>(v);
             } else {
-                float v = quantize_element<QUANT == 2, D>(src.regs[slot][r], word_of(col));
+                float v = quantize_element<QUANT == 2, D>(src.regs[slot][r], word_of(col), sat_inf);
                 if constexpr (relu == ReluPreMode::NormalRelu)
                     v = v > 0 ? v : 0;
                 *reinterpret_cast<D*>(d + dst.ByteOffset(dr, dc)) = static_cast<D>(v);

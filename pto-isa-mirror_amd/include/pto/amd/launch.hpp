@@ -112,6 +112,14 @@ inline int device_status()
     return v;
 }
 
+// sets the task cookie the cores of this translation unit read (reference: set_task_cookie, common/cpu_stub.hpp:498);
+// a synchronous copy: launches that follow see it
+inline int set_task_cookie(uint64_t cookie)
+{
+    const unsigned long long v = cookie;
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_task_cookie), &v, sizeof v);
+}
+
 // clears the status word (after a test that provoked a violation on purpose)
 inline int reset_device_status()
 {

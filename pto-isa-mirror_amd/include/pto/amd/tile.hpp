@@ -64,6 +64,11 @@ static_assert(LDS_TOTAL <= 160 * 1024, "the on-chip regions must fit the 160 KiB
 // (1: TASSIGN address outside its region, 2: TQUANT NZ mode on a tile that is not whole 16-row x 2-group boxes).
 // pto::amd::device_status() reads it on the host.
 static __device__ int g_status = 0;
+// The task cookie of this translation unit's cores (reference: get_task_cookie(), common/cpu_stub.hpp:606-612): control
+// bits the fix-pipe consults; bit 48 = saturate non-finite results of the half / bfloat16 quantising drains
+// (cpu/common.hpp:143-171).  pto::amd::set_task_cookie() writes it from the host.
+static __device__ unsigned long long g_task_cookie = 0;
+__device__ __forceinline__ uint64_t get_task_cookie() { return g_task_cookie; }
 __device__ __forceinline__ void report(int code)
 {
     if (threadIdx.x == 0)

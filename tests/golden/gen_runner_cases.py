@@ -1,7 +1,7 @@
 """Writes the data of the framework-free case runner (tests/pto_kernels/case_runner.hip): inputs and goldens of the
 reference's own test lists for the matmul path -- tests/cpu/st/testcase/tmatmul/main.cpp:96-252 (case1-4, gemm_1/2, bf16_1,
 bias_1/2/5/gemm, bf16_bias_1), tmatmul_mx/main.cpp:151-330 (case1-19), tstore_acc2gm/main.cpp:220-247 (nz2nd and scalar
-quantisation cases), tdequant/gen_data.py:69-72 -- with shapes, element types and value distributions taken from those
+quantisation cases), tstore_quant/main.cpp:112-130 (ND_1 ... ND_10), tquant/main.cpp:161-777, tdequant/gen_data.py:69-72 -- with shapes, element types and value distributions taken from those
 files and their gen_data.py, the inputs drawn from this script's own seeds, and every golden computed by the oracle
 (oracle/pto_oracle.c), not by the runner.
 
@@ -181,6 +181,112 @@ for case, dt, rows, cols in (("case1", np.int8, 64, 64), ("case2", np.int16, 32,
     scale, off = rng.uniform(0.01, 2.0, rows).astype(np.float32), rng.uniform(-20, 20, rows).astype(np.float32)
     put("tdequant", case, x1_gm=src, x2_gm=scale, bias_gm=off, golden=orc.tdequant(src, scale, off))
     line("tdequant", case, "dequant", rows, 0, cols, "i8" if dt == np.int8 else "i16", "f32", "f32", 0, 0.001)
+
+# ---- tstore_quant (tstore_quant/main.cpp:112-130, tstore_quant/gen_data.py:46-64,170-186): a Vec tile of float / int32
+# integers in [-5, 5) leaves through the quantising TSTORE; ND cases are [g0 g1 g2 g3][g4] row-major, DN cases
+# [g3][g0 g1 g2 g4] stored column by column.  Words: scale in [0, 5), offset in [0, 512), a shift count, bit 46 for int8.
+def quant_words(dst, count):
+    out = []
+    for _ in range(count):
+        bits = int(np.float32(rng.uniform(0.0, 5.0)).view(np.uint32))
+        out.append((int(rng.integers(0, 16)) << 32) | ((1 << 46) if dst == "i8" else 0) | (int(rng.integers(0, 512)) << 37) | bits)
+    return np.array(out, np.uint64)
+
+
+ST["i16"] = ob.ST_I16
+for cid, (fmt, src, dst, g, vq, sat, relu) in enumerate([
+        ("ND", "f32", "i8", (1, 1, 1, 2, 128), True, True, True), ("ND", "i32", "i16", (1, 2, 1, 23, 121), True, True, False),
+        ("ND", "i32", "i8", (2, 2, 3, 23, 47), True, False, True), ("DN", "f32", "f16", (1, 1, 1, 4, 21), False, True, True),
+        ("DN", "f32", "f16", (3, 1, 1, 1, 124), False, False, False), ("DN", "i32", "i8", (2, 1, 2, 32, 32), False, True, False),
+        ("DN", "f32", "f16", (1, 1, 1, 16, 8), False, False, True), ("DN", "i32", "i16", (2, 2, 2, 16, 16), False, False, False),
+        ("DN", "i32", "i8", (1, 2, 1, 16, 32), True, True, True), ("ND", "f32", "f16", (1, 1, 1, 16, 16), True, False, False)], 1):
+    rows, cols = (g[0] * g[1] * g[2] * g[3], g[4]) if fmt == "ND" else (g[3], g[0] * g[1] * g[2] * g[4])
+    x = rng.integers(-5, 5, (rows, cols)).astype(np.float32 if src == "f32" else np.int32)
+    words = quant_words(dst, cols if vq else 1)
+    golden = orc.store_quant(x, ST[dst], words, int(vq), relu=relu, saturate_inf=int(sat))
+    if fmt == "DN":  # memory holds the matrix column by column
+        x, golden = np.ascontiguousarray(x.T), np.ascontiguousarray(golden.T)
+    case = f"{fmt}_{cid}"
+    put("tstore_quant", case, input=x, quant=words, golden=golden)
+    line("tstore_quant", case, "storeq_tile", rows, 0, cols, src, src, dst, f"{cid}:{int(sat)}", 0, f"q{cid}")
+
+
+# ---- tquant (tquant/main.cpp:161-777: INT8 sym / asym, MXFP8 OCP / NV from f32, f16 and bf16 sources, the 2 x 256
+# boundary patterns, the MXFP4 pattern families from f16 and bf16 sources, the NZ re-ordering of the exponents).  The
+# value patterns are this script's own renderings of what the case names say; the goldens are the oracle's.
+SRC = {"f32": ob.SRC_F32, "f16": ob.SRC_F16, "bf16": ob.SRC_BF16}
+
+
+def as_source(x, kind):
+    """The f32 values a source of that precision holds, and the array the kernel reads."""
+    x = np.asarray(x, np.float32)
+    if kind == "f16":
+        with np.errstate(over="ignore"):
+            h = x.astype(np.float16)
+        return h.astype(np.float32), h.view(np.uint16)
+    if kind == "bf16":
+        bits = x.view(np.uint32)
+        rounded = ((bits.astype(np.uint64) + 0x7FFF + ((bits >> 16) & 1)) >> 16).astype(np.uint16)
+        rounded = np.where(np.isnan(x), np.uint16(0x7FC0), rounded)
+        return (rounded.astype(np.uint32) << 16).view(np.float32), rounded
+    return x, x
+
+
+def tquant_case(case, x, kind, alg, nz=False):
+    vals, stored = as_source(x, kind)
+    codes, exp, _, _ = orc.tquant_mx(vals, alg, axis=1, src_kind=SRC[kind])
+    rows, cols = vals.shape
+    put("tquant", case, input=stored, golden=codes, golden_exp=orc.reorder_exp_zz(exp) if nz else exp)
+    line("tquant", case, "tquant_mx", rows, 0, cols, kind, kind, "u8", f"{alg}:{int(nz)}", 0)
+
+
+def pattern(name, rows, cols, fp4):
+    top = 6.0 if fp4 else 448.0
+    if name == "special":
+        base = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, top, -top, top * 2, 1.0, -1.0, 0.5, 3.0], np.float32)
+        return np.resize(base, (rows, cols)).astype(np.float32)
+    if name == "subnormal":
+        return (rng.standard_normal((rows, cols)) * 2.0 ** rng.integers(-149, -120, (rows, cols // 32)).repeat(32, 1)).astype(np.float32)
+    if name == "rounding":  # values on and next to the ties between neighbouring codes of the group's binade
+        steps = np.arange(rows * cols, dtype=np.float32).reshape(rows, cols) % 64
+        x = (steps * 0.125 + 0.0625).astype(np.float32)
+        x[:, ::3] = np.nextafter(x[:, ::3], np.float32(np.inf))
+        x[:, 1::3] = -x[:, 1::3]
+        return x
+    if name in ("exp_a", "exp_b"):
+        lo, hi = (-30, 30) if name == "exp_a" else (-126, 127)
+        return (rng.uniform(1, 2, (rows, cols)) * 2.0 ** rng.integers(lo, hi, (rows, cols)) * rng.choice([-1, 1], (rows, cols))).astype(np.float32)
+    x = (rng.standard_normal((rows, cols)) * 5).astype(np.float32)  # mixed
+    x.ravel()[::7] = 0.0
+    x.ravel()[3::11] *= np.float32(1e-30)
+    x.ravel()[5::13] *= np.float32(1e30)
+    x.ravel()[17::97] = np.nan
+    x.ravel()[29::101] = -np.inf
+    return x
+
+
+q8 = (rng.standard_normal((64, 128)) * 40).astype(np.float32)
+q8.ravel()[::5] = np.round(q8.ravel()[::5]) + 0.5
+q8_scale, q8_off = rng.uniform(0.5, 4.0, 64).astype(np.float32), rng.uniform(0, 200, 64).astype(np.float32)
+put("tquant", "Int8Sym", input=q8, scale=q8_scale, golden=orc.tquant_int8(q8, q8_scale))
+line("tquant", "Int8Sym", "tquant_i8", 64, 0, 128, "f32", "f32", "i8", 0, 0)
+put("tquant", "Int8Asym", input=q8, scale=q8_scale, offset=q8_off, golden=orc.tquant_int8(q8, q8_scale, q8_off))
+line("tquant", "Int8Asym", "tquant_i8", 64, 0, 128, "f32", "f32", "u8", 1, 0)
+for kind, tag in (("f32", ""), ("f16", "FP16"), ("bf16", "BF16")):
+    tquant_case(f"MxFp8{tag}Nd", (rng.standard_normal((32, 128)) * 10 ** rng.uniform(-3, 3, (32, 1))).astype(np.float32), kind, 0)
+    tquant_case(f"MxFp8{tag}Nz", (rng.standard_normal((32, 128)) * 10 ** rng.uniform(-3, 3, (32, 1))).astype(np.float32), kind, 0, nz=True)
+tquant_case("MxFp8NvNd", (rng.standard_normal((32, 128)) * 10 ** rng.uniform(-3, 3, (32, 1))).astype(np.float32), "f32", 1)
+edges = np.array([0.0, -0.0, 1e-45, 2.0 ** -130, np.nextafter(np.float32(448), 0), 448.0, -448.0, np.nextafter(np.float32(448), np.inf),
+                  896.0, np.inf, -np.inf, np.nan, 6.0, 0.75, 2.0 ** 127, -2.0 ** -126], np.float32)
+for kind, alg, tag in (("f32", 0, "OcpFp32"), ("f32", 1, "NvFp32"), ("f16", 1, "NvFp16"), ("bf16", 1, "NvBf16")):
+    tquant_case(f"MxFp8{tag}Boundary2x256", np.resize(edges, (2, 256)).astype(np.float32), kind, alg)
+for kind, tag in (("f16", "Fp16"), ("bf16", "Bf16")):
+    for name, label in (("special", "Special"), ("subnormal", "Subnormal"), ("rounding", "Rounding"), ("exp_a", "ExpRandomA"),
+                        ("exp_b", "ExpRandomB"), ("mixed", "Mixed")):
+        tquant_case(f"MxFp4E2M1{tag}Nd{label}", pattern(name, 2, 256, True), kind, 2)
+    tquant_case(f"MxFp4E2M1{tag}NdMixed32x1024", pattern("mixed", 32, 1024, True), kind, 2)
+    for name, label in (("special", "Special"), ("rounding", "Rounding"), ("mixed", "Mixed")):
+        tquant_case(f"MxFp4E2M1NV{tag}Nd{label}", pattern(name, 2, 256, True), kind, 3)
 
 np.savez_compressed(os.path.join(HERE, "runner_cases.npz"), **arrays)
 with open(os.path.join(HERE, "runner_cases.txt"), "w") as f:

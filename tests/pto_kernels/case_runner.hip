@@ -32,6 +32,8 @@
 
 extern "C" int pto_kernels_launch(int id, void* out, void* src0, void* src1, void* src2, void* stream);
 extern "C" int pto_kernels_status();
+extern "C" int pto_store_quant_launch(int id, void* out, void* src, void* words, int saturate, void* stream);
+extern "C" int pto_store_quant_status();
 extern "C" int pto_boundary_launch_mx(int id, void* out, void* a, void* b, void* sa, void* sb, void* bias, void* stream);
 extern "C" int pto_boundary_status();
 
@@ -445,6 +447,43 @@ static bool run_data_case(const std::string& dir, const CaseLine& c, void* strea
             RT(aclrtSynchronizeStream(stream));
         }
         ok = check(c, ptoamd_last_kernel(), dc, PTOAMD_F32, vm, vn, n, golden);
+    } else if (c.op == "storeq_tile") {  // a Vec tile through the quantising TSTORE, as a kernel written in the tile ISA
+        int id = 0, sat = 0;
+        sscanf(c.extra.c_str(), "%d:%d", &id, &sat);
+        const size_t count = (size_t)m * n;
+        const auto src = read_bin(dir, c, "input", count * type_bits(at) / 8), words = read_bin(dir, c, "quant", 0);
+        const auto golden = read_bin(dir, c, "golden", count * type_bits(ct) / 8);
+        DeviceBuffer ds(src.data(), src.size()), dw(words.data(), words.size()), dc(count * 4);
+        RT(pto_store_quant_launch(id, dc.dev, ds.dev, dw.dev, sat, stream));
+        RT(aclrtSynchronizeStream(stream));
+        // (source, output and golden share one memory order, row by row or column by column: compared as a flat run)
+        ok = pto_store_quant_status() == 0 && check(c, "pto kernel", dc, ct, 1, (int)count, (int)count, golden);
+    } else if (c.op == "tquant_mx") {
+        int alg = 0, nz = 0;
+        sscanf(c.extra.c_str(), "%d:%d", &alg, &nz);
+        const bool fp4 = alg >= 2;
+        const size_t count = (size_t)m * n, code_bytes = fp4 ? count / 2 : count, groups = count / 32;
+        const auto src = read_bin(dir, c, "input", count * type_bits(at) / 8);
+        const auto golden = read_bin(dir, c, "golden", code_bytes), golden_exp = read_bin(dir, c, "golden_exp", groups);
+        DeviceBuffer ds(src.data(), src.size()), dcodes(code_bytes + 16), dexp(groups + 16), dzz(groups + 16);
+        RT(ptoamd_tquant_mx((uint8_t*)dcodes.dev, (uint8_t*)dexp.dev, nullptr, nullptr, ds.dev, at, m, n, alg, 1, stream));
+        if (nz)  // the exponents in 16-row x 2-group boxes (the NZ store mode of TQUANT<MXFP8>)
+            RT(ptoamd_mx_scale_relayout((uint8_t*)dzz.dev, PTOAMD_MX_A_ZZ, (const uint8_t*)dexp.dev, PTOAMD_MX_A_ND, m, n / 32, stream));
+        RT(aclrtSynchronizeStream(stream));
+        ok = check(c, "codes", dcodes, PTOAMD_U8, 1, (int)code_bytes, (int)code_bytes, golden);
+        ok = check(c, "exponents", nz ? dzz : dexp, PTOAMD_U8, 1, (int)groups, (int)groups, golden_exp) && ok;
+    } else if (c.op == "tquant_i8") {
+        const bool asym = atoi(c.extra.c_str()) != 0;
+        const size_t count = (size_t)m * n;
+        const auto src = read_bin(dir, c, "input", count * 4), scale = read_bin(dir, c, "scale", (size_t)m * 4);
+        const auto golden = read_bin(dir, c, "golden", count);
+        std::vector<uint8_t> off;
+        if (asym)
+            off = read_bin(dir, c, "offset", (size_t)m * 4);
+        DeviceBuffer ds(src.data(), src.size()), dsc(scale.data(), scale.size()), dof(asym ? off.data() : scale.data(), (size_t)m * 4), dc(count + 16);
+        RT(ptoamd_tquant_int8(dc.dev, (const float*)ds.dev, (const float*)dsc.dev, asym ? (const float*)dof.dev : nullptr, m, n, stream));
+        RT(aclrtSynchronizeStream(stream));
+        ok = check(c, ptoamd_last_kernel(), dc, ct, m, n, n, golden);
     } else if (c.op == "dequant") {
         const auto src = read_bin(dir, c, "x1_gm", (size_t)m * n * type_bits(at) / 8);
         const auto scale = read_bin(dir, c, "x2_gm", (size_t)m * 4), off = read_bin(dir, c, "bias_gm", (size_t)m * 4);

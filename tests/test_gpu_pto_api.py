@@ -479,7 +479,7 @@ def _expand_runner_cases(tmp_path):
 
 def test_case_runner_reference_case_lists(tmp_path):
     """The framework-free runner over the reference's own case lists (tmatmul case1-4 / gemm / bias, tmatmul_mx case1-19,
-    tstore_acc2gm, tdequant): inputs and goldens come from files (goldens made by the oracle), every case runs through the
+    tstore_acc2gm, tstore_quant ND_1 ... ND_10 as tile-ISA kernels, tquant, tdequant): inputs and goldens come from files (goldens made by the oracle), every case runs through the
     C ABI, those with a compiled PTO kernel through that too, and the comparison is the reference's ResultCmp.  -l lists,
     -t selects a suite or a case, an unknown selection is exit status 2."""
     if not os.path.exists(RUNNER):
@@ -488,14 +488,16 @@ def test_case_runner_reference_case_lists(tmp_path):
     base = [RUNNER, "--data", str(tmp_path), "--manifest", manifest]
     listed = subprocess.run(base + ["-l"], capture_output=True, text=True, timeout=60)
     names = listed.stdout.split()
-    assert listed.returncode == 0 and len(names) == 50
-    assert {"tmatmul.case1", "tmatmul.case_bias_5", "tmatmul_mx.case19", "tstore_acc2gm.case_relu_21", "tdequant.case2"} <= set(names)
+    assert listed.returncode == 0 and len(names) == 93
+    assert {"tmatmul.case1", "tmatmul.case_bias_5", "tmatmul_mx.case19", "tstore_acc2gm.case_relu_21", "tdequant.case2",
+            "tstore_quant.DN_9", "tquant.MxFp4E2M1NVBf16NdMixed", "tquant.Int8Asym"} <= set(names)
     res = subprocess.run(base, capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stdout[-4000:] + res.stderr[-2000:]
-    assert "50 cases run, 0 failed" in res.stdout
+    assert "93 cases run, 0 failed" in res.stdout
     for name in names:
         assert f"{name}: PASS" in res.stdout, name
-    assert res.stdout.count("[pto kernel]") == 6  # tmatmul case1, 2, 3, gemm_1, bf16_1, bias_1 also ran as tile-ISA kernels
+    # tmatmul case1, 2, 3, gemm_1, bf16_1, bias_1 also ran as tile-ISA kernels; the ten tstore_quant cases only so
+    assert res.stdout.count("[pto kernel]") == 16
     one = subprocess.run(base + ["-t", "tmatmul_mx.case2"], capture_output=True, text=True, timeout=60)
     assert one.returncode == 0 and "1 cases run, 0 failed" in one.stdout
     suite = subprocess.run(base + ["-t", "tdequant"], capture_output=True, text=True, timeout=60)
