@@ -14,7 +14,7 @@ import pytest
 REF = "/root/reference/tests/cpu/st/testcase"
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SOURCES = ["tmatmul/tmatmul_kernel.cpp", "tmatmul_mx/tmatmul_mx_kernel.cpp", "tmatmul_mx_nddn/tmatmul_mx_nddn_kernel.cpp",
-           "tdequant/tdequant_kernel.cpp"]
+           "tdequant/tdequant_kernel.cpp", "tstore_quant/tstore_quant_kernel.cpp"]
 
 
 @pytest.mark.parametrize("source", SOURCES)
