@@ -67,17 +67,24 @@ template <typename TileData, typename GlobalData>
 PTO_INST bool tload_dma(TileData& dst, GlobalData& src)
 {
     using T = typename TileData::DType;
+    // (the E8M0 scale matrices: MX_A_ND keeps a row's K-groups contiguous like ND, MX_B_DN a column's like DN; their
+    // shapes are (1, 1, lines, groups / 2, 2) with strides (., ., line pitch, 2, 1))
+    constexpr bool nd = GlobalData::layout == Layout::ND, dn = GlobalData::layout == Layout::DN;
+    constexpr bool mx_a = GlobalData::layout == Layout::MX_A_ND, mx_b = GlobalData::layout == Layout::MX_B_DN;
     if constexpr (TileData::MatLines && TileData::LineBytes % 16 == 0 && sizeof(T) == sizeof(typename GlobalData::DType) &&
-                  ((GlobalData::layout == Layout::ND && TileData::LinesAreRows) ||
-                   (GlobalData::layout == Layout::DN && !TileData::LinesAreRows))) {
-        constexpr bool nd = GlobalData::layout == Layout::ND;
+                  (((nd || mx_a) && TileData::LinesAreRows) || ((dn || mx_b) && !TileData::LinesAreRows))) {
         // ND: element (r, c) at r * stride[3] + c * stride[4]; DN: the same with the unit stride on the rows
-        const int64_t line_stride = src.GetStride(nd ? 3 : 4), unit_stride = src.GetStride(nd ? 4 : 3);
+        const int64_t line_stride = src.GetStride((mx_a || mx_b) ? 2 : (nd ? 3 : 4));
         const int64_t gbytes = line_stride * (int64_t)sizeof(T);
         const uintptr_t gaddr = reinterpret_cast<uintptr_t>(src.data());
-        const bool ok = src.GetShape(0) == 1 && src.GetShape(1) == 1 && src.GetShape(2) == 1 && unit_stride == 1 &&
-                        src.GetShape(3) >= TileData::Rows && src.GetShape(4) >= TileData::Cols &&
-                        dst.GetValidRow() == TileData::Rows && dst.GetValidCol() == TileData::Cols && (gbytes & 15) == 0 &&
+        bool shape_ok;
+        if constexpr (mx_a || mx_b)
+            shape_ok = src.GetShape(0) == 1 && src.GetShape(1) == 1 && src.GetStride(3) == 2 && src.GetStride(4) == 1 &&
+                       src.GetShape(4) == 2 && src.GetShape(2) >= TileData::Lines && src.GetShape(3) * 2 >= TileData::LineBytes;
+        else
+            shape_ok = src.GetShape(0) == 1 && src.GetShape(1) == 1 && src.GetShape(2) == 1 && src.GetStride(nd ? 4 : 3) == 1 &&
+                       src.GetShape(3) >= TileData::Rows && src.GetShape(4) >= TileData::Cols;
+        const bool ok = shape_ok && dst.GetValidRow() == TileData::Rows && dst.GetValidCol() == TileData::Cols && (gbytes & 15) == 0 &&
                         (gaddr & 15u) == 0 && gbytes > 0 &&
                         (int64_t)(TileData::Lines - 1) * gbytes + TileData::LineBytes <= (int64_t)0xFFFFFFFFll;
         if (!ok)
@@ -180,11 +187,12 @@ template <typename DstTile, typename SrcTile>
 PTO_INST bool textract_window(DstTile& dst, SrcTile& src, int row0, int col0)
 {
     using T = typename DstTile::DType;
-    if constexpr (SrcTile::MatLines && !is_packed4<T> &&
-                  ((DstTile::Loc == TileType::Left && SrcTile::LinesAreRows) || (DstTile::Loc == TileType::Right && !SrcTile::LinesAreRows))) {
-        constexpr bool left = DstTile::Loc == TileType::Left;
+    if constexpr (SrcTile::MatLines && !is_packed4<T> && DstTile::OperandLoc && DstTile::LinesAreRows == SrcTile::LinesAreRows) {
+        constexpr bool left = DstTile::LinesAreRows;
+        // (fragments are read as 16-byte chunks; the bytes of a scale tile are read one by one, from any offset)
+        constexpr bool scale = DstTile::Loc == TileType::ScaleLeft || DstTile::Loc == TileType::ScaleRight;
         const uint32_t kb0 = (uint32_t)(left ? col0 : row0) * (uint32_t)sizeof(T);
-        const bool ok = (kb0 & 15u) == 0 && row0 >= 0 && col0 >= 0 && row0 + DstTile::Rows <= src.GetValidRow() &&
+        const bool ok = (scale || (kb0 & 15u) == 0) && row0 >= 0 && col0 >= 0 && row0 + DstTile::Rows <= src.GetValidRow() &&
                         col0 + DstTile::Cols <= src.GetValidCol() && dst.GetValidRow() == DstTile::Rows &&
                         dst.GetValidCol() == DstTile::Cols;
         if (!ok)
@@ -210,7 +218,7 @@ PTO_INST void textract_lds(DstTile& dst, SrcTile& src, int row0, int col0)
 {
     using T = typename DstTile::DType;
     static_assert(std::is_same_v<T, typename SrcTile::DType>, "TMOV / TEXTRACT: element types differ");
-    if constexpr (DstTile::Loc == TileType::Left || DstTile::Loc == TileType::Right) {
+    if constexpr (DstTile::OperandLoc) {
         if constexpr (WINDOW_OK) {
             if (textract_window(dst, src, row0, col0))
                 return;
@@ -511,6 +519,57 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kpad = min((a.GetValidCol() + 63) / 64 * 64, TileRightT::Rows);
     const uint8_t *pa = a.Storage(), *pb = b.Storage(), *psa = as.Storage(), *psb = bs.Storage();
+    if constexpr (TileRes::BLOCKED && !is_packed4<TA> && !via_fp8 && !gemv) {
+        // fp8 on a wave grid: per k-step (two MX blocks) the wave reads the fragments and scale bytes of its MB row blocks
+        // and NB column blocks once and issues MB * NB scaled MFMAs (as tmatmul does for the plain types)
+        constexpr int MB = TileRes::MB, NB = TileRes::NB;
+        const int wr = wave / TileRes::grid.wc, wc = wave % TileRes::grid.wc;
+        int aline[MB], bline[NB];
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+            aline[i] = min((wr * MB + i) * 32 + l32, TileLeftT::Rows - 1);
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+            bline[j] = min((wc * NB + j) * 32 + l32, TileRightT::Cols - 1);
+        if constexpr (INIT) {
+#pragma unroll
+            for (int slot = 0; slot < TileRes::NBLK; ++slot)
+                c.regs[slot] = typename TileRes::Vec16(0);
+        }
+        auto kstep = [&](int k0) __attribute__((always_inline)) {
+            const int g = k0 / 32 + lhi;
+            i32x8v fa[MB], fb[NB];
+            int sa[MB], sb[NB];
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 16 * lhi, bline[j]));
+                const uint4 b1 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 + 16 * lhi, bline[j]));
+                fb[j] = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                sb[j] = psb[bs.ByteOffset(g, bline[j])];
+            }
+#pragma unroll
+            for (int i = 0; i < MB; ++i) {
+                const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(aline[i], k0 + 16 * lhi));
+                const uint4 a1 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(aline[i], k0 + 32 + 16 * lhi));
+                fa[i] = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                sa[i] = psa[as.ByteOffset(aline[i], g)];
+            }
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+                    c.regs[i * NB + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[j], fa[i], c.regs[i * NB + j], MxFormat<TB>::code,
+                                                                                         MxFormat<TA>::code, 0, sb[j], 0, sa[i]);
+        };
+        if constexpr (TileLeftT::ValidCol != DYNAMIC) {
+            constexpr int kp = (TileLeftT::ValidCol + 63) / 64 * 64 < TileRightT::Rows ? (TileLeftT::ValidCol + 63) / 64 * 64 : TileRightT::Rows;
+            static_for<kp / 64>([&](auto sc) { kstep(decltype(sc)::value * 64); });
+        } else {
+            for (int k0 = 0; k0 < kpad; k0 += 64)
+                kstep(k0);
+        }
+        return;
+    }
 #pragma unroll
     for (int slot = 0; slot < TileRes::NBLK; ++slot) {
         int bi, bj;

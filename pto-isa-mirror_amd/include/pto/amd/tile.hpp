@@ -164,7 +164,13 @@ struct LdsStorage {
     uint32_t addr_ = 0;  // the TASSIGN address (offset inside the tile's region)
     uint32_t pend_ = 0;  // Mat tiles: an asynchronous TLOAD into the tile may still be in flight
 };
-// Left / Right tiles: where the lines live (the tile's own storage, or a window onto a Mat tile)
+// The tiles the matrix unit reads -- Left / Right and their scale tiles -- are stored as lines along K (rows of the A
+// side, columns of the B side) and may be windows onto a Mat tile instead of owning bytes.
+constexpr bool is_operand_loc(TileType l)
+{
+    return l == TileType::Left || l == TileType::Right || l == TileType::ScaleLeft || l == TileType::ScaleRight;
+}
+// Left / Right / ScaleLeft / ScaleRight tiles: where the lines live (the tile's own storage, or a window onto a Mat tile)
 struct WindowStorage : LdsStorage {
     uint32_t pitch_ = 0, sh_ = 0, mask_ = 0;  // line pitch in bytes and the swizzle of the storage the lines live in
     uint32_t line0_ = 0, kb0_ = 0;            // first line / first byte along a line of the window
@@ -178,7 +184,7 @@ template <TileType Loc_, typename Element_, const int Rows_, const int Cols_, co
           const int SFractalSize_ = TileConfig::fractalABSize, auto PadVal_ = PadValue::Null,
           const CompactMode Compact_ = CompactMode::Null>
 struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_, Rows_, Cols_>,
-                                 std::conditional_t<Loc_ == TileType::Left || Loc_ == TileType::Right, amd::WindowStorage, amd::LdsStorage>> {
+                                 std::conditional_t<amd::is_operand_loc(Loc_), amd::WindowStorage, amd::LdsStorage>> {
     using DType = Element_;
     static constexpr TileType Loc = Loc_;
     static constexpr int Rows = Rows_, Cols = Cols_, ValidRow = RowValid_, ValidCol = ColValid_;
@@ -210,8 +216,9 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
     // Mat tiles with a box layout are stored as swizzled lines; lines are rows for SLayout::RowMajor boxes, columns for
     // SLayout::ColMajor boxes
     static constexpr bool MatLines = Loc_ == TileType::Mat && SFractal_ != SLayout::NoneBox && !is_packed4;
-    static constexpr bool Lined = MatLines || Loc_ == TileType::Left || Loc_ == TileType::Right;
-    static constexpr bool LinesAreRows = Loc_ == TileType::Left || (MatLines && SFractal_ == SLayout::RowMajor);
+    static constexpr bool OperandLoc = amd::is_operand_loc(Loc_);
+    static constexpr bool Lined = MatLines || OperandLoc;
+    static constexpr bool LinesAreRows = Loc_ == TileType::Left || Loc_ == TileType::ScaleLeft || (MatLines && SFractal_ == SLayout::RowMajor);
     static constexpr int Lines = LinesAreRows ? Rows_ : Cols_;
     static constexpr int LineBytes = (LinesAreRows ? Cols_ : Rows_) * amd::ElemTraits<Element_>::bytes2 / 2;
     using Swz = amd::LineSwizzle<LineBytes>;
@@ -220,7 +227,7 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
     {
         if constexpr (Loc_ != TileType::Acc)
             this->lds_ = amd::Region<Loc_>::base;
-        if constexpr (Loc_ == TileType::Left || Loc_ == TileType::Right) {
+        if constexpr (OperandLoc) {
             this->own_ok_ = Bytes <= amd::Region<Loc_>::size;
             BindOwnLines();
         }
@@ -228,7 +235,7 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
     // the lines are the tile's own storage (not a window onto a Mat tile)
     PTO_INST void BindOwnLines()
     {
-        if constexpr (Loc_ == TileType::Left || Loc_ == TileType::Right) {
+        if constexpr (OperandLoc) {
             this->lds_ = amd::Region<Loc_>::base + this->addr_;
             this->pitch_ = LineBytes;
             this->sh_ = Swz::sh;
@@ -245,7 +252,7 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
     PTO_INST uint32_t ByteOffset(int r, int c) const
     {
         constexpr int b2 = amd::ElemTraits<Element_>::bytes2;
-        if constexpr (Loc_ == TileType::Left || Loc_ == TileType::Right) {
+        if constexpr (OperandLoc) {
             const uint32_t line = (uint32_t)(LinesAreRows ? r : c) + this->line0_;
             const uint32_t kb = (uint32_t)((LinesAreRows ? c : r) * b2 / 2) + this->kb0_;
             return amd::line_offset(line, kb, this->pitch_, this->sh_, this->mask_);
@@ -353,8 +360,8 @@ PTO_INST uint64_t GetScaleAddr(uint64_t addr) { return addr >> 4; }
 template <typename T, typename AddrType>
 PTO_INST void TASSIGN(T& obj, AddrType addr)
 {
-    if constexpr (T::Loc == TileType::Left || T::Loc == TileType::Right) {
-        // a Left / Right tile needs its own bytes only when an extraction has to copy; one that does not fit its region
+    if constexpr (T::OperandLoc) {
+        // a Left / Right (or scale) tile needs its own bytes only when an extraction has to copy; one that does not fit its region
         // can still be a window onto a Mat tile, so the range check is deferred to the copy
         using R = amd::Region<T::Loc>;
         uint32_t a = (uint32_t)(uint64_t)addr;
@@ -380,7 +387,7 @@ PTO_INST void TASSIGN(T& obj, AddrType addr)
 template <std::size_t Addr, typename T>
 PTO_INST std::enable_if_t<is_tile_data_v<T>> TASSIGN(T& obj)
 {
-    if constexpr (T::Loc == TileType::Left || T::Loc == TileType::Right) {
+    if constexpr (T::OperandLoc) {
         static_assert(Addr % 16 == 0, "TASSIGN: address not 16-byte aligned");
     } else if constexpr (T::Loc != TileType::Acc) {
         static_assert(Addr + T::Bytes <= amd::Region<T::Loc>::size && Addr % 16 == 0,
