@@ -176,6 +176,31 @@ def pto_api_bf16(pa, ev, gen, steps, warmup):
                 cpu="headline")
 
 
+def pto_api_mxfp8(pa, ev, gen, steps, warmup):
+    """configs[3] through the reference's own programming interface: kernels/mxmatmul_performance.hip is a core program of
+    TLOAD / TEXTRACT / TMATMUL_MX / TSTORE calls (operand panels and E8M0 scale tiles double-buffered in L1)."""
+    C, lib = _pto_lib("mxmatmul_performance")
+    m, n, k = 4096, 14336, 4096
+    a, sa = pa.tquant_mx(torch.randn((m, k), generator=gen, device=DEV), pa.OCP_MXFP8, want_aux=False)
+    b, sb = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP8, want_aux=False)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+
+    def step():
+        rc = lib.pto_mxmatmul_performance(0, *(C.c_void_p(t.data_ptr()) for t in (out, a, b, sa, sb)),
+                                          C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, rc
+
+    wall, ker = time_launches(ev, step, steps, warmup)
+    ref = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E4M3, pa.E4M3, pa.BF16)
+    torch.cuda.synchronize()
+    assert lib.pto_mxmatmul_performance_status() == 0 and torch.equal(out, ref), "the PTO-style MX GEMM and the launcher disagree"
+    flops = 2 * m * n * k
+    return dict(config="configs[3] MXFP8 E4M3 4096x14336x4096 -> bf16 written in the PTO tile ISA (TLOAD / TEXTRACT / TMATMUL_MX / "
+                       "TSTORE, 256 x 256 tiles, K panels of 128, scale tiles of 16 K-groups)",
+                kernel="MxMatmulPerformance<e4m3, 256, 256, 128> (header layer)", ms=ker, wall_ms=wall, tflops=flops / ker / 1e9,
+                bound="mfma", frac_of_peak=flops / ker / 1e9 / PEAK_TFLOPS["fp8"], cpu="config4")
+
+
 def pto_api_config1(pa, ev, gen, steps, warmup):
     """configs[0] through the tile ISA (kernels/gemm_tiled.hip): 128 x 128 tiles as BASELINE.json words it, and 64 x 64."""
     C, lib = _pto_lib("gemm_tiled")
@@ -502,10 +527,10 @@ def main():
                     help="untimed run-in of the same launches before the warmup steps, for the GPU clock to settle")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-config measurements after the headline")
-    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10], default=None,
+    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11], default=None,
                     help="measure just BASELINE.json configs[N] (a per_config entry) and print it: for profiling one kernel; "
-                         "5-8 are the elementwise kernels (TQUANT MXFP8, TQUANT MXFP4, TQUANT INT8, TDEQUANT), 9 and 10 "
-                         "configs[1] and configs[0] written in the PTO tile ISA")
+                         "5-8 are the elementwise kernels (TQUANT MXFP8, TQUANT MXFP4, TQUANT INT8, TDEQUANT), 9, 10 and 11 "
+                         "configs[1], configs[0] and configs[3] written in the PTO tile ISA")
     ap.add_argument("--published", action="store_true",
                     help="measure only the shapes the reference publishes wall times for and print those rows")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -532,7 +557,7 @@ def main():
         return
     if args.only is not None:
         fn = {0: config1, 2: config3, 3: config4, 4: config5, 5: quant_mxfp8, 6: quant_mxfp4, 7: quant_int8,
-              8: dequant_int8, 9: pto_api_bf16, 10: pto_api_config1}[args.only]
+              8: dequant_int8, 9: pto_api_bf16, 10: pto_api_config1, 11: pto_api_mxfp8}[args.only]
         entry = fn(pa, ev, gen, args.steps, args.warmup)
         entry.pop("cpu", None)
         print(json.dumps(entry))
@@ -560,7 +585,7 @@ def main():
     }
     if not args.no_extra:
         per = []
-        for fn in (config1, config3, config4, config5, pto_api_bf16, pto_api_config1, quant_mxfp8, quant_mxfp4, quant_int8,
+        for fn in (config1, config3, config4, config5, pto_api_bf16, pto_api_config1, pto_api_mxfp8, quant_mxfp8, quant_mxfp4, quant_int8,
                    dequant_int8):
             per.append(fn(pa, ev, gen, 50, 5))
             torch.cuda.empty_cache()

@@ -536,21 +536,42 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
             for (int slot = 0; slot < TileRes::NBLK; ++slot)
                 c.regs[slot] = typename TileRes::Vec16(0);
         }
+        // Fragment addresses.  A lane reads line l32 of every block of its wave tile; blocks are 32 lines apart, which
+        // leaves the swizzle term (line >> sh) & mask unchanged, so the chunk at 16-byte index c of block i lies at
+        //     line0 * pitch + ((c ^ swz) << 4) + i * 32 * pitch.
+        // With c = c0 + lhi and c0 even, (c0 + lhi) ^ swz = c0 ^ (lhi ^ swz): one lane constant per operand XOR a literal,
+        // plus a literal block offset that goes into the read instruction.  Written out here because, computed block by
+        // block through ByteOffset, every address is its own loop-invariant value, and a program's worth of them does not
+        // fit the register file next to the accumulators.  (Needs a power-of-two number of chunks per line and windows
+        // that start on 32-byte boundaries along K; anything else takes ByteOffset.)
+        const uint8_t* arena = lds_arena();
+        const uint32_t a_l0 = (uint32_t)(wr * MB * 32 + l32) + a.line0_, b_l0 = (uint32_t)(wc * NB * 32 + l32) + b.line0_;
+        const bool fast_addr = (a.pitch_ & (a.pitch_ - 1)) == 0 && (b.pitch_ & (b.pitch_ - 1)) == 0 && a.pitch_ >= 64 && b.pitch_ >= 64 &&
+                               (a.kb0_ & 31u) == 0 && (b.kb0_ & 31u) == 0;
+        const uint32_t a_lane = a.lds_ + a_l0 * a.pitch_ + (((uint32_t)lhi ^ ((a_l0 >> a.sh_) & a.mask_)) << 4);
+        const uint32_t b_lane = b.lds_ + b_l0 * b.pitch_ + (((uint32_t)lhi ^ ((b_l0 >> b.sh_) & b.mask_)) << 4);
+        auto frag = [&](bool left, int blk, int kbyte) __attribute__((always_inline)) -> uint4 {
+            // kbyte: 0 or 32 past the k-step's first byte, i.e. a literal multiple of 32
+            if (fast_addr) {
+                const uint32_t lane_c = left ? a_lane : b_lane, pitch = left ? a.pitch_ : b.pitch_, kb0 = left ? a.kb0_ : b.kb0_;
+                return *reinterpret_cast<const uint4*>(arena + ((lane_c ^ (kb0 + (uint32_t)kbyte)) + (uint32_t)blk * 32u * pitch));
+            }
+            return left ? *reinterpret_cast<const uint4*>(pa + a.ByteOffset(aline[blk], kbyte + 16 * lhi))
+                        : *reinterpret_cast<const uint4*>(pb + b.ByteOffset(kbyte + 16 * lhi, bline[blk]));
+        };
         auto kstep = [&](int k0) __attribute__((always_inline)) {
             const int g = k0 / 32 + lhi;
             i32x8v fa[MB], fb[NB];
             int sa[MB], sb[NB];
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
-                const uint4 b0 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 16 * lhi, bline[j]));
-                const uint4 b1 = *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k0 + 32 + 16 * lhi, bline[j]));
+                const uint4 b0 = frag(false, j, k0), b1 = frag(false, j, k0 + 32);
                 fb[j] = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
                 sb[j] = psb[bs.ByteOffset(g, bline[j])];
             }
 #pragma unroll
             for (int i = 0; i < MB; ++i) {
-                const uint4 a0 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(aline[i], k0 + 16 * lhi));
-                const uint4 a1 = *reinterpret_cast<const uint4*>(pa + a.ByteOffset(aline[i], k0 + 32 + 16 * lhi));
+                const uint4 a0 = frag(true, i, k0), a1 = frag(true, i, k0 + 32);
                 fa[i] = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
                 sa[i] = psa[as.ByteOffset(aline[i], g)];
             }
@@ -568,6 +589,12 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
             for (int k0 = 0; k0 < kpad; k0 += 64)
                 kstep(k0);
         }
+        // The MFMAs are register-to-register operations that the compiler may move freely, and it sinks them past the
+        // next instructions' barriers and branches to where the accumulators are next needed -- with every fragment
+        // they read kept live until then.  An empty statement that "uses" the accumulators pins them to this call.
+#pragma unroll
+        for (int slot = 0; slot < TileRes::NBLK; ++slot)
+            asm volatile("" : "+v"(c.regs[slot]));
         return;
     }
 #pragma unroll
@@ -674,6 +701,8 @@ PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
                           (uint32_t)(WAVES * pair_band) <= (uint32_t)PTO_AMD_STAGE_BYTES) {
                 if (vr == TileRes::Rows && vc == TileRes::Cols && ((ld * (int64_t)sizeof(G)) & 15) == 0 &&
                     (reinterpret_cast<uintptr_t>(g) & 15u) == 0) {
+                    if constexpr (STAGE_ALIASES_L1)
+                        __syncthreads();  // every wave has read its last operands out of L1
                     uint8_t* stage = lds_arena() + STAGE_BASE + wave * pair_band;
 #pragma unroll
                     for (int slot = 0; slot < TileRes::NBLK; slot += 2) {
@@ -715,6 +744,8 @@ PTO_INST void tstore_acc(GlobalData& dst, TileRes& src)
             if constexpr (TileRes::Rows % 32 == 0 && TileRes::Cols % 32 == 0 && (uint32_t)(WAVES * band) <= (uint32_t)PTO_AMD_STAGE_BYTES) {
                 if (vr == TileRes::Rows && vc == TileRes::Cols && ((ld * (int64_t)sizeof(G)) & 15) == 0 &&
                     (reinterpret_cast<uintptr_t>(g) & 15u) == 0) {
+                    if constexpr (STAGE_ALIASES_L1)
+                        __syncthreads();
                     uint8_t* stage = lds_arena() + STAGE_BASE + wave * band;
                     constexpr int lanes_per_row = row_bytes / 16, rows_per_pass = 64 / lanes_per_row;
                     const int rrow = lane / lanes_per_row, rchunk = lane % lanes_per_row;

@@ -53,9 +53,21 @@ struct Region {
                                      : L == TileType::Scaling ? PTO_AMD_FB_BYTES
                                                               : PTO_AMD_L0S_BYTES / 2;
 };
-constexpr uint32_t STAGE_BASE = PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES +
-                                PTO_AMD_BIAS_BYTES + PTO_AMD_FB_BYTES + PTO_AMD_L0S_BYTES;
+// The fix-pipe staging bytes follow the regions -- or, with PTO_AMD_STAGE_IN_L1 defined, lie over the start of L1: a
+// kernel whose L1 tiles are dead by the time it stores (the usual GEMM shape) then needs no LDS for them; TSTORE puts a
+// workgroup barrier in front of its first staging write so that every wave is done reading L1.
+constexpr uint32_t REGIONS_END = PTO_AMD_L1_BYTES + PTO_AMD_L0A_BYTES + PTO_AMD_L0B_BYTES + PTO_AMD_UB_BYTES +
+                                 PTO_AMD_BIAS_BYTES + PTO_AMD_FB_BYTES + PTO_AMD_L0S_BYTES;
+#ifdef PTO_AMD_STAGE_IN_L1
+constexpr bool STAGE_ALIASES_L1 = true;
+constexpr uint32_t STAGE_BASE = 0;
+constexpr uint32_t LDS_TOTAL = REGIONS_END;
+static_assert(PTO_AMD_STAGE_BYTES <= PTO_AMD_L1_BYTES, "the staging bytes lie inside L1");
+#else
+constexpr bool STAGE_ALIASES_L1 = false;
+constexpr uint32_t STAGE_BASE = REGIONS_END;
 constexpr uint32_t LDS_TOTAL = STAGE_BASE + PTO_AMD_STAGE_BYTES;
+#endif
 #ifndef PTO_AMD_CHECK_REFERENCE_SOURCE
 static_assert(LDS_TOTAL <= 160 * 1024, "the on-chip regions must fit the 160 KiB LDS of a CU");
 #endif

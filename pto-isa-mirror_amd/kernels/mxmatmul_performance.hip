@@ -1,0 +1,172 @@
+// A block-scaled GEMM written in the PTO tile ISA for the gfx950 backend: C[M, N] = sum over K-groups of 32 of
+// (A . 2^(sa - 127)) (B . 2^(sb - 127)), A [M][K] fp8 row-major (ND), B the DN view of [N][K] memory, E8M0 scales
+// [M][K / 32] (MX_A_ND) and [N][K / 32] (MX_B_DN), fp32 accumulation, bf16 C.  The program has the shape of the
+// reference's kernel (kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:159-282): a core owns
+// one baseM x baseN tile of C; operand panels of baseK are double-buffered in L1 by TLOAD, the scales are loaded for
+// several panels at a time (stepKscale of them) into double-buffered scale tiles, TEXTRACT slices both, TMATMUL_MX
+// accumulates, one TSTORE drains.
+//
+// Sized for this backend: a core is a workgroup of 512 threads; L1 holds two A panels, two B panels (32 KiB each) and two
+// scale tiles per side (4 KiB each: 256 lines of 16 groups, the smallest tile whose lines a 16-byte copy can move); the
+// Left / Right tiles and their scale tiles are windows onto those, so the L0 regions need no bytes; the fix-pipe staging
+// lies over the start of L1, whose panels are dead when the tile is stored.  As in the bf16 kernel, a panel's copy-in is
+// issued before the TMATMUL_MX of the panel before it, and the event flags of the reference program are not written out.
+#define PTO_AMD_THREADS 512
+#define PTO_AMD_L1_BYTES (144 * 1024)
+#define PTO_AMD_L0A_BYTES 256
+#define PTO_AMD_L0B_BYTES 256
+#define PTO_AMD_UB_BYTES 256
+#define PTO_AMD_BIAS_BYTES 256
+#define PTO_AMD_FB_BYTES 256
+#define PTO_AMD_L0S_BYTES 512
+#define PTO_AMD_STAGE_IN_L1
+#define PTO_AMD_STAGE_BYTES (8 * 16 * (128 + 16))  // 16-bit results: a wave stages 16 rows of two side-by-side blocks
+#include <pto/pto-inst.hpp>
+
+using namespace pto;
+
+template <int tilesM, int tilesN, int groupM>
+AICORE inline void OwnTile(int& tm, int& tn)
+{
+    constexpr int cores = tilesM * tilesN;
+    int id = (int)get_block_idx();
+    if constexpr (cores % 8 == 0)
+        id = (id & 7) * (cores / 8) + (id >> 3);
+    constexpr int perGroup = groupM * tilesN;
+    const int firstM = (id / perGroup) * groupM;
+    const int rows = (tilesM - firstM) < groupM ? (tilesM - firstM) : groupM;
+    tm = firstM + (id % perGroup) % rows;
+    tn = (id % perGroup) / rows;
+}
+
+template <typename OutT, typename InT, int M, int K, int N, int baseM, int baseN, int baseK, int stepKscale>
+__global__ AICORE void MxMatmulPerformance(__gm__ OutT* out, __gm__ InT* a, __gm__ InT* b, __gm__ float8_e8m0_t* sa, __gm__ float8_e8m0_t* sb)
+{
+    using X = float8_e8m0_t;
+    constexpr int panels = K / baseK, groups = baseK / 32, chunkGroups = groups * stepKscale, kGroups = K / 32;
+    static_assert(M % baseM == 0 && N % baseN == 0 && K % (baseK * stepKscale) == 0, "whole tiles, panels and scale chunks only");
+
+    using GlobalA = GlobalTensor<InT, TileShape2D<InT, baseM, baseK, Layout::ND>, BaseShape2D<InT, M, K, Layout::ND>, Layout::ND>;
+    using GlobalB = GlobalTensor<InT, TileShape2D<InT, baseK, baseN, Layout::DN>, BaseShape2D<InT, K, N, Layout::DN>, Layout::DN>;
+    using GlobalSA = GlobalTensor<X, TileShape2D<X, baseM, chunkGroups, Layout::MX_A_ND>, BaseShape2D<X, M, kGroups, Layout::MX_A_ND>, Layout::MX_A_ND>;
+    using GlobalSB = GlobalTensor<X, TileShape2D<X, chunkGroups, baseN, Layout::MX_B_DN>, BaseShape2D<X, kGroups, N, Layout::MX_B_DN>, Layout::MX_B_DN>;
+    using GlobalC = GlobalTensor<OutT, TileShape2D<OutT, baseM, baseN, Layout::ND>, BaseShape2D<OutT, M, N, Layout::ND>, Layout::ND>;
+
+    using TileMatA = Tile<TileType::Mat, InT, baseM, baseK, BLayout::ColMajor, baseM, baseK, SLayout::RowMajor>;
+    using TileMatB = Tile<TileType::Mat, InT, baseK, baseN, BLayout::RowMajor, baseK, baseN, SLayout::ColMajor>;
+    using TileScaleA = Tile<TileType::Mat, X, baseM, chunkGroups, BLayout::RowMajor, baseM, chunkGroups, SLayout::RowMajor, 32>;
+    using TileScaleB = Tile<TileType::Mat, X, chunkGroups, baseN, BLayout::ColMajor, chunkGroups, baseN, SLayout::ColMajor, 32>;
+    using LeftTile = TileLeft<InT, baseM, baseK, baseM, baseK>;
+    using RightTile = TileRight<InT, baseK, baseN, baseK, baseN>;
+    using LeftScaleTile = TileLeftScale<X, baseM, groups, baseM, groups>;
+    using RightScaleTile = TileRightScale<X, groups, baseN, groups, baseN>;
+    using ResTile = TileAcc<float, baseM, baseN, baseM, baseN>;
+
+    TileMatA aMat[2];
+    TileMatB bMat[2];
+    TileScaleA aScaleMat[2];
+    TileScaleB bScaleMat[2];
+    LeftTile aTile;
+    RightTile bTile;
+    LeftScaleTile aScale;
+    RightScaleTile bScale;
+    ResTile cTile;
+    constexpr uint32_t bytesA = baseM * baseK, bytesB = baseK * baseN, bytesSA = baseM * chunkGroups, bytesSB = chunkGroups * baseN;
+    constexpr uint32_t scales0 = 2 * bytesA + 2 * bytesB;
+    TASSIGN(aMat[0], 0x0);
+    TASSIGN(aMat[1], bytesA);
+    TASSIGN(bMat[0], 2 * bytesA);
+    TASSIGN(bMat[1], 2 * bytesA + bytesB);
+    TASSIGN(aScaleMat[0], scales0);
+    TASSIGN(aScaleMat[1], scales0 + bytesSA);
+    TASSIGN(bScaleMat[0], scales0 + 2 * bytesSA);
+    TASSIGN(bScaleMat[1], scales0 + 2 * bytesSA + bytesSB);
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(aScale, 0x0);
+    TASSIGN(bScale, 0x0);
+    TASSIGN(cTile, 0x0);
+
+    int tm, tn;
+    OwnTile<M / baseM, N / baseN, 4>(tm, tn);
+    __gm__ InT* aRows = a + (size_t)tm * baseM * K;
+    __gm__ InT* bCols = b + (size_t)tn * baseN * K;
+    __gm__ X* saRows = sa + (size_t)tm * baseM * kGroups;
+    __gm__ X* sbCols = sb + (size_t)tn * baseN * kGroups;
+
+    // One scale chunk: stepKscale panels, walked with literal indices so that every window offset and buffer choice is a
+    // constant of the instruction stream.  Panel q of the chunk (L1 slot q % 2): slice operands and scales, start the next
+    // copies (the last panel of a chunk also requests the next chunk's scales), multiply.
+    auto chunk = [&](auto sslotc, int p0) __attribute__((always_inline)) {
+        constexpr int scur = decltype(sslotc)::value;
+        pto::amd::static_for<stepKscale>([&](auto qc) {
+            constexpr int q = decltype(qc)::value, cur = q & 1, nxt = cur ^ 1;
+            const int p = p0 + q;
+            TEXTRACT(aTile, aMat[cur], 0, 0);
+            TEXTRACT(bTile, bMat[cur], 0, 0);
+            TEXTRACT(aScale, aScaleMat[scur], 0, q * groups);
+            TEXTRACT(bScale, bScaleMat[scur], q * groups, 0);
+            if (p + 1 < panels) {
+                GlobalA gmA(aRows + (size_t)(p + 1) * baseK);
+                GlobalB gmB(bCols + (size_t)(p + 1) * baseK);
+                TLOAD(aMat[nxt], gmA);
+                TLOAD(bMat[nxt], gmB);
+                if constexpr (q == stepKscale - 1) {
+                    GlobalSA gmSA(saRows + (size_t)(p + 1) * groups);
+                    GlobalSB gmSB(sbCols + (size_t)(p + 1) * groups);
+                    TLOAD(aScaleMat[scur ^ 1], gmSA);
+                    TLOAD(bScaleMat[scur ^ 1], gmSB);
+                }
+            }
+            if (p == 0)
+                TMATMUL_MX(cTile, aTile, aScale, bTile, bScale);
+            else
+                TMATMUL_MX(cTile, cTile, aTile, aScale, bTile, bScale);
+        });
+    };
+
+    {
+        GlobalA gmA(aRows);
+        GlobalB gmB(bCols);
+        GlobalSA gmSA(saRows);
+        GlobalSB gmSB(sbCols);
+        TLOAD(aMat[0], gmA);
+        TLOAD(bMat[0], gmB);
+        TLOAD(aScaleMat[0], gmSA);
+        TLOAD(bScaleMat[0], gmSB);
+    }
+    static_assert(stepKscale % 2 == 0, "a chunk starts in L1 slot 0");
+    for (int p = 0; p < panels; p += 2 * stepKscale) {
+        chunk(std::integral_constant<int, 0>{}, p);
+        if (p + stepKscale < panels)
+            chunk(std::integral_constant<int, 1>{}, p + stepKscale);
+    }
+
+    GlobalC gmC(out + (size_t)tm * baseM * N + (size_t)tn * baseN);
+    TSTORE(gmC, cTile);
+}
+
+// id 0: configs[3] of the baseline list: E4M3 4096 x 14336 x 4096 -> bf16 (896 cores: 3.5 rounds of a 256-CU part)
+// id 1: the same -> f32
+// id 2: E4M3 512 x 768 x 1024 -> f32 (6 cores; a small case for parity tests)
+// id 3: E5M2 4096^3 -> bf16 (a shape the reference publishes a time for)
+template <typename OutT, typename InT, int M, int K, int N>
+static int run(void* out, void* a, void* b, void* sa, void* sb, void* stream)
+{
+    constexpr int cores = (M / 256) * (N / 256);
+    return pto::amd::launch<&MxMatmulPerformance<OutT, InT, M, K, N, 256, 256, 128, 4>>(cores, stream, (OutT*)out, (InT*)a, (InT*)b,
+                                                                                         (float8_e8m0_t*)sa, (float8_e8m0_t*)sb);
+}
+
+extern "C" int pto_mxmatmul_performance(int id, void* out, void* a, void* b, void* sa, void* sb, void* stream)
+{
+    switch (id) {
+    case 0: return run<bfloat16_t, float8_e4m3_t, 4096, 4096, 14336>(out, a, b, sa, sb, stream);
+    case 1: return run<float, float8_e4m3_t, 4096, 4096, 14336>(out, a, b, sa, sb, stream);
+    case 2: return run<float, float8_e4m3_t, 512, 1024, 768>(out, a, b, sa, sb, stream);
+    case 3: return run<bfloat16_t, float8_e5m2_t, 4096, 4096, 4096>(out, a, b, sa, sb, stream);
+    default: return -1;
+    }
+}
+
+extern "C" int pto_mxmatmul_performance_status() { return pto::amd::device_status(); }

@@ -100,3 +100,72 @@ def test_configs0_tiled_gemm_in_the_tile_isa(pa, oracle, case):
     ref = oracle.matmul_f16(a.view(np.uint16), b.view(np.uint16), b_dn=False)
     absdot = np.abs(a.astype(np.float64)) @ np.abs(b.astype(np.float64))
     check_f32_drain(host(out), ref, absdot, 512, f"PTO-style tiled GEMM f16 512^3, case {case}")
+
+
+# ---- the block-scaled GEMM written in the tile ISA (kernels/mxmatmul_performance.hip) ------------------------------------
+MX_LIB = os.path.join(ge.PKG_DIR, "lib", "libpto_mxmatmul_performance.so")
+
+
+@pytest.fixture(scope="module")
+def mxperf():
+    assert os.path.exists(MX_LIB), "build first: make -C pto-isa-mirror_amd"
+    lib = C.CDLL(MX_LIB)
+
+    def run(case, out, a, b, sa, sb):
+        rc = lib.pto_mxmatmul_performance(case, *(C.c_void_p(t.data_ptr()) for t in (out, a, b, sa, sb)),
+                                          C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, f"launch failed with HIP error {rc}"
+        torch.cuda.synchronize()
+        assert lib.pto_mxmatmul_performance_status() == 0
+        return out
+
+    return run
+
+
+def test_mxfp8_512x768x1024_whole_matrix(pa, oracle, mxperf):
+    """Case 2: E4M3 codes over the whole finite range, scales 2^-8 .. 2^7, six cores; every output against the oracle (the
+    bar of fp8 data that spans all codes: 2^-11 sum|a||b| element-wise, 1e-3 normalised), and bit for bit against the
+    C-ABI launcher, which issues the same scaled MFMAs in the same k order."""
+    m, n, k = 512, 768, 1024
+    r = np.random.default_rng(123)
+    a = r.integers(0, 256, (m, k)).astype(np.uint8)
+    b = r.integers(0, 256, (n, k)).astype(np.uint8)
+    a[(a & 0x7F) == 0x7F] = 0x12
+    b[(b & 0x7F) == 0x7F] = 0x12
+    sa = r.integers(119, 135, (m, k // 32)).astype(np.uint8)
+    sb = r.integers(119, 135, (n, k // 32)).astype(np.uint8)
+    d = [torch.from_numpy(x).to(DEV) for x in (a, b, sa, sb)]
+    out = mxperf(2, torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV), *d)
+    got = host(out)
+    ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ob.E4M3, ob.E4M3)
+    table = oracle.mx_decode_table(ob.E4M3)
+    wa = np.abs(table[a]) * np.repeat(2.0 ** (sa.astype(np.float64) - 127), 32, 1)
+    wb = np.abs(table[b]) * np.repeat(2.0 ** (sb.astype(np.float64) - 127), 32, 1)
+    check_f32_drain(got, ref, wa @ wb.T, k, "PTO-style MXFP8 512x768x1024", max_rel=1e-3, eps=2.0 ** -11)
+    launcher = pa.gemm_mx(d[0], d[1], d[2], d[3], m, n, k, pa.E4M3, pa.E4M3, pa.F32)
+    assert torch.equal(out, launcher)
+
+
+def test_mxfp8_config3_full_size(pa, oracle, mxperf):
+    """Cases 0 and 1: configs[3] (E4M3 4096 x 14336 x 4096, operands quantised from N(0,1) by TQUANT<MXFP8>) written in
+    the tile ISA: the fp32 drain equals the launcher's bit for bit (itself held to the oracle in test_gpu_parity), the bf16
+    drain is its rounding, every output is written, and a sample is checked against the oracle directly."""
+    m, n, k = 4096, 14336, 4096
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    a, sa = pa.tquant_mx(torch.randn((m, k), generator=gen, device=DEV), pa.OCP_MXFP8, want_aux=False)
+    b, sb = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP8, want_aux=False)
+    f = mxperf(1, torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV), a, b, sa, sb)
+    out = mxperf(0, torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV), a, b, sa, sb)
+    assert not bool(torch.isnan(f).any())
+    launcher = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E4M3, pa.E4M3, pa.F32)
+    assert torch.equal(f, launcher)
+    del launcher
+    assert torch.equal(out, f.to(torch.bfloat16))
+    rows = np.unique(np.concatenate([[0, 255, 256, 2049, 4095], np.arange(7, m, 131)]))[:32]
+    cols = np.arange(0, n, 448) + np.arange(32) % 448
+    ar, bc, sar, sbc = host(sel(a, rows)), host(sel(b, cols)), host(sel(sa, rows)), host(sel(sb, cols))
+    ref = oracle.matmul_mx(ar, bc, sar, sbc, len(rows), k, len(cols), ob.E4M3, ob.E4M3)
+    table = oracle.mx_decode_table(ob.E4M3)
+    wa = np.abs(table[ar]) * np.repeat(2.0 ** (sar.astype(np.float64) - 127), 32, 1)
+    wb = np.abs(table[bc]) * np.repeat(2.0 ** (sbc.astype(np.float64) - 127), 32, 1)
+    check_f32_drain(host(f)[np.ix_(rows, cols)], ref, wa @ wb.T, k, "PTO-style MXFP8 configs[3], samples")
