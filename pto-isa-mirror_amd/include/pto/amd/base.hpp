@@ -41,6 +41,15 @@
 #ifndef PTO_AMD_STAGE_BYTES
 #define PTO_AMD_STAGE_BYTES 0
 #endif
+// PTO_AMD_TLOAD_AFTER_ACQUIRE (defined by the kernel source, off by default): a promise about program order that saves
+// the asynchronous TLOAD its own workgroup barrier.  Before it overwrites a Mat tile, TLOAD must know that no wave is
+// still reading the tile's old contents -- directly, or through Left / Right / scale windows in a TMATMUL.  By default it
+// runs a barrier of its own.  With the macro defined the kernel promises that, between the last instruction that read
+// the tile and the TLOAD, every core executes an instruction that waits for a pending load (the first TEXTRACT / TMOV /
+// TSTORE of any freshly loaded tile: that wait ends in a barrier).  The double-buffered order of the reference's
+// kernels -- TEXTRACT(panel p) ... TLOAD(panel p + 1 into the other buffer) ... TMATMUL(panel p) -- keeps the promise:
+// the other buffer's last readers were the TMATMULs of panel p - 1, before the TEXTRACT of panel p waited for its load.
+// It is what the reference writes as wait_flag(PIPE_MTE1, PIPE_MTE2) in front of such a TLOAD.
 
 // A PTO kernel entry is written `__global__ AICORE void f(...)`; here it is a device function run by pto::amd::launch.
 // (PTO_AMD_CHECK_REFERENCE_SOURCE: a device-only syntax pass over an unmodified reference kernel file, whose

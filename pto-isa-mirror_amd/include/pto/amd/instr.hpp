@@ -90,7 +90,9 @@ PTO_INST bool tload_dma(TileData& dst, GlobalData& src)
         if (!ok)
             return false;
         acquire(dst);     // an earlier asynchronous load of the same tile has landed before it is overwritten
+#ifndef PTO_AMD_TLOAD_AFTER_ACQUIRE
         __syncthreads();  // earlier readers of the tile (TMATMULs through windows, TMOVs) are done
+#endif
         constexpr int C = TileData::LineBytes / 16, total = TileData::Lines * C;
         constexpr int iters = (total + PTO_AMD_THREADS - 1) / PTO_AMD_THREADS;
         const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);

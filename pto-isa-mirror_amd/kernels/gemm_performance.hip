@@ -21,6 +21,8 @@
 #define PTO_AMD_BIAS_BYTES (1 * 1024)
 #define PTO_AMD_FB_BYTES (1 * 1024)
 #define PTO_AMD_L0S_BYTES (1 * 1024)
+// every TLOAD below follows the TEXTRACT of a freshly loaded panel and targets the buffer whose last readers came before it
+#define PTO_AMD_TLOAD_AFTER_ACQUIRE
 #define PTO_AMD_STAGE_BYTES (8 * 32 * (64 + 16))  // a band of 32 rows x (64 + 16) bytes per wave: 16-bit results leave as whole rows
 #include <pto/pto-inst.hpp>
 

@@ -19,6 +19,8 @@
 #define PTO_AMD_BIAS_BYTES 256
 #define PTO_AMD_FB_BYTES 256
 #define PTO_AMD_L0S_BYTES 512
+// every TLOAD below follows the TEXTRACT of a freshly loaded panel and targets the buffer whose last readers came before it
+#define PTO_AMD_TLOAD_AFTER_ACQUIRE
 #define PTO_AMD_STAGE_IN_L1
 #define PTO_AMD_STAGE_BYTES (8 * 16 * (128 + 16))  // 16-bit results: a wave stages 16 rows of two side-by-side blocks
 #include <pto/pto-inst.hpp>
