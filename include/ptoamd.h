@@ -82,7 +82,7 @@ enum { PTOAMD_MEMCPY_H2H = 0, PTOAMD_MEMCPY_H2D = 1, PTOAMD_MEMCPY_D2H = 2, PTOA
  * caller that captures them into a HIP graph needs.  Without it the first call per kernel and device sets up lazily. */
 int ptoamd_init(int device);
 int ptoamd_finalize(void);                      /* aclrtResetDevice + aclFinalize */
-/* The dispatchers' environment switches (PTOAMD_TILE, PTOAMD_NO_TAIL_SPLIT, PTOAMD_FORCE_GENERIC,
+/* The dispatchers' environment switches (PTOAMD_TILE, PTOAMD_NO_TAIL_SPLIT, PTOAMD_MX_16X16, PTOAMD_FORCE_GENERIC,
  * PTOAMD_B_ND_TRANSPOSE, PTOAMD_GEMV_*) are read once per process; this reads them again.  No counterpart in the
  * reference (its simulator reads PTO_CPU_MAX_THREADS and the buffer sizes once too, cpu/NPUMemoryModel.hpp:128-135). */
 int ptoamd_reload_options(void);

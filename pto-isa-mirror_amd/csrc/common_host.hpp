@@ -25,6 +25,7 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 // tests plain fields instead of calling getenv.
 struct Options {
     int tile = -1;               // PTOAMD_TILE=0..6: run this tile shape; -1 = choose by problem size
+    bool mx_16x16 = false;       // PTOAMD_MX_16X16=1: the block-scaled fp8 256 x 256 tile runs on the 16x16x128 instruction
     bool no_tail_split = false;  // PTOAMD_NO_TAIL_SPLIT=1: never split a half-full last round off as smaller tiles
     int tail_tile = 0;           // PTOAMD_TAIL_TILE=5|6|7: the tail's tile; 0 = 256x128 ring-3 tiles (block-scaled) or 128x128
     bool force_generic = false;  // PTOAMD_FORCE_GENERIC=1: everything runs on the order-exact generic kernels

@@ -294,8 +294,6 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
         int t = options().tile;
         if (ragged_k && t > 5)  // tiles 6 and 7 exist for whole slabs only
             t = 5;
-        if (t == 3)  // the four-wave form of the 256 x 256 DMA tile is no longer built
-            t = 4;
         if (t == 0)  // nor is the register-staged 256 x 256 tile (it spilled: 315 against 176 us for the 128 x 128 one on
             t = 1;   // bf16 4096 x 4096 x 4104)
         if (t < 3 || dtl_ok)
@@ -327,9 +325,9 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
 // then costs a half or a quarter of a 256x256 tile's time instead of a whole round (MXFP8 4096 x 14336 x 4096, 3.5
 // rounds of 256 CUs).  PTOAMD_TILE (an explicit tile) and PTOAMD_NO_TAIL_SPLIT=1 switch the split off;
 // PTOAMD_TAIL_TILE=5|6|7 picks the tail's tile (default: 7 for the block-scaled types, 5 otherwise).
-static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStream_t stream)
+static hipError_t launch_tiles_as(int tile, int op, const TileGemmParams& p, hipStream_t stream)
 {
-    if (tile == 4 && options().tile < 0 && !options().no_tail_split) {
+    if ((tile == 4 || tile == 3) && options().tile < 0 && !options().no_tail_split) {
         const int cus = device_compute_units();
         const int tiles_m = (p.m + 255) / 256, tiles_n = (p.n + 255) / 256;
         int whole = tiles_n;  // tile columns that make whole rounds
@@ -340,7 +338,7 @@ static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStr
             const int n1 = whole * 256;
             TileGemmParams head = p;
             head.n = n1;
-            const hipError_t e = launch_gemm_tile(4, op, head, stream);
+            const hipError_t e = launch_gemm_tile(tile, op, head, stream);
             if (e != hipSuccess)
                 return e;
             TileGemmParams tail = p;
@@ -368,13 +366,34 @@ static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStr
     return launch_gemm_tile(tile, op, p, stream);
 }
 
+static hipError_t launch_tiles(int tile, int op, const TileGemmParams& p, hipStream_t stream)
+{
+    // tile id 3: the 16x16x128 form of the block-scaled fp8 types' large tile (the other types have one form, under both
+    // ids).  Same results bit for bit and, on MXFP8 4096 x 14336 x 4096, the same time: 2 718 clocks per slab at 1.71 GHz
+    // against 2 500 at 1.58 GHz on one box -- what the part sustains under this kernel is a rate of matrix work, not a
+    // clock.  The 32x32x64 form also takes ragged edges and stays the default; PTOAMD_MX_16X16=1 selects the other.
+    const int big = options().mx_16x16 ? 3 : 4;
+    if (tile == 4)
+        return launch_tiles_as(big, op, p, stream);
+    return launch_tiles_as(tile, op, p, stream);
+}
+
 static bool force_generic() { return options().force_generic; }
+
+// the tile id a launch of `tile` ends up on (the block-scaled fp8 types' large tile has two forms, see launch_tiles)
+static int tile_as_launched(int tile, int op, int m, int n)
+{
+    const bool fp8 = op >= TOP_FP8_E4E4 && op != TOP_FP4;
+    if (fp8 && m % 256 == 0 && n % 256 == 0 && ((tile == 4 && options().mx_16x16) || tile == 3))
+        return 3;
+    return tile == 3 ? 4 : tile;
+}
 
 static const char* tile_kernel_name(int tile, int op)
 {
     static const char* ops[TOP_COUNT] = {"bf16", "f16", "i8", "fp8_e4m3_e4m3", "fp8_e5m2_e5m2", "fp8_e4m3_e5m2",
                                          "fp8_e5m2_e4m3", "fp4_e2m1"};
-    static const char* tiles[8] = {"tile256x256", "tile128x128", "tile64x64", "tile256x256w4_dtl", "tile256x256w8_dtl",
+    static const char* tiles[8] = {"tile256x256", "tile128x128", "tile64x64", "tile256x256w8x16_dtl", "tile256x256w8_dtl",
                                    "tile128x128_dtl", "tile256x128_dtl", "tile256x128r3_dtl"};
     static thread_local char buf[64];
     snprintf(buf, sizeof buf, "%s_%s", tiles[tile], ops[op]);
@@ -618,7 +637,7 @@ static int gemm_common(void* c, int c_type, const void* a, const void* b, int ab
                         dma_offsets_fit(m, n, lda_b, ldb_kmajor, k_bytes);
     const int tile = pick_tile(m, n, k_bytes, false, false, dma_ok, op == TOP_BF16 || op == TOP_F16 || op == TOP_I8);
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
-    set_last_kernel(tile_kernel_name(tile, op));
+    set_last_kernel(tile_kernel_name(tile_as_launched(tile, op, m, n), op));
     return PTOAMD_OK;
 }
 
@@ -781,7 +800,7 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
     const int tile = e1m2 ? pick_tile(m, n, k, true, false, false)
                           : pick_tile(m, n, k_bytes, true, a4, scale_dma_ok && dma_offsets_fit(m, n, lda_b, ldb_b, k_bytes));
     PTOAMD_HIP_CHECK(launch_tiles(tile, op, p, stream));
-    set_last_kernel(tile_kernel_name(tile, op));
+    set_last_kernel(tile_kernel_name(tile_as_launched(tile, op, m, n), op));
     return PTOAMD_OK;
 }
 

@@ -220,6 +220,26 @@ struct OpFP8 {
         c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c, BFMT, AFMT, SEL, (int)sb, SEL, (int)sa);
     }
 };
+// The same operands on the 16x16x128 scaled MFMA: a lane holds 32 bytes of one of 16 rows, the whole 128-element K
+// extent of a slab goes in one instruction, and each lane supplies one scale byte (lane group b: MX block b of the row).
+template <int AFMT, int BFMT>
+struct OpFP8x16 {
+    static constexpr int BLK = 16, ACC_REGS = 4;
+    using Acc = f32x4;
+    using Elem = float;
+    static constexpr int FRAG_BYTES = 32;
+    static constexpr bool SCALED = true;
+    static constexpr int GROUPS_PER_SLAB = 4;
+    __device__ static __forceinline__ void mma(Acc& c, const uint4* a, const uint4* b, uint32_t sa, uint32_t sb)
+    {
+        i32x8 av, bv;
+        av.s0 = a[0].x; av.s1 = a[0].y; av.s2 = a[0].z; av.s3 = a[0].w;
+        av.s4 = a[1].x; av.s5 = a[1].y; av.s6 = a[1].z; av.s7 = a[1].w;
+        bv.s0 = b[0].x; bv.s1 = b[0].y; bv.s2 = b[0].z; bv.s3 = b[0].w;
+        bv.s4 = b[1].x; bv.s5 = b[1].y; bv.s6 = b[1].z; bv.s7 = b[1].w;
+        c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, c, BFMT, AFMT, 0, (int)sb, 0, (int)sa);
+    }
+};
 // 16 packed fp4 codes (8 bytes, even k in the low nibble) -> the 16 E4M3 bytes of the same values.  mode 1: E2M1
 // (0, 0.5, 1, 1.5, 2, 3, 4, 6), mode 2: E1M2 (0, 0.25, ... 1.75); bit 3 of a code is the sign.
 __device__ __forceinline__ uint4 expand_fp4_to_e4m3(uint2 x, int mode)
@@ -302,7 +322,7 @@ struct TileCfg {
     static_assert(LDS_BYTES <= 160 * 1024, "the ring and the scale buffers fit the CU's LDS");
     static constexpr int LA = BM * 8 / THREADS, LB = BN * 8 / THREADS;  // 16-byte chunks per thread per slab
     static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "wave tiles are made of 32x32 blocks");
-    static_assert(BLK == 32 || Op::FRAG_BYTES == 16, "the 16x16 instructions take 16-byte fragments");
+    static_assert(BLK == 32 || Op::FRAG_BYTES == 16 || Op::SCALED, "the plain 16x16 instructions take 16-byte fragments");
     static_assert((BM * 8) % THREADS == 0 && (BN * 8) % THREADS == 0, "slab chunks must divide over the workgroup");
 };
 

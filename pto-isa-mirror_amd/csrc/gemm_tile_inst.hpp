@@ -3,6 +3,7 @@
 // parallel translation units.
 #include "common_host.hpp"
 #include "gemm_tile_dtl.hpp"
+#include "gemm_tile_mx16.hpp"
 
 namespace ptoamd {
 
@@ -48,6 +49,20 @@ static hipError_t launch_dtl(const TileGemmParams& p, hipStream_t stream)
     return hipGetLastError();
 }
 
+// the 256 x 256 tile of the block-scaled fp8 types on the 16x16x128 instruction (whole 128-byte slabs of K only)
+template <class Cfg>
+static hipError_t launch_mx16(const TileGemmParams& p, hipStream_t stream)
+{
+    const hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(&gemm_tile_mx16_kernel<Cfg>), Cfg::LDS_BYTES);
+    if (e != hipSuccess || p.m <= 0)
+        return e;
+    if (p.k_bytes % 128 != 0)
+        return hipErrorInvalidValue;
+    const int tiles = ((p.m + Cfg::BM - 1) / Cfg::BM) * ((p.n + Cfg::BN - 1) / Cfg::BN);
+    hipLaunchKernelGGL((gemm_tile_mx16_kernel<Cfg>), dim3(tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream, p);
+    return hipGetLastError();
+}
+
 #ifdef PTOAMD_TILE_RAGGED_K
 #define PTOAMD_RK true
 #else
@@ -58,7 +73,7 @@ hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 {
     if (tile == TILE_PREPARE_ALL) {  // every kernel of this unit gets its launch attributes on the current device
         TileGemmParams none{};
-        for (int t : {4, 5, 6, 7, 1, 2}) {
+        for (int t : {4, 3, 5, 6, 7, 1, 2}) {
             const hipError_t e = PTOAMD_TILE_FN(t, none, stream);
             if (e != hipSuccess)
                 return e;
@@ -71,6 +86,12 @@ hipError_t PTOAMD_TILE_FN(int tile, const TileGemmParams& p, hipStream_t stream)
 #ifdef PTOAMD_TILE_OP16  // the large eight-wave tile runs on the 16x16 instructions where the operand type has them
         case 3:
         case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP16>, PTOAMD_RK>(p, stream);
+#elif defined(PTOAMD_TILE_MX16)  // block-scaled fp8: id 3 is the large tile on the 16x16x128 instruction
+        case 3:  // (tiles that lie inside the matrix; a ragged edge takes the 32x32x64 form, whose loader clamps its rows)
+            if (p.m % 256 == 0 && p.n % 256 == 0)
+                return launch_mx16<TileCfg<256, 256, 2, 4, PTOAMD_TILE_MX16>>(p, stream);
+            return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>, PTOAMD_RK>(p, stream);
+        case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>, PTOAMD_RK>(p, stream);
 #else
         case 3:
         case 4: return launch_dtl<TileCfg<256, 256, 2, 4, PTOAMD_TILE_OP>, PTOAMD_RK>(p, stream);

@@ -47,6 +47,7 @@ void read_options()
     if (t != nullptr && t[0] >= '0' && t[0] <= '7')
         o.tile = t[0] - '0';
     o.no_tail_split = getenv("PTOAMD_NO_TAIL_SPLIT") != nullptr;
+    o.mx_16x16 = getenv("PTOAMD_MX_16X16") != nullptr;
     const char* tt = getenv("PTOAMD_TAIL_TILE");
     if (tt != nullptr && tt[0] >= '5' && tt[0] <= '7')
         o.tail_tile = tt[0] - '0';

@@ -187,9 +187,9 @@ def test_operands_past_4_gib_leave_the_dma_tiles(pa, oracle):
     del base, a
 
 
-TILE_NAMES = ("tile256x256_", "tile128x128_", "tile64x64_", "tile256x256w4_dtl", "tile256x256w8_dtl", "tile128x128_dtl",
+TILE_NAMES = ("tile256x256_", "tile128x128_", "tile64x64_", "tile256x256w8x16_dtl", "tile256x256w8_dtl", "tile128x128_dtl",
               "tile256x128_dtl")
-ALL_TILES = [1, 2, 4, 5, 6]  # (ids 0 and 3, a register-staged and a four-wave 256 x 256 tile, are no longer built: they select 1 and 4)
+ALL_TILES = [1, 2, 4, 5, 6]  # (id 0, a register-staged 256 x 256 tile, is no longer built and selects 1; id 3 is tile 4 except for block-scaled fp8)
 
 
 def expect_tile(pa, tile, k_bytes, ragged_k_form=False):
@@ -861,6 +861,89 @@ def test_mx_scale_chunks_across_slabs(pa, oracle, typ, tile):
             got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[typ], PA_T[typ], pa.F32))
             assert "_dtl_" in pa.last_kernel(), pa.last_kernel()
         assert relerr(got, ref) <= 2e-2, (g, pa.last_kernel())
+
+
+@pytest.mark.parametrize("ta,tb", [(ob.E4M3, ob.E4M3), (ob.E5M2, ob.E5M2), (ob.E4M3, ob.E5M2), (ob.E5M2, ob.E4M3)])
+def test_mx_large_tile_on_the_16x16x128_instruction(pa, oracle, ta, tb):
+    """The second form of the block-scaled fp8 256 x 256 tile (one 16x16x128 scaled MFMA k-step per 128-byte slab, one
+    fragment set refilled in place, scales read as bytes): the oracle's bars, and the bits of the 32x32x64 form.  It
+    takes tiles that lie inside the matrix; a ragged edge falls back to the other form."""
+    r = np.random.default_rng(ta * 16 + tb + 900)
+    for m, n, k in ((256, 256, 512), (256, 512, 1024), (512, 256, 2048)):
+        a, _, sa, sb = _mx_inputs(r, ta, m, n, k)
+        _, b, _, _ = _mx_inputs(r, tb, m, n, k)
+        ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ta, tb)
+        with tile_env(PTOAMD_TILE=3):
+            got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[ta], PA_T[tb], pa.F32))
+            assert pa.last_kernel().startswith("tile256x256w8x16_dtl_fp8"), pa.last_kernel()
+        ua = _mx_unpack(oracle, a, ta) * np.repeat(2.0 ** (sa.astype(np.float64) - 127), 32, 1)
+        ub = _mx_unpack(oracle, b, tb) * np.repeat(2.0 ** (sb.astype(np.float64) - 127), 32, 1)
+        check_f32_drain(got, ref, np.abs(ua) @ np.abs(ub).T, k, f"MX 16x16x128 {ta}x{tb} {m}x{n}x{k}", max_rel=1e-3, eps=2.0 ** -11)
+        with tile_env(PTOAMD_TILE=4):
+            other = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[ta], PA_T[tb], pa.F32))
+            assert pa.last_kernel().startswith("tile256x256w8_dtl_fp8"), pa.last_kernel()
+        assert np.array_equal(got.view(np.uint32), other.view(np.uint32))
+    with tile_env(PTOAMD_TILE=3):  # a ragged edge: the 32x32x64 form
+        m, n, k = 300, 256, 512
+        a, b, sa, sb = _mx_inputs(r, ta, m, n, k)
+        got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, PA_T[ta], PA_T[ta], pa.F32))
+        assert pa.last_kernel().startswith("tile256x256w8_dtl_fp8"), pa.last_kernel()
+        assert relerr(got, oracle.matmul_mx(a, b, sa, sb, m, k, n, ta, ta)) <= 2e-2
+
+
+def test_mx_16x16x128_form_scale_bytes_and_slab_counts(pa, oracle):
+    """Which scale byte meets which 32 elements: a single non-zero element per row at a random K position, scales from a
+    14-binade range, products and sums exact in fp32 -- bit-equal to the oracle; a large exponent either side of every
+    16-byte scale chunk boundary; plain fp8 (no scale arrays) over 1 - 9 slabs; and configs[3]'s shape under
+    PTOAMD_MX_16X16=1 (head launch on this form, tail on the 256 x 128 tile) against the default's bits."""
+    m, n, k = 256, 256, 512
+    r = np.random.default_rng(902)
+    a = np.zeros((m, k), np.uint8)
+    b = np.full((n, k), 0x38, np.uint8)  # 1.0
+    a[np.arange(m), r.integers(0, k, m)] = 0x40  # 2.0
+    sa = r.integers(120, 134, (m, k // 32)).astype(np.uint8)
+    sb = r.integers(120, 134, (n, k // 32)).astype(np.uint8)
+    ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ob.E4M3, ob.E4M3)
+    with tile_env(PTOAMD_TILE=3):
+        got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, pa.E4M3, pa.E4M3, pa.F32))
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    k = 2048
+    a, b, _, _ = _mx_inputs(r, ob.E4M3, m, n, k)
+    for g in (0, 1, 2, 3, 4, 15, 16, 17, 31, 32, 47, 48, 63):
+        sa = np.full((m, k // 32), 121, np.uint8)
+        sb = np.full((n, k // 32), 122, np.uint8)
+        sa[:, g] = 133
+        sb[1::2, g] = 130
+        sa[m - 1, (g + 5) % 64] = 129
+        sa[17, (g + 9) % 64] = 131
+        sb[35, (g + 11) % 64] = 128
+        ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ob.E4M3, ob.E4M3)
+        with tile_env(PTOAMD_TILE=3):
+            got = host(pa.gemm_mx(dev(a), dev(b), dev(sa), dev(sb), m, n, k, pa.E4M3, pa.E4M3, pa.F32))
+            assert pa.last_kernel().startswith("tile256x256w8x16_dtl"), pa.last_kernel()
+        assert relerr(got, ref) <= 2e-2, g
+    for k in (128, 256, 384, 512, 640, 1152):
+        a = r.integers(0, 256, (m, k)).astype(np.uint8)
+        b = r.integers(0, 256, (n, k)).astype(np.uint8)
+        a[(a & 0x7F) == 0x7F] = 0x12
+        b[(b & 0x7F) == 0x7F] = 0x12
+        with tile_env(PTOAMD_TILE=3):
+            got = host(pa.gemm_fp8(dev(a), dev(b), pa.E4M3, pa.E4M3, pa.F32))
+            assert pa.last_kernel().startswith("tile256x256w8x16_dtl"), pa.last_kernel()
+        with tile_env(PTOAMD_TILE=4):
+            other = host(pa.gemm_fp8(dev(a), dev(b), pa.E4M3, pa.E4M3, pa.F32))
+        assert np.array_equal(got.view(np.uint32), other.view(np.uint32)), k
+        assert relerr(got, oracle.matmul_fp8(a, b, b_dn=True)) <= 2e-2, k
+    m, n, k = 4096, 14336, 4096
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    a, sa = pa.tquant_mx(torch.randn((m, k), generator=gen, device=DEV), pa.OCP_MXFP8, want_aux=False)
+    b, sb = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP8, want_aux=False)
+    ref = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E4M3, pa.E4M3, pa.BF16)
+    assert pa.last_kernel() == "tile256x256w8_dtl_fp8_e4m3_e4m3"
+    with tile_env(PTOAMD_MX_16X16=1):
+        got = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E4M3, pa.E4M3, pa.BF16)
+        assert pa.last_kernel() == "tile256x256w8x16_dtl_fp8_e4m3_e4m3"
+    assert torch.equal(got, ref)
 
 
 def test_mx_scale_rows_that_are_not_16_byte_multiples_take_the_register_tiles(pa, oracle):
