@@ -56,6 +56,19 @@ PTO_INST void acquire(TileData& t)
     }
 }
 
+// Several freshly loaded Mat tiles at once: one wait and one workgroup barrier for all of them, where acquiring them one
+// by one (the first TEXTRACT / TMOV of each) brings a barrier per tile.
+template <typename... Tiles>
+PTO_INST void acquire_all(Tiles&... t)
+{
+    static_assert(((Tiles::Loc == TileType::Mat) && ...), "only Mat tiles are loaded asynchronously");
+    if ((... || (t.pend_ != 0))) {  // the same value in every thread of the core
+        dma_wait();
+        __syncthreads();
+        ((t.pend_ = 0), ...);
+    }
+}
+
 // ---- TLOAD as LDS-DMA -------------------------------------------------------------------------------------------------
 // A boxed Mat tile is stored as swizzled lines (rows for the A-side layouts, columns for the B-side ones).  When the
 // global tensor delivers those lines contiguously -- ND for row lines, DN for column lines -- every 16-byte chunk of
@@ -1302,3 +1315,13 @@ PTO_INST RecordEvent TGEMV_BIAS(TileRes& c, TileLeftT& a, TileRightT& b, TileBia
 }
 
 }  // namespace pto
+
+// wait_flag(PIPE_MTE2, PIPE_MTE1, id, tiles...): the reference's "the loads have arrived" flag, given the Mat tiles it
+// stands for.  Plain wait_flag orders nothing here (every instruction waits for what it reads); this form lets a kernel
+// wait for the asynchronous TLOADs of several tiles with one barrier, in the place where the reference program has its
+// wait_flag(PIPE_MTE2, PIPE_MTE1, ...) (kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:131-136).
+template <typename... Tiles, typename = std::enable_if_t<(sizeof...(Tiles) > 0)>>
+PTO_INST void wait_flag(pto::pipe_t, pto::pipe_t, pto::event_t, Tiles&... tiles)
+{
+    pto::amd::acquire_all(tiles...);
+}

@@ -11,8 +11,9 @@
 //   * 20 KiB of fix-pipe staging let TSTORE turn the accumulator blocks into whole 64-byte rows of bf16;
 //   * a core executes its tile instructions in program order, so the copy-in of panel p + 1 is issued *before* the
 //     TMATMULs of panel p (TLOAD only starts the copies; the TEXTRACT of the next iteration waits for them), where the
-//     reference issues it in the same iteration and lets the MTE2 queue run ahead.  The event flags of the reference
-//     program have nothing left to order and are not written out.
+//     reference issues it in the same iteration and lets the MTE2 queue run ahead.  Of the event flags of the reference
+//     program one is left: wait_flag(PIPE_MTE2, PIPE_MTE1) names the two tiles of a panel, so that their arrival costs
+//     one barrier instead of one per tile; the others have nothing left to order and are not written out.
 #define PTO_AMD_THREADS 512
 #define PTO_AMD_L1_BYTES (128 * 1024)
 #define PTO_AMD_L0A_BYTES (1 * 1024)
@@ -90,6 +91,7 @@ __global__ AICORE void GemmPerformance(__gm__ OutT* out, __gm__ InT* a, __gm__ I
     // one panel: make its slices the operands, start the copy-in of the next panel into the other L1 slot, multiply
     auto panel = [&](auto slot, int p) __attribute__((always_inline)) {
         constexpr int cur = decltype(slot)::value, nxt = cur ^ 1;
+        wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0, aMat[cur], bMat[cur]);  // the panel has landed: one wait for both tiles
         for (int s = 0; s < stepK; ++s) {
             TEXTRACT(aTile, aMat[cur], 0, s * baseK);
             TEXTRACT(bTile, bMat[cur], s * baseK, 0);

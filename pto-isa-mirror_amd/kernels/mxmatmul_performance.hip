@@ -10,7 +10,8 @@
 // scale tiles per side (4 KiB each: 256 lines of 16 groups, the smallest tile whose lines a 16-byte copy can move); the
 // Left / Right tiles and their scale tiles are windows onto those, so the L0 regions need no bytes; the fix-pipe staging
 // lies over the start of L1, whose panels are dead when the tile is stored.  As in the bf16 kernel, a panel's copy-in is
-// issued before the TMATMUL_MX of the panel before it, and the event flags of the reference program are not written out.
+// issued before the TMATMUL_MX of the panel before it.  Of the reference program's event flags one is written out:
+// wait_flag(PIPE_MTE2, PIPE_MTE1) names the tiles of a panel, whose arrival then costs one barrier instead of one per tile.
 #define PTO_AMD_THREADS 512
 #define PTO_AMD_L1_BYTES (144 * 1024)
 #define PTO_AMD_L0A_BYTES 256
@@ -104,6 +105,8 @@ __global__ AICORE void MxMatmulPerformance(__gm__ OutT* out, __gm__ InT* a, __gm
         pto::amd::static_for<stepKscale>([&](auto qc) {
             constexpr int q = decltype(qc)::value, cur = q & 1, nxt = cur ^ 1;
             const int p = p0 + q;
+            // the panel (and, at a chunk's first panel, the scale chunk) has landed: one wait for all four tiles
+            wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0, aMat[cur], bMat[cur], aScaleMat[scur], bScaleMat[scur]);
             TEXTRACT(aTile, aMat[cur], 0, 0);
             TEXTRACT(bTile, bMat[cur], 0, 0);
             TEXTRACT(aScale, aScaleMat[scur], 0, q * groups);
