@@ -238,12 +238,17 @@ int ptoamd_gemm_mx_bias(void* c, int c_type, const void* a, const void* b, int a
  * (the TLOAD + TMOV of a scale tile, cpu/TLoad.hpp:287-321 with the MX_* maps of cpu/tile_offsets.hpp:233-268) are
  * re-laid into the workspace first, and the fastest (direct-to-LDS) kernels run.  ptoamd_gemm_mx reads such scales where
  * they lie instead, with the register-staged kernels; neither form allocates.  workspace: 256-byte aligned, at least ptoamd_gemm_mx_workspace_bytes(...) bytes (0 for the
- * two natural layouts: workspace may then be NULL).
+ * two natural layouts: workspace may then be NULL).  A row-major B (PTOAMD_B_ND) of fp8 codes is transposed inside the
+ * register-staged kernels' loader, every element once per row tile; a workspace of
+ * ptoamd_gemm_mx_workspace_bytes_b_nd(...) bytes (the scales' part, rounded up to 256 bytes, plus a [N][K] copy of B with
+ * rows padded to 16 bytes) lets the call transpose B once and run the direct-to-LDS kernels instead (M above 128; a
+ * smaller workspace keeps the in-loader form).  Packed fp4 codes are never transposed.
  */
 int ptoamd_gemm_mx_ws(void* c, int c_type, const void* a, const void* b, int a_type, int b_type, const uint8_t* sa,
                       const uint8_t* sb, int sa_layout, int sb_layout, const float* c_in, int m, int n, int k, int lda,
                       int ldb, int ldc, int b_layout, void* workspace, size_t workspace_bytes, void* stream);
 size_t ptoamd_gemm_mx_workspace_bytes(int m, int n, int k, int sa_layout, int sb_layout);
+size_t ptoamd_gemm_mx_workspace_bytes_b_nd(int m, int n, int k, int sa_layout, int sb_layout, int b_type);
 
 /*
  * ptoamd_gemm_mx_ws with the workspace inside the library: a static device array of PTOAMD_STATIC_SCRATCH_BYTES, one

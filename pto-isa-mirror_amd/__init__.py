@@ -35,6 +35,7 @@ _lib = C.CDLL(LIB_PATH)
 _lib.ptoamd_last_error.restype = C.c_char_p
 _lib.ptoamd_last_kernel.restype = C.c_char_p
 _lib.ptoamd_gemm_mx_workspace_bytes.restype = C.c_size_t
+_lib.ptoamd_gemm_mx_workspace_bytes_b_nd.restype = C.c_size_t
 _lib.ptoamd_gemm_workspace_bytes.restype = C.c_size_t
 
 EXPORTS = [
@@ -44,7 +45,7 @@ EXPORTS = [
     "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
     "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_ws", "ptoamd_gemm_workspace_bytes", "ptoamd_gemm_fp8", "ptoamd_gemm_requant", "ptoamd_gemm_atomic_add", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
     "ptoamd_gemm_mx_ws",
-    "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
+    "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_workspace_bytes_b_nd", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
     "ptoamd_tquant_int8_para", "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_tdequant_para", "ptoamd_mx_scale_relayout",
     "ptoamd_last_kernel", "ptoamd_reload_options",
 ]
@@ -193,7 +194,11 @@ def gemm_mx_static(a, b, sa, sb, m, n, k, a_type, b_type, out, sa_layout=MX_A_ND
     return out
 
 
-def gemm_mx_workspace_bytes(m, n, k, sa_layout=MX_A_ND, sb_layout=MX_B_DN):
+def gemm_mx_workspace_bytes(m, n, k, sa_layout=MX_A_ND, sb_layout=MX_B_DN, b_layout=B_DN, b_type=E4M3):
+    """Bytes of workspace gemm_mx(..., workspace=...) needs; with b_layout=B_ND it includes the room for a transposed
+    copy of a row-major fp8 B, which lets the direct-to-LDS kernels run."""
+    if b_layout == B_ND:
+        return int(_lib.ptoamd_gemm_mx_workspace_bytes_b_nd(m, n, k, sa_layout, sb_layout, b_type))
     return int(_lib.ptoamd_gemm_mx_workspace_bytes(m, n, k, sa_layout, sb_layout))
 
 

@@ -715,14 +715,38 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
         PTOAMD_REQUIRE(lda % 2 == 0 && ldb % 2 == 0, PTOAMD_E_ALIGNMENT, "%s: fp4 leading dimensions must be even", who);
     const int out_kind = c_type == PTOAMD_F32 ? OUT_F32 : (c_type == PTOAMD_F16 ? OUT_F16 : OUT_BF16);
     const int bits = a8 ? 8 : 4;
-    const long k_bytes = (long)k * bits / 8, lda_b = (long)lda * bits / 8, ldb_b = (long)ldb * bits / 8;
+    const long k_bytes = (long)k * bits / 8, lda_b = (long)lda * bits / 8;
+    long ldb_b = (long)ldb * bits / 8;
     // The scaled MFMA has no E1M2 operand format, but every E1M2 (and E2M1) value is an E4M3 value: a product with an
     // E1M2 operand runs on the E4M3 x E4M3 instruction, the register-staged loader expanding both operands' packed
     // nibbles to E4M3 bytes on their way into LDS (the block scales are per 32 elements in either form).
     const bool e1m2 = a_type == PTOAMD_E1M2 || b_type == PTOAMD_E1M2;
     const bool expand_ok = e1m2 && b_layout == PTOAMD_B_DN && (k % 128) == 0 && (reinterpret_cast<uintptr_t>(a) & 7u) == 0 &&
                            (reinterpret_cast<uintptr_t>(b) & 7u) == 0 && (lda_b % 8) == 0 && (ldb_b % 8) == 0;
-    // a row-major B of one-byte codes is transposed on its way into LDS by the register-staged tiles; packed fp4 is not
+    // Workspace layout: [M][K/32] scales of A (when they need re-laying), rounded up to 256 bytes, the [N][K/32] scales of
+    // B likewise, then -- when B is row-major fp8 and the room is there -- a [N][K] copy of B, rows padded to 16 bytes.
+    const int kg = k / 32;
+    int sa_mode = sa_layout == PTOAMD_MX_A_ND ? 0 : (sa_layout == PTOAMD_MX_A_ZZ ? 1 : 2);
+    int sb_mode = sb_layout == PTOAMD_MX_B_DN ? 0 : (sb_layout == PTOAMD_MX_B_NN ? 1 : 2);
+    const size_t need_a = sa_mode != 0 ? (((size_t)m * kg + 255) & ~(size_t)255) : 0;
+    const size_t need_b = sb_mode != 0 ? (size_t)n * kg : 0;
+    const size_t bt_at = (need_a + need_b + 255) & ~(size_t)255;
+    const long bt_pitch = ws_row_bytes(k_bytes);
+    // A row-major B of one-byte codes: with room in the workspace it is transposed there first and the DMA tiles run (a
+    // large product: every B element would otherwise be scattered into LDS once per row tile); without, the
+    // register-staged tiles transpose it on its way into LDS.  Packed fp4 has neither.
+    const bool b_via_ws = b_layout == PTOAMD_B_ND && a8 && ws != nullptr && !force_generic() && m > 128 &&
+                          ws_bytes >= bt_at + (size_t)n * (size_t)bt_pitch && (k_bytes % 128) == 0;
+    if (b_via_ws) {  // from here on B is the column-major copy
+        const int rc = transpose_b<uint8_t>(ws + bt_at, b, k, n, ldb_b, bt_pitch, stream);
+        if (rc != PTOAMD_OK)
+            return rc;
+        b = ws + bt_at;
+        b_layout = PTOAMD_B_DN;
+        ldb = (int)bt_pitch;
+        ldb_b = bt_pitch;
+        ws_bytes = bt_at;
+    }
     const bool b_in_kernel = b_layout == PTOAMD_B_ND && a8 && (n % 16) == 0;
     const bool tile_ok = !force_generic() &&
                          (e1m2 ? expand_ok
@@ -738,17 +762,11 @@ static int gemm_mx_common(const char* who, void* c, int c_type, const void* a, c
         g.sa_layout = sa_layout; g.sb_layout = sb_layout;
         return launch_generic(g, stream);
     }
-    const int kg = k / 32;
     // Scales that are not plain [M][K/32] / [N][K/32] rows: with a workspace they are re-laid into it and the DMA tiles run
     // (the fastest form for a large product); without one the register-staged tiles address the pairs of the caller's
     // layout directly.  Nothing is allocated either way.
     const uint8_t* sa_use = sa;
     const uint8_t* sb_use = sb;
-    int sa_mode = sa_layout == PTOAMD_MX_A_ND ? 0 : (sa_layout == PTOAMD_MX_A_ZZ ? 1 : 2);
-    int sb_mode = sb_layout == PTOAMD_MX_B_DN ? 0 : (sb_layout == PTOAMD_MX_B_NN ? 1 : 2);
-    // workspace layout: [M][K/32] scales of A, rounded up to 256 bytes, then [N][K/32] scales of B
-    const size_t need_a = sa_mode != 0 ? (((size_t)m * kg + 255) & ~(size_t)255) : 0;
-    const size_t need_b = sb_mode != 0 ? (size_t)n * kg : 0;
     if (ws != nullptr && need_a + need_b > 0) {
         PTOAMD_REQUIRE(need_a + need_b <= ws_bytes, PTOAMD_E_INVALID,
                        "%s: the scale layouts need %zu bytes of workspace, %zu available", who, need_a + need_b, ws_bytes);
@@ -844,6 +862,16 @@ int ptoamd_gemm_mx_static(void* c, int c_type, const void* a, const void* b, int
         return rc;
     return gemm_mx_common("ptoamd_gemm_mx_static", c, c_type, a, b, a_type, b_type, sa, sb, sa_layout, sb_layout, c_in, m, n, k,
                           lda, ldb, ldc, b_layout, ws, PTOAMD_STATIC_SCRATCH_BYTES, stream_);
+}
+
+size_t ptoamd_gemm_mx_workspace_bytes_b_nd(int m, int n, int k, int sa_layout, int sb_layout, int b_type)
+{
+    if (m <= 0 || n <= 0 || k <= 0)
+        return 0;
+    const size_t scales = (ptoamd_gemm_mx_workspace_bytes(m, n, k, sa_layout, sb_layout) + 255) & ~(size_t)255;
+    if (b_type != PTOAMD_E4M3 && b_type != PTOAMD_E5M2)
+        return scales;  // packed fp4 codes are not transposed
+    return scales + (size_t)n * (size_t)ws_row_bytes(k);
 }
 
 size_t ptoamd_gemm_mx_workspace_bytes(int m, int n, int k, int sa_layout, int sb_layout)

@@ -1005,6 +1005,52 @@ def test_gemm_mx_workspace_form(pa, oracle):
                    workspace=ws[:need - 256])
 
 
+def test_gemm_mx_row_major_b_through_the_workspace(pa, oracle):
+    """A row-major (B_ND) fp8 B: the register-staged tiles transpose it in their loader, every element once per row tile.
+    With a workspace of gemm_mx_workspace_bytes(..., b_layout=B_ND) the call transposes it once into the workspace and the
+    DMA tiles run -- same bits; boxed scales share the workspace; a workspace that only holds the scales keeps the
+    in-loader form; the static-scratch entry point does the same inside the library's array."""
+    r = np.random.default_rng(78)
+    m, n, k = 512, 384, 1024
+    a, b, sa, sb = _mx_inputs(r, ob.E4M3, m, n, k)
+    ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ob.E4M3, ob.E4M3)
+    da, db_nd = dev(a), dev(np.ascontiguousarray(b.T))  # [k][n]
+    dsa, dsb = dev(sa), dev(sb)
+    need = pa.gemm_mx_workspace_bytes(m, n, k, b_layout=pa.B_ND)
+    assert need == n * k and pa.gemm_mx_workspace_bytes(m, n, k, b_layout=pa.B_ND, b_type=pa.E2M1) == 0
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    with tile_env(PTOAMD_TILE=5):
+        in_loader = host(pa.gemm_mx(da, db_nd, dsa, dsb, m, n, k, pa.E4M3, pa.E4M3, pa.F32, b_layout=pa.B_ND))
+        assert pa.last_kernel().startswith("tile128x128_fp8"), pa.last_kernel()
+        got = host(pa.gemm_mx(da, db_nd, dsa, dsb, m, n, k, pa.E4M3, pa.E4M3, pa.F32, b_layout=pa.B_ND, workspace=ws))
+        assert pa.last_kernel().startswith("tile128x128_dtl_fp8"), pa.last_kernel()
+    assert np.array_equal(got.view(np.uint32), in_loader.view(np.uint32))
+    assert relerr(got, ref) <= 2e-2
+    # boxed scales and the copy of B in one workspace
+    sa_zz = pa.mx_scale_relayout(dsa, pa.MX_A_ND, pa.MX_A_ZZ, m, k // 32)
+    sb_nn = pa.mx_scale_relayout(dsb, pa.MX_B_DN, pa.MX_B_NN, k // 32, n)
+    need2 = pa.gemm_mx_workspace_bytes(m, n, k, pa.MX_A_ZZ, pa.MX_B_NN, b_layout=pa.B_ND)
+    assert need2 == (m + n) * (k // 32) + n * k
+    ws2 = torch.empty(need2, dtype=torch.uint8, device=DEV)
+    with tile_env(PTOAMD_TILE=5):
+        got2 = host(pa.gemm_mx(da, db_nd, sa_zz, sb_nn, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sa_layout=pa.MX_A_ZZ,
+                               sb_layout=pa.MX_B_NN, b_layout=pa.B_ND, workspace=ws2))
+        assert pa.last_kernel().startswith("tile128x128_dtl_fp8"), pa.last_kernel()
+        # room for the scales only: B stays where it is and the loader transposes it
+        got3 = host(pa.gemm_mx(da, db_nd, sa_zz, sb_nn, m, n, k, pa.E4M3, pa.E4M3, pa.F32, sa_layout=pa.MX_A_ZZ,
+                               sb_layout=pa.MX_B_NN, b_layout=pa.B_ND, workspace=ws2[:(m + n) * (k // 32)]))
+        assert pa.last_kernel().startswith("tile128x128_fp8"), pa.last_kernel()
+    assert np.array_equal(got2.view(np.uint32), got.view(np.uint32))
+    assert np.array_equal(got3.view(np.uint32), got.view(np.uint32))
+    # the entry point that allocates nothing: the copy of B goes into the library's static array; accumulator input
+    cin = dev(r.standard_normal((m, n)).astype(np.float32))
+    out = torch.empty((m, n), dtype=torch.float32, device=DEV)
+    with tile_env(PTOAMD_TILE=5):
+        pa.gemm_mx_static(da, db_nd, dsa, dsb, m, n, k, pa.E4M3, pa.E4M3, out, b_layout=pa.B_ND, c_in=cin)
+        assert pa.last_kernel().startswith("tile128x128_dtl_fp8"), pa.last_kernel()
+    assert relerr(host(out), ref + host(cin)) <= 2e-2
+
+
 @pytest.mark.parametrize("tile", [1, 2])
 @pytest.mark.parametrize("typ", [ob.E4M3, ob.E2M1])
 @pytest.mark.parametrize("la,lb", [("MX_A_ZZ", "MX_B_NN"), ("MX_A_DN", "MX_B_ND"), ("MX_A_ND", "MX_B_NN"), ("MX_A_ZZ", "MX_B_DN")])
