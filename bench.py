@@ -142,6 +142,35 @@ def config5(pa, ev, gen, steps, warmup):
                 frac_of_peak=nbytes / ker / 1e6 / PEAK_HBM_GBPS, cpu="config5")
 
 
+def config5_packed(pa, ev, gen, steps, warmup):
+    """configs[4] with the weights packed ahead of time into the kernel's stage order (same sums, same bits)."""
+    m, n, k = 16, 28672, 8192
+    a = randn_bf16((m, k), gen)
+    copies = []
+    for _ in range(4):
+        w, sw = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
+        copies.append(pa.gemv_mxfp4_pack(w, sw, n, k))
+    ref = pa.gemv_mxfp4(a, w, sw, n, k, pa.BF16)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    pa.gemv_mxfp4_packed(a, copies[3], n, k, pa.BF16, out=out)
+    if not torch.equal(out, ref):
+        raise RuntimeError("the packed GEMV does not reproduce the plain one")
+    del w, sw
+    state = {"i": 0}
+
+    def step():
+        packed = copies[state["i"] % 4]
+        state["i"] += 1
+        pa.gemv_mxfp4_packed(a, packed, n, k, pa.BF16, out=out)
+
+    wall, ker = time_launches(ev, step, steps, warmup)
+    nbytes = n * k // 2 + n * k // 32 + m * k * 2 + m * n * 2
+    return dict(config="configs[4] MXFP4 decode GEMV 16x28672x8192 -> bf16, weights pre-packed by ptoamd_gemv_mxfp4_pack "
+                       "(rotated over 4 copies)",
+                kernel=pa.last_kernel(), ms=ker, wall_ms=wall, gbps=nbytes / ker / 1e6, bound="hbm",
+                frac_of_peak=nbytes / ker / 1e6 / PEAK_HBM_GBPS, cpu="config5")
+
+
 def _pto_lib(name):
     """A library of kernels written in the PTO tile ISA against the header layer (pto-isa-mirror_amd/kernels/<name>.hip)."""
     import ctypes as C
@@ -527,10 +556,10 @@ def main():
                     help="untimed run-in of the same launches before the warmup steps, for the GPU clock to settle")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-config measurements after the headline")
-    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11], default=None,
+    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12], default=None,
                     help="measure just BASELINE.json configs[N] (a per_config entry) and print it: for profiling one kernel; "
                          "5-8 are the elementwise kernels (TQUANT MXFP8, TQUANT MXFP4, TQUANT INT8, TDEQUANT), 9, 10 and 11 "
-                         "configs[1], configs[0] and configs[3] written in the PTO tile ISA")
+                         "configs[1], configs[0] and configs[3] written in the PTO tile ISA, 12 configs[4] on pre-packed weights")
     ap.add_argument("--published", action="store_true",
                     help="measure only the shapes the reference publishes wall times for and print those rows")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -557,7 +586,7 @@ def main():
         return
     if args.only is not None:
         fn = {0: config1, 2: config3, 3: config4, 4: config5, 5: quant_mxfp8, 6: quant_mxfp4, 7: quant_int8,
-              8: dequant_int8, 9: pto_api_bf16, 10: pto_api_config1, 11: pto_api_mxfp8}[args.only]
+              8: dequant_int8, 9: pto_api_bf16, 10: pto_api_config1, 11: pto_api_mxfp8, 12: config5_packed}[args.only]
         entry = fn(pa, ev, gen, args.steps, args.warmup)
         entry.pop("cpu", None)
         print(json.dumps(entry))
@@ -585,7 +614,7 @@ def main():
     }
     if not args.no_extra:
         per = []
-        for fn in (config1, config3, config4, config5, pto_api_bf16, pto_api_config1, pto_api_mxfp8, quant_mxfp8, quant_mxfp4, quant_int8,
+        for fn in (config1, config3, config4, config5, config5_packed, pto_api_bf16, pto_api_config1, pto_api_mxfp8, quant_mxfp8, quant_mxfp4, quant_int8,
                    dequant_int8):
             per.append(fn(pa, ev, gen, 50, 5))
             torch.cuda.empty_cache()

@@ -275,6 +275,22 @@ int ptoamd_gemm_mx_static(void* c, int c_type, const void* a, const void* b, int
 int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, const uint8_t* w, const uint8_t* sw, int m, int n,
                       int k, int lda, int ldw, int ldc, void* stream);
 
+/*
+ * The same product with the weights stored once in the order the kernel consumes them (k a multiple of 2048): per
+ * 16 rows x 2048 k one 16 KiB block of codes -- the 16 row pieces, their 16-byte chunks at the LDS positions the kernel
+ * reads them from -- and, in a second region behind all code blocks, one 1 KiB block of the 16 x 64 scale bytes, so that
+ * a stage is two contiguous runs of memory.  Same arithmetic in the same order as ptoamd_gemv_mxfp4 on the loader-wave
+ * kernel (bit-identical outputs), 4 - 5 % faster on 16 x 28672 x 8192.  It is to this kernel what the NZ / fractal GM layouts are to the reference's cube unit
+ * (include/pto/cpu/tile_offsets.hpp: data laid out in the consumer's order, once, ahead of time); the packed buffer is
+ * only meaningful to ptoamd_gemv_mxfp4_packed.
+ *   ptoamd_gemv_mxfp4_packed_bytes : size of the packed buffer (0 when k is not a multiple of 2048)
+ *   ptoamd_gemv_mxfp4_pack         : w [n][ldw / 2] bytes (16-byte aligned rows), sw [n][k / 32] -> packed
+ */
+size_t ptoamd_gemv_mxfp4_packed_bytes(int n, int k);
+int ptoamd_gemv_mxfp4_pack(void* packed, const uint8_t* w, const uint8_t* sw, int n, int k, int ldw, void* stream);
+int ptoamd_gemv_mxfp4_packed(void* out, int c_type, const void* a_bf16, const void* packed, int m, int n, int k, int lda,
+                             int ldc, void* stream);
+
 /* TQUANT<INT8_SYM / INT8_ASYM> (cpu/TQuant.hpp:496-522): dst = clamp(nearbyint(src * scale[row] (+ offset[row]))).
  * offset == NULL selects the symmetric form (int8 output); otherwise the output is uint8.  src is [rows][cols] f32. */
 int ptoamd_tquant_int8(void* dst, const float* src, const float* scale, const float* offset, int rows, int cols,

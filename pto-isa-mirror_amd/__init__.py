@@ -37,6 +37,7 @@ _lib.ptoamd_last_kernel.restype = C.c_char_p
 _lib.ptoamd_gemm_mx_workspace_bytes.restype = C.c_size_t
 _lib.ptoamd_gemm_mx_workspace_bytes_b_nd.restype = C.c_size_t
 _lib.ptoamd_gemm_workspace_bytes.restype = C.c_size_t
+_lib.ptoamd_gemv_mxfp4_packed_bytes.restype = C.c_size_t
 
 EXPORTS = [
     "ptoamd_init", "ptoamd_finalize", "ptoamd_last_error", "ptoamd_device_info", "ptoamd_malloc", "ptoamd_free",
@@ -45,7 +46,7 @@ EXPORTS = [
     "ptoamd_event_destroy", "ptoamd_event_record", "ptoamd_event_synchronize", "ptoamd_event_elapsed_ms",
     "ptoamd_gemm", "ptoamd_gemm_bias", "ptoamd_gemm_ws", "ptoamd_gemm_workspace_bytes", "ptoamd_gemm_fp8", "ptoamd_gemm_requant", "ptoamd_gemm_atomic_add", "ptoamd_gemm_w8a8", "ptoamd_gemm_mx", "ptoamd_gemm_mx_bias",
     "ptoamd_gemm_mx_ws",
-    "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_workspace_bytes_b_nd", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_tquant_int8",
+    "ptoamd_gemm_mx_workspace_bytes", "ptoamd_gemm_mx_workspace_bytes_b_nd", "ptoamd_gemm_mx_static", "ptoamd_gemv_mxfp4", "ptoamd_gemv_mxfp4_packed_bytes", "ptoamd_gemv_mxfp4_pack", "ptoamd_gemv_mxfp4_packed", "ptoamd_tquant_int8",
     "ptoamd_tquant_int8_para", "ptoamd_tquant_mx", "ptoamd_tdequant", "ptoamd_tdequant_para", "ptoamd_mx_scale_relayout",
     "ptoamd_last_kernel", "ptoamd_reload_options",
 ]
@@ -234,6 +235,26 @@ def gemv_mxfp4(a_bf16, w, sw, n, k, c_type=F32, stream=None, out=None):
         out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=w.device)
     _check(_lib.ptoamd_gemv_mxfp4(_ptr(out, True), c_type, _ptr(a_bf16, True), _ptr(w), _ptr(sw), m, n, k, a_bf16.stride(0), k,
                                   out.stride(0), _stream(stream)), "ptoamd_gemv_mxfp4")
+    return out
+
+
+def gemv_mxfp4_pack(w, sw, n, k, stream=None):
+    """MXFP4 weights [n, k/2] + E8M0 scales [n, k/32] -> the packed buffer gemv_mxfp4_packed consumes (k % 2048 == 0)."""
+    size = int(_lib.ptoamd_gemv_mxfp4_packed_bytes(n, k))
+    if size == 0:
+        raise PtoAmdError(f"gemv_mxfp4_pack: k = {k} must be a positive multiple of 2048")
+    packed = torch.empty(size, dtype=torch.uint8, device=w.device)
+    _check(_lib.ptoamd_gemv_mxfp4_pack(_ptr(packed), _ptr(w), _ptr(sw), n, k, k, _stream(stream)), "ptoamd_gemv_mxfp4_pack")
+    return packed
+
+
+def gemv_mxfp4_packed(a_bf16, packed, n, k, c_type=F32, stream=None, out=None):
+    """Decode GEMV on weights packed by gemv_mxfp4_pack: the same sums in the same order as gemv_mxfp4."""
+    m = a_bf16.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=_TORCH_OUT[c_type], device=packed.device)
+    _check(_lib.ptoamd_gemv_mxfp4_packed(_ptr(out, True), c_type, _ptr(a_bf16, True), _ptr(packed), m, n, k, a_bf16.stride(0),
+                                         out.stride(0), _stream(stream)), "ptoamd_gemv_mxfp4_packed")
     return out
 
 

@@ -35,6 +35,7 @@ struct GemvParams {
     int ldc;
     int out_bf16;
     int n_groups;       // ceil(n / 16)
+    const uint8_t* wp;  // packed weights (gemv_mxfp4_pack_kernel), loader-wave kernel only: w and sw are then unused
 };
 
 constexpr int GEMV_CHUNK = 512;  // k per chunk
@@ -388,7 +389,13 @@ static_assert(WD_LDS <= 160 * 1024, "LDS capacity");
 
 __device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
-template <bool HW_CVT>
+// PACKED: the weights come as the stages this kernel consumes.  Block number strip * (k / 2048) + chunk of the packed
+// buffer's first region holds the 16 row pieces of (strip of 16 rows, chunk of 2048 k), their 16-byte chunks already at
+// the swizzled positions (16 KiB); the same block number of the second region holds the 16 x 64 scale bytes (1 KiB).  A
+// stage is then two contiguous runs of memory instead of 16 pieces 1 KiB long and a row pitch apart plus 16 scale
+// pieces, and streams 4 - 5 % faster (23.4 against 24.5 us on 16 x 28672 x 8192; with the scales inside one 17 KiB block
+// per stage, which takes the code blocks off their 16 KiB alignment, 23.8 us).
+template <bool HW_CVT, bool PACKED = false>
 __global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvParams p, int strips_per_wg)
 {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -417,16 +424,26 @@ __global__ void __launch_bounds__(512) gemv_mxfp4_splitk_wide_kernel(const GemvP
         const int kc = (kc_first + nx_kc) % kchunks;
         const uint32_t dst = lds0 + (issued % WD_RING) * WD_STAGE;
         const int rlim = min(15, p.n - 1 - strip * 16);
-        const uint8_t* wbase = p.w + (long)strip * 16 * p.ldw_bytes + (long)kc * (WD_CHUNK / 2);
+        const int e = wc * 64 + lane;   // 64 dwords = the scales of four rows
+        if constexpr (PACKED) {
+            const long idx = (long)strip * kchunks + kc;
+            const uint8_t* blk = p.wp + idx * WD_WBYTES;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const int r = 4 * wc + d;   // a loader takes four neighbouring rows (slightly faster than every fourth)
-            lds_dma16_off_nt(wbase, (uint32_t)(min(r, rlim) * (int)p.ldw_bytes) + (uint32_t)((lane ^ r) << 4), dst + r * 1024);
+            for (int d = 0; d < 4; ++d) {
+                const int r = 4 * wc + d;
+                lds_dma16_off_nt(blk, (uint32_t)(r * 1024 + (lane << 4)), dst + r * 1024);
+            }
+            lds_dma4_off_nt(p.wp + (long)p.n_groups * kchunks * WD_WBYTES + idx * WD_SBYTES, (uint32_t)(e * 4), dst + WD_WBYTES + wc * 256);
+        } else {
+            const uint8_t* wbase = p.w + (long)strip * 16 * p.ldw_bytes + (long)kc * (WD_CHUNK / 2);
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const int r = 4 * wc + d;   // a loader takes four neighbouring rows (slightly faster than every fourth)
+                lds_dma16_off_nt(wbase, (uint32_t)(min(r, rlim) * (int)p.ldw_bytes) + (uint32_t)((lane ^ r) << 4), dst + r * 1024);
+            }
+            lds_dma4_off_nt(p.sw + (long)strip * 16 * sb + (long)kc * (WD_CHUNK / 32), (uint32_t)(min(e >> 4, rlim) * sb + (e & 15) * 4),
+                            dst + WD_WBYTES + wc * 256);
         }
-        // 64 dwords = the scales of four rows
-        const int e = wc * 64 + lane;
-        lds_dma4_off_nt(p.sw + (long)strip * 16 * sb + (long)kc * (WD_CHUNK / 32), (uint32_t)(min(e >> 4, rlim) * sb + (e & 15) * 4),
-                        dst + WD_WBYTES + wc * 256);
         ++issued;
         if (++nx_i == min(SK_RMAX, nsteps - nx_b0)) {
             nx_i = 0;
@@ -609,8 +626,32 @@ __global__ void gemv_mxfp4_generic_kernel(const GemvParams p)
         reinterpret_cast<float*>(p.out)[(long)gi * p.ldc + gj] = acc;
 }
 
+// Weights [n][ldw_bytes] + scales [n][k / 32] -> the stage blocks of the PACKED loader-wave kernel.  One workgroup per
+// block (strip, chunk): thread t moves 16-byte position t % 64 of rows t / 64, t / 64 + 4, ...; a row past n - 1 repeats
+// row n - 1, as the loader of the plain form does (its outputs are never stored).
+__global__ void __launch_bounds__(256) gemv_mxfp4_pack_kernel(uint8_t* __restrict__ packed, const uint8_t* __restrict__ w,
+                                                               const uint8_t* __restrict__ sw, int n, int k, long ldw_bytes, long ldsw)
+{
+    const int kchunks = k / WD_CHUNK, strip = blockIdx.x / kchunks, kc = blockIdx.x % kchunks;
+    uint8_t* blk = packed + (long)blockIdx.x * WD_WBYTES;
+    uint8_t* sblk = packed + (long)gridDim.x * WD_WBYTES + (long)blockIdx.x * WD_SBYTES;
+    const int pos = threadIdx.x & 63;
+    for (int r = threadIdx.x >> 6; r < 16; r += 4) {
+        const long row = min(strip * 16 + r, n - 1);
+        const uint4 v = *reinterpret_cast<const uint4*>(w + row * ldw_bytes + (long)kc * (WD_CHUNK / 2) + ((pos ^ r) << 4));
+        *reinterpret_cast<uint4*>(blk + r * 1024 + (pos << 4)) = v;
+    }
+    {
+        const int e = threadIdx.x;  // dword e of the 16 x 64 scale bytes
+        const long row = min(strip * 16 + (e >> 4), n - 1);
+        *reinterpret_cast<uint32_t*>(sblk + e * 4) =
+            *reinterpret_cast<const uint32_t*>(sw + row * ldsw + (long)kc * (WD_CHUNK / 32) + (e & 15) * 4);
+    }
+}
+
 int prepare_gemv_kernels()
 {
+    PTOAMD_HIP_CHECK(ensure_dynamic_lds(reinterpret_cast<const void*>(gemv_mxfp4_splitk_wide_kernel<true, true>), WD_LDS));
     PTOAMD_HIP_CHECK(ensure_dynamic_lds(reinterpret_cast<const void*>(gemv_mxfp4_splitk_wide_kernel<false>), WD_LDS));
     PTOAMD_HIP_CHECK(ensure_dynamic_lds(reinterpret_cast<const void*>(gemv_mxfp4_splitk_wide_kernel<true>), WD_LDS));
     PTOAMD_HIP_CHECK(ensure_dynamic_lds(reinterpret_cast<const void*>(gemv_mxfp4_splitk_kernel<false>), SK_LDS));
@@ -711,3 +752,63 @@ extern "C" int ptoamd_gemv_mxfp4(void* out, int c_type, const void* a_bf16, cons
     PTOAMD_HIP_CHECK(hipGetLastError());
     return PTOAMD_OK;
 }
+
+// ---- the pre-packed form: weights stored once in the order the loader waves consume them ------------------------------
+extern "C" size_t ptoamd_gemv_mxfp4_packed_bytes(int n, int k)
+{
+    if (n <= 0 || k <= 0 || k % WD_CHUNK != 0)
+        return 0;
+    return (size_t)((n + 15) / 16) * (size_t)(k / WD_CHUNK) * (size_t)WD_STAGE;
+}
+
+extern "C" int ptoamd_gemv_mxfp4_pack(void* packed, const uint8_t* w, const uint8_t* sw, int n, int k, int ldw, void* stream_)
+{
+    hipStream_t stream = as_stream(stream_);
+    PTOAMD_REQUIRE(packed && w && sw, PTOAMD_E_INVALID, "ptoamd_gemv_mxfp4_pack: null operand");
+    PTOAMD_REQUIRE(n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemv_mxfp4_pack: n, k must be positive");
+    PTOAMD_REQUIRE(k % WD_CHUNK == 0, PTOAMD_E_UNSUPPORTED, "ptoamd_gemv_mxfp4_pack: k = %d must be a multiple of %d", k, WD_CHUNK);
+    PTOAMD_REQUIRE(ldw >= k && ldw % 32 == 0, PTOAMD_E_INVALID, "ptoamd_gemv_mxfp4_pack: ldw must be at least k and a multiple of 32");
+    PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(packed) & 15u) == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0 &&
+                       (reinterpret_cast<uintptr_t>(sw) & 3u) == 0,
+                   PTOAMD_E_ALIGNMENT, "ptoamd_gemv_mxfp4_pack: packed and w must be 16-byte aligned, sw 4-byte aligned");
+    const long blocks = (long)((n + 15) / 16) * (k / WD_CHUNK);
+    PTOAMD_REQUIRE(blocks < (1L << 31), PTOAMD_E_UNSUPPORTED, "ptoamd_gemv_mxfp4_pack: too many blocks");
+    hipLaunchKernelGGL(gemv_mxfp4_pack_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, reinterpret_cast<uint8_t*>(packed), w, sw,
+                       n, k, (long)ldw / 2, (long)k / 32);
+    PTOAMD_HIP_CHECK(hipGetLastError());
+    set_last_kernel("gemv_mxfp4_pack");
+    return PTOAMD_OK;
+}
+
+extern "C" int ptoamd_gemv_mxfp4_packed(void* out, int c_type, const void* a_bf16, const void* packed, int m, int n, int k,
+                                        int lda, int ldc, void* stream_)
+{
+    hipStream_t stream = as_stream(stream_);
+    TraceScope trace("TGEMV_MX", "cube", m, n, k);
+    trace.in(a_bf16, m, k, "ND", PTOAMD_BF16).in(packed, k, n, "packed", PTOAMD_E2M1).out(out, m, n, "ND", c_type);
+    PTOAMD_REQUIRE(out && a_bf16 && packed, PTOAMD_E_INVALID, "ptoamd_gemv_mxfp4_packed: null operand");
+    PTOAMD_REQUIRE(m > 0 && n > 0 && k > 0, PTOAMD_E_INVALID, "ptoamd_gemv_mxfp4_packed: m, n, k must be positive");
+    PTOAMD_REQUIRE(m <= 16, PTOAMD_E_UNSUPPORTED, "ptoamd_gemv_mxfp4_packed: m = %d exceeds the decode batch of 16", m);
+    PTOAMD_REQUIRE(k % WD_CHUNK == 0, PTOAMD_E_UNSUPPORTED, "ptoamd_gemv_mxfp4_packed: k = %d must be a multiple of %d", k, WD_CHUNK);
+    PTOAMD_REQUIRE(c_type == PTOAMD_F32 || c_type == PTOAMD_BF16, PTOAMD_E_UNSUPPORTED, "ptoamd_gemv_mxfp4_packed: output is f32 or bf16");
+    PTOAMD_REQUIRE(lda >= k && ldc >= n && lda % 8 == 0 && (long)lda * 2 * 16 < (1L << 31), PTOAMD_E_INVALID,
+                   "ptoamd_gemv_mxfp4_packed: lda must be at least k and a multiple of 8, ldc at least n");
+    PTOAMD_REQUIRE((reinterpret_cast<uintptr_t>(a_bf16) & 15u) == 0 && (reinterpret_cast<uintptr_t>(packed) & 15u) == 0,
+                   PTOAMD_E_ALIGNMENT, "ptoamd_gemv_mxfp4_packed: a and packed must be 16-byte aligned");
+    GemvParams p{};
+    p.a = reinterpret_cast<const uint16_t*>(a_bf16);
+    p.wp = reinterpret_cast<const uint8_t*>(packed);
+    p.out = out;
+    p.m = m; p.n = n; p.k = k; p.lda = lda; p.ldc = ldc;
+    p.out_bf16 = c_type == PTOAMD_BF16;
+    p.n_groups = (n + 15) / 16;
+    const int cus = device_compute_units();
+    const int spw = (p.n_groups + cus - 1) / cus;
+    const int grid = (p.n_groups + spw - 1) / spw;
+    PTOAMD_HIP_CHECK(ensure_dynamic_lds(reinterpret_cast<const void*>(gemv_mxfp4_splitk_wide_kernel<true, true>), WD_LDS));
+    hipLaunchKernelGGL((gemv_mxfp4_splitk_wide_kernel<true, true>), dim3(grid), dim3(512), WD_LDS, stream, p, spw);
+    PTOAMD_HIP_CHECK(hipGetLastError());
+    set_last_kernel("gemv_mxfp4_splitk_wide_packed");
+    return PTOAMD_OK;
+}
+

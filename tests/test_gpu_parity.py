@@ -1268,6 +1268,10 @@ def test_config5_mxfp4_decode_full_size(pa, oracle):
     assert torch.equal(out2, out * 0.125)
     one = pa.gemv_mxfp4(a[3:4].contiguous(), w, sw, n, k, pa.F32)
     assert torch.equal(one[0], out[3])
+    # the pre-packed weight form: identical bits, bf16 drain included
+    packed = pa.gemv_mxfp4_pack(w, sw, n, k)
+    assert torch.equal(pa.gemv_mxfp4_packed(a, packed, n, k, pa.F32), out)
+    assert torch.equal(pa.gemv_mxfp4_packed(a, packed, n, k, pa.BF16), pa.gemv_mxfp4(a, w, sw, n, k, pa.BF16))
 
 
 # ------------------------------------------------------------------------------------------- TQUANT / TDEQUANT
