@@ -319,8 +319,8 @@ static int pick_tile(int m, int n, long k_bytes, bool scaled, bool fp4 = false, 
     return 2;
 }
 
-// Launch on the chosen tile.  When the 256x256 grid is some whole rounds of the CUs plus a last one that is at most half
-// full, the columns of that last round run as smaller tiles in a second launch on the same stream: 256x128 tiles (at most
+// Launch on the chosen tile.  When the 256x256 grid is some (nearly) whole rounds of the CUs plus at most half a round,
+// the columns of that remainder run as smaller tiles in a second launch on the same stream: 256x128 tiles (at most
 // one workgroup per CU, same wave tile as the large form) or 128x128 tiles (two workgroups per CU); a tile of the tail
 // then costs a half or a quarter of a 256x256 tile's time instead of a whole round (MXFP8 4096 x 14336 x 4096, 3.5
 // rounds of 256 CUs).  PTOAMD_TILE (an explicit tile) and PTOAMD_NO_TAIL_SPLIT=1 switch the split off;
@@ -330,11 +330,22 @@ static hipError_t launch_tiles_as(int tile, int op, const TileGemmParams& p, hip
     if ((tile == 4 || tile == 3) && options().tile < 0 && !options().no_tail_split) {
         const int cus = device_compute_units();
         const int tiles_m = (p.m + 255) / 256, tiles_n = (p.n + 255) / 256;
-        int whole = tiles_n;  // tile columns that make whole rounds
-        while (whole > 0 && ((long)tiles_m * whole) % cus != 0)
-            --whole;
-        const long tail_tiles = (long)tiles_m * (tiles_n - whole);
-        if (whole > 0 && whole < tiles_n && tail_tiles <= cus / 2) {  // a last round at most half full
+        // `whole`: the most tile columns whose tiles make (nearly) whole rounds -- at most a sixteenth of a round idle --
+        // with at most half a round's worth of tiles left over.  Looked for only when the grid's own last round is at most
+        // five eighths full (a fuller one is better left alone).
+        const long all = (long)tiles_m * tiles_n;
+        const long last_fill = all - (all - 1) / cus * cus;
+        int whole = 0;
+        if (last_fill <= 5 * cus / 8) {
+            for (int w = tiles_n - 1; w > 0 && (long)tiles_m * (tiles_n - w) <= cus / 2; --w) {
+                const long head_tiles = (long)tiles_m * w;
+                if ((head_tiles + cus - 1) / cus * cus - head_tiles <= cus / 16) {
+                    whole = w;
+                    break;
+                }
+            }
+        }
+        if (whole > 0) {
             const int n1 = whole * 256;
             TileGemmParams head = p;
             head.n = n1;

@@ -661,6 +661,28 @@ def test_tail_round_runs_as_a_second_launch(pa, oracle):
     assert relerr(host(got)[np.ix_(rows, cols)], ref) <= 2e-2
 
 
+def test_tail_split_after_nearly_whole_rounds(pa, oracle):
+    """6 x 44 tiles of 256 x 256 are one round of a 256-CU chip plus 8 tiles; no number of whole tile columns makes an exact
+    round, but 42 columns (252 tiles) leave 4 CUs idle: those run as the head launch and the last two columns as
+    128 x 128 tiles.  Same bits as the single launch; the seam columns against the oracle."""
+    if torch.cuda.get_device_properties(0).multi_processor_count != 256:
+        pytest.skip("the shape is chosen for a 256-CU part")
+    r = np.random.default_rng(79)
+    m, n, k = 6 * 256, 44 * 256 - 24, 256
+    a = bf16_bits(r.standard_normal((m, k)) * 0.05)
+    b = bf16_bits(r.standard_normal((n, k)) * 0.05)
+    da, db = dev(a).view(torch.bfloat16), dev(b).view(torch.bfloat16)
+    got = host(pa.gemm(da, db, pa.BF16, pa.F32, pa.B_DN))
+    assert pa.last_kernel() == "tile256x256w8_dtl_bf16"
+    with tile_env(PTOAMD_NO_TAIL_SPLIT="1"):
+        one = host(pa.gemm(da, db, pa.BF16, pa.F32, pa.B_DN))
+    assert np.array_equal(got.view(np.uint32), one.view(np.uint32))
+    rows = np.array([0, 255, 256, 1000, m - 1])
+    cols = np.concatenate([np.arange(42 * 256 - 8, 42 * 256 + 8), np.arange(0, n, 517), [n - 1]])
+    ref = oracle.matmul_bf16(a[rows], b[cols], b_dn=True)
+    assert relerr(got[np.ix_(rows, cols)], ref) <= 1e-3
+
+
 # ------------------------------------------------------------------------------------------- TMATMUL_MX
 def _mx_inputs(r, typ, m, n, k, spread=8):
     packed = typ in (ob.E2M1, ob.E1M2)
