@@ -230,6 +230,34 @@ def pto_api_mxfp8(pa, ev, gen, steps, warmup):
                 bound="mfma", frac_of_peak=flops / ker / 1e9 / PEAK_TFLOPS["fp8"], cpu="config4")
 
 
+def pto_api_mxfp4(pa, ev, gen, steps, warmup):
+    """MXFP4 2048 x 8192 (K) x 8192 -> bf16 (a shape the reference publishes a time for) through the same core program as
+    pto_api_mxfp8, on packed E2M1 operand tiles."""
+    C, lib = _pto_lib("mxmatmul_performance")
+    m, n, k = 2048, 8192, 8192
+    a, sa = pa.tquant_mx(torch.randn((m, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
+    b, sb = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+
+    def step():
+        rc = lib.pto_mxmatmul_performance(4, *(C.c_void_p(t.data_ptr()) for t in (out, a, b, sa, sb)),
+                                          C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, rc
+
+    wall, ker = time_launches(ev, step, steps, warmup)
+    ref = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E2M1, pa.E2M1, pa.BF16)
+    launcher = pa.last_kernel()
+    torch.cuda.synchronize()
+    assert lib.pto_mxmatmul_performance_status() == 0 and torch.equal(out, ref), "the PTO-style MXFP4 GEMM and the launcher disagree"
+    lwall, lker = time_launches(ev, lambda: pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E2M1, pa.E2M1, pa.BF16, out=out), steps, warmup)
+    flops = 2 * m * n * k
+    return dict(config="MXFP4 E2M1 2048x8192x8192 (m, k, n) -> bf16 written in the PTO tile ISA (TLOAD / TEXTRACT / TMATMUL_MX / TSTORE, "
+                       "256 x 256 tiles, K panels of 256 codes, scale tiles of 16 K-groups)",
+                kernel="MxMatmulPerformance<e2m1, 256, 256, 256> (header layer)", ms=ker, wall_ms=wall, tflops=flops / ker / 1e9,
+                bound="mfma", frac_of_peak=flops / ker / 1e9 / PEAK_TFLOPS["fp4"], launcher_kernel=launcher, launcher_ms=lker,
+                cpu=None)
+
+
 def pto_api_config1(pa, ev, gen, steps, warmup):
     """configs[0] through the tile ISA (kernels/gemm_tiled.hip): 128 x 128 tiles as BASELINE.json words it, and 64 x 64."""
     C, lib = _pto_lib("gemm_tiled")
@@ -556,10 +584,10 @@ def main():
                     help="untimed run-in of the same launches before the warmup steps, for the GPU clock to settle")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-config measurements after the headline")
-    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12], default=None,
+    ap.add_argument("--only", type=int, choices=[0, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13], default=None,
                     help="measure just BASELINE.json configs[N] (a per_config entry) and print it: for profiling one kernel; "
                          "5-8 are the elementwise kernels (TQUANT MXFP8, TQUANT MXFP4, TQUANT INT8, TDEQUANT), 9, 10 and 11 "
-                         "configs[1], configs[0] and configs[3] written in the PTO tile ISA, 12 configs[4] on pre-packed weights")
+                         "configs[1], configs[0] and configs[3] written in the PTO tile ISA, 12 configs[4] on pre-packed weights, 13 an MXFP4 GEMM in the tile ISA")
     ap.add_argument("--published", action="store_true",
                     help="measure only the shapes the reference publishes wall times for and print those rows")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -586,7 +614,7 @@ def main():
         return
     if args.only is not None:
         fn = {0: config1, 2: config3, 3: config4, 4: config5, 5: quant_mxfp8, 6: quant_mxfp4, 7: quant_int8,
-              8: dequant_int8, 9: pto_api_bf16, 10: pto_api_config1, 11: pto_api_mxfp8, 12: config5_packed}[args.only]
+              8: dequant_int8, 9: pto_api_bf16, 10: pto_api_config1, 11: pto_api_mxfp8, 12: config5_packed, 13: pto_api_mxfp4}[args.only]
         entry = fn(pa, ev, gen, args.steps, args.warmup)
         entry.pop("cpu", None)
         print(json.dumps(entry))
@@ -614,7 +642,7 @@ def main():
     }
     if not args.no_extra:
         per = []
-        for fn in (config1, config3, config4, config5, config5_packed, pto_api_bf16, pto_api_config1, pto_api_mxfp8, quant_mxfp8, quant_mxfp4, quant_int8,
+        for fn in (config1, config3, config4, config5, config5_packed, pto_api_bf16, pto_api_config1, pto_api_mxfp8, pto_api_mxfp4, quant_mxfp8, quant_mxfp4, quant_int8,
                    dequant_int8):
             per.append(fn(pa, ev, gen, 50, 5))
             torch.cuda.empty_cache()
@@ -629,7 +657,9 @@ def main():
             return memo[tag]
         line["cpu_baseline"] = leg("headline")
         for entry in line.get("per_config", []):
-            entry["cpu_baseline"] = leg(entry.pop("cpu"))
+            tag = entry.pop("cpu")
+            if tag is not None:  # (entries outside BASELINE.json's configs carry no CPU leg)
+                entry["cpu_baseline"] = leg(tag)
     for entry in line.get("per_config", []):
         entry.pop("cpu", None)
     print(json.dumps(line))

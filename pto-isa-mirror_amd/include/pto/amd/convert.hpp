@@ -204,18 +204,25 @@ PTO_INST void tfillpad_lds(DstTile& dst, SrcTile& src)
     uint8_t* d = dst.Storage();
     const bool in_place = s == d;
     __syncthreads();
-    if constexpr (is_packed4<T>) {  // two codes per byte along a row
+    if constexpr (is_packed4<T>) {
+        // two codes per byte, neighbours along a row or down a column (each tile says which); a thread builds one
+        // destination byte from the two codes it holds, zero where the source has no valid element
+        auto code = [&](int r, int c) -> uint32_t {
+            if (r < vr && c < vc)
+                return (s[src.ByteOffset(r, c)] >> (4 * SrcTile::Nibble(r, c))) & 0xFu;
+            return 0u;
+        };
         for (int idx = threadIdx.x; idx < DstTile::Rows * DstTile::Cols / 2; idx += PTO_AMD_THREADS) {
-            const int r = idx / (DstTile::Cols / 2), c = 2 * (idx - r * (DstTile::Cols / 2));
-            uint32_t v = 0;
-            if (r < vr && c < SrcTile::Cols) {
-                v = s[src.ByteOffset(r, c)];
-                if (c >= vc)
-                    v = 0;
-                else if (c + 1 >= vc)
-                    v &= 0x0Fu;
+            int r, c;
+            uint32_t lo, hi;
+            if constexpr (DstTile::PairsDownColumns) {
+                r = 2 * (idx / DstTile::Cols), c = idx - (r / 2) * DstTile::Cols;
+                lo = code(r, c), hi = code(r + 1, c);
+            } else {
+                r = idx / (DstTile::Cols / 2), c = 2 * (idx - r * (DstTile::Cols / 2));
+                lo = code(r, c), hi = code(r, c + 1);
             }
-            d[dst.ByteOffset(r, c)] = (uint8_t)v;
+            d[dst.ByteOffset(r, c)] = (uint8_t)(lo | (hi << 4));
         }
     } else {
         const T pad = pad_element<T, P>();

@@ -88,7 +88,7 @@ PTO_INST bool tload_dma(TileData& dst, GlobalData& src)
                   (((nd || mx_a) && TileData::LinesAreRows) || ((dn || mx_b) && !TileData::LinesAreRows))) {
         // ND: element (r, c) at r * stride[3] + c * stride[4]; DN: the same with the unit stride on the rows
         const int64_t line_stride = src.GetStride((mx_a || mx_b) ? 2 : (nd ? 3 : 4));
-        const int64_t gbytes = line_stride * (int64_t)sizeof(T);
+        const int64_t gbytes = line_stride * (int64_t)ElemTraits<T>::bytes2 / 2;  // (packed fp4: strides count codes)
         const uintptr_t gaddr = reinterpret_cast<uintptr_t>(src.data());
         bool shape_ok;
         if constexpr (mx_a || mx_b)
@@ -141,11 +141,40 @@ PTO_INST void tload_lds(TileData& dst, GlobalData& src)
     const auto* g = reinterpret_cast<const T*>(src.data());
     uint8_t* base = dst.Storage();
     __syncthreads();
-    if constexpr (is_packed4<T>) {  // two codes per byte along a row: move bytes (element offsets are even)
-        static_assert(GlobalData::layout == Layout::ND, "packed fp4 tiles load from row-major global tensors");
-        for (int idx = threadIdx.x; idx < vr * (vc / 2); idx += PTO_AMD_THREADS) {
-            const int r = idx / (vc / 2), c = 2 * (idx - r * (vc / 2));
-            base[dst.ByteOffset(r, c)] = reinterpret_cast<const uint8_t*>(g)[src.Offset(r, c) / 2];
+    if constexpr (is_packed4<T>) {
+        // Two codes per byte.  In global memory the pair runs along the unit-stride direction (a row of an ND tensor, a
+        // column of a DN one; offsets count codes); in the tile along a row, or down a column where columns are the
+        // tile's lines.  Same direction on both sides: bytes move.  Otherwise a thread builds each tile byte from the
+        // two codes it holds.
+        static_assert(GlobalData::layout == Layout::ND || GlobalData::layout == Layout::DN, "packed fp4 tiles load from ND or DN tensors");
+        const auto* g8 = reinterpret_cast<const uint8_t*>(g);
+        constexpr bool down = TileData::PairsDownColumns;
+        if constexpr (down == (GlobalData::layout == Layout::DN)) {
+            for (int idx = threadIdx.x; idx < vr * vc / 2; idx += PTO_AMD_THREADS) {
+                int r, c;
+                if constexpr (down)
+                    c = idx / (vr / 2), r = 2 * (idx - c * (vr / 2));
+                else
+                    r = idx / (vc / 2), c = 2 * (idx - r * (vc / 2));
+                base[dst.ByteOffset(r, c)] = g8[src.Offset(r, c) / 2];
+            }
+        } else {
+            auto code = [&](int r, int c) -> uint32_t {
+                const int64_t off = src.Offset(r, c);
+                return (g8[off >> 1] >> (4 * (int)(off & 1))) & 0xFu;
+            };
+            for (int idx = threadIdx.x; idx < vr * vc / 2; idx += PTO_AMD_THREADS) {
+                int r, c;
+                uint32_t lo, hi;
+                if constexpr (down) {
+                    r = 2 * (idx / vc), c = idx - (r / 2) * vc;
+                    lo = code(r, c), hi = code(r + 1, c);
+                } else {
+                    c = 2 * (idx / vr), r = idx - (c / 2) * vr;
+                    lo = code(r, c), hi = code(r, c + 1);
+                }
+                base[dst.ByteOffset(r, c)] = (uint8_t)(lo | (hi << 4));
+            }
         }
     } else if constexpr (GlobalData::layout == Layout::DN) {  // rows are the contiguous direction in memory
         for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
@@ -175,7 +204,13 @@ PTO_INST void tstore_lds(GlobalData& dst, TileData& src)
         static_assert(GlobalData::layout == Layout::ND && sizeof(G) == 1, "packed fp4 tiles store to row-major global tensors");
         for (int idx = threadIdx.x; idx < vr * (vc / 2); idx += PTO_AMD_THREADS) {
             const int r = idx / (vc / 2), c = 2 * (idx - r * (vc / 2));
-            reinterpret_cast<uint8_t*>(g)[dst.Offset(r, c) / 2] = base[src.ByteOffset(r, c)];
+            if constexpr (TileData::PairsDownColumns) {  // the tile pairs codes down its columns, memory along the row
+                const uint32_t lo = (base[src.ByteOffset(r, c)] >> (4 * TileData::Nibble(r, c))) & 0xFu;
+                const uint32_t hi = (base[src.ByteOffset(r, c + 1)] >> (4 * TileData::Nibble(r, c + 1))) & 0xFu;
+                reinterpret_cast<uint8_t*>(g)[dst.Offset(r, c) / 2] = (uint8_t)(lo | (hi << 4));
+            } else {
+                reinterpret_cast<uint8_t*>(g)[dst.Offset(r, c) / 2] = base[src.ByteOffset(r, c)];
+            }
         }
     } else {
         for (int idx = threadIdx.x; idx < vr * vc; idx += PTO_AMD_THREADS) {
@@ -202,11 +237,11 @@ template <typename DstTile, typename SrcTile>
 PTO_INST bool textract_window(DstTile& dst, SrcTile& src, int row0, int col0)
 {
     using T = typename DstTile::DType;
-    if constexpr (SrcTile::MatLines && !is_packed4<T> && DstTile::OperandLoc && DstTile::LinesAreRows == SrcTile::LinesAreRows) {
+    if constexpr (SrcTile::MatLines && DstTile::OperandLoc && DstTile::LinesAreRows == SrcTile::LinesAreRows) {
         constexpr bool left = DstTile::LinesAreRows;
         // (fragments are read as 16-byte chunks; the bytes of a scale tile are read one by one, from any offset)
         constexpr bool scale = DstTile::Loc == TileType::ScaleLeft || DstTile::Loc == TileType::ScaleRight;
-        const uint32_t kb0 = (uint32_t)(left ? col0 : row0) * (uint32_t)sizeof(T);
+        const uint32_t kb0 = (uint32_t)(left ? col0 : row0) * (uint32_t)ElemTraits<T>::bytes2 / 2u;  // (packed fp4: two codes per byte)
         const bool ok = (scale || (kb0 & 15u) == 0) && row0 >= 0 && col0 >= 0 && row0 + DstTile::Rows <= src.GetValidRow() &&
                         col0 + DstTile::Cols <= src.GetValidCol() && dst.GetValidRow() == DstTile::Rows &&
                         dst.GetValidCol() == DstTile::Cols;
@@ -285,7 +320,7 @@ PTO_INST void textract_lds(DstTile& dst, SrcTile& src, int row0, int col0)
                 return (s[src.ByteOffset(sr, sc)] >> (4 * SrcTile::Nibble(sr, sc))) & 0xFu;
             return 0u;
         };
-        constexpr bool along_rows = DstTile::Loc == TileType::Right;
+        constexpr bool along_rows = DstTile::PairsDownColumns;
         static_assert(along_rows ? DstTile::Rows % 2 == 0 : DstTile::Cols % 2 == 0, "packed fp4 tiles hold element pairs");
         for (int idx = threadIdx.x; idx < DstTile::Rows * DstTile::Cols / 2; idx += PTO_AMD_THREADS) {
             int r, c;
@@ -534,9 +569,11 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kpad = min((a.GetValidCol() + 63) / 64 * 64, TileRightT::Rows);
     const uint8_t *pa = a.Storage(), *pb = b.Storage(), *psa = as.Storage(), *psb = bs.Storage();
-    if constexpr (TileRes::BLOCKED && !is_packed4<TA> && !via_fp8 && !gemv) {
-        // fp8 on a wave grid: per k-step (two MX blocks) the wave reads the fragments and scale bytes of its MB row blocks
-        // and NB column blocks once and issues MB * NB scaled MFMAs (as tmatmul does for the plain types)
+    if constexpr (TileRes::BLOCKED && !via_fp8 && !gemv) {
+        // fp8 / fp4 on a wave grid: per k-step (two MX blocks) the wave reads the fragments and scale bytes of its MB row
+        // blocks and NB column blocks once and issues MB * NB scaled MFMAs (as tmatmul does for the plain types).  A k-step
+        // is 64 bytes of a line of fp8 codes -- a lane holds 16 bytes of either block -- and 32 bytes of packed fp4 codes --
+        // a lane holds the 16 bytes that are block lhi.
         constexpr int MB = TileRes::MB, NB = TileRes::NB;
         const int wr = wave / TileRes::grid.wc, wc = wave % TileRes::grid.wc;
         int aline[MB], bline[NB];
@@ -565,14 +602,16 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
                                (a.kb0_ & 31u) == 0 && (b.kb0_ & 31u) == 0;
         const uint32_t a_lane = a.lds_ + a_l0 * a.pitch_ + (((uint32_t)lhi ^ ((a_l0 >> a.sh_) & a.mask_)) << 4);
         const uint32_t b_lane = b.lds_ + b_l0 * b.pitch_ + (((uint32_t)lhi ^ ((b_l0 >> b.sh_) & b.mask_)) << 4);
+        constexpr bool fp4 = is_packed4<TA>;
         auto frag = [&](bool left, int blk, int kbyte) __attribute__((always_inline)) -> uint4 {
-            // kbyte: 0 or 32 past the k-step's first byte, i.e. a literal multiple of 32
+            // kbyte: the k-step's first byte along the line, or 32 past it (fp8): a literal multiple of 32
             if (fast_addr) {
                 const uint32_t lane_c = left ? a_lane : b_lane, pitch = left ? a.pitch_ : b.pitch_, kb0 = left ? a.kb0_ : b.kb0_;
                 return *reinterpret_cast<const uint4*>(arena + ((lane_c ^ (kb0 + (uint32_t)kbyte)) + (uint32_t)blk * 32u * pitch));
             }
-            return left ? *reinterpret_cast<const uint4*>(pa + a.ByteOffset(aline[blk], kbyte + 16 * lhi))
-                        : *reinterpret_cast<const uint4*>(pb + b.ByteOffset(kbyte + 16 * lhi, bline[blk]));
+            const int k_el = fp4 ? 2 * (kbyte + 16 * lhi) : kbyte + 16 * lhi;  // ByteOffset takes element indices
+            return left ? *reinterpret_cast<const uint4*>(pa + a.ByteOffset(aline[blk], k_el))
+                        : *reinterpret_cast<const uint4*>(pb + b.ByteOffset(k_el, bline[blk]));
         };
         auto kstep = [&](int k0) __attribute__((always_inline)) {
             const int g = k0 / 32 + lhi;
@@ -580,14 +619,24 @@ PTO_INST void tmatmul_mx(TileRes& c, TileLeftT& a, TileLeftScaleT& as, TileRight
             int sa[MB], sb[NB];
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
-                const uint4 b0 = frag(false, j, k0), b1 = frag(false, j, k0 + 32);
-                fb[j] = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                if constexpr (fp4) {
+                    const uint4 b0 = frag(false, j, k0 / 2);
+                    fb[j] = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, 0, 0, 0, 0};
+                } else {
+                    const uint4 b0 = frag(false, j, k0), b1 = frag(false, j, k0 + 32);
+                    fb[j] = i32x8v{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                }
                 sb[j] = psb[bs.ByteOffset(g, bline[j])];
             }
 #pragma unroll
             for (int i = 0; i < MB; ++i) {
-                const uint4 a0 = frag(true, i, k0), a1 = frag(true, i, k0 + 32);
-                fa[i] = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                if constexpr (fp4) {
+                    const uint4 a0 = frag(true, i, k0 / 2);
+                    fa[i] = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, 0, 0, 0, 0};
+                } else {
+                    const uint4 a0 = frag(true, i, k0), a1 = frag(true, i, k0 + 32);
+                    fa[i] = i32x8v{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+                }
                 sa[i] = psa[as.ByteOffset(aline[i], g)];
             }
 #pragma unroll

@@ -227,7 +227,8 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
     static constexpr bool is_packed4 = amd::ElemTraits<Element_>::bytes2 == 1;
     // Mat tiles with a box layout are stored as swizzled lines; lines are rows for SLayout::RowMajor boxes, columns for
     // SLayout::ColMajor boxes
-    static constexpr bool MatLines = Loc_ == TileType::Mat && SFractal_ != SLayout::NoneBox && !is_packed4;
+    // (a line of packed fp4 codes keeps the two codes of a byte neighbours along the line)
+    static constexpr bool MatLines = Loc_ == TileType::Mat && SFractal_ != SLayout::NoneBox;
     static constexpr bool OperandLoc = amd::is_operand_loc(Loc_);
     static constexpr bool Lined = MatLines || OperandLoc;
     static constexpr bool LinesAreRows = Loc_ == TileType::Left || Loc_ == TileType::ScaleLeft || (MatLines && SFractal_ == SLayout::RowMajor);
@@ -275,9 +276,11 @@ struct Tile : std::conditional_t<Loc_ == TileType::Acc, amd::AccStorage<Element_
             return (uint32_t)(((int64_t)r * Cols_ + c) * b2 / 2);
         }
     }
-    // which nibble of that byte holds element (r, c) of a packed fp4 tile: pairs run along k for Left / Right tiles,
-    // along a row otherwise
-    PTO_INST static int Nibble(int r, int c) { return Loc_ == TileType::Right ? (r & 1) : (c & 1); }
+    // which nibble of that byte holds element (r, c) of a packed fp4 tile: the two codes of a byte are neighbours along a
+    // line where the tile is stored as lines (down a column for Right tiles and column-lined Mat tiles), along a row
+    // otherwise
+    static constexpr bool PairsDownColumns = Loc_ == TileType::Right || (MatLines && !LinesAreRows);
+    PTO_INST static int Nibble(int r, int c) { return PairsDownColumns ? (r & 1) : (c & 1); }
     // the tile's on-chip address as TASSIGN bound it (what the reference's data() pointer stands for)
     PTO_INST uint64_t data() const
     {

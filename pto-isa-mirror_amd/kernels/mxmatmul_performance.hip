@@ -46,6 +46,8 @@ template <typename OutT, typename InT, int M, int K, int N, int baseM, int baseN
 __global__ AICORE void MxMatmulPerformance(__gm__ OutT* out, __gm__ InT* a, __gm__ InT* b, __gm__ float8_e8m0_t* sa, __gm__ float8_e8m0_t* sb)
 {
     using X = float8_e8m0_t;
+    // (packed fp4: two codes per byte -- extents and strides count codes, pointers and TASSIGN addresses count bytes)
+    constexpr int perByte = (std::is_same_v<InT, float4_e2m1x2_t> || std::is_same_v<InT, float4_e1m2x2_t>) ? 2 : 1;
     constexpr int panels = K / baseK, groups = baseK / 32, chunkGroups = groups * stepKscale, kGroups = K / 32;
     static_assert(M % baseM == 0 && N % baseN == 0 && K % (baseK * stepKscale) == 0, "whole tiles, panels and scale chunks only");
 
@@ -74,7 +76,7 @@ __global__ AICORE void MxMatmulPerformance(__gm__ OutT* out, __gm__ InT* a, __gm
     LeftScaleTile aScale;
     RightScaleTile bScale;
     ResTile cTile;
-    constexpr uint32_t bytesA = baseM * baseK, bytesB = baseK * baseN, bytesSA = baseM * chunkGroups, bytesSB = chunkGroups * baseN;
+    constexpr uint32_t bytesA = baseM * baseK / perByte, bytesB = baseK * baseN / perByte, bytesSA = baseM * chunkGroups, bytesSB = chunkGroups * baseN;
     constexpr uint32_t scales0 = 2 * bytesA + 2 * bytesB;
     TASSIGN(aMat[0], 0x0);
     TASSIGN(aMat[1], bytesA);
@@ -92,8 +94,8 @@ __global__ AICORE void MxMatmulPerformance(__gm__ OutT* out, __gm__ InT* a, __gm
 
     int tm, tn;
     OwnTile<M / baseM, N / baseN, 4>(tm, tn);
-    __gm__ InT* aRows = a + (size_t)tm * baseM * K;
-    __gm__ InT* bCols = b + (size_t)tn * baseN * K;
+    __gm__ InT* aRows = a + (size_t)tm * baseM * K / perByte;
+    __gm__ InT* bCols = b + (size_t)tn * baseN * K / perByte;
     __gm__ X* saRows = sa + (size_t)tm * baseM * kGroups;
     __gm__ X* sbCols = sb + (size_t)tn * baseN * kGroups;
 
@@ -112,8 +114,8 @@ __global__ AICORE void MxMatmulPerformance(__gm__ OutT* out, __gm__ InT* a, __gm
             TEXTRACT(aScale, aScaleMat[scur], 0, q * groups);
             TEXTRACT(bScale, bScaleMat[scur], q * groups, 0);
             if (p + 1 < panels) {
-                GlobalA gmA(aRows + (size_t)(p + 1) * baseK);
-                GlobalB gmB(bCols + (size_t)(p + 1) * baseK);
+                GlobalA gmA(aRows + (size_t)(p + 1) * baseK / perByte);
+                GlobalB gmB(bCols + (size_t)(p + 1) * baseK / perByte);
                 TLOAD(aMat[nxt], gmA);
                 TLOAD(bMat[nxt], gmB);
                 if constexpr (q == stepKscale - 1) {
@@ -155,12 +157,16 @@ __global__ AICORE void MxMatmulPerformance(__gm__ OutT* out, __gm__ InT* a, __gm
 // id 1: the same -> f32
 // id 2: E4M3 512 x 768 x 1024 -> f32 (6 cores; a small case for parity tests)
 // id 3: E5M2 4096^3 -> bf16 (a shape the reference publishes a time for)
+// id 4: MXFP4 E2M1 2048 x 8192 x 8192 -> bf16 (a shape the reference publishes a time for); K panels of 256 codes = 128 bytes
+// id 5: MXFP4 E2M1 512 x 1024 x 768 -> f32 (a small case for parity tests)
 template <typename OutT, typename InT, int M, int K, int N>
 static int run(void* out, void* a, void* b, void* sa, void* sb, void* stream)
 {
     constexpr int cores = (M / 256) * (N / 256);
-    return pto::amd::launch<&MxMatmulPerformance<OutT, InT, M, K, N, 256, 256, 128, 4>>(cores, stream, (OutT*)out, (InT*)a, (InT*)b,
-                                                                                         (float8_e8m0_t*)sa, (float8_e8m0_t*)sb);
+    constexpr bool fp4 = std::is_same_v<InT, float4_e2m1x2_t>;
+    // a panel is 128 bytes of every row either way; a scale tile line is 16 groups: four fp8 panels, two fp4 panels
+    return pto::amd::launch<&MxMatmulPerformance<OutT, InT, M, K, N, 256, 256, fp4 ? 256 : 128, fp4 ? 2 : 4>>(
+        cores, stream, (OutT*)out, (InT*)a, (InT*)b, (float8_e8m0_t*)sa, (float8_e8m0_t*)sb);
 }
 
 extern "C" int pto_mxmatmul_performance(int id, void* out, void* a, void* b, void* sa, void* sb, void* stream)
@@ -170,6 +176,8 @@ extern "C" int pto_mxmatmul_performance(int id, void* out, void* a, void* b, voi
     case 1: return run<float, float8_e4m3_t, 4096, 4096, 14336>(out, a, b, sa, sb, stream);
     case 2: return run<float, float8_e4m3_t, 512, 1024, 768>(out, a, b, sa, sb, stream);
     case 3: return run<bfloat16_t, float8_e5m2_t, 4096, 4096, 4096>(out, a, b, sa, sb, stream);
+    case 4: return run<bfloat16_t, float4_e2m1x2_t, 2048, 8192, 8192>(out, a, b, sa, sb, stream);
+    case 5: return run<float, float4_e2m1x2_t, 512, 1024, 768>(out, a, b, sa, sb, stream);
     default: return -1;
     }
 }

@@ -169,3 +169,41 @@ def test_mxfp8_config3_full_size(pa, oracle, mxperf):
     wa = np.abs(table[ar]) * np.repeat(2.0 ** (sar.astype(np.float64) - 127), 32, 1)
     wb = np.abs(table[bc]) * np.repeat(2.0 ** (sbc.astype(np.float64) - 127), 32, 1)
     check_f32_drain(host(f)[np.ix_(rows, cols)], ref, wa @ wb.T, k, "PTO-style MXFP8 configs[3], samples")
+
+
+def test_mxfp4_512x768x1024_whole_matrix(pa, oracle, mxperf):
+    """Case 5: packed E2M1 codes over all 16 values, scales 2^-8 .. 2^7: the same program with fp4 operand tiles (Mat
+    tiles of packed codes stored as lines along K, loaded by LDS-DMA from an ND A and a DN B; Left / Right windows; the
+    register-blocked TMATMUL_MX with one 16-byte fragment per block and k-step).  Every output against the oracle with the
+    plain fp32 bars, and bit for bit against the C-ABI launcher."""
+    m, n, k = 512, 768, 1024
+    r = np.random.default_rng(321)
+    a = r.integers(0, 256, (m, k // 2)).astype(np.uint8)
+    b = r.integers(0, 256, (n, k // 2)).astype(np.uint8)
+    sa = r.integers(119, 135, (m, k // 32)).astype(np.uint8)
+    sb = r.integers(119, 135, (n, k // 32)).astype(np.uint8)
+    d = [torch.from_numpy(x).to(DEV) for x in (a, b, sa, sb)]
+    out = mxperf(5, torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV), *d)
+    got = host(out)
+    ref = oracle.matmul_mx(a, b, sa, sb, m, k, n, ob.E2M1, ob.E2M1)
+    table = oracle.mx_decode_table(ob.E2M1)
+    unpack = lambda x: np.stack([table[x & 0xF], table[x >> 4]], -1).reshape(x.shape[0], -1)
+    wa = np.abs(unpack(a)) * np.repeat(2.0 ** (sa.astype(np.float64) - 127), 32, 1)
+    wb = np.abs(unpack(b)) * np.repeat(2.0 ** (sb.astype(np.float64) - 127), 32, 1)
+    check_f32_drain(got, ref, wa @ wb.T, k, "PTO-style MXFP4 512x768x1024")
+    launcher = pa.gemm_mx(d[0], d[1], d[2], d[3], m, n, k, pa.E2M1, pa.E2M1, pa.F32)
+    assert torch.equal(out, launcher)
+
+
+def test_mxfp4_2048x8192x8192_against_the_launcher(pa, mxperf):
+    """Case 4: MXFP4 2048 x 8192 (K) x 8192, operands quantised from N(0,1) by TQUANT<MXFP4> -> bf16: every output written
+    and equal to the launcher's (held to the oracle in test_gpu_parity)."""
+    m, n, k = 2048, 8192, 8192
+    gen = torch.Generator(device=DEV).manual_seed(44)
+    a, sa = pa.tquant_mx(torch.randn((m, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
+    b, sb = pa.tquant_mx(torch.randn((n, k), generator=gen, device=DEV), pa.OCP_MXFP4, want_aux=False)
+    out = mxperf(4, torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV), a, b, sa, sb)
+    assert not bool(torch.isnan(out).any())
+    launcher = pa.gemm_mx(a, b, sa, sb, m, n, k, pa.E2M1, pa.E2M1, pa.BF16)
+    assert torch.equal(out, launcher)
+

@@ -31,3 +31,36 @@ def test_reference_kernel_source_compiles_against_the_header_layer(source):
            "-I" + os.path.join(ROOT, "pto-isa-mirror_amd", "include"), path]
     res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stderr[-4000:]
+
+
+# The reference's hand-tuned kernels for this path are written in the same tile ISA.  Their core programs -- everything
+# but one statement -- are checked the same way.  The statement is the CANN launch configuration
+# `<<<blockDim, nullptr, stream>>>` (block count, an L2 control pointer, a stream), which is not HIP's
+# `<<<grid, block, shared bytes, stream>>>`: it is taken out of a temporary copy (the kernel is then named as an ordinary
+# function call, which instantiates the whole core program for the shape the file launches), nothing else is touched and
+# the copy lives in pytest's temporary directory only.
+MANUAL = "/root/reference/kernels/manual"
+MANUAL_SOURCES = ["a2a3/gemm_performance/gemm_performance_kernel.cpp", "a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp",
+                  "a5/matmul_mxfp4_performance/mxmatmul_performance_kernel.cpp"]
+CANN_LAUNCH = "<<<blockDim, nullptr, stream>>>"
+
+
+@pytest.mark.parametrize("source", MANUAL_SOURCES)
+def test_reference_performance_kernel_core_program_compiles_against_the_header_layer(source, tmp_path):
+    path = os.path.join(MANUAL, source)
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(path):
+        pytest.skip("reference tree not mounted")
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not installed")
+    text = open(path).read()
+    assert text.count(CANN_LAUNCH) == 1, "the file's one launch statement"
+    copy = tmp_path / os.path.basename(source)
+    copy.write_text(text.replace(CANN_LAUNCH, ""))
+    cmd = [hipcc, "-std=c++17", "-O1", "--offload-arch=gfx950", "-x", "hip", "--cuda-device-only", "-fsyntax-only",
+           "-DPTO_AMD_CHECK_REFERENCE_SOURCE", "-DPTO_AMD_L1_BYTES=524288", "-DPTO_AMD_L0A_BYTES=65536",
+           "-DPTO_AMD_L0B_BYTES=65536", "-DPTO_AMD_UB_BYTES=262144", "-DPTO_AMD_L0S_BYTES=16384",
+           "-I" + os.path.join(ROOT, "pto-isa-mirror_amd", "include"), str(copy)]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-4000:]
+
