@@ -520,6 +520,55 @@ __global__ AICORE void RunQUANT_TMATMUL_MX(__gm__ float* out, __gm__ float* src0
     TSTORE(outGlobal, cTile);
 }
 
+// Packed fp4 operands from either global layout, through the element-wise TLOAD (the tiles are not fully valid, so the
+// LDS-DMA form does not apply): A as ND (codes paired along a row, as the row-lined Mat tile pairs them) or DN (paired
+// down a column: every tile byte is built from two bytes of memory); B as DN (paired down a column, as the column-lined
+// Mat tile pairs them) or ND.  The Left / Right tiles are copies (zero-filled past the valid region).
+template <bool A_DN, bool B_DN, int validM, int validK, int validN>
+__global__ AICORE void RunTMATMULMX_FP4_LAYOUTS(__gm__ float* out, __gm__ float4_e2m1x2_t* src0, __gm__ float4_e2m1x2_t* src1,
+                                                __gm__ float8_e8m0_t* src2, __gm__ float8_e8m0_t* src3)
+{
+    using F4 = float4_e2m1x2_t;
+    using X = float8_e8m0_t;
+    constexpr int M = CeilAlign<int>(validM, 32), N = CeilAlign<int>(validN, 32), K = CeilAlign<int>(validK, 64), kMX = K / 32;
+    constexpr Layout LA = A_DN ? Layout::DN : Layout::ND, LB = B_DN ? Layout::DN : Layout::ND;
+    GlobalTensor<F4, TileShape2D<F4, validM, validK, LA>, BaseShape2D<F4, validM, validK, LA>, LA> aGlobal(src0);
+    GlobalTensor<F4, TileShape2D<F4, validK, validN, LB>, BaseShape2D<F4, validK, validN, LB>, LB> bGlobal(src1);
+    GlobalTensor<X, TileShape2D<X, validM, validK / 32, Layout::MX_A_ND>, BaseShape2D<X, validM, validK / 32, Layout::MX_A_ND>, Layout::MX_A_ND>
+        saGlobal(src2);
+    GlobalTensor<X, TileShape2D<X, validK / 32, validN, Layout::MX_B_DN>, BaseShape2D<X, validK / 32, validN, Layout::MX_B_DN>, Layout::MX_B_DN>
+        sbGlobal(src3);
+    GlobalTensor<float, TileShape2D<float, validM, validN>, BaseShape2D<float, validM, validN>> outGlobal(out);
+    Tile<TileType::Mat, F4, M, K, BLayout::ColMajor, validM, validK, SLayout::RowMajor> aMat;
+    Tile<TileType::Mat, F4, K, N, BLayout::RowMajor, validK, validN, SLayout::ColMajor> bMat;
+    Tile<TileType::Mat, X, M, kMX, BLayout::RowMajor, validM, validK / 32, SLayout::RowMajor, 32> saMat;
+    Tile<TileType::Mat, X, kMX, N, BLayout::ColMajor, validK / 32, validN, SLayout::ColMajor, 32> sbMat;
+    TASSIGN(aMat, 0x0);
+    TASSIGN(bMat, M * K / 2);
+    TASSIGN(saMat, M * K / 2 + K * N / 2);
+    TASSIGN(sbMat, M * K / 2 + K * N / 2 + M * kMX);
+    TileLeft<F4, M, K, validM, validK> aTile;
+    TileRight<F4, K, N, validK, validN> bTile;
+    TileLeftScale<X, M, kMX, validM, validK / 32> saTile;
+    TileRightScale<X, kMX, N, validK / 32, validN> sbTile;
+    TileAcc<float, M, N, validM, validN> cTile;
+    TASSIGN(aTile, 0x0);
+    TASSIGN(bTile, 0x0);
+    TASSIGN(cTile, 0x0);
+    TASSIGN(saTile, 0x0);
+    TASSIGN(sbTile, 0x0);
+    TLOAD(aMat, aGlobal);
+    TLOAD(bMat, bGlobal);
+    TLOAD(saMat, saGlobal);
+    TLOAD(sbMat, sbGlobal);
+    TMOV(aTile, aMat);
+    TMOV(bTile, bMat);
+    TMOV(saTile, saMat);
+    TMOV(sbTile, sbMat);
+    TMATMUL_MX(cTile, aTile, saTile, bTile, sbTile);
+    TSTORE(outGlobal, cTile);
+}
+
 extern "C" int pto_boundary_launch_mx(int id, void* out, void* a, void* b, void* sa, void* sb, void* bias, void* stream)
 {
     using S = float8_e8m0_t;
@@ -536,6 +585,11 @@ extern "C" int pto_boundary_launch_mx(int id, void* out, void* a, void* b, void*
     case 11: return run<&RunTGEMVMX<F12, F12, 128, 62, Layout::MX_B_ND, true>>(stream, 1, (float*)out, (F12*)a, (F12*)b, (S*)sa, (S*)sb);
     case 12: return run<&RunTGEMVMX<E4, E5, 256, 20, Layout::MX_B_ND, false>>(stream, 1, (float*)out, (E4*)a, (E5*)b, (S*)sa, (S*)sb);
     case 21: return run<&RunTGEMVMX<F21, F21, 192, 40, Layout::MX_B_DN, true>>(stream, 1, (float*)out, (F21*)a, (F21*)b, (S*)sa, (S*)sb);
+    // 30-33: fp4 operands from ND / DN global tensors (30 + (A is DN) + 2 (B is DN)), 30 x 128 x 60 valid
+    case 30: return run<&RunTMATMULMX_FP4_LAYOUTS<false, false, 30, 128, 60>>(stream, 1, (float*)out, (F21*)a, (F21*)b, (S*)sa, (S*)sb);
+    case 31: return run<&RunTMATMULMX_FP4_LAYOUTS<true, false, 30, 128, 60>>(stream, 1, (float*)out, (F21*)a, (F21*)b, (S*)sa, (S*)sb);
+    case 32: return run<&RunTMATMULMX_FP4_LAYOUTS<false, true, 30, 128, 60>>(stream, 1, (float*)out, (F21*)a, (F21*)b, (S*)sa, (S*)sb);
+    case 33: return run<&RunTMATMULMX_FP4_LAYOUTS<true, true, 30, 128, 60>>(stream, 1, (float*)out, (F21*)a, (F21*)b, (S*)sa, (S*)sb);
     default: return -1;
     }
 }

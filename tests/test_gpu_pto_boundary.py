@@ -225,6 +225,33 @@ def test_tgemv_mx(lib, oracle, case, dist):
         assert_sum_close(got, ref, absdot, k, f"gemv mx case {case}", **_mx_bound(ta))
 
 
+@pytest.mark.parametrize("dist", ["ints", "codes"])
+@pytest.mark.parametrize("case", [30, 31, 32, 33])
+def test_fp4_operands_from_nd_and_dn_global_tensors(lib, oracle, case, dist):
+    """Packed fp4 codes pair along the unit-stride direction of the global tensor (a row of ND, a column of DN), and in
+    a boxed Mat tile along its lines (rows on the A side, columns on the B side).  All four combinations through the
+    element-wise TLOAD (tiles with a ragged valid region): bytes move where the directions agree, and are built from two
+    source nibbles where they do not.  Case 30 + (A is DN) + 2 (B is DN)."""
+    m, k, n = 30, 128, 60
+    r = np.random.default_rng(3000 + case)
+    a, b, sa, sb, ref, exact, absdot, kg = _mx_problem(oracle, r, ob.E2M1, ob.E2M1, m, k, n, dist)
+    a_dn, b_dn = (case - 30) & 1, (case - 30) & 2
+    a_gm = _pack(np.ascontiguousarray(a.T), ob.E2M1) if a_dn else _pack(a, ob.E2M1)
+    b_gm = _pack(np.ascontiguousarray(b.T), ob.E2M1) if b_dn else _pack(b, ob.E2M1)
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
+    d = [dev(x) for x in (a_gm, b_gm, sa.reshape(-1), np.ascontiguousarray(sb.T).reshape(-1))]
+    rc = lib.pto_boundary_launch_mx(case, ptr(out), ptr(d[0]), ptr(d[1]), ptr(d[2]), ptr(d[3]), None, stream())
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert lib.pto_boundary_status() == 0
+    got = out.cpu().numpy()
+    if dist == "ints":
+        assert np.array_equal(got, exact.astype(np.float32))
+        assert np.array_equal(got, ref)
+    else:
+        assert_sum_close(got, ref, absdot, k, f"fp4 layouts case {case}", **_mx_bound(ob.E2M1))
+
+
 # ------------------------------------------------------------------------------------------------------- TCVT
 R, C, V = 16, 72, 70
 RINT, ROUND, FLOOR, CEIL, TRUNC, ODD = 1, 2, 3, 4, 5, 6
